@@ -1,0 +1,195 @@
+"""TEST INFRASTRUCTURE — numpy/ctypes access to the parity checkers.  Never imported by the product package.
+
+``sdpa_f32`` and friends call ``oracle/libsdpa_oracle.so`` (this repository's C restatement of TinyTorch's fp32 CPU
+attention, reference src/Function/FuncNNLayer.h:231-266).  ``ref_*`` call ``oracle/_ref/libtt_ref.so``, the real
+TinyTorch CPU library compiled by ``oracle/Makefile``, when that file is present.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+ORACLE_SO = os.path.join(_HERE, "libsdpa_oracle.so")
+REF_SO = os.path.join(_HERE, "_ref", "libtt_ref.so")
+
+F32, F16, BF16 = 0, 1, 2
+MASK_NONE, MASK_BOOL, MASK_FLOAT = 0, 1, 2
+_DTYPES = {"f32": F32, "fp32": F32, "f16": F16, "fp16": F16, "bf16": BF16}
+
+_c_f32p = ctypes.POINTER(ctypes.c_float)
+_c_u16p = ctypes.POINTER(ctypes.c_uint16)
+_c_i64p = ctypes.POINTER(ctypes.c_int64)
+_i64 = ctypes.c_int64
+
+
+def build(ref=True):
+    """Compile the C restatement (always) and, where the reference tree is mounted, oracle/_ref."""
+    subprocess.run(["make", "-C", _HERE, "oracle"], check=True)
+    if ref and os.path.isdir("/root/reference/src"):
+        subprocess.run(["make", "-C", _HERE, "ref", "-j8"], check=True)
+
+
+_lib = None
+_ref = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(ORACLE_SO):
+            build(ref=False)
+        L = ctypes.CDLL(ORACLE_SO)
+        L.oracle_round_array.argtypes = [_c_f32p, _c_f32p, _c_u16p, _i64, ctypes.c_int]
+        L.oracle_round_array.restype = None
+        L.oracle_bits_to_f32_array.argtypes = [_c_u16p, _c_f32p, _i64, ctypes.c_int]
+        L.oracle_bits_to_f32_array.restype = None
+        L.oracle_randn.argtypes = [ctypes.c_uint64, ctypes.c_uint64, _i64, ctypes.c_float, _c_f32p, ctypes.c_int]
+        L.oracle_randn.restype = None
+        L.oracle_sdpa_f32.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p] + [_i64] * 6 + [
+            ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_int]
+        L.oracle_sdpa_f32.restype = ctypes.c_int
+        L.oracle_sdpa_rows_f32.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p] + [_i64] * 6 + [
+            ctypes.c_int, ctypes.c_float, _c_i64p, _i64, ctypes.c_int]
+        L.oracle_sdpa_rows_f32.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def have_ref():
+    return os.path.exists(REF_SO)
+
+
+def ref():
+    global _ref
+    if _ref is None:
+        R = ctypes.CDLL(REF_SO)
+        R.tt_ref_round_trip.argtypes = [_c_f32p, _c_f32p, _i64, ctypes.c_int]
+        R.tt_ref_round_trip.restype = ctypes.c_int
+        R.tt_ref_sdpa_f32.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p] + [_i64] * 6 + [
+            ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_void_p]
+        R.tt_ref_sdpa_f32.restype = ctypes.c_int
+        R.tt_ref_sdpa_f32_gqa5d.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p] + [_i64] * 6 + [ctypes.c_int]
+        R.tt_ref_sdpa_f32_gqa5d.restype = ctypes.c_int
+        _ref = R
+    return _ref
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _p(a):
+    return a.ctypes.data_as(_c_f32p)
+
+
+def default_threads():
+    return max(1, min(16, os.cpu_count() or 1))
+
+
+def randn(seed, stream, shape, mul=1.0, nthreads=None):
+    """i.i.d. N(0,1)*mul as float32; element i depends only on (seed, stream, i)."""
+    n = int(np.prod(shape, dtype=np.int64))
+    out = np.empty(n, dtype=np.float32)
+    lib().oracle_randn(seed, stream, n, mul, _p(out), nthreads or default_threads())
+    return out.reshape(shape)
+
+
+def round_to(x, dtype):
+    """Round fp32 -> dtype (RNE) -> (fp32 values of the rounded numbers, uint16 bit patterns or None)."""
+    d = _DTYPES[dtype] if isinstance(dtype, str) else dtype
+    x = _f32(x)
+    if d == F32:
+        return x.copy(), None
+    vals = np.empty_like(x)
+    bits = np.empty(x.shape, dtype=np.uint16)
+    lib().oracle_round_array(_p(x), _p(vals), bits.ctypes.data_as(_c_u16p), x.size, d)
+    return vals, bits
+
+
+def bits_to_f32(bits, dtype):
+    d = _DTYPES[dtype] if isinstance(dtype, str) else dtype
+    bits = np.ascontiguousarray(bits, dtype=np.uint16)
+    out = np.empty(bits.shape, dtype=np.float32)
+    lib().oracle_bits_to_f32_array(bits.ctypes.data_as(_c_u16p), _p(out), bits.size, d)
+    return out
+
+
+def _dims(q, k, v):
+    B, Hq, L, D = q.shape
+    Bk, Hkv, S, Dk = k.shape
+    assert v.shape == k.shape and Bk == B and Dk == D and Hq % Hkv == 0
+    return B, Hq, Hkv, L, S, D
+
+
+def _mask_args(mask, L, S):
+    if mask is None:
+        return MASK_NONE, None, None
+    if mask.dtype == np.bool_ or mask.dtype == np.uint8:
+        m = np.ascontiguousarray(mask, dtype=np.uint8)
+        kind = MASK_BOOL
+    else:
+        m = _f32(mask)
+        kind = MASK_FLOAT
+    assert m.shape == (L, S)
+    return kind, m, ctypes.c_void_p(m.ctypes.data)
+
+
+def sdpa_f32(q, k, v, causal=False, scale=None, mask=None, nthreads=None):
+    """The restated reference CPU path: q [B,Hq,L,D], k/v [B,Hkv,S,D] float32 -> [B,Hq,L,D] float32."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    B, Hq, Hkv, L, S, D = _dims(q, k, v)
+    sc = np.float32(1.0) / np.sqrt(np.float32(D)) if scale is None else np.float32(scale)
+    kind, keep, mp = _mask_args(mask, L, S)
+    out = np.empty(q.shape, dtype=np.float32)
+    rc = lib().oracle_sdpa_f32(_p(q), _p(k), _p(v), _p(out), B, Hq, Hkv, L, S, D, int(bool(causal)), float(sc), kind,
+                               mp, nthreads or default_threads())
+    if rc != 0:
+        raise RuntimeError("oracle_sdpa_f32 failed: %d" % rc)
+    return out
+
+
+def sdpa_rows_f32(q, k, v, rows, causal=False, scale=None, nthreads=None):
+    """Restated path for selected (b, h, l) triples only -> [len(rows), D]."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    B, Hq, Hkv, L, S, D = _dims(q, k, v)
+    sc = np.float32(1.0) / np.sqrt(np.float32(D)) if scale is None else np.float32(scale)
+    rows = np.ascontiguousarray(rows, dtype=np.int64).reshape(-1, 3)
+    out = np.empty((rows.shape[0], D), dtype=np.float32)
+    rc = lib().oracle_sdpa_rows_f32(_p(q), _p(k), _p(v), _p(out), B, Hq, Hkv, L, S, D, int(bool(causal)), float(sc),
+                                    rows.ctypes.data_as(_c_i64p), rows.shape[0], nthreads or default_threads())
+    if rc != 0:
+        raise RuntimeError("oracle_sdpa_rows_f32 failed: %d" % rc)
+    return out
+
+
+def ref_sdpa_f32(q, k, v, causal=False, scale=None, mask=None):
+    """tinytorch::function::sdpAttention of the compiled reference (single-threaded, fp32 CPU)."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    B, Hq, Hkv, L, S, D = _dims(q, k, v)
+    kind, keep, mp = _mask_args(mask, L, S)
+    out = np.empty(q.shape, dtype=np.float32)
+    rc = ref().tt_ref_sdpa_f32(_p(q), _p(k), _p(v), _p(out), B, Hq, Hkv, L, S, D, int(bool(causal)),
+                               0 if scale is None else 1, 0.0 if scale is None else float(scale), kind, mp)
+    if rc != 0:
+        raise RuntimeError("tt_ref_sdpa_f32 failed: %d" % rc)
+    return out
+
+
+def ref_sdpa_f32_gqa5d(q, k, v, causal=False):
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    B, Hq, Hkv, L, S, D = _dims(q, k, v)
+    out = np.empty(q.shape, dtype=np.float32)
+    rc = ref().tt_ref_sdpa_f32_gqa5d(_p(q), _p(k), _p(v), _p(out), B, Hq, Hkv, L, S, D, int(bool(causal)))
+    if rc != 0:
+        raise RuntimeError("tt_ref_sdpa_f32_gqa5d failed: %d" % rc)
+    return out
+
+
+def ref_round_trip(x, dtype):
+    d = _DTYPES[dtype] if isinstance(dtype, str) else dtype
+    x = _f32(x).reshape(-1)
+    out = np.empty_like(x)
+    ref().tt_ref_round_trip(_p(x), _p(out), x.size, d)
+    return out

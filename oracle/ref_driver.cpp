@@ -1,0 +1,108 @@
+// TEST INFRASTRUCTURE — not part of the product.
+//
+// C-ABI shim over the *real* TinyTorch CPU library (compiled by oracle/Makefile from the sources where they lie
+// under /root/reference; nothing of the reference is copied into this repository).  It calls
+// tinytorch::function::sdpAttention (reference src/Function/FuncNNLayer.h:298-302) on CPU fp32 tensors and hands
+// the result back through plain pointers, so the tests can pin oracle/sdpa_oracle.c against the reference itself
+// and write the golden fixtures under tests/golden/.
+//
+// Built only where /root/reference exists; the resulting oracle/_ref/libtt_ref.so travels to the GPU box.
+
+#include <cstdint>
+#include <cstring>
+#include <limits>
+#include <vector>
+
+#include "TinyTorch.h"
+
+using namespace tinytorch;
+
+namespace {
+
+Tensor fromF32(const float* p, const std::vector<int64_t>& shape) {
+  int64_t n = 1;
+  for (auto s : shape) n *= s;
+  std::vector<float> buf(p, p + n);
+  Tensor t(buf);
+  t.reshape_(IntArrayView(shape));
+  return t;
+}
+
+void ensureCpu() {
+  static bool done = false;
+  if (!done) {
+    setDefaultDevice(DeviceType::CPU);
+    done = true;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+// Round-trip fp32 -> {1: Float16, 2: BFloat16} -> fp32 through the reference's own dtype cast
+// (Tensor::to, reference src/Tensor/Tensor.cpp:224-233; Half.h:226-257; BFloat16.h:72-85).
+int tt_ref_round_trip(const float* in, float* out, int64_t n, int dtype) {
+  ensureCpu();
+  Tensor t = fromF32(in, {n});
+  Tensor r = t.to(dtype == 1 ? DType::Float16 : DType::BFloat16).to(DType::Float32);
+  auto v = r.toList<float>();
+  std::memcpy(out, v.data(), sizeof(float) * n);
+  return 0;
+}
+
+// function::sdpAttention on fp32 CPU tensors.
+//   q [B,Hq,L,D]; k,v [B,Hkv,S,D]; out [B,Hq,L,D].
+//   Hkv != Hq: grouped-query attention through op::repeatInterleave(k, Hq/Hkv, 1)
+//   (reference src/Operation/OpTransformCpu.h:399-442), i.e. kv_head = q_head / (Hq/Hkv).
+//   mask_kind: 0 none, 1 Bool [mask_rows,S] (uint8 0/1), 2 additive float [mask_rows,S]; mask_rows is L.
+//   has_scale == 0 -> default 1/sqrt(D).
+int tt_ref_sdpa_f32(const float* q, const float* k, const float* v, float* out, int64_t B, int64_t Hq, int64_t Hkv,
+                    int64_t L, int64_t S, int64_t D, int causal, int has_scale, float scale, int mask_kind,
+                    const void* mask) {
+  ensureCpu();
+  NoGradGuard guard;
+  Tensor tq = fromF32(q, {B, Hq, L, D});
+  Tensor tk = fromF32(k, {B, Hkv, S, D});
+  Tensor tv = fromF32(v, {B, Hkv, S, D});
+  if (Hkv != Hq) {
+    if (Hq % Hkv != 0) return -1;
+    tk = op::repeatInterleave(tk, Hq / Hkv, 1);
+    tv = op::repeatInterleave(tv, Hq / Hkv, 1);
+  }
+  Tensor tm;
+  if (mask_kind == 1) {
+    const auto* m = static_cast<const uint8_t*>(mask);
+    std::vector<uint8_t> buf(m, m + L * S);
+    tm = Tensor(buf, options::dtype(DType::Bool));
+    tm.reshape_({L, S});
+  } else if (mask_kind == 2) {
+    tm = fromF32(static_cast<const float*>(mask), {L, S});
+  }
+  std::optional<float> sc = has_scale ? std::optional<float>(scale) : std::nullopt;
+  Tensor y = function::sdpAttention(tq, tk, tv, causal != 0, tm, 0.f, sc);
+  auto r = y.toList<float>();
+  if (static_cast<int64_t>(r.size()) != B * Hq * L * D) return -2;
+  std::memcpy(out, r.data(), sizeof(float) * r.size());
+  return 0;
+}
+
+// Same call through the matmul batch-broadcast form of GQA (5-D q [B,Hkv,G,L,D] x kv [B,Hkv,1,S,D],
+// reference src/Operation/OpLinalg.cpp:205-223) — used to check that both GQA spellings agree.
+int tt_ref_sdpa_f32_gqa5d(const float* q, const float* k, const float* v, float* out, int64_t B, int64_t Hq,
+                          int64_t Hkv, int64_t L, int64_t S, int64_t D, int causal) {
+  ensureCpu();
+  NoGradGuard guard;
+  if (Hq % Hkv != 0) return -1;
+  int64_t G = Hq / Hkv;
+  Tensor tq = fromF32(q, {B, Hkv, G, L, D});
+  Tensor tk = fromF32(k, {B, Hkv, 1, S, D});
+  Tensor tv = fromF32(v, {B, Hkv, 1, S, D});
+  Tensor y = function::sdpAttention(tq, tk, tv, causal != 0);
+  auto r = y.toList<float>();
+  if (static_cast<int64_t>(r.size()) != B * Hq * L * D) return -2;
+  std::memcpy(out, r.data(), sizeof(float) * r.size());
+  return 0;
+}
+
+}  // extern "C"

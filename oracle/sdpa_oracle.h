@@ -1,0 +1,62 @@
+/* TEST INFRASTRUCTURE — the parity checker, never the product.
+ *
+ * CPU restatement of TinyTorch's scaled-dot-product attention as its CPU path computes it in fp32
+ * (reference src/Function/FuncNNLayer.h:231-266 and the CPU ops it calls).  Only tests/, the smoke check and the
+ * cpu_baseline leg of bench.py may load this library; the shipped library (include/ttsdpa.h) never does.
+ *
+ * Pinning status (tests/test_oracle.py):
+ *   oracle_sdpa_f32            pinned: reference KATs (test/test_function.cpp:393-419), bit-exact against the compiled
+ *                              reference (oracle/_ref) and against fixtures written from it, fp64 closed form,
+ *                              invariants (causal row 0 == v[0], rows of P sum to 1, uniform-K running mean).
+ *   oracle_round_bf16 / _f16   pinned: bit-exact against the reference's own casts over a sweep that includes
+ *                              ties, subnormals, overflow, inf and NaN; and against numpy float16 casts.
+ *   oracle_randn               not a reference function (the harness's own PRNG); pinned by moments and by a
+ *                              pure-numpy restatement of the same counter-based construction.
+ */
+#ifndef SDPA_ORACLE_H
+#define SDPA_ORACLE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { ORACLE_MASK_NONE = 0, ORACLE_MASK_BOOL = 1, ORACLE_MASK_FLOAT = 2 };
+enum { ORACLE_F32 = 0, ORACLE_F16 = 1, ORACLE_BF16 = 2 }; /* same numbering as the reference DType enum */
+
+/* fp32 -> 16-bit pattern, round-to-nearest-even. */
+uint16_t oracle_f32_to_bf16_bits(float x);
+uint16_t oracle_f32_to_f16_bits(float x);
+float oracle_bf16_bits_to_f32(uint16_t b);
+float oracle_f16_bits_to_f32(uint16_t b);
+/* Array forms: round `in` to dtype (ORACLE_F16/ORACLE_BF16; ORACLE_F32 copies); writes the fp32 value of the rounded
+ * number to out_f32 (may be NULL) and the bit pattern to out_bits (may be NULL). */
+void oracle_round_array(const float* in, float* out_f32, uint16_t* out_bits, int64_t n, int dtype);
+void oracle_bits_to_f32_array(const uint16_t* in, float* out, int64_t n, int dtype);
+
+/* Counter-based N(0,1) generator: element i of (seed, stream) never depends on n or on the thread count.
+ * out[i] = (float)(mul * z_i). */
+void oracle_randn(uint64_t seed, uint64_t stream, int64_t n, float mul, float* out, int nthreads);
+
+/* The reference CPU path, fp32, for q [B,Hq,L,D], k/v [B,Hkv,S,D] (all dense row-major) -> out [B,Hq,L,D].
+ * kv head of query head h is h / (Hq/Hkv) (what op::repeatInterleave(k, Hq/Hkv, 1) feeds the reference).
+ * causal: top-left aligned lower triangle, key j visible to query i iff j <= i (tril(ones(L,S), 0)).
+ * mask: NULL, or [L,S] uint8 (ORACLE_MASK_BOOL: 0 = hidden) or [L,S] float (ORACLE_MASK_FLOAT: added to the scores).
+ * nthreads > 1 spreads (batch, head) slices over threads; every slice is computed by the same sequential code, so
+ * the result does not depend on nthreads.  Returns 0, or -1 on bad arguments / out of memory. */
+int oracle_sdpa_f32(const float* q, const float* k, const float* v, float* out, int64_t B, int64_t Hq, int64_t Hkv,
+                    int64_t L, int64_t S, int64_t D, int causal, float scale, int mask_kind, const void* mask,
+                    int nthreads);
+
+/* Same arithmetic for a subset of the (batch, head, query-row) triples: rows[3*i..3*i+2] = (b, h, l);
+ * out is [nrows, D].  A row's result does not depend on the other rows, so this equals the matching rows of
+ * oracle_sdpa_f32 bit for bit. */
+int oracle_sdpa_rows_f32(const float* q, const float* k, const float* v, float* out, int64_t B, int64_t Hq,
+                         int64_t Hkv, int64_t L, int64_t S, int64_t D, int causal, float scale, const int64_t* rows,
+                         int64_t nrows, int nthreads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
