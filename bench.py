@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3] [--no-secondary] [--no-cpu]
+
+A step is one call of the hot path (ttsdpa_forward through the C ABI) over one batch of synthetic input already
+resident in HBM.  The headline workload is BASELINE.json's configs[2] (bf16 causal GQA prefill, B2 32q/8kv S4096
+D128: the shape the prefill target is quoted on); the decode workload configs[3] (bf16, B64 32q/8kv KV 8192) is
+measured in the same run and reported under "secondary".  One JSON line is printed.
+
+Algorithmic work per launch (what "achieved" divides by the measured launch time):
+  prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)
+  prefill, full:    4 * B * Hq * L * S * D flop
+  decode:           2 * B*Hkv*S*D*2 bytes (K and V once) + 2 * B*Hq*D*2 bytes (q in, out)
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}  # MI355X dense MFMA peaks
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (B, Hq, Hkv, L, S, D, dtype, causal, input multiplier, bound)
+    "config1": (1, 4, 4, 128, 128, 64, "f32", True, 1.0, "mfma"),
+    "config2": (4, 32, 32, 2048, 2048, 128, "f16", True, 0.5, "mfma"),
+    "config3": (2, 32, 8, 4096, 4096, 128, "bf16", True, 1.0, "mfma"),
+    "config4": (64, 32, 8, 1, 8192, 128, "bf16", False, 1.0, "hbm"),
+    "config5": (1, 28, 4, 16384, 16384, 128, "bf16", True, 1.0, "mfma"),
+}
+DESCR = {
+    "config1": "fp32 causal SDPA B1 H4 S128 D64",
+    "config2": "fp16 causal MHA prefill B4 H32 S2048 D128",
+    "config3": "bf16 causal GQA prefill B2 32q/8kv S4096 D128",
+    "config4": "bf16 decode B64 32q/8kv L1 KV8192 D128 (isCausal=false)",
+    "config5": "bf16 causal GQA prefill B1 28q/4kv S16384 D128",
+}
+
+
+def algorithmic_work(B, Hq, Hkv, L, S, D, dtype, causal):
+    esz = 4 if dtype == "f32" else 2
+    if causal:
+        vis = sum(min(i + 1, S) for i in range(L)) if L != S else S * (S + 1) // 2
+        flops = 4 * B * Hq * D * vis
+    else:
+        flops = 4 * B * Hq * L * S * D
+    nbytes = 2 * B * Hkv * S * D * esz + 2 * B * Hq * L * D * esz
+    return flops, nbytes
+
+
+def run_gpu(name, steps, warmup):
+    import torch
+    from tinytorch_amd import _capi, build_params
+
+    B, Hq, Hkv, L, S, D, dtype, causal, mul, bound = WORKLOADS[name]
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    gen = torch.Generator(device="cuda").manual_seed(0x5EED)
+    q = (torch.randn(B, Hq, L, D, device="cuda", generator=gen) * mul).to(td)
+    k = (torch.randn(B, Hkv, S, D, device="cuda", generator=gen) * mul).to(td)
+    v = (torch.randn(B, Hkv, S, D, device="cuda", generator=gen) * mul).to(td)
+    out = torch.empty_like(q)
+    p = build_params(q, k, v, out, causal)
+    lib = _capi.lib()
+    rc, route = _capi.plan(p)
+    assert rc == 0, _capi.status_string(rc)
+    nbytes = lib.ttsdpa_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream()
+
+    def step():
+        rc = lib.ttsdpa_forward(ctypes.byref(p), ws.data_ptr(), nbytes, stream.cuda_stream)
+        if rc != 0:
+            raise RuntimeError("ttsdpa_forward: %s" % _capi.status_string(rc))
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    dev_ms = e0.elapsed_time(e1) / steps  # HIP events on the launch stream: average duration per launch
+
+    flops, abytes = algorithmic_work(B, Hq, Hkv, L, S, D, dtype, causal)
+    if bound == "mfma":
+        achieved, peak, unit = flops / (dev_ms * 1e-3) / 1e12, PEAK_TFLOPS[dtype], "TFLOP/s"
+        value = flops / (wall_ms * 1e-3) / 1e12
+    else:
+        achieved, peak, unit = abytes / (dev_ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+        value = abytes / (wall_ms * 1e-3) / 1e9
+    res = {
+        "workload": name, "description": DESCR[name], "route": _capi.ROUTE_NAMES[route], "dtype": dtype,
+        "value": round(value, 3), "unit": unit, "ms_per_step": round(wall_ms, 5),
+        "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel_ms": round(dev_ms, 5), "algorithmic_flops": flops, "algorithmic_bytes": abytes},
+    }
+    return res, (q, k, v, out)
+
+
+def run_cpu_baseline(name, tensors, budget_s=20.0):
+    """The reference CPU path (compiled reference if oracle/_ref is present, else this repository's C restatement)
+    on one host core, over as many (batch, head) slices of the same inputs as fit the time budget."""
+    import numpy as np
+    import oracle
+
+    B, Hq, Hkv, L, S, D, dtype, causal, mul, bound = WORKLOADS[name]
+    q, k, v, out = tensors
+    kind = "reference" if oracle.have_ref() else "port"
+    fn = oracle.ref_sdpa_f32 if kind == "reference" else (lambda *a, **kw: oracle.sdpa_f32(*a, nthreads=1, **kw))
+    G = Hq // Hkv
+    flops_slice, _ = algorithmic_work(1, 1, 1, L, S, D, dtype, causal)
+    done, spent, worst = 0, 0.0, 0.0
+    slices = [(b, h) for b in range(B) for h in range(Hq)]
+    for (b, h) in slices:
+        qs = q[b:b + 1, h:h + 1].float().cpu().numpy()
+        ks = k[b:b + 1, h // G:h // G + 1].float().cpu().numpy()
+        vs = v[b:b + 1, h // G:h // G + 1].float().cpu().numpy()
+        t0 = time.perf_counter()
+        ref = fn(qs, ks, vs, causal=causal)
+        dt = time.perf_counter() - t0
+        err = float(np.abs(ref - out[b:b + 1, h:h + 1].float().cpu().numpy()).max())
+        worst = max(worst, err)
+        done += 1
+        spent += dt
+        if spent + dt > budget_s:
+            break
+    if bound == "mfma":
+        val, unit = flops_slice * done / spent / 1e12, "TFLOP/s"
+    else:
+        esz = 4 if dtype == "f32" else 2
+        slice_bytes = (2 * S * D * esz) / G + 2 * L * D * esz  # a query head's share of its KV head + q + out
+        val, unit = slice_bytes * done / spent / 1e9, "GB/s"
+    return {"value": float("%.4g" % val), "unit": unit, "cores": 1, "host_cores": os.cpu_count(), "kind": kind,
+            "sample": "%d of %d (batch, head) slices of the same inputs, %.1f s, one thread; whole-job estimate %.1f s"
+                      % (done, len(slices), spent, spent / done * len(slices)),
+            "max_abs_err_gpu_vs_cpu": float("%.3g" % worst)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS))
+    ap.add_argument("--secondary", default="config4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the attention path shards by batch / KV head with no "
+                 "exchange; no multi-GPU figure is produced). Run with --gpus 1.")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback.")
+
+    main_res, tensors = run_gpu(args.workload, args.steps, args.warmup)
+    cpu = None if args.no_cpu else run_cpu_baseline(args.workload, tensors, args.cpu_seconds)
+    del tensors
+    torch.cuda.empty_cache()
+    line = {
+        "metric": "attn prefill TFLOP/s + decode KV GB/s on 1 MI355X (% of roofline)",
+        "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": main_res["dtype"], "data": "synthetic (torch.randn on device, seed 0x5EED)",
+        "config": {"workload": "%s: %s" % (args.workload, main_res["description"]), "route": main_res["route"]},
+        "roofline": main_res["roofline"], "cpu_baseline": cpu,
+    }
+    if not args.no_secondary and args.secondary != args.workload:
+        sec, tensors = run_gpu(args.secondary, args.steps, args.warmup)
+        sec["cpu_baseline"] = None if args.no_cpu else run_cpu_baseline(args.secondary, tensors, args.cpu_seconds)
+        del tensors
+        line["secondary"] = sec
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

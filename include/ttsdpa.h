@@ -1,0 +1,126 @@
+/*
+ * ttsdpa — scaled-dot-product attention for AMD MI355X (gfx950), C ABI.
+ *
+ * This is the device boundary behind TinyTorch's attention call
+ *     tinytorch::function::sdpAttention(query, key, value, isCausal, attnMask, dropoutP, scale)
+ * (reference src/Function/FuncNNLayer.h:298-302; forward composite at :231-266).  In the reference that call expands
+ * to ~11 generic device ops (transpose, batched GEMM, scale, mask build, broadcast add, softmax, GEMM; reference
+ * src/Operation/OpLinalgCuda.cuh:239-293, src/Operation/OpNNLayerCuda.cuh:36-145,359-380,
+ * src/Tensor/TensorIterator.cuh:72-161, src/Operation/OpTransformCuda.cuh:79,193).  Here the whole forward is one
+ * entry point; the GPU slot of the {device, dtype} dispatch table (reference src/Tensor/Dispatch.h:32-48) binds to it.
+ *
+ * Conventions (they follow the reference's device ops, src/Utils/CUDAUtils.h:36-83 and src/Tensor/TensorImpl.cpp:234-241):
+ *   - plain device pointers and sizes, no framework types; tensors are row-major with unit stride on the last
+ *     (head_dim) axis and caller-given element strides on batch / head / sequence, so KV-cache views and
+ *     grouped-query layouts pass without copies;
+ *   - work is enqueued on the caller's HIP stream and the call returns without synchronising;
+ *   - the library never allocates or frees device memory: the output and the decode workspace are the caller's;
+ *   - no exceptions, no abort: every entry point returns a status.  0 = enqueued; negative = the arguments are
+ *     outside what the library handles (nothing was launched, the caller may take another route);
+ *     positive = a hipError_t from the runtime.
+ */
+#ifndef TTSDPA_H
+#define TTSDPA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TTSDPA_ABI_VERSION 1
+
+/* Element types; numbering is the reference's DType enum (reference src/Tensor/DType.h:20-28). */
+enum ttsdpa_dtype { TTSDPA_F32 = 0, TTSDPA_F16 = 1, TTSDPA_BF16 = 2 };
+
+/* Kind of attnMask (reference src/Function/FuncNNLayer.h:249-256). */
+enum ttsdpa_mask_kind {
+  TTSDPA_MASK_NONE = 0,
+  TTSDPA_MASK_BOOL = 1, /* uint8, 0 = key hidden (bias -inf), non-zero = visible */
+  TTSDPA_MASK_ADD = 2   /* additive bias, same element type as q */
+};
+
+enum ttsdpa_status {
+  TTSDPA_OK = 0,
+  TTSDPA_ERR_NULL = -1,        /* a required pointer is NULL */
+  TTSDPA_ERR_DTYPE = -2,       /* dtype not one of ttsdpa_dtype */
+  TTSDPA_ERR_SHAPE = -3,       /* negative size, Hq not a multiple of Hkv, head_dim unsupported */
+  TTSDPA_ERR_STRIDE = -4,      /* stride / pointer alignment the kernels cannot use */
+  TTSDPA_ERR_MASK = -5,        /* mask_kind invalid, or causal together with a mask (the reference asserts) */
+  TTSDPA_ERR_WORKSPACE = -6,   /* workspace NULL or smaller than ttsdpa_workspace_bytes() */
+  TTSDPA_ERR_UNSUPPORTED = -7, /* valid call, but not for the kernel asked for (e.g. ttsdpa_decode with L > limit) */
+  TTSDPA_ERR_ABI = -8          /* struct_size does not match this library */
+};
+
+/* Which kernel a call maps to (ttsdpa_plan). */
+enum ttsdpa_route {
+  TTSDPA_ROUTE_NONE = 0,    /* nothing to launch (an empty output) */
+  TTSDPA_ROUTE_GENERAL = 1, /* any dtype / head_dim % 4 == 0 / mask; fp32 arithmetic on the vector ALUs */
+  TTSDPA_ROUTE_PREFILL = 2, /* fp16/bf16, head_dim 128 or 64, no attnMask: MFMA flash-attention forward */
+  TTSDPA_ROUTE_DECODE = 3,  /* fp16/bf16, head_dim 128, few query rows against a long KV cache: split-KV streaming */
+  TTSDPA_ROUTE_ZERO = 4     /* S == 0: the reference's empty contraction yields zeros */
+};
+
+/*
+ * One attention call.  Shapes follow the reference op: q [B,Hq,L,D], k and v [B,Hkv,S,D], out [B,Hq,L,D].
+ * Query head h reads KV head h / (Hq/Hkv) — what op::repeatInterleave(k, Hq/Hkv, 1) (reference
+ * src/Operation/OpTransformCpu.h:399-442) or the 5-D matmul broadcast (src/Operation/OpLinalg.cpp:205-223) feeds
+ * the reference; Hkv == Hq is plain multi-head attention.
+ * Strides are in elements: {batch, head, sequence}; the head_dim stride is 1.  A dense tensor [B,H,N,D] has
+ * {H*N*D, N*D, D}.
+ * causal: key j is visible to query i iff j <= i (top-left aligned, tril(ones(L,S),0), reference
+ * src/Function/FuncNNLayer.h:241-247) — a decode step with L == 1 must therefore pass causal = 0.
+ * mask: [L,S] dense, or NULL.  scale multiplies q.k^T before the bias; the reference default is 1/sqrt(D).
+ */
+typedef struct ttsdpa_params {
+  uint32_t struct_size; /* sizeof(ttsdpa_params) */
+  int32_t dtype;        /* ttsdpa_dtype of q, k, v, out */
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  int32_t B, Hq, Hkv, L, S, D;
+  int64_t q_stride[3];
+  int64_t k_stride[3];
+  int64_t v_stride[3];
+  int64_t o_stride[3];
+  float scale;
+  int32_t causal;
+  int32_t mask_kind; /* ttsdpa_mask_kind */
+  const void* mask;
+} ttsdpa_params;
+
+/* Library identification.  No counterpart in the reference (its device ops are linked statically). */
+int ttsdpa_abi_version(void);
+const char* ttsdpa_status_string(int status);
+
+/* Fill *p for dense tensors: sizes, dense strides, scale = 1/sqrt(D) (reference src/Function/FuncNNLayer.h:235),
+ * no mask, not causal.  Pointers are left NULL. */
+void ttsdpa_params_init(ttsdpa_params* p, int dtype, int B, int Hq, int Hkv, int L, int S, int D);
+
+/* Validate *p and report the kernel ttsdpa_forward would pick (enum ttsdpa_route) in *route.  Launches nothing and
+ * needs no GPU.  Plays the role of the reference's shape checks before a device op (src/Operation/OpLinalg.cpp:62-89). */
+int ttsdpa_plan(const ttsdpa_params* p, int* route);
+
+/* Bytes of device scratch ttsdpa_forward / ttsdpa_decode need for *p (0 for routes that need none).
+ * The reference's precedent for op-owned device scratch is src/Operation/OpNNLayerCuda.cuh:415. */
+size_t ttsdpa_workspace_bytes(const ttsdpa_params* p);
+
+/* The whole of FuncSDPAttention::forward (reference src/Function/FuncNNLayer.h:231-266, dropoutP == 0) on the GPU:
+ * out = softmax(q.k^T * scale + bias) . v, enqueued on `stream` (a hipStream_t; NULL = the default stream).
+ * Chooses the route of ttsdpa_plan. */
+int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The three kernels individually (same contract; TTSDPA_ERR_UNSUPPORTED when *p is outside the kernel's domain).
+ * ttsdpa_prefill replaces the reference's GEMM -> scale -> bias -> softmax -> GEMM chain for training/prefill shapes;
+ * ttsdpa_decode replaces it for one (or a few) query rows against a long contiguous KV cache;
+ * ttsdpa_general covers everything else the reference op accepts (masks, fp32, other head sizes). */
+int ttsdpa_prefill(const ttsdpa_params* p, void* stream);
+int ttsdpa_decode(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream);
+int ttsdpa_general(const ttsdpa_params* p, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTSDPA_H */

@@ -1,0 +1,132 @@
+"""Host-only checks of the C ABI (no GPU, no kernel launch): the library loads, exports every symbol that
+include/ttsdpa.h declares, lays out ttsdpa_params as the header says, validates arguments and picks routes."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from conftest import ROOT
+from tinytorch_amd import _capi
+
+FAKE = 0x10000  # a non-NULL, 16-byte aligned address; nothing is launched in this file
+
+
+def params(*dims, **kw):
+    """dims = (dtype, B, Hq, Hkv, L, S, D); kw overrides struct fields afterwards."""
+    p = _capi.make_params(*dims)
+    p.q = p.k = p.v = p.out = FAKE
+    for k, v in kw.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_exports_match_header():
+    text = open(os.path.join(ROOT, "include", "ttsdpa.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(ttsdpa_[a-z_]+)\s*\(", text)))
+    assert declared == sorted(_capi.EXPORTS)
+    L = _capi.lib()
+    for name in declared:
+        assert getattr(L, name) is not None
+    assert L.ttsdpa_abi_version() == 1
+
+
+def test_struct_layout_matches_header():
+    # 4+4, 4 pointers, 6 ints, 12 int64, float, 2 ints, (pad), pointer
+    assert ctypes.sizeof(_capi.Params) == 8 + 32 + 24 + 96 + 12 + 4 + 8
+    p = _capi.make_params(_capi.BF16, 2, 32, 8, 4096, 4096, 128)
+    assert p.struct_size == ctypes.sizeof(_capi.Params)
+    assert list(p.q_stride) == [32 * 4096 * 128, 4096 * 128, 128]
+    assert list(p.k_stride) == [8 * 4096 * 128, 4096 * 128, 128]
+    assert abs(p.scale - 128 ** -0.5) < 1e-8 and p.causal == 0 and p.mask_kind == 0
+
+
+@pytest.mark.parametrize("args,route", [
+    ((_capi.F32, 1, 4, 4, 128, 128, 64), _capi.ROUTE_GENERAL),       # config 1
+    ((_capi.F16, 4, 32, 32, 2048, 2048, 128), _capi.ROUTE_PREFILL),  # config 2
+    ((_capi.BF16, 2, 32, 8, 4096, 4096, 128), _capi.ROUTE_PREFILL),  # config 3
+    ((_capi.BF16, 64, 32, 8, 1, 8192, 128), _capi.ROUTE_DECODE),     # config 4
+    ((_capi.BF16, 1, 28, 4, 16384, 16384, 128), _capi.ROUTE_PREFILL),  # config 5
+    ((_capi.BF16, 1, 28, 4, 1, 4096, 128), _capi.ROUTE_DECODE),      # 7 heads per KV head
+    ((_capi.BF16, 1, 8, 8, 300, 300, 64), _capi.ROUTE_PREFILL),
+    ((_capi.BF16, 1, 8, 8, 300, 300, 96), _capi.ROUTE_GENERAL),
+    ((_capi.BF16, 1, 64, 2, 1, 4096, 128), _capi.ROUTE_PREFILL),     # 32 rows per KV head: too many for decode
+    ((_capi.BF16, 1, 8, 8, 0, 16, 128), _capi.ROUTE_NONE),
+    ((_capi.BF16, 0, 8, 8, 4, 16, 128), _capi.ROUTE_NONE),
+    ((_capi.BF16, 1, 8, 8, 4, 0, 128), _capi.ROUTE_ZERO),
+])
+def test_routes(args, route):
+    rc, r = _capi.plan(params(*args))
+    assert rc == 0, _capi.status_string(rc)
+    assert r == route, _capi.ROUTE_NAMES[r]
+
+
+def test_routes_depend_on_flags():
+    base = (_capi.BF16, 2, 8, 2, 512, 512, 128)
+    assert _capi.plan(params(*base, causal=1))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(*base, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(*base, scale=-1.0))[1] == _capi.ROUTE_GENERAL
+    p = params(*base)
+    p.k_stride[2] = 132  # rows not 16-byte aligned
+    assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL
+    p = params(*base)
+    p.q = FAKE + 2
+    assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL
+    # decode with causal set is the top-left triangle (only key 0 visible): not the streaming kernel's case
+    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 1, 1024, 128, causal=1))[1] == _capi.ROUTE_PREFILL
+
+
+@pytest.mark.parametrize("mutate,status", [
+    (dict(struct_size=8), _capi.ERR_ABI),
+    (dict(dtype=3), _capi.ERR_DTYPE),
+    (dict(q=0), _capi.ERR_NULL),
+    (dict(out=0), _capi.ERR_NULL),
+    (dict(Hkv=3), _capi.ERR_SHAPE),
+    (dict(D=0), _capi.ERR_SHAPE),
+    (dict(D=512), _capi.ERR_SHAPE),
+    (dict(L=-1), _capi.ERR_SHAPE),
+    (dict(mask_kind=7), _capi.ERR_MASK),
+    (dict(mask_kind=_capi.MASK_BOOL), _capi.ERR_NULL),                      # mask kind without a mask
+    (dict(mask_kind=_capi.MASK_BOOL, mask=FAKE, causal=1), _capi.ERR_MASK),  # reference asserts on this
+])
+def test_validation_errors(mutate, status):
+    p = params(_capi.BF16, 2, 8, 2, 64, 64, 128, **mutate)
+    L = _capi.lib()
+    assert _capi.plan(p)[0] == status
+    # every launching entry point refuses the same way, before touching the GPU
+    assert L.ttsdpa_forward(ctypes.byref(p), None, 0, None) == status
+    assert L.ttsdpa_general(ctypes.byref(p), None) == status
+    assert L.ttsdpa_prefill(ctypes.byref(p), None) == status
+    assert L.ttsdpa_decode(ctypes.byref(p), None, 0, None) == status
+    assert _capi.status_string(status) not in ("ok", "unknown status")
+
+
+def test_kernel_domains_and_workspace():
+    L = _capi.lib()
+    fp32 = params(_capi.F32, 1, 4, 4, 128, 128, 64)
+    assert L.ttsdpa_prefill(ctypes.byref(fp32), None) == _capi.ERR_UNSUPPORTED
+    assert L.ttsdpa_decode(ctypes.byref(fp32), None, 0, None) == _capi.ERR_UNSUPPORTED
+    dec = params(_capi.BF16, 64, 32, 8, 1, 8192, 128)
+    need = L.ttsdpa_workspace_bytes(ctypes.byref(dec))
+    assert need > 0 and need % 4 == 0
+    assert L.ttsdpa_decode(ctypes.byref(dec), None, 0, None) == _capi.ERR_WORKSPACE
+    assert L.ttsdpa_decode(ctypes.byref(dec), FAKE, need - 1, None) == _capi.ERR_WORKSPACE
+    assert L.ttsdpa_forward(ctypes.byref(dec), FAKE, need - 1, None) == _capi.ERR_WORKSPACE
+    short = params(_capi.BF16, 2, 8, 2, 1, 64, 128)
+    assert L.ttsdpa_workspace_bytes(ctypes.byref(short)) == 0          # one split: no scratch
+    assert L.ttsdpa_workspace_bytes(ctypes.byref(fp32)) == 0
+    big = params(_capi.BF16, 1, 64, 2, 1, 4096, 128)
+    assert L.ttsdpa_decode(ctypes.byref(big), None, 0, None) == _capi.ERR_UNSUPPORTED
+
+
+def test_host_wrapper_argument_errors():
+    import torch
+    from tinytorch_amd import sdpAttention
+    q = torch.zeros(1, 2, 4, 8)
+    with pytest.raises(RuntimeError, match="GPU only"):   # no CPU fallback behind this package
+        sdpAttention(q, q, q)
+    with pytest.raises(NotImplementedError):
+        sdpAttention(q, q, q, dropoutP=0.1)
+    with pytest.raises(ValueError):
+        sdpAttention(q[0], q[0], q[0])

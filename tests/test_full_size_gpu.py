@@ -1,0 +1,97 @@
+"""The benchmark configurations at their full sizes.  The CPU oracle needs minutes for whole outputs of these
+shapes, so each run is checked on a few hundred query rows drawn at random (a row's result depends on no other row;
+oracle.sdpa_rows_f32 is the same arithmetic, bit for bit, as the full oracle) plus size-independent properties:
+the first causal row returns v[0], linearity in V, and agreement of the grouped-query kernel with repeated K/V."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import TOL, call, make_inputs, to_host_f32
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {
+    # name: B, Hq, Hkv, L, S, D, dtype, causal, mul, entry
+    "config2_f16_mha_prefill": (4, 32, 32, 2048, 2048, 128, "f16", True, 0.5, "prefill"),
+    "config3_bf16_gqa_prefill": (2, 32, 8, 4096, 4096, 128, "bf16", True, 1.0, "prefill"),
+    "config4_bf16_decode": (64, 32, 8, 1, 8192, 128, "bf16", False, 1.0, "decode"),
+    "config5_bf16_long_prefill": (1, 28, 4, 16384, 16384, 128, "bf16", True, 1.0, "prefill"),
+}
+
+
+def sample_rows(B, Hq, L, n, seed):
+    rng = np.random.RandomState(seed)
+    rows = np.stack([rng.randint(0, B, n), rng.randint(0, Hq, n), rng.randint(0, L, n)], axis=1)
+    rows[0] = (0, 0, 0)
+    rows[1] = (B - 1, Hq - 1, L - 1)
+    if L > 200:
+        for i, l in enumerate((31, 32, 63, 64, 127, 128, 129)):  # tile and wavefront boundaries
+            rows[2 + i] = (rng.randint(0, B), rng.randint(0, Hq), l)
+    return rows
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_full_size_sampled_rows(name):
+    B, Hq, Hkv, L, S, D, dtype, causal, mul, entry = CONFIGS[name]
+    print("full size", name, flush=True)
+    host, dev = make_inputs(0x5EED0000 + len(name), B, Hq, Hkv, L, S, D, dtype, mul)
+    rc, out = call("forward", *dev, causal=causal)
+    assert rc == 0
+    rc2, out2 = call(entry, *dev, causal=causal)       # forward picked the kernel the config is about
+    assert rc2 == 0 and torch.equal(out.view(torch.int16), out2.view(torch.int16))
+    y = to_host_f32(out)
+    assert np.isfinite(y).all()
+    rows = sample_rows(B, Hq, L, 384, 7)
+    exp = oracle.sdpa_rows_f32(*host, rows, causal=causal)
+    got = y[rows[:, 0], rows[:, 1], rows[:, 2]]
+    err = float(np.abs(got - exp).max())
+    print("   max-abs-err over %d sampled rows: %.3e" % (len(rows), err), flush=True)
+    assert err <= TOL[dtype]
+    if causal:  # query 0 sees key 0 only: the output row is v[0] of its KV head, exactly
+        G = Hq // Hkv
+        v0 = np.repeat(host[2][:, :, 0, :], G, axis=1)
+        assert np.array_equal(y[:, :, 0, :], v0)
+    # every output lies inside the convex hull of the value rows it may see (weights are a distribution)
+    vmax = np.repeat(host[2].max(axis=2), Hq // Hkv, axis=1)[:, :, None, :]
+    vmin = np.repeat(host[2].min(axis=2), Hq // Hkv, axis=1)[:, :, None, :]
+    assert (y <= vmax + 2e-2).all() and (y >= vmin - 2e-2).all()
+
+
+def test_config3_linearity_in_v_and_gqa():
+    B, Hq, Hkv, L, S, D = 1, 32, 8, 4096, 4096, 128
+    host, dev = make_inputs(99, B, Hq, Hkv, L, S, D, "bf16")
+    q, k, v1 = dev
+    v2 = torch.roll(v1, shifts=17, dims=2).contiguous()
+    o1 = call("prefill", q, k, v1, causal=True)[1].float()
+    o2 = call("prefill", q, k, v2, causal=True)[1].float()
+    o12 = call("prefill", q, k, ((v1.float() + v2.float()) * 0.5).to(torch.bfloat16), causal=True)[1].float()
+    # out is linear in V: out((v1+v2)/2) == (out(v1)+out(v2))/2 up to the 16-bit roundings of v and out
+    assert float((o12 - 0.5 * (o1 + o2)).abs().max()) <= 2e-2
+    kr, vr = k.repeat_interleave(4, dim=1), v1.repeat_interleave(4, dim=1)
+    o1r = call("prefill", q, kr, vr, causal=True)[1]
+    assert torch.equal(o1r.view(torch.int16), call("prefill", q, k, v1, causal=True)[1].view(torch.int16))
+
+
+def test_config4_decode_split_invariance():
+    """The split-KV merge is a re-association of one softmax: a cache given in one piece or as its two halves
+    (merged by hand with the same log-sum-exp rule on the host) gives the same answer."""
+    B, Hq, Hkv, S, D = 8, 32, 8, 8192, 128
+    host, dev = make_inputs(123, B, Hq, Hkv, 1, S, D, "bf16")
+    q, k, v = dev
+    full = to_host_f32(call("decode", q, k, v)[1]).astype(np.float64)
+    h = S // 2
+    qa = host[0].astype(np.float64)
+    G = Hq // Hkv
+    parts = []
+    for lo, hi in ((0, h), (h, S)):
+        o = to_host_f32(call("decode", q, k[:, :, lo:hi], v[:, :, lo:hi])[1]).astype(np.float64)
+        kk = np.repeat(host[1][:, :, lo:hi].astype(np.float64), G, axis=1)
+        s = np.einsum("bhld,bhsd->bhls", qa, kk) / np.sqrt(D)
+        m = s.max(-1, keepdims=True)
+        lse = m + np.log(np.exp(s - m).sum(-1, keepdims=True))
+        parts.append((o, lse))
+    (o1, l1), (o2, l2) = parts
+    w1 = 1.0 / (1.0 + np.exp(l2 - l1))
+    merged = o1 * w1 + o2 * (1 - w1)
+    assert np.abs(merged - full).max() <= 2e-2

@@ -1,0 +1,264 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle on identical seeded inputs.
+
+Bars (north-star statement): max-abs-error <= 1e-4 for fp32, <= 2e-2 for fp16/bf16 (fp32 accumulation; the oracle is
+the reference's fp32 CPU path applied to the inputs rounded to the 16-bit type)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import golden_names, load_golden
+from gpu_util import TOL, call, make_inputs, max_abs_err, route_of, to_device, to_host_f32
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+# ---- fixtures written from the compiled reference ---------------------------------------------------------------
+
+@pytest.mark.parametrize("name", golden_names())
+def test_golden_fp32(name):
+    g = load_golden(name)
+    say("golden fp32", name)
+    q, k, v = [torch.from_numpy(g[x]).cuda() for x in ("q", "k", "v")]
+    mask = None
+    if g["mask"] is not None:
+        mask = torch.from_numpy(g["mask"]).cuda()
+        mask = mask.bool() if g["mask"].dtype == np.uint8 else mask
+    rc, out = call("forward", q, k, v, causal=g["causal"], mask=mask, scale=g["scale"])
+    assert rc == 0
+    y, exp = to_host_f32(out), g["out"]
+    assert np.array_equal(np.isnan(y), np.isnan(exp))  # rows with every key hidden are NaN on both sides
+    ok = ~np.isnan(exp)
+    assert np.abs(y[ok] - exp[ok]).max() <= TOL["f32"]
+
+
+@pytest.mark.parametrize("name,dtype", [("bf16_inputs_causal", "bf16"), ("f16_inputs_causal", "f16"),
+                                        ("decode_l1_s64", "bf16"), ("decode_l1_s300_scale", "f16"),
+                                        ("gqa_hq8_hkv2", "bf16"), ("boolmask_l9_s12", "bf16"),
+                                        ("floatmask_l9_s12", "f16")])
+def test_golden_16bit(name, dtype):
+    g = load_golden(name)
+    say("golden", dtype, name)
+    host, dev = [], []
+    for x in ("q", "k", "v"):
+        vals, bits = oracle.round_to(g[x], dtype)
+        host.append(vals)
+        dev.append(to_device(vals, bits, dtype))
+    mask_h, mask_d = g["mask"], None
+    if mask_h is not None:
+        if mask_h.dtype == np.uint8:
+            mask_d = torch.from_numpy(mask_h).cuda().bool()
+        else:
+            mv, mb = oracle.round_to(mask_h, dtype)
+            mask_h, mask_d = mv, to_device(mv, mb, dtype)
+    exp = oracle.sdpa_f32(*host, causal=g["causal"], scale=g["scale"], mask=mask_h)
+    rc, out = call("forward", *dev, causal=g["causal"], mask=mask_d, scale=g["scale"])
+    assert rc == 0
+    assert max_abs_err(out, exp) <= TOL[dtype]
+
+
+# ---- config 1 exactly --------------------------------------------------------------------------------------------
+
+def test_config1_fp32_causal():
+    host, dev = make_inputs(0x5EED0001, 1, 4, 4, 128, 128, 64, "f32")
+    g = load_golden("c1_f32_causal")
+    assert np.array_equal(host[0], g["q"])  # the fixture holds these very inputs
+    rc, out = call("forward", *dev, causal=True)
+    assert rc == 0
+    err = max_abs_err(out, g["out"])
+    say("config1 fp32 max-abs-err vs reference output:", err)
+    assert err <= 1e-4
+
+
+# ---- prefill kernel ------------------------------------------------------------------------------------------------
+
+PREFILL_CASES = [
+    # B, Hq, Hkv, L, S, D, dtype, causal, mul
+    (1, 4, 4, 512, 512, 128, "f16", True, 0.5),     # config 2, scaled down
+    (1, 8, 2, 1024, 1024, 128, "bf16", True, 1.0),  # config 3, scaled down
+    (1, 7, 1, 768, 768, 128, "bf16", True, 1.0),    # config 5's 7-heads-per-KV-head grouping
+    (2, 4, 2, 256, 256, 128, "bf16", False, 1.0),
+    (1, 2, 2, 128, 128, 128, "f16", True, 1.0),
+    (1, 2, 1, 100, 100, 128, "bf16", True, 1.0),    # ragged: not a multiple of any tile
+    (1, 2, 2, 130, 257, 128, "bf16", False, 1.0),
+    (1, 2, 2, 200, 77, 128, "f16", True, 1.0),      # L > S, top-left causal
+    (1, 2, 2, 77, 200, 128, "bf16", True, 1.0),     # L < S
+    (1, 3, 3, 33, 64, 128, "bf16", False, 1.0),
+    (1, 4, 2, 300, 300, 64, "bf16", True, 1.0),     # head_dim 64
+    (2, 2, 2, 129, 65, 64, "f16", False, 1.0),
+    (1, 2, 2, 16, 16, 128, "bf16", True, 1.0),
+    (8, 16, 8, 192, 192, 128, "bf16", True, 1.0),   # (batch x kv heads) multiple of 8: the XCD-aware order
+]
+
+
+@pytest.mark.parametrize("case", PREFILL_CASES, ids=lambda c: "B%dH%dk%dL%dS%dD%d-%s-c%d" % c[:8])
+def test_prefill_against_oracle(case):
+    B, Hq, Hkv, L, S, D, dtype, causal, mul = case
+    say("prefill", case)
+    host, dev = make_inputs(1000 + L + S, B, Hq, Hkv, L, S, D, dtype, mul)
+    exp = oracle.sdpa_f32(*host, causal=causal)
+    rc, out = call("prefill", *dev, causal=causal)
+    assert rc == 0
+    err = max_abs_err(out, exp)
+    say("   max-abs-err", err)
+    assert err <= TOL[dtype]
+    assert route_of(*dev, causal=causal) in ("prefill", "decode")
+    rc, out2 = call("forward", *dev, causal=causal)
+    assert rc == 0 and max_abs_err(out2, exp) <= TOL[dtype]
+
+
+def test_prefill_custom_scale_and_strided_views():
+    B, Hq, Hkv, L, S, D = 2, 4, 2, 160, 160, 128
+    host, dev = make_inputs(77, B, Hq, Hkv, L, S, D, "bf16")
+    exp = oracle.sdpa_f32(*host, causal=True, scale=0.03)
+    # q arrives as a transposed view of a [B, L, H, D] buffer; k/v as the first S rows of a longer cache
+    qbuf = dev[0].permute(0, 2, 1, 3).contiguous()
+    qv = qbuf.permute(0, 2, 1, 3)
+    assert not qv.is_contiguous()
+    cache_k = torch.zeros(B, Hkv, S + 96, D, dtype=dev[1].dtype, device="cuda")
+    cache_v = torch.zeros_like(cache_k)
+    cache_k[:, :, :S] = dev[1]
+    cache_v[:, :, :S] = dev[2]
+    rc, out = call("prefill", qv, cache_k[:, :, :S], cache_v[:, :, :S], causal=True, scale=0.03)
+    assert rc == 0
+    assert max_abs_err(out, exp) <= TOL["bf16"]
+
+
+def test_gqa_equals_repeated_kv_bitwise():
+    """kv head = q head / G inside the kernel must be the same arithmetic as feeding repeat-interleaved K/V
+    (what the reference does, src/Operation/OpTransformCpu.h:399-442)."""
+    host, dev = make_inputs(5, 1, 8, 2, 384, 384, 128, "bf16")
+    rc, a = call("prefill", *dev, causal=True)
+    kr = dev[1].repeat_interleave(4, dim=1)
+    vr = dev[2].repeat_interleave(4, dim=1)
+    rc2, b = call("prefill", dev[0], kr, vr, causal=True)
+    assert rc == 0 and rc2 == 0
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+# ---- decode kernel -------------------------------------------------------------------------------------------------
+
+DECODE_CASES = [
+    # B, Hq, Hkv, L, S, dtype
+    (4, 32, 8, 1, 2048, "bf16"),   # config 4, scaled down (several splits)
+    (2, 8, 2, 1, 1, "bf16"),
+    (2, 8, 2, 1, 31, "bf16"),
+    (2, 8, 2, 1, 32, "f16"),
+    (2, 8, 2, 1, 33, "bf16"),
+    (1, 4, 4, 1, 255, "bf16"),     # one query head per KV head
+    (1, 8, 2, 1, 1000, "f16"),
+    (3, 28, 4, 1, 777, "bf16"),    # 7 heads per KV head
+    (1, 16, 2, 1, 4100, "bf16"),   # 8 per KV head, ragged tail
+    (1, 16, 1, 1, 513, "bf16"),    # 16 per KV head
+    (2, 4, 1, 4, 640, "bf16"),     # 4 query rows x 4 heads = 16 rows (multi-token decode)
+    (2, 6, 2, 2, 300, "f16"),      # 2 rows x 3 heads
+    (1, 32, 8, 1, 16384, "bf16"),  # long cache, many splits
+]
+
+
+@pytest.mark.parametrize("case", DECODE_CASES, ids=lambda c: "B%dH%dk%dL%dS%d-%s" % c)
+def test_decode_against_oracle(case):
+    B, Hq, Hkv, L, S, dtype = case
+    say("decode", case)
+    host, dev = make_inputs(2000 + S, B, Hq, Hkv, L, S, 128, dtype)
+    exp = oracle.sdpa_f32(*host, causal=False)
+    rc, out = call("decode", *dev)
+    assert rc == 0
+    err = max_abs_err(out, exp)
+    say("   max-abs-err", err)
+    assert err <= TOL[dtype]
+
+
+def test_decode_cache_view_and_key_permutation():
+    B, Hq, Hkv, S, D = 4, 8, 2, 1500, 128
+    host, dev = make_inputs(31, B, Hq, Hkv, 1, S, D, "bf16")
+    exp = oracle.sdpa_f32(*host)
+    cache_k = torch.zeros(B, Hkv, 2048, D, dtype=torch.bfloat16, device="cuda")
+    cache_v = torch.zeros_like(cache_k)
+    cache_k[:, :, :S] = dev[1]
+    cache_v[:, :, :S] = dev[2]
+    rc, out = call("forward", dev[0], cache_k[:, :, :S], cache_v[:, :, :S])
+    assert rc == 0 and max_abs_err(out, exp) <= TOL["bf16"]
+    # attention without a mask does not care about the order of the cache entries
+    perm = torch.randperm(S, generator=torch.Generator().manual_seed(1)).cuda()
+    rc, outp = call("forward", dev[0], dev[1][:, :, perm].contiguous(), dev[2][:, :, perm].contiguous())
+    assert rc == 0
+    assert np.abs(to_host_f32(out) - to_host_f32(outp)).max() <= 1e-2
+
+
+def test_all_routes_agree():
+    """The three kernels are three schedules of the same function."""
+    host, dev = make_inputs(41, 2, 8, 2, 4, 512, 128, "bf16")
+    exp = oracle.sdpa_f32(*host)
+    outs = {}
+    for entry in ("general", "prefill", "decode"):
+        rc, o = call(entry, *dev)
+        assert rc == 0, entry
+        outs[entry] = o
+        assert max_abs_err(o, exp) <= TOL["bf16"], entry
+    a, b, c = [to_host_f32(outs[e]) for e in ("general", "prefill", "decode")]
+    assert np.abs(a - b).max() <= 1e-2 and np.abs(a - c).max() <= 1e-2
+
+
+# ---- general kernel ------------------------------------------------------------------------------------------------
+
+GENERAL_CASES = [
+    (1, 2, 2, 70, 70, 64, "f32", True), (2, 4, 2, 33, 90, 96, "f32", False), (1, 2, 1, 65, 65, 256, "f32", True),
+    (1, 3, 3, 5, 7, 20, "f32", False), (1, 2, 2, 64, 64, 96, "bf16", True), (1, 2, 2, 40, 50, 32, "f16", False),
+    (1, 1, 1, 1, 1, 4, "f32", True), (1, 2, 2, 130, 64, 6, "f32", True),
+]
+
+
+@pytest.mark.parametrize("case", GENERAL_CASES, ids=lambda c: "B%dH%dk%dL%dS%dD%d-%s-c%d" % c)
+def test_general_against_oracle(case):
+    B, Hq, Hkv, L, S, D, dtype, causal = case
+    say("general", case)
+    host, dev = make_inputs(3000 + D, B, Hq, Hkv, L, S, D, dtype)
+    exp = oracle.sdpa_f32(*host, causal=causal)
+    rc, out = call("general", *dev, causal=causal)
+    assert rc == 0
+    assert max_abs_err(out, exp) <= TOL[dtype]
+    if dtype == "f32":
+        assert route_of(*dev, causal=causal) == "general"
+
+
+def test_general_masks_large():
+    B, Hq, Hkv, L, S, D = 2, 4, 2, 150, 170, 128
+    host, dev = make_inputs(55, B, Hq, Hkv, L, S, D, "bf16")
+    rng = np.random.RandomState(2)
+    bm = (rng.rand(L, S) > 0.5).astype(np.uint8)
+    bm[:, 3] = 1
+    exp = oracle.sdpa_f32(*host, mask=bm)
+    rc, out = call("forward", *dev, mask=torch.from_numpy(bm).cuda().bool())
+    assert rc == 0 and max_abs_err(out, exp) <= TOL["bf16"]
+    fm_v, fm_b = oracle.round_to(oracle.randn(56, 9, (L, S)), "bf16")
+    exp = oracle.sdpa_f32(*host, mask=fm_v)
+    rc, out = call("forward", *dev, mask=to_device(fm_v, fm_b, "bf16"))
+    assert rc == 0 and max_abs_err(out, exp) <= TOL["bf16"]
+
+
+def test_empty_and_degenerate_shapes():
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device="cuda")
+    rc, out = call("forward", z(2, 4, 0, 128), z(2, 4, 16, 128), z(2, 4, 16, 128))
+    assert rc == 0 and out.numel() == 0
+    rc, out = call("forward", z(0, 4, 8, 128), z(0, 4, 16, 128), z(0, 4, 16, 128))
+    assert rc == 0 and out.numel() == 0
+    # S == 0: the reference's empty contraction gives zeros
+    out = torch.full((2, 4, 8, 128), 7.0, dtype=torch.bfloat16, device="cuda")
+    rc, out = call("forward", z(2, 4, 8, 128) + 1, z(2, 4, 0, 128), z(2, 4, 0, 128), out=out)
+    assert rc == 0 and float(out.float().abs().max()) == 0.0
+
+
+def test_host_wrapper_matches_capi():
+    from tinytorch_amd import sdpAttention
+    host, dev = make_inputs(61, 1, 8, 2, 256, 256, 128, "bf16")
+    y = sdpAttention(*dev, isCausal=True)
+    rc, out = call("forward", *dev, causal=True)
+    assert rc == 0 and torch.equal(y.view(torch.int16), out.view(torch.int16))
+    hostd, devd = make_inputs(62, 2, 8, 2, 1, 3000, 128, "bf16")
+    y = sdpAttention(*devd)
+    assert max_abs_err(y, oracle.sdpa_f32(*hostd)) <= TOL["bf16"]

@@ -1,0 +1,12 @@
+"""MI355X-native scaled-dot-product attention behind TinyTorch's ``function::sdpAttention`` interface.
+
+The compute path is the HIP library ``tinytorch_amd/lib/libttsdpa.so`` (C ABI: include/ttsdpa.h).  Importing this
+package loads it and fails if it has not been built.
+"""
+from . import _capi
+
+_capi.lib()  # fail loudly when the extension is missing
+
+from .function import sdpAttention, build_params  # noqa: E402
+
+__all__ = ["sdpAttention", "build_params"]

@@ -1,0 +1,96 @@
+"""ctypes binding of the C ABI declared in include/ttsdpa.h (tinytorch_amd/lib/libttsdpa.so).
+
+The library is the product: when it is missing the import fails loudly — there is no other compute path.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libttsdpa.so")
+
+F32, F16, BF16 = 0, 1, 2
+MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
+ROUTE_NONE, ROUTE_GENERAL, ROUTE_PREFILL, ROUTE_DECODE, ROUTE_ZERO = 0, 1, 2, 3, 4
+ROUTE_NAMES = {0: "none", 1: "general", 2: "prefill", 3: "decode", 4: "zero"}
+
+OK = 0
+ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_STRIDE, ERR_MASK, ERR_WORKSPACE, ERR_UNSUPPORTED, ERR_ABI = range(-1, -9, -1)
+
+EXPORTS = [
+    "ttsdpa_abi_version", "ttsdpa_status_string", "ttsdpa_params_init", "ttsdpa_plan", "ttsdpa_workspace_bytes",
+    "ttsdpa_forward", "ttsdpa_prefill", "ttsdpa_decode", "ttsdpa_general",
+]
+
+
+class Params(ctypes.Structure):
+    """struct ttsdpa_params"""
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("dtype", ctypes.c_int32),
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("B", ctypes.c_int32), ("Hq", ctypes.c_int32), ("Hkv", ctypes.c_int32),
+        ("L", ctypes.c_int32), ("S", ctypes.c_int32), ("D", ctypes.c_int32),
+        ("q_stride", ctypes.c_int64 * 3),
+        ("k_stride", ctypes.c_int64 * 3),
+        ("v_stride", ctypes.c_int64 * 3),
+        ("o_stride", ctypes.c_int64 * 3),
+        ("scale", ctypes.c_float),
+        ("causal", ctypes.c_int32),
+        ("mask_kind", ctypes.c_int32),
+        ("mask", ctypes.c_void_p),
+    ]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "tinytorch_amd: %s is missing — build it with `make -C tinytorch_amd/csrc` "
+                "(or __graft_entry__.build()); there is no fallback path" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        P = ctypes.POINTER(Params)
+        L.ttsdpa_abi_version.restype = ctypes.c_int
+        L.ttsdpa_status_string.argtypes = [ctypes.c_int]
+        L.ttsdpa_status_string.restype = ctypes.c_char_p
+        L.ttsdpa_params_init.argtypes = [P] + [ctypes.c_int] * 7
+        L.ttsdpa_params_init.restype = None
+        L.ttsdpa_plan.argtypes = [P, ctypes.POINTER(ctypes.c_int)]
+        L.ttsdpa_plan.restype = ctypes.c_int
+        L.ttsdpa_workspace_bytes.argtypes = [P]
+        L.ttsdpa_workspace_bytes.restype = ctypes.c_size_t
+        L.ttsdpa_forward.argtypes = [P, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        L.ttsdpa_forward.restype = ctypes.c_int
+        L.ttsdpa_prefill.argtypes = [P, ctypes.c_void_p]
+        L.ttsdpa_prefill.restype = ctypes.c_int
+        L.ttsdpa_decode.argtypes = [P, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        L.ttsdpa_decode.restype = ctypes.c_int
+        L.ttsdpa_general.argtypes = [P, ctypes.c_void_p]
+        L.ttsdpa_general.restype = ctypes.c_int
+        if L.ttsdpa_abi_version() != 1:
+            raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
+        _lib = L
+    return _lib
+
+
+def status_string(rc):
+    return lib().ttsdpa_status_string(rc).decode()
+
+
+def make_params(dtype, B, Hq, Hkv, L, S, D):
+    p = Params()
+    lib().ttsdpa_params_init(ctypes.byref(p), dtype, B, Hq, Hkv, L, S, D)
+    return p
+
+
+def plan(p):
+    """-> (status, route)"""
+    r = ctypes.c_int(-1)
+    rc = lib().ttsdpa_plan(ctypes.byref(p), ctypes.byref(r))
+    return rc, r.value

@@ -1,0 +1,96 @@
+// Shared device-side definitions for the gfx950 attention kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ttsdpa {
+
+// Kernel argument block: the validated contents of ttsdpa_params plus derived values.
+struct KArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  const void* mask;
+  int B, Hq, Hkv, L, S, D;
+  int G;  // Hq / Hkv: query heads per KV head
+  int causal;
+  int mask_kind;
+  float scale;
+  long long qs[3], ks[3], vs[3], os[3];  // element strides: batch, head, sequence
+};
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// Element-type traits: storage is 16-bit (or fp32 for the general kernel), arithmetic is fp32.
+struct BF16 {
+  typedef __bf16 elem;
+  typedef bf16x8 vec8;
+  typedef bf16x4 vec4;
+  static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  // fp32 value of the low / high 16-bit half of a packed pair
+  static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+};
+
+struct F16 {
+  typedef _Float16 elem;
+  typedef f16x8 vec8;
+  typedef f16x4 vec4;
+  static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float lo(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+  }
+  static __device__ __forceinline__ float hi(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+  }
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float load_as_float(const float* p) { return *p; }
+__device__ __forceinline__ float load_as_float(const __bf16* p) { return (float)*p; }
+__device__ __forceinline__ float load_as_float(const _Float16* p) { return (float)*p; }
+__device__ __forceinline__ void store_from_float(float* p, float x) { *p = x; }
+__device__ __forceinline__ void store_from_float(__bf16* p, float x) { *p = (__bf16)x; }
+__device__ __forceinline__ void store_from_float(_Float16* p, float x) { *p = (_Float16)x; }
+
+// Host-side launchers (one per kernel family); each returns a hipError_t as int.
+int launch_general(const KArgs& a, int dtype, hipStream_t stream);
+int launch_prefill(const KArgs& a, int dtype, hipStream_t stream);
+int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream);
+int launch_zero(const KArgs& a, int dtype, hipStream_t stream);
+
+// Decode tiling, shared by the workspace-size query and the launcher.
+struct DecodePlan {
+  int splits;      // KV splits per (batch, kv head)
+  int chunk;       // keys per split (multiple of the per-wave key block)
+  int rows;        // query rows handled together per KV head: L * G
+  size_t ws_bytes; // workspace: per (batch, kv head, split): rows * (D + 2) floats
+};
+DecodePlan plan_decode(const KArgs& a);
+
+constexpr int kDecodeMaxRows = 16;  // L * (Hq/Hkv) handled by one MFMA row block
+
+}  // namespace ttsdpa

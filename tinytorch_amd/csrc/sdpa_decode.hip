@@ -1,0 +1,322 @@
+// Split-KV attention for decode: a few query rows per KV head against a long, contiguous KV cache (fp16 / bf16,
+// head_dim 128).  Memory-bound: every K and V byte is read exactly once with 16-byte loads, whatever the number of
+// query heads sharing the KV head, instead of the reference's GEMM -> scale -> softmax -> GEMM chain over a
+// materialised score tensor (reference src/Function/FuncNNLayer.h:237-265).
+//
+// Work split.  Grid = splits x Hkv x B workgroups of 4 wavefronts.  A split is a contiguous range of keys; its
+// wavefronts take 32-key blocks round-robin.  All query rows that read this KV head — the L * (Hq/Hkv) rows
+// (l, g), at most 16 — are handled together, so the cache is streamed once for the whole group.
+//
+// Per 32-key block and wavefront:
+//   scores  v_mfma_f32_16x16x32: A = the query rows (16 x 32 slice of head_dim, zero rows where unused), B = K^T taken
+//           straight from global memory: lane l supplies key l%16 and the 8 head_dim elements of group l/16, i.e. one
+//           16-byte load; four MFMAs cover head_dim 128.  Query row x sits at MFMA row 4*(x%4) + x/4, so the
+//           result lane (key l%16, group l/16) holds rows l/16, l/16+4, ... in registers 0, 1, ...
+//   softmax running max per row (reduced over the 16 key lanes with DPP row rotations), exp2 with scale*log2e folded
+//   P.V     on the vector ALUs: lane l owns head_dim elements 8*(l%16) .. +7 of keys l/16, l/16+4, ... (one 16-byte
+//           load per key, a wavefront load instruction covers 4 whole V rows = 1 KiB contiguous); the probabilities
+//           travel from the score lanes to the value lanes through a per-wavefront LDS patch.
+// Each wavefront ends with (max, sum, acc) per row; the workgroup merges its four, then either writes the final
+// output (splits == 1) or a partial (max, sum, acc) record that merge_kernel combines by log-sum-exp.
+
+#include "sdpa_common.h"
+
+namespace ttsdpa {
+
+namespace {
+
+constexpr int KB = 32;       // keys per wavefront block
+constexpr int DD = 128;      // head_dim
+constexpr int NWAVE = 4;
+
+// max over the 16 lanes of a DPP row (lanes 16*i .. 16*i+15), result in every lane of the row
+__device__ __forceinline__ float row16_max(float x) {
+  x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x128, 0xf, 0xf, false)));  // row_ror:8
+  x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x124, 0xf, 0xf, false)));  // row_ror:4
+  x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x122, 0xf, 0xf, false)));  // row_ror:2
+  x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x121, 0xf, 0xf, false)));  // row_ror:1
+  return x;
+}
+__device__ __forceinline__ float row16_sum(float x) {
+  x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x128, 0xf, 0xf, false));
+  x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x124, 0xf, 0xf, false));
+  x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x122, 0xf, 0xf, false));
+  x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x121, 0xf, 0xf, false));
+  return x;
+}
+
+// Make this wavefront's LDS writes visible to its own later reads and keep the compiler from reordering across.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// R = registers of query rows per score lane: rows handled = up to 4*R.
+template <typename TR, int R>
+__global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int chunk, float* __restrict__ ws) {
+  typedef typename TR::elem T;
+  typedef typename TR::vec8 vec8;
+  constexpr int NR = 4 * R;  // row slots
+
+  // per-wavefront patch: probabilities [KB keys][NR rows] + rescale factors [NR]; reused for the final merge
+  __shared__ __attribute__((aligned(16))) float Pl[NWAVE][KB * NR + NR];
+  __shared__ __attribute__((aligned(16))) float Om[NWAVE][NR][DD + 2];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l16 = lane & 15;  // score lanes: key within a 16-key group | value lanes: 16-byte chunk of the row
+  const int lg = lane >> 4;   // score lanes: row group              | value lanes: key phase
+
+  int n = blockIdx.x;
+  const int split = n % splits;
+  n /= splits;
+  const int hk = n % a.Hkv;
+  const int b = n / a.Hkv;
+  const int rows = a.L * a.G;  // query rows sharing this KV head, row x = (l, g) = (x / G, x % G)
+
+  const T* kp = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
+  const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
+
+  // ---- query rows as MFMA A operands: lane l supplies MFMA row l%16, head_dim 32*ks + 8*(l/16) .. +7 --------------
+  vec8 qa[4];
+  {
+    int mrow = l16;                       // MFMA row
+    int x = (mrow & 3) * 4 + (mrow >> 2); // query row stored there: row x sits at 4*(x%4) + x/4
+    bool used = (mrow & 3) < R && x < rows;
+    int xl = used ? x / a.G : 0, xg = used ? x % a.G : 0;
+    const T* qr = (const T*)a.q + b * a.qs[0] + (hk * a.G + xg) * a.qs[1] + xl * a.qs[2] + 8 * lg;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      vec8 t = *(const vec8*)(qr + 32 * ks);
+#pragma unroll
+      for (int i = 0; i < 8; i++) qa[ks][i] = used ? t[i] : (T)0.f;
+    }
+  }
+
+  // lane-local state: score lanes track rows lg + 4r; value lanes accumulate all rows for their 8 dims
+  float m_run[R], l_run[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) m_run[r] = -1e30f, l_run[r] = 0.f;
+  float acc[NR][8];
+#pragma unroll
+  for (int x = 0; x < NR; x++)
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[x][i] = 0.f;
+  const float c = a.scale * kLog2e;
+
+  const int s_begin = split * chunk;
+  const int s_end = s_begin + chunk < a.S ? s_begin + chunk : a.S;
+  float* pl = Pl[wave];
+
+  for (int k0 = s_begin + wave * KB; k0 < s_end; k0 += NWAVE * KB) {
+    // ---- issue all loads of the block: K for the score MFMAs, V for the accumulation ----------------------------------
+    u32x4 kreg[2][4];
+#pragma unroll
+    for (int gi = 0; gi < 2; gi++) {
+      int key = k0 + 16 * gi + l16;
+      key = key < a.S ? key : a.S - 1;
+      const T* kr = kp + key * a.ks[2] + 8 * lg;
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) kreg[gi][ks] = *(const u32x4*)(kr + 32 * ks);
+    }
+    u32x4 vreg[KB / 4];
+#pragma unroll
+    for (int i = 0; i < KB / 4; i++) {
+      int key = k0 + 4 * i + lg;
+      key = key < a.S ? key : a.S - 1;
+      vreg[i] = *(const u32x4*)(vp + key * a.vs[2] + 8 * l16);
+    }
+
+    // ---- scores --------------------------------------------------------------------------------------------------------
+    f32x4 sc[2];
+#pragma unroll
+    for (int gi = 0; gi < 2; gi++) {
+      sc[gi] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++)
+        sc[gi] = TR::mfma16(qa[ks], __builtin_bit_cast(vec8, kreg[gi][ks]), sc[gi]);
+      if (k0 + 16 * gi + l16 >= s_end) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) sc[gi][r] = -INFINITY;
+      }
+    }
+
+    // ---- running softmax per row (register r of score-lane group lg is row lg + 4r) -----------------------------------
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      float mloc = row16_max(fmaxf(sc[0][r], sc[1][r]));
+      float m_new = fmaxf(m_run[r], mloc);
+      float alpha = fast_exp2((m_run[r] - m_new) * c);
+      float mc = m_new * c;
+      m_run[r] = m_new;
+      float p0 = fast_exp2(fmaf(sc[0][r], c, -mc));
+      float p1 = fast_exp2(fmaf(sc[1][r], c, -mc));
+      l_run[r] = l_run[r] * alpha + p0 + p1;
+      pl[(l16)*NR + 4 * r + lg] = p0;
+      pl[(16 + l16) * NR + 4 * r + lg] = p1;
+      if (l16 == 0) pl[KB * NR + 4 * r + lg] = alpha;
+    }
+    wave_lds_sync();
+
+    // ---- rescale and accumulate P.V -------------------------------------------------------------------------------------
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      f32x4 al = *(const f32x4*)(pl + KB * NR + 4 * r);
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[4 * r + j][i] *= al[j];
+    }
+#pragma unroll
+    for (int i = 0; i < KB / 4; i++) {
+      float vf[8];
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        vf[2 * w] = TR::lo(vreg[i][w]);
+        vf[2 * w + 1] = TR::hi(vreg[i][w]);
+      }
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        f32x4 p = *(const f32x4*)(pl + (4 * i + lg) * NR + 4 * r);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+          for (int e = 0; e < 8; e++) acc[4 * r + j][e] = fmaf(p[j], vf[e], acc[4 * r + j][e]);
+      }
+    }
+    wave_lds_sync();
+  }
+
+  // ---- wavefront totals: sums over the 16 key lanes; accumulators over the 4 key phases ------------------------------------
+#pragma unroll
+  for (int r = 0; r < R; r++) l_run[r] = row16_sum(l_run[r]);
+#pragma unroll
+  for (int x = 0; x < NR; x++)
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      float t = acc[x][i];
+      t += __shfl_xor(t, 16);
+      t += __shfl_xor(t, 32);
+      acc[x][i] = t;
+    }
+  if (lg == 0) {
+#pragma unroll
+    for (int x = 0; x < NR; x++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) Om[wave][x][8 * l16 + i] = acc[x][i];
+  }
+  if (l16 == 0) {
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      Om[wave][4 * r + lg][DD] = m_run[r];
+      Om[wave][4 * r + lg][DD + 1] = l_run[r];
+    }
+  }
+  __syncthreads();
+
+  // ---- merge the four wavefronts; thread t handles (row slot, dim) pairs ------------------------------------------------------
+  for (int e = tid; e < NR * DD; e += 256) {
+    int x = e / DD, d = e % DD;  // row slot x holds query row x (slot index == query row index)
+    if (x >= rows) continue;
+    float mx = Om[0][x][DD];
+#pragma unroll
+    for (int w = 1; w < NWAVE; w++) mx = fmaxf(mx, Om[w][x][DD]);
+    float lsum = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < NWAVE; w++) {
+      float f = fast_exp2((Om[w][x][DD] - mx) * c);
+      lsum += f * Om[w][x][DD + 1];
+      o += f * Om[w][x][d];
+    }
+    if (splits == 1) {
+      int xl = x / a.G, xg = x % a.G;
+      T* op = (T*)a.out + b * a.os[0] + (hk * a.G + xg) * a.os[1] + xl * a.os[2];
+      store_from_float(op + d, o / lsum);
+    } else {
+      float* rec = ws + ((long long)blockIdx.x * rows + x) * (DD + 2);
+      rec[d] = o;
+      if (d == 0) {
+        rec[DD] = mx;
+        rec[DD + 1] = lsum;
+      }
+    }
+  }
+}
+
+// Combine the per-split records of one (batch, kv head): one workgroup, thread t handles (row, dim) pairs.
+template <typename T>
+__global__ __launch_bounds__(256) void merge_kernel(KArgs a, int splits, const float* __restrict__ ws) {
+  const int pair = blockIdx.x;  // b * Hkv + hk
+  const int hk = pair % a.Hkv, b = pair / a.Hkv;
+  const int rows = a.L * a.G;
+  const float c = a.scale * kLog2e;
+  for (int e = threadIdx.x; e < rows * DD; e += 256) {
+    int x = e / DD, d = e % DD;
+    const float* rec0 = ws + ((long long)pair * splits * rows + x) * (DD + 2);
+    const long long step = (long long)rows * (DD + 2);
+    float mx = -1e30f;
+    for (int s = 0; s < splits; s++) mx = fmaxf(mx, rec0[s * step + DD]);
+    float lsum = 0.f, o = 0.f;
+    for (int s = 0; s < splits; s++) {
+      float f = fast_exp2((rec0[s * step + DD] - mx) * c);
+      lsum += f * rec0[s * step + DD + 1];
+      o += f * rec0[s * step + d];
+    }
+    int xl = x / a.G, xg = x % a.G;
+    T* op = (T*)a.out + b * a.os[0] + (hk * a.G + xg) * a.os[1] + xl * a.os[2];
+    store_from_float(op + d, o / lsum);
+  }
+}
+
+template <typename TR>
+int launch_decode_t(const KArgs& a, const DecodePlan& pl, float* ws, hipStream_t stream) {
+  typedef typename TR::elem T;
+  dim3 grid((unsigned)((long long)a.B * a.Hkv * pl.splits)), block(256);
+  int R = (pl.rows + 3) / 4;
+  switch (R) {
+    case 1: hipLaunchKernelGGL((decode_kernel<TR, 1>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
+    case 2: hipLaunchKernelGGL((decode_kernel<TR, 2>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
+    case 3: hipLaunchKernelGGL((decode_kernel<TR, 3>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
+    default: hipLaunchKernelGGL((decode_kernel<TR, 4>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
+  }
+  int rc = (int)hipGetLastError();
+  if (rc != 0 || pl.splits == 1) return rc;
+  hipLaunchKernelGGL((merge_kernel<T>), dim3((unsigned)(a.B * a.Hkv)), block, 0, stream, a, pl.splits, ws);
+  return (int)hipGetLastError();
+}
+
+}  // namespace
+
+// Splits: enough workgroups to cover the 256 CUs several times over, each split at least 256 keys, chunk a
+// multiple of the 128 keys a workgroup consumes per round.
+DecodePlan plan_decode(const KArgs& a) {
+  DecodePlan p;
+  p.rows = a.L * a.G;
+  const int round = NWAVE * KB;
+  long long pairs = (long long)a.B * a.Hkv;
+  int max_splits = (a.S + 2 * round - 1) / (2 * round);
+  if (max_splits < 1) max_splits = 1;
+  long long want = (8 * 256 + pairs - 1) / pairs;  // aim for >= 8 workgroups per CU
+  int splits = (int)(want < 1 ? 1 : want);
+  if (splits > max_splits) splits = max_splits;
+  if (splits > 64) splits = 64;
+  int chunk = (a.S + splits - 1) / splits;
+  chunk = (chunk + round - 1) / round * round;
+  if (chunk < round) chunk = round;
+  splits = (a.S + chunk - 1) / chunk;
+  if (splits < 1) splits = 1;
+  p.splits = splits;
+  p.chunk = chunk;
+  p.ws_bytes = splits > 1 ? (size_t)pairs * splits * p.rows * (DD + 2) * sizeof(float) : 0;
+  return p;
+}
+
+int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream) {
+  DecodePlan pl = plan_decode(a);
+  if (dtype == 1) return launch_decode_t<F16>(a, pl, (float*)workspace, stream);
+  return launch_decode_t<BF16>(a, pl, (float*)workspace, stream);
+}
+
+}  // namespace ttsdpa

@@ -1,0 +1,185 @@
+// C ABI of the attention library (declarations and contract: include/ttsdpa.h).
+// Validates a call, picks the kernel family, and enqueues it on the caller's stream.  Nothing here allocates device
+// memory, synchronises, throws or aborts.
+
+#include <math.h>
+#include <string.h>
+
+#include "../../include/ttsdpa.h"
+#include "sdpa_common.h"
+
+using namespace ttsdpa;
+
+namespace {
+
+bool dense_last_ok(const int64_t* st, int align) { return st[0] % align == 0 && st[1] % align == 0 && st[2] % align == 0; }
+
+bool ptr_aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+// Validation shared by every entry point; fills the kernel argument block.
+int validate(const ttsdpa_params* p, KArgs* a) {
+  if (!p) return TTSDPA_ERR_NULL;
+  if (p->struct_size != sizeof(ttsdpa_params)) return TTSDPA_ERR_ABI;
+  if (p->dtype != TTSDPA_F32 && p->dtype != TTSDPA_F16 && p->dtype != TTSDPA_BF16) return TTSDPA_ERR_DTYPE;
+  if (p->B < 0 || p->Hq < 1 || p->Hkv < 1 || p->L < 0 || p->S < 0 || p->D < 1 || p->D > 256) return TTSDPA_ERR_SHAPE;
+  if (p->Hq % p->Hkv != 0) return TTSDPA_ERR_SHAPE;
+  if (p->mask_kind < TTSDPA_MASK_NONE || p->mask_kind > TTSDPA_MASK_ADD) return TTSDPA_ERR_MASK;
+  if (p->mask_kind != TTSDPA_MASK_NONE && p->causal) return TTSDPA_ERR_MASK;  // reference FuncNNLayer.h:242
+  const bool empty_out = p->B == 0 || p->L == 0;
+  if (!empty_out) {
+    if (!p->q || !p->out) return TTSDPA_ERR_NULL;
+    if (p->S > 0 && (!p->k || !p->v)) return TTSDPA_ERR_NULL;
+    if (p->mask_kind != TTSDPA_MASK_NONE && !p->mask) return TTSDPA_ERR_NULL;
+  }
+  for (int i = 0; i < 3; i++) {
+    if (p->q_stride[i] < 0 || p->k_stride[i] < 0 || p->v_stride[i] < 0 || p->o_stride[i] < 0) return TTSDPA_ERR_STRIDE;
+  }
+  if (p->q_stride[2] < p->D && p->L > 1) return TTSDPA_ERR_STRIDE;
+  if (p->o_stride[2] < p->D && p->L > 1) return TTSDPA_ERR_STRIDE;
+  if ((p->k_stride[2] < p->D || p->v_stride[2] < p->D) && p->S > 1) return TTSDPA_ERR_STRIDE;
+  const size_t esz = p->dtype == TTSDPA_F32 ? 4 : 2;
+  if (!ptr_aligned(p->q, esz) || !ptr_aligned(p->k, esz) || !ptr_aligned(p->v, esz) || !ptr_aligned(p->out, esz))
+    return TTSDPA_ERR_STRIDE;
+  a->q = p->q, a->k = p->k, a->v = p->v, a->out = p->out, a->mask = p->mask;
+  a->B = p->B, a->Hq = p->Hq, a->Hkv = p->Hkv, a->L = p->L, a->S = p->S, a->D = p->D;
+  a->G = p->Hq / p->Hkv;
+  a->causal = p->causal ? 1 : 0;
+  a->mask_kind = p->mask_kind;
+  a->scale = p->scale;
+  for (int i = 0; i < 3; i++) {
+    a->qs[i] = p->q_stride[i], a->ks[i] = p->k_stride[i], a->vs[i] = p->v_stride[i], a->os[i] = p->o_stride[i];
+  }
+  return TTSDPA_OK;
+}
+
+// 16-bit tensors the MFMA kernels can read with 16-byte loads and write with 8-byte stores.
+bool fast_layout_ok(const ttsdpa_params* p) {
+  if (p->dtype != TTSDPA_F16 && p->dtype != TTSDPA_BF16) return false;
+  if (p->mask_kind != TTSDPA_MASK_NONE) return false;
+  if (!(p->scale > 0.f) || !isfinite(p->scale)) return false;  // the row maximum is taken on unscaled scores
+  if (!dense_last_ok(p->q_stride, 8) || !dense_last_ok(p->k_stride, 8) || !dense_last_ok(p->v_stride, 8) ||
+      !dense_last_ok(p->o_stride, 8))
+    return false;
+  return ptr_aligned(p->q, 16) && ptr_aligned(p->k, 16) && ptr_aligned(p->v, 16) && ptr_aligned(p->out, 16);
+}
+
+bool prefill_ok(const ttsdpa_params* p) {
+  return fast_layout_ok(p) && (p->D == 128 || p->D == 64) && p->S >= 1 && p->L >= 1;
+}
+
+bool decode_ok(const ttsdpa_params* p) {
+  if (!fast_layout_ok(p) || p->D != 128 || p->causal || p->S < 1 || p->L < 1) return false;
+  return (long long)p->L * (p->Hq / p->Hkv) <= kDecodeMaxRows;
+}
+
+int pick_route(const ttsdpa_params* p) {
+  if (p->B == 0 || p->L == 0) return TTSDPA_ROUTE_NONE;
+  if (p->S == 0) return TTSDPA_ROUTE_ZERO;
+  // Few query rows against many keys: streaming the cache once for the whole head group beats a 128-row tile.
+  if (decode_ok(p) && p->S >= 256) return TTSDPA_ROUTE_DECODE;
+  if (prefill_ok(p) && p->L >= 16) return TTSDPA_ROUTE_PREFILL;
+  if (decode_ok(p)) return TTSDPA_ROUTE_DECODE;
+  if (prefill_ok(p)) return TTSDPA_ROUTE_PREFILL;
+  return TTSDPA_ROUTE_GENERAL;
+}
+
+int check_grid(long long nwg) { return nwg > 0x7fffffffLL ? TTSDPA_ERR_SHAPE : TTSDPA_OK; }
+
+}  // namespace
+
+extern "C" {
+
+int ttsdpa_abi_version(void) { return TTSDPA_ABI_VERSION; }
+
+const char* ttsdpa_status_string(int status) {
+  switch (status) {
+    case TTSDPA_OK: return "ok";
+    case TTSDPA_ERR_NULL: return "required pointer is NULL";
+    case TTSDPA_ERR_DTYPE: return "unsupported dtype";
+    case TTSDPA_ERR_SHAPE: return "invalid or unsupported shape";
+    case TTSDPA_ERR_STRIDE: return "unsupported stride or alignment";
+    case TTSDPA_ERR_MASK: return "invalid mask arguments";
+    case TTSDPA_ERR_WORKSPACE: return "workspace missing or too small";
+    case TTSDPA_ERR_UNSUPPORTED: return "arguments outside this kernel's domain";
+    case TTSDPA_ERR_ABI: return "ttsdpa_params.struct_size mismatch";
+    default: return status > 0 ? hipGetErrorString((hipError_t)status) : "unknown status";
+  }
+}
+
+void ttsdpa_params_init(ttsdpa_params* p, int dtype, int B, int Hq, int Hkv, int L, int S, int D) {
+  memset(p, 0, sizeof(*p));
+  p->struct_size = sizeof(*p);
+  p->dtype = dtype;
+  p->B = B, p->Hq = Hq, p->Hkv = Hkv, p->L = L, p->S = S, p->D = D;
+  p->q_stride[0] = (int64_t)Hq * L * D, p->q_stride[1] = (int64_t)L * D, p->q_stride[2] = D;
+  p->k_stride[0] = (int64_t)Hkv * S * D, p->k_stride[1] = (int64_t)S * D, p->k_stride[2] = D;
+  p->v_stride[0] = p->k_stride[0], p->v_stride[1] = p->k_stride[1], p->v_stride[2] = D;
+  p->o_stride[0] = p->q_stride[0], p->o_stride[1] = p->q_stride[1], p->o_stride[2] = D;
+  p->scale = D > 0 ? 1.f / sqrtf((float)D) : 1.f;
+  p->causal = 0;
+  p->mask_kind = TTSDPA_MASK_NONE;
+  p->mask = nullptr;
+}
+
+int ttsdpa_plan(const ttsdpa_params* p, int* route) {
+  KArgs a;
+  int rc = validate(p, &a);
+  if (rc != TTSDPA_OK) return rc;
+  if (route) *route = pick_route(p);
+  return TTSDPA_OK;
+}
+
+size_t ttsdpa_workspace_bytes(const ttsdpa_params* p) {
+  KArgs a;
+  if (validate(p, &a) != TTSDPA_OK) return 0;
+  if (p->B == 0 || p->L == 0 || p->S == 0 || !decode_ok(p)) return 0;
+  return plan_decode(a).ws_bytes;
+}
+
+int ttsdpa_general(const ttsdpa_params* p, void* stream) {
+  KArgs a;
+  int rc = validate(p, &a);
+  if (rc != TTSDPA_OK) return rc;
+  if (p->B == 0 || p->L == 0) return TTSDPA_OK;
+  if (p->S == 0) return launch_zero(a, p->dtype, (hipStream_t)stream);
+  if ((rc = check_grid((long long)a.B * a.Hq * ((a.L + 63) / 64))) != TTSDPA_OK) return rc;
+  return launch_general(a, p->dtype, (hipStream_t)stream);
+}
+
+int ttsdpa_prefill(const ttsdpa_params* p, void* stream) {
+  KArgs a;
+  int rc = validate(p, &a);
+  if (rc != TTSDPA_OK) return rc;
+  if (p->B == 0 || p->L == 0) return TTSDPA_OK;
+  if (!prefill_ok(p)) return TTSDPA_ERR_UNSUPPORTED;
+  if ((rc = check_grid((long long)a.B * a.Hq * ((a.L + 127) / 128))) != TTSDPA_OK) return rc;
+  return launch_prefill(a, p->dtype, (hipStream_t)stream);
+}
+
+int ttsdpa_decode(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream) {
+  KArgs a;
+  int rc = validate(p, &a);
+  if (rc != TTSDPA_OK) return rc;
+  if (p->B == 0 || p->L == 0) return TTSDPA_OK;
+  if (!decode_ok(p)) return TTSDPA_ERR_UNSUPPORTED;
+  DecodePlan pl = plan_decode(a);
+  if (pl.ws_bytes > 0 && (!workspace || workspace_bytes < pl.ws_bytes || !ptr_aligned(workspace, 16)))
+    return TTSDPA_ERR_WORKSPACE;
+  if ((rc = check_grid((long long)a.B * a.Hkv * pl.splits)) != TTSDPA_OK) return rc;
+  return launch_decode(a, p->dtype, workspace, (hipStream_t)stream);
+}
+
+int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream) {
+  KArgs a;
+  int rc = validate(p, &a);
+  if (rc != TTSDPA_OK) return rc;
+  switch (pick_route(p)) {
+    case TTSDPA_ROUTE_NONE: return TTSDPA_OK;
+    case TTSDPA_ROUTE_ZERO: return launch_zero(a, p->dtype, (hipStream_t)stream);
+    case TTSDPA_ROUTE_DECODE: return ttsdpa_decode(p, workspace, workspace_bytes, stream);
+    case TTSDPA_ROUTE_PREFILL: return ttsdpa_prefill(p, stream);
+    default: return ttsdpa_general(p, stream);
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,96 @@
+"""Host-side mirror of TinyTorch's attention interface for torch device tensors.
+
+``sdpAttention`` keeps the name, argument order, defaults and error behaviour of
+``tinytorch::function::sdpAttention`` (reference src/Function/FuncNNLayer.h:298-302) and of
+``FuncSDPAttention::forward`` (:231-266); the work itself is one call through the C ABI of include/ttsdpa.h.
+torch is only the owner of device memory and of the current stream here.
+"""
+import ctypes
+import math
+
+import torch
+
+from . import _capi
+
+_DTYPES = {torch.float32: _capi.F32, torch.float16: _capi.F16, torch.bfloat16: _capi.BF16}
+_workspaces = {}
+
+
+def _workspace(device, nbytes):
+    """Device scratch for the decode route, grown on demand and kept per device (the reference's ops take such
+    scratch from the caching allocator, src/Operation/OpNNLayerCuda.cuh:415)."""
+    buf = _workspaces.get(device)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[device] = buf
+    return buf
+
+
+def _strides3(t):
+    assert t.stride(-1) == 1 or t.size(-1) == 1
+    return (t.stride(0), t.stride(1), t.stride(2))
+
+
+def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=None):
+    """Fill a ttsdpa_params for 4-D tensors [B,H,N,D]."""
+    B, Hq, L, D = query.shape
+    Bk, Hkv, S, Dk = key.shape
+    if value.shape != key.shape or Bk != B or Dk != D:
+        raise ValueError("sdpAttention: key/value shape %s / %s do not match query %s"
+                         % (tuple(key.shape), tuple(value.shape), tuple(query.shape)))
+    if Hkv < 1 or Hq % Hkv != 0:
+        raise ValueError("sdpAttention: %d query heads cannot share %d key/value heads" % (Hq, Hkv))
+    if query.dtype not in _DTYPES or key.dtype != query.dtype or value.dtype != query.dtype:
+        raise TypeError("sdpAttention: dtype must be one of float32/float16/bfloat16 and equal for q, k, v")
+    p = _capi.make_params(_DTYPES[query.dtype], B, Hq, Hkv, L, S, D)
+    p.q, p.k, p.v, p.out = query.data_ptr(), key.data_ptr(), value.data_ptr(), out.data_ptr()
+    for name, t in (("q_stride", query), ("k_stride", key), ("v_stride", value), ("o_stride", out)):
+        st = _strides3(t)
+        for i in range(3):
+            getattr(p, name)[i] = st[i]
+    p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(float(D))
+    p.causal = 1 if isCausal else 0
+    if attnMask is not None:
+        if isCausal:
+            raise ValueError("sdpAttention: isCausal and attnMask are exclusive")  # reference FuncNNLayer.h:242
+        if tuple(attnMask.shape) != (L, S):
+            raise ValueError("sdpAttention: attnMask must be [L, S]")
+        if attnMask.dtype == torch.bool:
+            p.mask_kind = _capi.MASK_BOOL
+        elif attnMask.dtype == query.dtype:
+            p.mask_kind = _capi.MASK_ADD
+        else:
+            raise TypeError("sdpAttention: attnMask must be bool or of the query dtype")
+        p.mask = attnMask.data_ptr()
+    return p
+
+
+def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0, scale=None):
+    """out = softmax(query @ key^T * scale + bias) @ value on the GPU.
+
+    query [B,Hq,L,D]; key/value [B,Hkv,S,D] with Hq a multiple of Hkv (query head h reads KV head h // (Hq//Hkv));
+    returns [B,Hq,L,D] in the dtype of query.  isCausal is top-left aligned (key j visible iff j <= i).
+    """
+    if dropoutP != 0.0:
+        raise NotImplementedError("sdpAttention: dropoutP must be 0 on this path")
+    if query.dim() != 4 or key.dim() != 4 or value.dim() != 4:
+        raise ValueError("sdpAttention: expected 4-D tensors [B, H, N, D]")
+    if not query.is_cuda:
+        raise RuntimeError("tinytorch_amd.sdpAttention runs on the GPU only; got a %s tensor" % query.device)
+    if key.device != query.device or value.device != query.device:
+        raise RuntimeError("sdpAttention: q, k, v must live on the same device")
+    fix = lambda t: t if (t.stride(-1) == 1 or t.size(-1) == 1) else t.contiguous()
+    query, key, value = fix(query), fix(key), fix(value)
+    if attnMask is not None:
+        attnMask = attnMask.contiguous()
+    out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
+    p = build_params(query, key, value, out, isCausal, attnMask, scale)
+    L = _capi.lib()
+    with torch.cuda.device(query.device):
+        nbytes = L.ttsdpa_workspace_bytes(ctypes.byref(p))
+        ws = _workspace(query.device, nbytes) if nbytes else None
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = L.ttsdpa_forward(ctypes.byref(p), ws.data_ptr() if ws is not None else None, nbytes, stream)
+    if rc != 0:
+        raise RuntimeError("ttsdpa_forward failed: %d (%s)" % (rc, _capi.status_string(rc)))
+    return out
