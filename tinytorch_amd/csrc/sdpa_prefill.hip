@@ -6,17 +6,20 @@
 // never leaves registers.
 //
 // Tiling.  A workgroup of 4 wavefronts owns 128 query rows of one (batch, query head); each wavefront owns 32 of
-// them.  Keys/values are consumed in tiles of 64, staged through LDS (K row-major, V transposed so that the key
-// axis is contiguous), the next tile's global loads being in flight while the current one is computed.
+// them.  Keys/values are consumed in tiles of 64 rows, staged row-major through a double-buffered LDS ring (one
+// barrier per tile); the global loads of tile j+2 are in flight while tile j is computed.
 //
 // Per wavefront and KV tile, with v_mfma_f32_32x32x16 (A: 32 rows x 16, B: 16 x 32 cols, lane l supplies row/col
 // l%32 and the 8 contraction elements of half l/32; C: lane l holds column l%32 and rows 8*(r/4) + 4*(l/32) + r%4):
-//   S^T[64 keys x 32 queries] = K_tile . Q^T      A = K rows from LDS, B = Q rows held in registers
-//   P^T = exp2((S^T - rowmax) * scale*log2e)      a query is one lane column: its keys sit in that lane's registers
+//   S^T[64 keys x 32 queries] = K_tile . Q^T      A = K rows from LDS (ds_read_b128), B = Q rows held in registers
+//   P^T = exp2((S^T - m) * scale*log2e)           a query is one lane column: its keys sit in that lane's registers
 //                                                 and in lane l^32, so a row reduction is one cross-lane step
-//   O^T[D x 32 queries] += V_tile^T . P^T         A = V^T rows from LDS, B = P^T taken straight from the S^T
-//                                                 accumulator registers (the contraction order is permuted
-//                                                 identically on the V^T side, see vt_pos)
+//   O^T[D x 32 queries] += V_tile^T . P^T         A = V^T, read from the row-major V tile with the LDS transpose
+//                                                 load ds_read_b64_tr_b16; B = P^T taken straight from the S^T
+//                                                 accumulator registers (the V side applies the same permutation
+//                                                 of the contraction index, see v_operand)
+// The running maximum m is only raised when a tile's maximum exceeds it by more than 2^8 in the exponent (the
+// probabilities stay <= 256, exact in fp32 sums and within bf16/fp16 range), so the accumulator rescale is rare.
 // Causal masking (key j visible to query i iff j <= i, reference src/Operation/OpTransformCpu.h:202-209) skips
 // tiles above the diagonal and applies the predicate only on tiles that straddle it.
 // Grouped-query attention: kv head = query head / (Hq/Hkv), resolved in the kernel; the workgroup order puts the
@@ -30,29 +33,48 @@ namespace {
 
 constexpr int BM = 128;  // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
-constexpr int VT_PITCH = BN + 8;  // elements per V^T row in LDS (144 B: 16 consecutive rows hit distinct banks)
+constexpr float kLazyExp = 8.f;  // raise the running maximum only when exceeded by 2^8 in the exponent
 
-// Position of key kv (0..63) inside a V^T row: the 8 keys one lane feeds to one MFMA become contiguous.
-// kv = 16*t + 8*a + 4*h + c  ->  16*t + 8*h + 4*a + c
-__device__ __forceinline__ int vt_pos(int kv) { return (kv & ~15) | ((kv & 4) << 1) | ((kv & 8) >> 1) | (kv & 3); }
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+
+template <int D>
+struct PrefillLds {
+  static constexpr int K_PITCH = D + 8;   // elements; rows 16 B apart in bank space: 32 rows x b128 conflict-free
+  static constexpr int V_PITCH = D + 32;  // elements; rows 64 B apart in bank space: 4 rows x 64 B conflict-free
+  static constexpr int STAGE = BN * (K_PITCH + V_PITCH);  // elements per stage
+  static constexpr int BYTES = 2 * STAGE * 2;
+};
+
+// One MFMA A operand of V^T from a row-major V tile: lane l (column d = d0 + l%32, half h = l/32) receives the
+// 8 keys kvbase + {4h + 0..3, 8 + 4h + 0..3}.  ds_read_b64_tr_b16 works on groups of 16 lanes: lane s of a group
+// supplies the address of 4 consecutive elements, and receives element s%4 of the segments of lanes s/4, 4 + s/4,
+// 8 + s/4, 12 + s/4.  With lane s pointing at V[k0 + s/4][c0 + 4*(s%4) ..], lane s ends up with V[k0 + 0..3][c0 + s].
+template <typename vec8>
+__device__ __forceinline__ vec8 v_operand(const void* lane_base, int byte_off_lo, int byte_off_hi) {
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)((const char*)lane_base + byte_off_lo));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)((const char*)lane_base + byte_off_hi));
+  s16x8 r = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(vec8, r);
+}
 
 template <typename TR, int D, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void prefill_kernel(KArgs a) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
-  constexpr int K_PITCH = D + 8;     // elements per K row in LDS
-  constexpr int KSTEPS = D / 16;     // MFMAs along head_dim for S^T
-  constexpr int DBLK = D / 32;       // 32-row blocks of O^T
-  constexpr int KLD = (BN * D / 8) / 256;  // 16-byte K chunks per thread per tile
-  constexpr int VBLOCKS = (BN / 4) * (D / 8);  // 4-key x 8-dim blocks per tile
-  constexpr int VLD = (VBLOCKS + 255) / 256;
+  typedef PrefillLds<D> Lds;
+  constexpr int K_PITCH = Lds::K_PITCH, V_PITCH = Lds::V_PITCH;
+  constexpr int KSTEPS = D / 16;           // MFMAs along head_dim for S^T
+  constexpr int DBLK = D / 32;             // 32-row blocks of O^T
+  constexpr int NLD = (BN * D / 8) / 256;  // 16-byte chunks per thread per tile, for K and for V
 
-  __shared__ __attribute__((aligned(16))) T Ks[BN * K_PITCH];
-  __shared__ __attribute__((aligned(16))) T Vt[D * VT_PITCH];
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  T* smem = (T*)smem_raw;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: branches on it are scalar
   const int lq = lane & 31;   // query column / operand row of this lane
   const int lh = lane >> 5;   // which half of the contraction elements this lane supplies
 
@@ -98,9 +120,11 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(KArgs a) {
   for (int i = 0; i < DBLK; i++)
 #pragma unroll
     for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
-  float m_run = -1e30f;  // running row maximum (raw scores), finite so that (m_run - m_new) never is inf - inf
-  float l_run = 0.f;     // this lane's share of the running row sum
   const float c = a.scale * kLog2e;
+  const float lazy = kLazyExp / c;  // the same margin in raw-score units
+  float m_use = -1e30f;  // maximum the exponentials are taken against (raw scores); finite: no inf - inf
+  float mc = m_use * c;
+  float l_run = 0.f;     // this lane's share of the running row sum
 
   int ntiles_kv = (a.S + BN - 1) / BN;
   if (CAUSAL) {
@@ -109,145 +133,148 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(KArgs a) {
     ntiles_kv = lastkv / BN + 1;
   }
 
-  // ---- global -> register staging of one K/V tile ------------------------------------------------------------
-  u32x4 kst[KLD];
-  u32x4 vst[VLD][4];
+  // ---- global -> register -> LDS staging of one K/V tile --------------------------------------------------------
+  // thread t moves chunks t, t+256, ...: chunk c is row c / (D/8), 16-byte column c % (D/8)
+  u32x4 kst[NLD], vst[NLD];
+  unsigned koff[NLD], voff[NLD];  // byte offsets of this thread's chunks inside a full tile
+  int lrow[NLD], lcol[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; i++) {
+    int cidx = tid + 256 * i;
+    lrow[i] = cidx / (D / 8);
+    lcol[i] = cidx % (D / 8);
+    koff[i] = (unsigned)(lrow[i] * a.ks[2] + 8 * lcol[i]) * 2u;
+    voff[i] = (unsigned)(lrow[i] * a.vs[2] + 8 * lcol[i]) * 2u;
+  }
   auto load_tile = [&](int kv0) {
+    const char* kt = (const char*)(kp + kv0 * a.ks[2]);
+    const char* vt = (const char*)(vp + kv0 * a.vs[2]);
+    if (kv0 + BN <= a.S) {
 #pragma unroll
-    for (int i = 0; i < KLD; i++) {
-      int cidx = tid + 256 * i;
-      int r = cidx / (D / 8), cc = cidx % (D / 8);
-      int key = kv0 + r;
-      key = key < a.S ? key : a.S - 1;
-      kst[i] = *(const u32x4*)(kp + key * a.ks[2] + 8 * cc);
-    }
+      for (int i = 0; i < NLD; i++) {
+        kst[i] = *(const u32x4*)(kt + koff[i]);
+        vst[i] = *(const u32x4*)(vt + voff[i]);
+      }
+    } else {  // ragged last tile: rows past the end re-read the last valid row (masked later)
 #pragma unroll
-    for (int i = 0; i < VLD; i++) {
-      int blk = tid + 256 * i;
-      if (VBLOCKS % 256 == 0 || blk < VBLOCKS) {
-        int kg = blk / (D / 8), dc = blk % (D / 8);
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          int key = kv0 + 4 * kg + j;
-          key = key < a.S ? key : a.S - 1;
-          vst[i][j] = *(const u32x4*)(vp + key * a.vs[2] + 8 * dc);
-        }
+      for (int i = 0; i < NLD; i++) {
+        int key = kv0 + lrow[i];
+        key = key < a.S ? key : a.S - 1;
+        kst[i] = *(const u32x4*)(kp + key * a.ks[2] + 8 * lcol[i]);
+        vst[i] = *(const u32x4*)(vp + key * a.vs[2] + 8 * lcol[i]);
       }
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](int stage) {
+    T* Ks = smem + stage * Lds::STAGE;
+    T* Vs = Ks + BN * K_PITCH;
 #pragma unroll
-    for (int i = 0; i < KLD; i++) {
-      int cidx = tid + 256 * i;
-      int r = cidx / (D / 8), cc = cidx % (D / 8);
-      *(u32x4*)(Ks + r * K_PITCH + 8 * cc) = kst[i];
-    }
-#pragma unroll
-    for (int i = 0; i < VLD; i++) {
-      int blk = tid + 256 * i;
-      if (VBLOCKS % 256 == 0 || blk < VBLOCKS) {
-        int kg = blk / (D / 8), dc = blk % (D / 8);
-        int pos = vt_pos(4 * kg);
-#pragma unroll
-        for (int w = 0; w < 4; w++) {
-          // dims 8*dc + 2w (low halves) and 8*dc + 2w + 1 (high halves) of the four keys 4*kg .. 4*kg+3
-          uint32_t r0 = vst[i][0][w], r1 = vst[i][1][w], r2 = vst[i][2][w], r3 = vst[i][3][w];
-          u32x2 lo, hi;
-          lo[0] = __builtin_amdgcn_perm(r1, r0, 0x05040100u);
-          lo[1] = __builtin_amdgcn_perm(r3, r2, 0x05040100u);
-          hi[0] = __builtin_amdgcn_perm(r1, r0, 0x07060302u);
-          hi[1] = __builtin_amdgcn_perm(r3, r2, 0x07060302u);
-          *(u32x2*)(Vt + (8 * dc + 2 * w) * VT_PITCH + pos) = lo;
-          *(u32x2*)(Vt + (8 * dc + 2 * w + 1) * VT_PITCH + pos) = hi;
-        }
-      }
+    for (int i = 0; i < NLD; i++) {
+      *(u32x4*)(Ks + lrow[i] * K_PITCH + 8 * lcol[i]) = kst[i];
+      *(u32x4*)(Vs + lrow[i] * V_PITCH + 8 * lcol[i]) = vst[i];
     }
   };
+
+  // lane-invariant part of the LDS operand addresses
+  const int k_lane = lq * K_PITCH + 8 * lh;                                              // elements
+  const int v_lane = (4 * lh + ((lane & 15) >> 2)) * V_PITCH + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);  // elements
 
   load_tile(0);
+  store_tile(0);
+  if (ntiles_kv > 1) load_tile(BN);
+  __syncthreads();
+
   for (int jt = 0; jt < ntiles_kv; jt++) {
     const int kv0 = jt * BN;
-    __syncthreads();  // every wavefront is done reading the previous tile
-    store_tile();
-    __syncthreads();
-    if (jt + 1 < ntiles_kv) load_tile(kv0 + BN);
-
-    if (CAUSAL && kv0 > qw0 + 31) continue;  // the whole tile is above this wavefront's diagonal
-
-    // ---- S^T = K . Q^T ------------------------------------------------------------------------------------------
-    f32x16 sacc[2];
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) sacc[blk][r] = 0.f;
-      const T* krow = Ks + (32 * blk + lq) * K_PITCH + 8 * lh;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-        vec8 ka = *(const vec8*)(krow + 16 * ks);
-        sacc[blk] = TR::mfma32(ka, qreg[ks], sacc[blk]);
-      }
+    const int cur = jt & 1;
+    if (jt + 1 < ntiles_kv) {
+      store_tile(cur ^ 1);  // stage cur^1 was last read before the barrier that ended the previous iteration
+      if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BN);
     }
 
-    // ---- mask the diagonal / ragged tile -------------------------------------------------------------------------
-    const bool need_mask = (CAUSAL && kv0 + BN - 1 > qw0) || (kv0 + BN > a.S);
-    if (need_mask) {
-      const int qi = qw0 + lq;
+    if (!CAUSAL || kv0 <= qw0 + 31) {  // else: the whole tile is above this wavefront's diagonal
+      const T* Ks = smem + cur * Lds::STAGE;
+      const T* Vs = Ks + BN * K_PITCH;
+
+      // ---- S^T = K . Q^T ----------------------------------------------------------------------------------------
+      f32x16 sacc[2];
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[blk][r] = 0.f;
+        const T* krow = Ks + k_lane + 32 * blk * K_PITCH;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) {
+          vec8 ka = *(const vec8*)(krow + 16 * ks);
+          sacc[blk] = TR::mfma32(ka, qreg[ks], sacc[blk]);
+        }
+      }
+
+      // ---- mask the diagonal / ragged tile -----------------------------------------------------------------------
+      const bool need_mask = (CAUSAL && kv0 + BN - 1 > qw0) || (kv0 + BN > a.S);
+      if (need_mask) {
+        const int qi = qw0 + lq;
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            int key = kv0 + 32 * blk + 8 * (r >> 2) + 4 * lh + (r & 3);
+            bool hidden = key >= a.S || (CAUSAL && key > qi);
+            if (hidden) sacc[blk][r] = -INFINITY;
+          }
+      }
+
+      // ---- online softmax with a lazily raised maximum ---------------------------------------------------------------
+      float mloc = sacc[0][0];
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, sacc[blk][r]);
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+      if (__builtin_amdgcn_ballot_w64(mloc > m_use + lazy) != 0) {  // some row of the wavefront must move its maximum
+        const float m_new = fmaxf(m_use, mloc);
+        const float alpha = fast_exp2((m_use - m_new) * c);
+        m_use = m_new;
+        mc = m_new * c;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DBLK; i++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+      }
+      float psum = 0.f;
 #pragma unroll
       for (int blk = 0; blk < 2; blk++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          int key = kv0 + 32 * blk + 8 * (r >> 2) + 4 * lh + (r & 3);
-          bool hidden = key >= a.S || (CAUSAL && key > qi);
-          if (hidden) sacc[blk][r] = -INFINITY;
+          float p = fast_exp2(fmaf(sacc[blk][r], c, -mc));
+          sacc[blk][r] = p;
+          psum += p;
         }
-    }
+      l_run += psum;
 
-    // ---- online softmax --------------------------------------------------------------------------------------------
-    float mloc = sacc[0][0];
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, sacc[blk][r]);
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    const float m_new = fmaxf(m_run, mloc);
-    const float alpha = fast_exp2((m_run - m_new) * c);
-    const float mc = m_new * c;
-    m_run = m_new;
-    float psum = 0.f;
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float p = fast_exp2(fmaf(sacc[blk][r], c, -mc));
-        sacc[blk][r] = p;
-        psum += p;
-      }
-    l_run = l_run * alpha + psum;
-#pragma unroll
-    for (int i = 0; i < DBLK; i++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
-
-    // ---- P^T as B operands: MFMA t consumes accumulator registers 8*(t%2) .. +7 of block t/2 ------------------------
-    vec8 pb[4];
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-      f32x8 x;
-#pragma unroll
-      for (int i = 0; i < 8; i++) x[i] = sacc[t >> 1][8 * (t & 1) + i];
-      pb[t] = __builtin_convertvector(x, vec8);
-    }
-
-    // ---- O^T += V^T . P^T ---------------------------------------------------------------------------------------------
-#pragma unroll
-    for (int db = 0; db < DBLK; db++) {
-      const T* vrow = Vt + (32 * db + lq) * VT_PITCH + 8 * lh;
+      // ---- P^T as B operands: MFMA t consumes accumulator registers 8*(t%2) .. +7 of block t/2 ------------------------
+      vec8 pb[4];
 #pragma unroll
       for (int t = 0; t < 4; t++) {
-        vec8 va = *(const vec8*)(vrow + 16 * t);
-        oacc[db] = TR::mfma32(va, pb[t], oacc[db]);
+        f32x8 x;
+#pragma unroll
+        for (int i = 0; i < 8; i++) x[i] = sacc[t >> 1][8 * (t & 1) + i];
+        pb[t] = __builtin_convertvector(x, vec8);
+      }
+
+      // ---- O^T += V^T . P^T ---------------------------------------------------------------------------------------------
+      const T* vl = Vs + v_lane;
+#pragma unroll
+      for (int db = 0; db < DBLK; db++) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          vec8 va = v_operand<vec8>(vl, ((16 * t) * V_PITCH + 32 * db) * 2, ((16 * t + 8) * V_PITCH + 32 * db) * 2);
+          oacc[db] = TR::mfma32(va, pb[t], oacc[db]);
+        }
       }
     }
+    __syncthreads();
   }
 
   // ---- normalise and store ----------------------------------------------------------------------------------------------
@@ -269,16 +296,21 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(KArgs a) {
   }
 }
 
+template <typename TR, int D, bool CAUSAL>
+int launch_prefill_k(const KArgs& a, dim3 grid, hipStream_t stream) {
+  // more than 64 KiB of dynamic LDS has to be granted per kernel once
+  static const hipError_t granted = hipFuncSetAttribute((const void*)prefill_kernel<TR, D, CAUSAL>,
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, PrefillLds<D>::BYTES);
+  if (granted != hipSuccess) return (int)granted;
+  hipLaunchKernelGGL((prefill_kernel<TR, D, CAUSAL>), grid, dim3(256), PrefillLds<D>::BYTES, stream, a);
+  return (int)hipGetLastError();
+}
+
 template <typename TR, int D>
 int launch_prefill_t(const KArgs& a, hipStream_t stream) {
   long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM);
-  dim3 grid((unsigned)nwg), block(256);
-  if (a.causal) {
-    hipLaunchKernelGGL((prefill_kernel<TR, D, true>), grid, block, 0, stream, a);
-  } else {
-    hipLaunchKernelGGL((prefill_kernel<TR, D, false>), grid, block, 0, stream, a);
-  }
-  return (int)hipGetLastError();
+  dim3 grid((unsigned)nwg);
+  return a.causal ? launch_prefill_k<TR, D, true>(a, grid, stream) : launch_prefill_k<TR, D, false>(a, grid, stream);
 }
 
 }  // namespace
