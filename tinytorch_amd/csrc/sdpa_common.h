@@ -78,7 +78,8 @@ __device__ __forceinline__ void store_from_float(_Float16* p, float x) { *p = (_
 
 // Host-side launchers (one per kernel family); each returns a hipError_t as int.
 int launch_general(const KArgs& a, int dtype, hipStream_t stream);
-int launch_prefill(const KArgs& a, int dtype, hipStream_t stream);
+int launch_prefill(const KArgs& a, int dtype, hipStream_t stream);       // 128-row workgroups; head_dim 64 or 128
+int launch_prefill_d128(const KArgs& a, int dtype, hipStream_t stream);  // 256-row workgroups, pipelined; head_dim 128
 int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream);
 int launch_zero(const KArgs& a, int dtype, hipStream_t stream);
 
