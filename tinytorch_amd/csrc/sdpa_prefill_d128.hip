@@ -8,7 +8,7 @@
 // Work split.  A workgroup of 8 wavefronts owns 256 query rows of one (batch, query head), 32 rows per wavefront,
 // two wavefronts per SIMD.  Keys/values are consumed in tiles of 64 rows shared by the 8 wavefronts.
 //
-// LDS.  Four K stages and three V stages of 16 KiB, filled by direct global->LDS loads (global_load_lds_dwordx4: no
+// LDS.  Four K stages and four V stages of 16 KiB, filled by direct global->LDS loads (global_load_lds_dwordx4: no
 // staging registers, no ds_write).  Such a load deposits the 64 lanes' 16-byte pieces contiguously, so rows cannot
 // be padded; instead the 16-byte chunk c of tile row r is stored at chunk slot c ^ f(r), f(r) = (r%4)*4 + (r/4)%4,
 // which makes both access patterns below bank-conflict free.  The swizzle is applied on the global side (a lane
@@ -26,8 +26,8 @@
 //                                                 index on both sides)
 // Software pipeline: the S^T MFMAs of half h+1 are issued in the same straight-line block as the exponentials of
 // half h, and the row maximum of half h+1 is taken while the P.V MFMAs of half h run, so the matrix pipe works under
-// the vector work.  K tiles are requested three tiles before use (four stages), V tiles two (three stages); one
-// barrier per 64-key tile.
+// the vector work.  K and V tiles are requested three tiles before use (four stages each); one barrier per 64-key
+// tile.
 // The running maximum m is raised only when a half's maximum exceeds it by more than 2^8 in the exponent (the
 // probabilities stay <= 256), so the accumulator rescale is rare.
 // Causal masking (key j visible to query i iff j <= i, reference src/Operation/OpTransformCpu.h:202-209) skips
@@ -48,7 +48,7 @@ constexpr int BM = NW * WM;  // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
 constexpr int ROW_BYTES = D * 2;
 constexpr int STAGE_BYTES = BN * ROW_BYTES;  // 16 KiB
-constexpr int KSTAGES = 4, VSTAGES = 3;     // K is fetched three tiles ahead of its use, V two
+constexpr int KSTAGES = 4, VSTAGES = 4;     // K and V tiles are requested three tiles before use
 constexpr int LDS_BYTES = (KSTAGES + VSTAGES) * STAGE_BYTES;
 constexpr float kLazyExp = 8.f;
 
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     ld_koff[i] = (unsigned)(row * a.ks[2] + 8 * chunk) * 2u;
     ld_voff[i] = (unsigned)(row * a.vs[2] + 8 * chunk) * 2u;
   }
-  auto dma_tile = [&](const T* base, long long rstride, const unsigned (&off)[2], int kv0, char* stage) {
+  auto dma_tile = [&](const T* base, long long rstride, const unsigned (&off)[2], int kv0, char* stage) __attribute__((always_inline)) {
     const char* src = (const char*)(base + kv0 * rstride);
     if (kv0 + BN <= a.S) {
 #pragma unroll
@@ -149,11 +149,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       }
     }
   };
-  auto dma_k = [&](int tile, int stage) { dma_tile(kp, a.ks[2], ld_koff, tile * BN, smem + stage * STAGE_BYTES); };
-  auto dma_v = [&](int tile, int stage) { dma_tile(vp, a.vs[2], ld_voff, tile * BN, smem + (KSTAGES + stage) * STAGE_BYTES); };
+  auto dma_k = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(kp, a.ks[2], ld_koff, tile * BN, smem + stage * STAGE_BYTES); };
+  auto dma_v = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(vp, a.vs[2], ld_voff, tile * BN, smem + (KSTAGES + stage) * STAGE_BYTES); };
   // Wait until at most `keep` of this wavefront's global->LDS loads are still in flight (they complete in issue
   // order), then meet the other wavefronts: what was issued before the newest `keep` loads is visible to all.
-  auto dma_wait_and_sync = [&](int keep) {
+  auto dma_wait_and_sync = [&](int keep) __attribute__((always_inline)) {
     if (keep >= 4) {
       asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     } else if (keep >= 2) {
@@ -184,7 +184,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #pragma unroll
       for (int db = 0; db < 4; db++) {
         int chunk = 4 * db + 2 * dhalf + ((s & 3) >> 1);
-        v_addr[db][ld] = (unsigned)(row * ROW_BYTES + 16 * (chunk ^ swz(row)) + 8 * (s & 1));
+        // the V region's base is folded in here so that stage and k-step offsets fit the 16-bit ds_read immediate
+        v_addr[db][ld] = (unsigned)(KSTAGES * STAGE_BYTES + row * ROW_BYTES + 16 * (chunk ^ swz(row)) + 8 * (s & 1));
       }
     }
   }
@@ -195,6 +196,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   if (ntiles_kv > 1) dma_k(1, 1);
   if (ntiles_kv > 1) dma_v(1, 1);
   if (ntiles_kv > 2) dma_k(2, 2);
+  if (ntiles_kv > 2) dma_v(2, 2);
 
   vec8 qreg[8];
   {
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   float l_run = 0.f;
 
   // S^T of one half tile (32 keys); kh = LDS address of the half's first K row
-  auto qk_half = [&](f32x16& s, const char* kh) {
+  auto qk_half = [&](f32x16& s, const char* kh) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < 16; r++) s[r] = 0.f;
 #pragma unroll
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     }
   };
 
-  auto mask_half = [&](f32x16& s, int kv0) {
+  auto mask_half = [&](f32x16& s, int kv0) __attribute__((always_inline)) {
     const int qi = qw0 + lq;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
@@ -237,7 +239,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     }
   };
 
-  auto row_max = [&](const f32x16& s) {
+  auto row_max = [&](const f32x16& s) __attribute__((always_inline)) {
     float m = s[0];
 #pragma unroll
     for (int r = 1; r < 16; r++) m = fmaxf(m, s[r]);
@@ -245,7 +247,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
 
   // raise the running maximum when some row needs it (rare), rescaling sum and accumulator
-  auto raise_max = [&](float mx) {
+  auto raise_max = [&](float mx) __attribute__((always_inline)) {
     if (__builtin_amdgcn_ballot_w64(mx > m_use + lazy) != 0) {
       const float m_new = fmaxf(m_use, mx);
       const float alpha = fast_exp2((m_use - m_new) * c);
@@ -260,7 +262,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
 
   // exponentials of one half -> P^T as MFMA B operands pb[k-step of 16 keys]
-  auto exp_half = [&](f32x16& s, vec8 (&pb)[2]) {
+  auto exp_half = [&](f32x16& s, vec8 (&pb)[2]) __attribute__((always_inline)) {
     float psum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
@@ -279,7 +281,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
 
   // O^T += V_half^T . P^T; vh = LDS address of the half's first V row
-  auto pv_half = [&](const vec8 (&pb)[2], const char* vh) {
+  auto pv_half = [&](const vec8 (&pb)[2], const char* vh) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < 2; t++)
 #pragma unroll
@@ -292,7 +294,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
 
   // Pipeline step, fast form: half hb needs no mask and half hb+1 is wanted.
-  auto fast_step = [&](f32x16& cur, float& mcur, f32x16& nxt, float& mnxt, const char* kn, const char* vc) {
+  auto fast_step = [&](f32x16& cur, float& mcur, f32x16& nxt, float& mnxt, const char* kn, const char* vc) __attribute__((always_inline)) {
     raise_max(mcur);
     vec8 pb[2];
     qk_half(nxt, kn);
@@ -302,7 +304,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
   // General form: half hb may be unwanted / masked, half hb+1 may be unwanted.
   auto slow_step = [&](f32x16& cur, float& mcur, f32x16& nxt, float& mnxt, int hb, const char* kn, const char* vc,
-                       bool do_nxt) {
+                       bool do_nxt) __attribute__((always_inline)) {
     const int kv0 = 32 * hb;
     if (do_nxt) qk_half(nxt, kn);
     if (hb < my_halves) {
@@ -323,40 +325,39 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   dma_wait_and_sync(0);
   qk_half(sP, smem);
   mP = row_max(sP);
-  // Stage of tile t: K in t % 4, V in t % 3.  Iteration j reads K(j) (second half), K(j+1) (first half) and V(j),
-  // and sends for K(j+3) and V(j+2), whose stages were last read in iteration j-1.  Its closing barrier publishes
-  // K(j+2) and V(j+1), issued one iteration earlier: only this iteration's own loads may still be in flight.
-  int kst = 0, vst = 0;  // stages of K(j), V(j)
-  auto issue_and_addresses = [&](int j, const char*& kc1, const char*& kn0, const char*& vc) {
+  // Tile t lives in stage t % 4 (K and V alike).  Iteration j reads K(j) (second half), K(j+1) (first half) and
+  // V(j), and sends for K(j+3) and V(j+3), whose stage was last read in iteration j-1.  Its closing barrier publishes
+  // tile j+2, requested one iteration earlier: only this iteration's own loads may still be in flight.
+  // The stage index is a compile-time constant in the unrolled fast loop, so every LDS address there is
+  // lane address + immediate.
+  auto tile_iter = [&](int j, const int st, const bool fast) __attribute__((always_inline)) {
     int keep = 0;
-    if (j + 3 < ntiles_kv) { dma_k(j + 3, (kst + 3) & 3); keep += 2; }
-    if (j + 2 < ntiles_kv) { dma_v(j + 2, vst >= 1 ? vst - 1 : vst + 2); keep += 2; }
-    kc1 = smem + kst * STAGE_BYTES + 32 * ROW_BYTES;
-    kn0 = smem + ((kst + 1) & 3) * STAGE_BYTES;
-    vc = smem + (KSTAGES + vst) * STAGE_BYTES;
-    return keep;
-  };
-  auto advance = [&]() {
-    kst = (kst + 1) & 3;
-    vst = vst == 2 ? 0 : vst + 1;
+    if (j + 3 < ntiles_kv) {
+      dma_k(j + 3, (st + 3) & 3);
+      dma_v(j + 3, (st + 3) & 3);
+      keep = 4;
+    }
+    const char* kc1 = smem + st * STAGE_BYTES + 32 * ROW_BYTES;
+    const char* kn0 = smem + ((st + 1) & 3) * STAGE_BYTES;
+    const char* vc = smem + st * STAGE_BYTES;  // v_addr carries the V region's base
+    if (fast) {
+      fast_step(sP, mP, sN, mN, kc1, vc);
+      fast_step(sN, mN, sP, mP, kn0, vc + 32 * ROW_BYTES);
+    } else {
+      slow_step(sP, mP, sN, mN, 2 * j, kc1, vc, 2 * j + 1 < my_halves);
+      slow_step(sN, mN, sP, mP, 2 * j + 1, kn0, vc + 32 * ROW_BYTES, j + 1 < ntiles_kv && 2 * j + 2 < my_halves);
+    }
+    dma_wait_and_sync(keep);
   };
   int j = 0;
-  for (; j < nfast; j++) {  // tiles that need no mask and whose successor half is wanted: straight-line pipeline
-    const char *kc1, *kn0, *vc;
-    int keep = issue_and_addresses(j, kc1, kn0, vc);
-    fast_step(sP, mP, sN, mN, kc1, vc);
-    fast_step(sN, mN, sP, mP, kn0, vc + 32 * ROW_BYTES);
-    dma_wait_and_sync(keep);
-    advance();
+  for (; j + 4 <= nfast; j += 4) {  // tiles that need no mask and whose successor half is wanted
+    tile_iter(j, 0, true);
+    tile_iter(j + 1, 1, true);
+    tile_iter(j + 2, 2, true);
+    tile_iter(j + 3, 3, true);
   }
-  for (; j < ntiles_kv; j++) {  // tiles on the diagonal, at the end of the keys, or not wanted by this wavefront
-    const char *kc1, *kn0, *vc;
-    int keep = issue_and_addresses(j, kc1, kn0, vc);
-    slow_step(sP, mP, sN, mN, 2 * j, kc1, vc, 2 * j + 1 < my_halves);
-    slow_step(sN, mN, sP, mP, 2 * j + 1, kn0, vc + 32 * ROW_BYTES, j + 1 < ntiles_kv && 2 * j + 2 < my_halves);
-    dma_wait_and_sync(keep);
-    advance();
-  }
+  for (; j < ntiles_kv; j++)  // the rest: diagonal tiles, the ragged end of the keys, tiles this wavefront skips
+    tile_iter(j, j & 3, false);
 
   // ---- normalise and store ----------------------------------------------------------------------------------------------
   {
