@@ -1,0 +1,193 @@
+// C++ test of the host layer on the GPU.  The first case restates TinyTorch's own attention unit test
+// (reference test/test_function.cpp:393-419: same literals, same 1e-3 VectorNear tolerance, reference
+// test/test.h:17-30) with the tensors on the accelerator; the others cover what the drop-in adds or must keep:
+// fp16/bf16 dispatch, grouped-query heads, a decode-shaped call, grad bookkeeping of Function::apply, and the loud
+// failure when a CPU tensor reaches an op that has no CPU slot.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "TinyTorch.h"
+
+using namespace tinytorch;
+
+static int g_failures = 0;
+static int g_asserts = 0;
+
+#define EXPECT_TRUE(x)                                                     \
+  do {                                                                     \
+    if (!(x)) {                                                            \
+      std::printf("  EXPECT_TRUE failed at line %d: %s\n", __LINE__, #x);  \
+      g_failures++;                                                        \
+    }                                                                      \
+  } while (0)
+
+static bool vectorNear(const std::vector<float>& a, const std::vector<float>& b, float eps = 1e-3f) {
+  if (a.size() != b.size()) return false;
+  for (size_t i = 0; i < a.size(); i++) {
+    if (std::isnan(a[i]) || std::isnan(b[i])) return false;
+    if (std::fabs(a[i] - b[i]) > eps) return false;
+  }
+  return true;
+}
+
+static void countingAssertHandler(const char*, const char*, int) { g_asserts++; }
+
+// fp64 closed form softmax(q k^T * scale + causal) v for [B,Hq,L,D] x [B,Hkv,S,D]
+static std::vector<float> closedForm(const std::vector<float>& q, const std::vector<float>& k, const std::vector<float>& v,
+                                     int B, int Hq, int Hkv, int L, int S, int D, bool causal) {
+  std::vector<float> out(static_cast<size_t>(B) * Hq * L * D);
+  const int G = Hq / Hkv;
+  const double scale = 1.0 / std::sqrt(static_cast<double>(D));
+  std::vector<double> w(S);
+  for (int b = 0; b < B; b++)
+    for (int h = 0; h < Hq; h++)
+      for (int i = 0; i < L; i++) {
+        const float* qr = &q[((static_cast<size_t>(b) * Hq + h) * L + i) * D];
+        const size_t kvbase = (static_cast<size_t>(b) * Hkv + h / G) * S * D;
+        double mx = -1e300;
+        for (int j = 0; j < S; j++) {
+          double s = 0;
+          for (int d = 0; d < D; d++) s += static_cast<double>(qr[d]) * k[kvbase + static_cast<size_t>(j) * D + d];
+          s *= scale;
+          if (causal && j > i) s = -INFINITY;
+          w[j] = s;
+          mx = std::fmax(mx, s);
+        }
+        double sum = 0;
+        for (int j = 0; j < S; j++) sum += (w[j] = std::exp(w[j] - mx));
+        for (int d = 0; d < D; d++) {
+          double o = 0;
+          for (int j = 0; j < S; j++) o += w[j] * v[kvbase + static_cast<size_t>(j) * D + d];
+          out[((static_cast<size_t>(b) * Hq + h) * L + i) * D + d] = static_cast<float>(o / sum);
+        }
+      }
+  return out;
+}
+
+static std::vector<float> pseudoRandom(size_t n, uint32_t seed) {
+  std::vector<float> x(n);
+  uint32_t s = seed * 2654435761u + 12345u;
+  for (size_t i = 0; i < n; i++) {
+    s = s * 1664525u + 1013904223u;
+    x[i] = (static_cast<float>((s >> 8) & 0xFFFF) / 65535.f - 0.5f) * 2.f;
+  }
+  return x;
+}
+
+static void test_func_sdpAttention_reference_vectors() {
+  std::printf("func_sdpAttention (reference vectors, GPU)\n");
+  const Options gpu = options::device(DeviceType::GPU);
+  Tensor query(std::vector<float>{0.6201, 0.5199, 0.2614, 0.9816, 0.9369, 0.8059, 0.8578, 0.7864, 0.8947, 0.4272,
+                                  0.7566, 0.2975, 0.4676, 0.1170, 0.1046, 0.7130},
+               {2, 2, 2, 2}, gpu);
+  Tensor key(std::vector<float>{0.8691, 0.8571, 0.9015, 0.3962, 0.7809, 0.0260, 0.7946, 0.6102, 0.0999, 0.9367,
+                                0.3174, 0.1418, 0.6388, 0.4654, 0.5967, 0.3617},
+             {2, 2, 2, 2}, gpu);
+  Tensor value(std::vector<float>{0.9904, 0.8726, 0.8662, 0.3096, 0.4391, 0.9327, 0.5259, 0.6763, 0.6314, 0.8901,
+                                  0.6936, 0.2933, 0.0599, 0.3249, 0.3593, 0.8228},
+               {2, 2, 2, 2}, gpu);
+
+  Tensor y = function::sdpAttention(query, key, value);
+  EXPECT_TRUE(y.shape() == value.shape());
+  EXPECT_TRUE(vectorNear(y.toList<float>(), {0.9331, 0.6129, 0.9380, 0.6349, 0.4899, 0.7828, 0.4897, 0.7833, 0.6609,
+                                             0.6070, 0.6617, 0.5993, 0.2079, 0.5711, 0.2054, 0.5670}));
+
+  y = function::sdpAttention(query, key, value, true);
+  EXPECT_TRUE(y.shape() == value.shape());
+  EXPECT_TRUE(vectorNear(y.toList<float>(), {0.9904, 0.8726, 0.9380, 0.6349, 0.4391, 0.9327, 0.4897, 0.7833, 0.6314,
+                                             0.8901, 0.6617, 0.5993, 0.0599, 0.3249, 0.2055, 0.5670}));
+
+  // Bool mask {{0,0},{1,0}}: query row 1 sees key 0 only; query row 0 sees nothing.  The reference lists 0.0000 for
+  // row 0 but computes 0 * inf = NaN there (its comparison cannot see a NaN); this library returns NaN as well.
+  Tensor mask(std::vector<uint8_t>{0, 0, 1, 0}, {2, 2}, options::device(DeviceType::GPU).dtype(DType::Bool));
+  y = function::sdpAttention(query, key, value, false, mask);
+  EXPECT_TRUE(y.shape() == value.shape());
+  std::vector<float> r = y.toList<float>();
+  const float expectRow1[8] = {0.9904, 0.8726, 0.4391, 0.9327, 0.6314, 0.8901, 0.0599, 0.3249};
+  for (int bh = 0; bh < 4; bh++) {
+    EXPECT_TRUE(std::isnan(r[bh * 4 + 0]) && std::isnan(r[bh * 4 + 1]));
+    EXPECT_TRUE(std::fabs(r[bh * 4 + 2] - expectRow1[bh * 2]) <= 1e-3f);
+    EXPECT_TRUE(std::fabs(r[bh * 4 + 3] - expectRow1[bh * 2 + 1]) <= 1e-3f);
+  }
+}
+
+static void test_half_dtypes_and_gqa() {
+  std::printf("bf16 / fp16 dispatch, grouped-query heads, decode shape\n");
+  struct Case { int B, Hq, Hkv, L, S, D; bool causal; DType dt; };
+  const Case cases[] = {{1, 8, 2, 160, 160, 128, true, DType::BFloat16},
+                        {2, 4, 4, 96, 96, 128, true, DType::Float16},
+                        {2, 8, 2, 1, 700, 128, false, DType::BFloat16},
+                        {1, 4, 2, 40, 56, 64, false, DType::Float32}};
+  for (const Case& c : cases) {
+    std::vector<float> q = pseudoRandom(static_cast<size_t>(c.B) * c.Hq * c.L * c.D, 1);
+    std::vector<float> k = pseudoRandom(static_cast<size_t>(c.B) * c.Hkv * c.S * c.D, 2);
+    std::vector<float> v = pseudoRandom(static_cast<size_t>(c.B) * c.Hkv * c.S * c.D, 3);
+    const Options o = options::device(DeviceType::GPU).dtype(c.dt);
+    Tensor tq(q, {c.B, c.Hq, c.L, c.D}, o), tk(k, {c.B, c.Hkv, c.S, c.D}, o), tv(v, {c.B, c.Hkv, c.S, c.D}, o);
+    // the closed form sees the values the device sees (after rounding to the 16-bit type)
+    std::vector<float> ref = closedForm(tq.toList<float>(), tk.toList<float>(), tv.toList<float>(), c.B, c.Hq, c.Hkv,
+                                        c.L, c.S, c.D, c.causal);
+    Tensor y = function::sdpAttention(tq, tk, tv, c.causal);
+    EXPECT_TRUE(y.defined() && y.dtype() == c.dt && y.shape() == tq.shape());
+    EXPECT_TRUE(vectorNear(y.toList<float>(), ref, c.dt == DType::Float32 ? 1e-4f : 2e-2f));
+  }
+}
+
+static void test_grad_bookkeeping_and_errors() {
+  std::printf("Function::apply bookkeeping, dispatcher failure, allocator reuse\n");
+  const Options gpu = options::device(DeviceType::GPU).dtype(DType::BFloat16);
+  Tensor q = Tensor::ones({1, 2, 16, 128}, gpu), k = Tensor::ones({1, 2, 16, 128}, gpu), v = Tensor::ones({1, 2, 16, 128}, gpu);
+  Tensor y = function::sdpAttention(q, k, v, true);
+  EXPECT_TRUE(!y.requiresGrad() && y.gradFn() == nullptr);
+  q.setRequiresGrad(true);
+  y = function::sdpAttention(q, k, v, true);
+  EXPECT_TRUE(y.requiresGrad() && y.gradFn() != nullptr);
+  {
+    NoGradGuard guard;
+    Tensor z = function::sdpAttention(q, k, v, true);
+    EXPECT_TRUE(!z.requiresGrad() && z.gradFn() == nullptr);
+  }
+  std::vector<float> ones = y.toList<float>();
+  bool allOne = true;
+  for (float f : ones) allOne = allOne && std::fabs(f - 1.f) < 1e-2f;
+  EXPECT_TRUE(allOne);
+
+  // backward is not implemented (as in the reference): it must fail through ASSERT
+  AssertHandler old = setAssertHandler(countingAssertHandler);
+  int before = g_asserts;
+  y.gradFn()->backward(y);
+  EXPECT_TRUE(g_asserts == before + 1);
+  // a CPU tensor has no implementation behind op::sdpAttention: loud failure, undefined result
+  Tensor cq = Tensor::ones({1, 1, 4, 64}, options::device(DeviceType::CPU));
+  before = g_asserts;
+  Tensor bad = function::sdpAttention(cq, cq, cq);
+  EXPECT_TRUE(g_asserts > before && !bad.defined());
+  // causal together with a mask is rejected before anything is launched (reference FuncNNLayer.h:242)
+  Tensor m = Tensor::ones({16, 16}, options::device(DeviceType::GPU).dtype(DType::Bool));
+  before = g_asserts;
+  bad = function::sdpAttention(q, k, v, true, m);
+  EXPECT_TRUE(g_asserts > before && !bad.defined());
+  setAssertHandler(old);
+
+  // repeated calls reuse cached device blocks instead of growing the pool
+  synchronizeCurrentStream(0);
+  size_t live0 = deviceAllocatorLiveBytes(0);
+  for (int i = 0; i < 8; i++) (void)function::sdpAttention(q, k, v, true);
+  synchronizeCurrentStream(0);
+  EXPECT_TRUE(deviceAllocatorLiveBytes(0) == live0);
+}
+
+int main() {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
+    std::printf("no GPU visible\n");
+    return 2;
+  }
+  test_func_sdpAttention_reference_vectors();
+  test_half_dtypes_and_gqa();
+  test_grad_bookkeeping_and_errors();
+  std::printf(g_failures == 0 ? "ALL PASSED\n" : "%d FAILURES\n", g_failures);
+  return g_failures == 0 ? 0 : 1;
+}

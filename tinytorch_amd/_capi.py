@@ -54,6 +54,9 @@ def lib():
             raise ImportError(
                 "tinytorch_amd: %s is missing — build it with `make -C tinytorch_amd/csrc` "
                 "(or __graft_entry__.build()); there is no fallback path" % LIB_PATH)
+        # torch ships its own HIP runtime (same SONAME as the system one).  Device pointers and streams handed to the
+        # library come from torch, so the library must bind to that copy: load torch's first.
+        import torch  # noqa: F401
         L = ctypes.CDLL(LIB_PATH)
         P = ctypes.POINTER(Params)
         L.ttsdpa_abi_version.restype = ctypes.c_int

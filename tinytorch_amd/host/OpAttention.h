@@ -1,0 +1,25 @@
+// Tensor-level attention op, declared and registered the way the reference adds a fused op (DEFINE_OP +
+// REGISTER_OP_IMPL per {device, dtype}; precedent reference src/Operation/OpFused.h:14-32, OpFusedCuda.cu:11-22).
+// The reference has no such op: its FuncSDPAttention::forward composes ~11 generic ops
+// (src/Function/FuncNNLayer.h:231-266).  Here the GPU slot of the table holds one implementation that hands the
+// whole forward to the C ABI of include/ttsdpa.h.  The CPU slot is deliberately empty: a CPU tensor reaching this op
+// fails loudly through the dispatcher instead of taking another route.
+#pragma once
+
+#include "Dispatch.h"
+
+namespace tinytorch::op {
+
+// query [B,Hq,L,D] (or [Hq,L,D]); key/value [B,Hkv,S,D] with Hq a multiple of Hkv (query head h reads KV head
+// h / (Hq/Hkv); Hkv == Hq is the reference's layout).  isCausal is top-left aligned, exclusive with attnMask.
+// attnMask: undefined, Bool [L,S] (false = hidden) or the query dtype [L,S] (added to the scores).
+// dropoutP must be 0.  Returns [B,Hq,L,D] in the query dtype, or an undefined Tensor after a failed ASSERT.
+using SdpAttentionOpFn = Tensor (*)(const Tensor& query, const Tensor& key, const Tensor& value, bool isCausal,
+                                    const Tensor& attnMask, float dropoutP, float scale);
+
+DEFINE_OP(sdpAttention, SdpAttentionOpFn)
+
+void registerAttentionGpu();
+STATIC_CALL(registerAttentionGpu);
+
+}  // namespace tinytorch::op
