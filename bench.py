@@ -54,6 +54,16 @@ def algorithmic_work(B, Hq, Hkv, L, S, D, dtype, causal):
     return flops, nbytes
 
 
+def measured_traffic(name):
+    """HBM bytes per launch of the workload's dominant kernel, as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    (profiles/traffic.json holds the figures and the commands that produced them); None when not measured."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        return json.load(f).get(name, {}).get("hbm_bytes_per_launch")
+
+
 def run_gpu(name, steps, warmup):
     import torch
     from tinytorch_amd import _capi, build_params
@@ -102,7 +112,7 @@ def run_gpu(name, steps, warmup):
         "workload": name, "description": DESCR[name], "route": _capi.ROUTE_NAMES[route], "dtype": dtype,
         "value": round(value, 3), "unit": unit, "ms_per_step": round(wall_ms, 5),
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "frac": round(achieved / peak, 4), "traffic": measured_traffic(name),
                      "kernel_ms": round(dev_ms, 5), "algorithmic_flops": flops, "algorithmic_bytes": abytes},
     }
     return res, (q, k, v, out)
@@ -157,6 +167,9 @@ def main():
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one device-to-device copy of 1 GiB (a kernel of known traffic that calibrates "
+                         "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the attention path shards by batch / KV head with no "
@@ -165,6 +178,12 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback.")
 
+    if args.copy_probe:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     main_res, tensors = run_gpu(args.workload, args.steps, args.warmup)
     cpu = None if args.no_cpu else run_cpu_baseline(args.workload, tensors, args.cpu_seconds)
     del tensors
