@@ -74,8 +74,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   const int lh = lane >> 5;
 
   // ---- workgroup -> (batch, kv head, query head in group, row tile) -------------------------------------------
+  // Under a causal mask a workgroup takes row tile t and then its mirror ntile-1-t: every workgroup sees the same
+  // number of KV tiles, so the launch has no long tail behind the heavy tiles.
   const int ntile = (a.L + BM - 1) / BM;
-  const int inner = a.G * ntile;
+  const int nslot = CAUSAL ? (ntile + 1) / 2 : ntile;
+  const int inner = a.G * nslot;
   const int npair = a.B * a.Hkv;
   int pair, in;
   {
@@ -91,14 +94,18 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }
   const int b = pair / a.Hkv, hk = pair % a.Hkv;
   const int g = in % a.G;
-  const int rt = CAUSAL ? ntile - 1 - in / a.G : in / a.G;  // longest rows first
+  const int slot_rt = in / a.G;
   const int h = hk * a.G + g;
-  const int q0 = rt * BM;
-  const int qw0 = q0 + wave * WM;
 
   const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
   const T* kp = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
   const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
+
+  for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
+  const int rt = (CAUSAL && part == 0) ? ntile - 1 - slot_rt : slot_rt;  // the long tile first
+  if (part == 1 && slot_rt >= ntile - 1 - slot_rt) break;                  // odd count: the middle tile has no mirror
+  const int q0 = rt * BM;
+  const int qw0 = q0 + wave * WM;
 
   int ntiles_kv = (a.S + BN - 1) / BN;
   if (CAUSAL) {
@@ -243,7 +250,10 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     float m = s[0];
 #pragma unroll
     for (int r = 1; r < 16; r++) m = fmaxf(m, s[r]);
-    return fmaxf(m, __shfl_xor(m, 32));
+    // the other 16 keys of this query sit in lane l^32: exchange the wavefront halves on the vector ALU
+    const unsigned u = __builtin_bit_cast(unsigned, m);
+    const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
   };
 
   // raise the running maximum when some row needs it (rare), rescaling sum and accumulator
@@ -378,6 +388,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
         }
     }
   }
+  }  // part
 }
 
 template <typename TR, bool CAUSAL>
@@ -392,7 +403,8 @@ int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
 }  // namespace
 
 int launch_prefill_d128(const KArgs& a, int dtype, hipStream_t stream) {
-  long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM);
+  const int ntile = (a.L + BM - 1) / BM;
+  long long nwg = (long long)a.B * a.Hq * (a.causal ? (ntile + 1) / 2 : ntile);
   dim3 grid((unsigned)nwg);
   if (dtype == 1) return a.causal ? launch_k<F16, true>(a, grid, stream) : launch_k<F16, false>(a, grid, stream);
   return a.causal ? launch_k<BF16, true>(a, grid, stream) : launch_k<BF16, false>(a, grid, stream);
