@@ -107,7 +107,9 @@ def test_kernel_domains_and_workspace():
     fp32 = params(_capi.F32, 1, 4, 4, 128, 128, 64)
     assert L.ttsdpa_prefill(ctypes.byref(fp32), None) == _capi.ERR_UNSUPPORTED
     assert L.ttsdpa_decode(ctypes.byref(fp32), None, 0, None) == _capi.ERR_UNSUPPORTED
-    dec = params(_capi.BF16, 64, 32, 8, 1, 8192, 128)
+    # config 4 has 512 (batch, kv head) pairs: enough workgroups without splitting the cache, hence no scratch
+    assert L.ttsdpa_workspace_bytes(ctypes.byref(params(_capi.BF16, 64, 32, 8, 1, 8192, 128))) == 0
+    dec = params(_capi.BF16, 2, 32, 8, 1, 8192, 128)  # few pairs: the cache is split and partials need scratch
     need = L.ttsdpa_workspace_bytes(ctypes.byref(dec))
     assert need > 0 and need % 4 == 0
     assert L.ttsdpa_decode(ctypes.byref(dec), None, 0, None) == _capi.ERR_WORKSPACE
