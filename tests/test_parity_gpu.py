@@ -111,6 +111,21 @@ def test_prefill_against_oracle(case):
     assert rc == 0 and max_abs_err(out2, exp) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("entry,shape", [("prefill", (1, 4, 2, 512, 512, 128)), ("prefill", (1, 2, 2, 200, 200, 64)),
+                                         ("decode", (2, 8, 2, 1, 2048, 128))])
+def test_large_score_range(entry, shape):
+    """Inputs scaled so that scores spread over hundreds of units: the running maximum has to follow every tile
+    (a maximum taken over only part of a row's keys would overflow the exponentials)."""
+    B, Hq, Hkv, L, S, D = shape
+    host, dev = make_inputs(4242, B, Hq, Hkv, L, S, D, "bf16", mul=6.0)
+    causal = entry == "prefill"
+    exp = oracle.sdpa_f32(*host, causal=causal)
+    rc, out = call(entry, *dev, causal=causal)
+    assert rc == 0
+    # values are 6x larger: the 2e-2 bar is relative to unit-variance inputs, scale it with the value range
+    assert max_abs_err(out, exp) <= 6.0 * TOL["bf16"]
+
+
 def test_prefill_custom_scale_and_strided_views():
     B, Hq, Hkv, L, S, D = 2, 4, 2, 160, 160, 128
     host, dev = make_inputs(77, B, Hq, Hkv, L, S, D, "bf16")

@@ -250,10 +250,12 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     float m = s[0];
 #pragma unroll
     for (int r = 1; r < 16; r++) m = fmaxf(m, s[r]);
-    // the other 16 keys of this query sit in lane l^32: exchange the wavefront halves on the vector ALU
-    const unsigned u = __builtin_bit_cast(unsigned, m);
-    const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+    // The other 16 keys of this query sit in lane l^32.  v_permlane32_swap exchanges the upper 32 lanes of its
+    // first operand with the lower 32 lanes of its second, so two copies of m become (lower half, lower half) and
+    // (upper half, upper half).  Written as asm: the compiler folds the two results of the builtin into one.
+    unsigned lo = __builtin_bit_cast(unsigned, m), hi = lo;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+    return fmaxf(__builtin_bit_cast(float, lo), __builtin_bit_cast(float, hi));
   };
 
   // raise the running maximum when some row needs it (rare), rescaling sum and accumulator
