@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TTSDPA_ABI_VERSION 1
+#define TTSDPA_ABI_VERSION 2
 
 /* Element types; numbering is the reference's DType enum (reference src/Tensor/DType.h:20-28). */
 enum ttsdpa_dtype { TTSDPA_F32 = 0, TTSDPA_F16 = 1, TTSDPA_BF16 = 2 };
@@ -71,7 +71,11 @@ enum ttsdpa_route {
  * {H*N*D, N*D, D}.
  * causal: key j is visible to query i iff j <= i (top-left aligned, tril(ones(L,S),0), reference
  * src/Function/FuncNNLayer.h:241-247) — a decode step with L == 1 must therefore pass causal = 0.
- * mask: [L,S] dense, or NULL.  scale multiplies q.k^T before the bias; the reference default is 1/sqrt(D).
+ * mask: NULL, or an attnMask of any shape that broadcasts to [B,Hq,L,S] — the reference adds it to the scores with
+ * a broadcasting add (src/Function/FuncNNLayer.h:249-260).  mask_stride gives its element strides along
+ * {batch, head, query row, key}; an axis the mask does not have, or has with size 1, gets stride 0.  A dense
+ * [L,S] mask is {0, 0, S, 1} (what ttsdpa_params_init fills), a per-batch key-padding mask [B,1,1,S] is {S, 0, 0, 1}.
+ * scale multiplies q.k^T before the bias; the reference default is 1/sqrt(D).
  */
 typedef struct ttsdpa_params {
   uint32_t struct_size; /* sizeof(ttsdpa_params) */
@@ -89,6 +93,7 @@ typedef struct ttsdpa_params {
   int32_t causal;
   int32_t mask_kind; /* ttsdpa_mask_kind */
   const void* mask;
+  int64_t mask_stride[4]; /* elements: batch, head, query row, key; 0 broadcasts the axis */
 } ttsdpa_params;
 
 /* Library identification.  No counterpart in the reference (its device ops are linked statically). */
@@ -96,7 +101,7 @@ int ttsdpa_abi_version(void);
 const char* ttsdpa_status_string(int status);
 
 /* Fill *p for dense tensors: sizes, dense strides, scale = 1/sqrt(D) (reference src/Function/FuncNNLayer.h:235),
- * no mask, not causal.  Pointers are left NULL. */
+ * no mask, not causal, mask strides of a dense [L,S] mask.  Pointers are left NULL. */
 void ttsdpa_params_init(ttsdpa_params* p, int dtype, int B, int Hq, int Hkv, int L, int S, int D);
 
 /* Validate *p and report the kernel ttsdpa_forward would pick (enum ttsdpa_route) in *route.  Launches nothing and

@@ -68,7 +68,8 @@ def ref():
         R.tt_ref_round_trip.argtypes = [_c_f32p, _c_f32p, _i64, ctypes.c_int]
         R.tt_ref_round_trip.restype = ctypes.c_int
         R.tt_ref_sdpa_f32.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p] + [_i64] * 6 + [
-            ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_void_p]
+            ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
+            ctypes.POINTER(ctypes.c_int64)]
         R.tt_ref_sdpa_f32.restype = ctypes.c_int
         R.tt_ref_sdpa_f32_gqa5d.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p] + [_i64] * 6 + [ctypes.c_int]
         R.tt_ref_sdpa_f32_gqa5d.restype = ctypes.c_int
@@ -123,7 +124,7 @@ def _dims(q, k, v):
     return B, Hq, Hkv, L, S, D
 
 
-def _mask_args(mask, L, S):
+def _mask_args(mask, L, S, any_shape=False):
     if mask is None:
         return MASK_NONE, None, None
     if mask.dtype == np.bool_ or mask.dtype == np.uint8:
@@ -132,7 +133,7 @@ def _mask_args(mask, L, S):
     else:
         m = _f32(mask)
         kind = MASK_FLOAT
-    assert m.shape == (L, S)
+    assert any_shape or m.shape == (L, S)
     return kind, m, ctypes.c_void_p(m.ctypes.data)
 
 
@@ -141,6 +142,17 @@ def sdpa_f32(q, k, v, causal=False, scale=None, mask=None, nthreads=None):
     q, k, v = _f32(q), _f32(k), _f32(v)
     B, Hq, Hkv, L, S, D = _dims(q, k, v)
     sc = np.float32(1.0) / np.sqrt(np.float32(D)) if scale is None else np.float32(scale)
+    if mask is not None and tuple(mask.shape) != (L, S):
+        # attnMask of another shape: the reference's bias add broadcasts it over [B,Hq,L,S] (reference
+        # src/Function/FuncNNLayer.h:249-260), so every (batch, head) slice sees its own [L,S] slice of the mask.
+        full = np.broadcast_to(mask, (B, Hq, L, S))
+        G = Hq // Hkv
+        out = np.empty(q.shape, dtype=np.float32)
+        for b in range(B):
+            for h in range(Hq):
+                out[b, h] = sdpa_f32(q[b:b + 1, h:h + 1], k[b:b + 1, h // G:h // G + 1], v[b:b + 1, h // G:h // G + 1],
+                                     scale=sc, mask=np.ascontiguousarray(full[b, h]), nthreads=nthreads)[0, 0]
+        return out
     kind, keep, mp = _mask_args(mask, L, S)
     out = np.empty(q.shape, dtype=np.float32)
     rc = lib().oracle_sdpa_f32(_p(q), _p(k), _p(v), _p(out), B, Hq, Hkv, L, S, D, int(bool(causal)), float(sc), kind,
@@ -168,10 +180,12 @@ def ref_sdpa_f32(q, k, v, causal=False, scale=None, mask=None):
     """tinytorch::function::sdpAttention of the compiled reference (single-threaded, fp32 CPU)."""
     q, k, v = _f32(q), _f32(k), _f32(v)
     B, Hq, Hkv, L, S, D = _dims(q, k, v)
-    kind, keep, mp = _mask_args(mask, L, S)
+    kind, keep, mp = _mask_args(mask, L, S, any_shape=True)
+    mdims = (ctypes.c_int64 * 8)(*(keep.shape if keep is not None else ()))
     out = np.empty(q.shape, dtype=np.float32)
     rc = ref().tt_ref_sdpa_f32(_p(q), _p(k), _p(v), _p(out), B, Hq, Hkv, L, S, D, int(bool(causal)),
-                               0 if scale is None else 1, 0.0 if scale is None else float(scale), kind, mp)
+                               0 if scale is None else 1, 0.0 if scale is None else float(scale), kind, mp,
+                               keep.ndim if keep is not None else 0, mdims)
     if rc != 0:
         raise RuntimeError("tt_ref_sdpa_f32 failed: %d" % rc)
     return out

@@ -55,11 +55,12 @@ int tt_ref_round_trip(const float* in, float* out, int64_t n, int dtype) {
 //   q [B,Hq,L,D]; k,v [B,Hkv,S,D]; out [B,Hq,L,D].
 //   Hkv != Hq: grouped-query attention through op::repeatInterleave(k, Hq/Hkv, 1)
 //   (reference src/Operation/OpTransformCpu.h:399-442), i.e. kv_head = q_head / (Hq/Hkv).
-//   mask_kind: 0 none, 1 Bool [mask_rows,S] (uint8 0/1), 2 additive float [mask_rows,S]; mask_rows is L.
+//   mask_kind: 0 none, 1 Bool (uint8 0/1), 2 additive float; the mask has shape mask_dims[0..mask_ndim) (any shape
+//   that broadcasts to [B,Hq,L,S]; mask_ndim == 0 means [L,S]).
 //   has_scale == 0 -> default 1/sqrt(D).
 int tt_ref_sdpa_f32(const float* q, const float* k, const float* v, float* out, int64_t B, int64_t Hq, int64_t Hkv,
                     int64_t L, int64_t S, int64_t D, int causal, int has_scale, float scale, int mask_kind,
-                    const void* mask) {
+                    const void* mask, int mask_ndim, const int64_t* mask_dims) {
   ensureCpu();
   NoGradGuard guard;
   Tensor tq = fromF32(q, {B, Hq, L, D});
@@ -71,13 +72,17 @@ int tt_ref_sdpa_f32(const float* q, const float* k, const float* v, float* out, 
     tv = op::repeatInterleave(tv, Hq / Hkv, 1);
   }
   Tensor tm;
+  std::vector<int64_t> mshape = {L, S};
+  if (mask_ndim > 0) mshape.assign(mask_dims, mask_dims + mask_ndim);
+  int64_t mcount = 1;
+  for (int64_t d : mshape) mcount *= d;
   if (mask_kind == 1) {
     const auto* m = static_cast<const uint8_t*>(mask);
-    std::vector<uint8_t> buf(m, m + L * S);
+    std::vector<uint8_t> buf(m, m + mcount);
     tm = Tensor(buf, options::dtype(DType::Bool));
-    tm.reshape_({L, S});
+    tm.reshape_(IntArrayView(mshape));
   } else if (mask_kind == 2) {
-    tm = fromF32(static_cast<const float*>(mask), {L, S});
+    tm = fromF32(static_cast<const float*>(mask), mshape);
   }
   std::optional<float> sc = has_scale ? std::optional<float>(scale) : std::nullopt;
   Tensor y = function::sdpAttention(tq, tk, tv, causal != 0, tm, 0.f, sc);

@@ -135,6 +135,47 @@ static void test_half_dtypes_and_gqa() {
   }
 }
 
+static void test_broadcast_masks() {
+  std::printf("attnMask shapes that broadcast to [B,H,L,S]\n");
+  const int B = 2, Hq = 4, Hkv = 2, L = 9, S = 40, D = 32, keep = 23;
+  std::vector<float> q = pseudoRandom(static_cast<size_t>(B) * Hq * L * D, 4);
+  std::vector<float> k = pseudoRandom(static_cast<size_t>(B) * Hkv * S * D, 5);
+  std::vector<float> v = pseudoRandom(static_cast<size_t>(B) * Hkv * S * D, 6);
+  const Options gpu = options::device(DeviceType::GPU);
+  Tensor tq(q, {B, Hq, L, D}, gpu), tk(k, {B, Hkv, S, D}, gpu), tv(v, {B, Hkv, S, D}, gpu);
+  // key padding [B,1,1,S]: batch 0 sees every key, batch 1 the first `keep`
+  std::vector<uint8_t> pad(static_cast<size_t>(B) * S, 1);
+  for (int j = keep; j < S; j++) pad[S + j] = 0;
+  Tensor tpad(pad, {B, 1, 1, S}, options::device(DeviceType::GPU).dtype(DType::Bool));
+  std::vector<float> y = function::sdpAttention(tq, tk, tv, false, tpad).toList<float>();
+  std::vector<float> full = closedForm(q, k, v, B, Hq, Hkv, L, S, D, false);
+  // batch 1 against the closed form over its first `keep` keys only
+  std::vector<float> k1(static_cast<size_t>(Hkv) * keep * D), v1(k1.size());
+  for (int h = 0; h < Hkv; h++)
+    for (int j = 0; j < keep; j++)
+      for (int d = 0; d < D; d++) {
+        k1[(static_cast<size_t>(h) * keep + j) * D + d] = k[((static_cast<size_t>(Hkv) + h) * S + j) * D + d];
+        v1[(static_cast<size_t>(h) * keep + j) * D + d] = v[((static_cast<size_t>(Hkv) + h) * S + j) * D + d];
+      }
+  const size_t half = static_cast<size_t>(Hq) * L * D;
+  std::vector<float> q1(q.begin() + half, q.end());
+  std::vector<float> cut = closedForm(q1, k1, v1, 1, Hq, Hkv, L, keep, D, false);
+  EXPECT_TRUE(vectorNear(std::vector<float>(y.begin(), y.begin() + half), std::vector<float>(full.begin(), full.begin() + half), 1e-4f));
+  EXPECT_TRUE(vectorNear(std::vector<float>(y.begin() + half, y.end()), cut, 1e-4f));
+  // an additive mask of zeros in any broadcastable shape changes nothing
+  using Shape = std::vector<int64_t>;
+  for (const Shape& shape : {Shape{S}, Shape{L, S}, Shape{Hq, 1, S}, Shape{B, Hq, L, S}}) {
+    Tensor z = Tensor::zeros(shape, gpu);
+    EXPECT_TRUE(vectorNear(function::sdpAttention(tq, tk, tv, false, z).toList<float>(), full, 1e-4f));
+  }
+  // a mask that does not broadcast is refused loudly
+  AssertHandler old = setAssertHandler(countingAssertHandler);
+  int before = g_asserts;
+  Tensor bad = function::sdpAttention(tq, tk, tv, false, Tensor::zeros({3, S}, gpu));
+  EXPECT_TRUE(g_asserts > before && !bad.defined());
+  setAssertHandler(old);
+}
+
 static void test_grad_bookkeeping_and_errors() {
   std::printf("Function::apply bookkeeping, dispatcher failure, allocator reuse\n");
   const Options gpu = options::device(DeviceType::GPU).dtype(DType::BFloat16);
@@ -187,6 +228,7 @@ int main() {
   }
   test_func_sdpAttention_reference_vectors();
   test_half_dtypes_and_gqa();
+  test_broadcast_masks();
   test_grad_bookkeeping_and_errors();
   std::printf(g_failures == 0 ? "ALL PASSED\n" : "%d FAILURES\n", g_failures);
   return g_failures == 0 ? 0 : 1;

@@ -33,6 +33,9 @@ def gen(seed, B, Hq, Hkv, L, S, D, mul=1.0, dtype="f32"):
 
 
 def case(name, q, k, v, causal=False, scale=None, mask=None):
+    if os.path.exists(os.path.join(HERE, name + ".npz")) and "--force" not in sys.argv:
+        print("%-28s kept (pass --force to rewrite)" % name)
+        return
     out = oracle.ref_sdpa_f32(q, k, v, causal=causal, scale=scale, mask=mask)
     extra = {}
     if mask is not None:
@@ -65,6 +68,16 @@ def main():
     case("boolmask_l9_s12", *gen(18, 2, 2, 2, 9, 12, 64), mask=bm)
     fm = oracle.randn(19, 7, (9, 12))
     case("floatmask_l9_s12", *gen(19, 2, 2, 1, 9, 12, 64), mask=fm)
+    # attnMask shapes other than [L,S]: the reference's bias add broadcasts them (reference FuncNNLayer.h:249-260)
+    pad = np.ones((3, 1, 1, 20), np.uint8)  # per-batch key padding [B,1,1,S]
+    pad[0, ..., 13:] = 0
+    pad[1, ..., 5:] = 0
+    case("boolmask_keypad_b3_s20", *gen(20, 3, 4, 2, 6, 20, 32), mask=pad)
+    case("floatmask_b2_h4_l5_s9", *gen(21, 2, 4, 4, 5, 9, 16), mask=oracle.randn(21, 7, (2, 4, 5, 9)))
+    hm = (np.random.RandomState(6).rand(4, 1, 11) > 0.5).astype(np.uint8)  # per-head key mask [H,1,S]
+    hm[..., 0] = 1
+    case("boolmask_h4_1_s11", *gen(22, 2, 4, 2, 3, 11, 16), mask=hm)
+    case("floatmask_row_s10", *gen(23, 1, 2, 2, 4, 10, 8), mask=oracle.randn(23, 7, (10,)))
 
 
 if __name__ == "__main__":

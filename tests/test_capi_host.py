@@ -17,7 +17,11 @@ def params(*dims, **kw):
     p = _capi.make_params(*dims)
     p.q = p.k = p.v = p.out = FAKE
     for k, v in kw.items():
-        setattr(p, k, v)
+        if isinstance(v, tuple):
+            for i, x in enumerate(v):
+                getattr(p, k)[i] = x
+        else:
+            setattr(p, k, v)
     return p
 
 
@@ -29,17 +33,19 @@ def test_exports_match_header():
     L = _capi.lib()
     for name in declared:
         assert getattr(L, name) is not None
-    assert L.ttsdpa_abi_version() == 1
+    header_version = int(re.search(r"#define\s+TTSDPA_ABI_VERSION\s+(\d+)", open(os.path.join(ROOT, "include", "ttsdpa.h")).read()).group(1))
+    assert L.ttsdpa_abi_version() == header_version
 
 
 def test_struct_layout_matches_header():
-    # 4+4, 4 pointers, 6 ints, 12 int64, float, 2 ints, (pad), pointer
-    assert ctypes.sizeof(_capi.Params) == 8 + 32 + 24 + 96 + 12 + 4 + 8
+    # 4+4, 4 pointers, 6 ints, 12 int64, float, 2 ints, (pad), pointer, 4 int64
+    assert ctypes.sizeof(_capi.Params) == 8 + 32 + 24 + 96 + 12 + 4 + 8 + 32
     p = _capi.make_params(_capi.BF16, 2, 32, 8, 4096, 4096, 128)
     assert p.struct_size == ctypes.sizeof(_capi.Params)
     assert list(p.q_stride) == [32 * 4096 * 128, 4096 * 128, 128]
     assert list(p.k_stride) == [8 * 4096 * 128, 4096 * 128, 128]
     assert abs(p.scale - 128 ** -0.5) < 1e-8 and p.causal == 0 and p.mask_kind == 0
+    assert list(p.mask_stride) == [0, 0, 4096, 1]  # a dense [L,S] mask shared by every batch and head
 
 
 @pytest.mark.parametrize("args,route", [
@@ -89,6 +95,8 @@ def test_routes_depend_on_flags():
     (dict(mask_kind=7), _capi.ERR_MASK),
     (dict(mask_kind=_capi.MASK_BOOL), _capi.ERR_NULL),                      # mask kind without a mask
     (dict(mask_kind=_capi.MASK_BOOL, mask=FAKE, causal=1), _capi.ERR_MASK),  # reference asserts on this
+    (dict(mask_kind=_capi.MASK_BOOL, mask=FAKE, mask_stride=(0, 0, -64, 1)), _capi.ERR_STRIDE),
+    (dict(mask_kind=_capi.MASK_ADD, mask=FAKE + 1), _capi.ERR_STRIDE),       # additive mask not element-aligned
 ])
 def test_validation_errors(mutate, status):
     p = params(_capi.BF16, 2, 8, 2, 64, 64, 128, **mutate)

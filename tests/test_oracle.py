@@ -166,6 +166,22 @@ def test_rounding_bf16_ties_and_roundtrip(oracle_mod):
     assert np.array_equal(b2[keep], allbits[keep])  # every bf16 value is a fixed point of the rounding
 
 
+@pytest.mark.parametrize("mshape", [(1, 7), (7,), (2, 1, 5, 7), (2, 4, 5, 7), (2, 1, 1, 7), (1, 4, 5, 1), (4, 1, 7)])
+@pytest.mark.parametrize("kind", ["bool", "float"])
+def test_broadcast_masks_against_compiled_reference(oracle_mod, mshape, kind):
+    _need_ref(oracle_mod)
+    B, Hq, Hkv, L, S, D = 2, 4, 2, 5, 7, 8
+    q = oracle_mod.randn(31, 0, (B, Hq, L, D))
+    k = oracle_mod.randn(31, 1, (B, Hkv, S, D))
+    v = oracle_mod.randn(31, 2, (B, Hkv, S, D))
+    if kind == "bool":
+        m = (np.random.RandomState(len(mshape)).rand(*mshape) > 0.4).astype(np.uint8)
+        m[..., 0] = 1
+    else:
+        m = oracle_mod.randn(32, 3, mshape)
+    assert np.array_equal(oracle_mod.sdpa_f32(q, k, v, mask=m), oracle_mod.ref_sdpa_f32(q, k, v, mask=m))
+
+
 # ---- mathematics ----------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("shape,causal", [((2, 4, 2, 19, 23, 32), False), ((1, 4, 4, 40, 40, 64), True),
@@ -182,8 +198,10 @@ def test_closed_form_fp64(oracle_mod, shape, causal):
 def test_closed_form_masks(oracle_mod):
     g = load_golden("boolmask_l9_s12")
     assert np.abs(g["out"] - closed_form_f64(g["q"], g["k"], g["v"], mask=g["mask"])).max() < 2e-5
-    g = load_golden("floatmask_l9_s12")
-    assert np.abs(g["out"] - closed_form_f64(g["q"], g["k"], g["v"], mask=g["mask"])).max() < 2e-5
+    for name in ("floatmask_l9_s12", "boolmask_keypad_b3_s20", "floatmask_b2_h4_l5_s9", "boolmask_h4_1_s11",
+                 "floatmask_row_s10"):
+        g = load_golden(name)
+        assert np.abs(g["out"] - closed_form_f64(g["q"], g["k"], g["v"], mask=g["mask"])).max() < 2e-5, name
 
 
 def test_invariants(oracle_mod):

@@ -256,6 +256,45 @@ def test_general_masks_large():
     assert rc == 0 and max_abs_err(out, exp) <= TOL["bf16"]
 
 
+@pytest.mark.parametrize("mshape", [(1, 1, 1, 170), (2, 1, 1, 170), (2, 1, 70, 170), (2, 4, 70, 170), (4, 70, 1), (170,)])
+@pytest.mark.parametrize("kind,dtype", [("bool", "bf16"), ("float", "f16"), ("float", "f32")])
+def test_broadcast_mask_shapes(mshape, kind, dtype):
+    # attnMask of any shape that broadcasts to [B,H,L,S] (reference src/Function/FuncNNLayer.h:249-260)
+    B, Hq, Hkv, L, S, D = 2, 4, 2, 70, 170, 64
+    host, dev = make_inputs(57, B, Hq, Hkv, L, S, D, dtype)
+    if kind == "bool":
+        m = (np.random.RandomState(len(mshape)).rand(*mshape) > 0.5).astype(np.uint8)
+        m[..., 0] = 1  # no row without a visible key
+        md = torch.from_numpy(m).cuda().bool()
+    else:
+        m, bits = oracle.round_to(oracle.randn(58, 9, mshape), dtype)
+        md = to_device(m, bits, dtype)
+    exp = oracle.sdpa_f32(*host, mask=m)
+    rc, out = call("forward", *dev, mask=md)
+    assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]
+
+
+def test_mask_views_with_strides():
+    # the mask is described by element strides: an expanded view (stride 0) and a sliced view (row and key strides
+    # that are not dense) give the result of their materialised copies
+    B, Hq, Hkv, L, S, D = 2, 4, 4, 33, 50, 32
+    host, dev = make_inputs(59, B, Hq, Hkv, L, S, D, "f32")
+    big = oracle.randn(60, 9, (B, 2 * L, 2 * S))
+    view = torch.from_numpy(big).cuda()[:, ::2, 1::2].unsqueeze(1)  # [B,1,L,S], strides (4LS, -, 4S, 2)
+    assert not view.is_contiguous()
+    exp = oracle.sdpa_f32(*host, mask=np.ascontiguousarray(big[:, None, ::2, 1::2]))
+    rc, out = call("forward", *dev, mask=view)
+    assert rc == 0 and max_abs_err(out, exp) <= TOL["f32"]
+    keypad = torch.ones(B, 1, 1, S, dtype=torch.bool, device="cuda")
+    keypad[0, ..., 20:] = False
+    rc, out2 = call("forward", *dev, mask=keypad.expand(B, Hq, L, S))
+    exp2 = oracle.sdpa_f32(*host, mask=keypad.cpu().numpy().astype(np.uint8))
+    assert rc == 0 and max_abs_err(out2, exp2) <= TOL["f32"]
+    # hidden keys do not influence the result at all: batch 0 equals attention over its first 20 keys
+    rc, out3 = call("forward", dev[0][:1], dev[1][:1, :, :20], dev[2][:1, :, :20])
+    assert rc == 0 and torch.allclose(out2[:1], out3, atol=1e-5)
+
+
 def test_empty_and_degenerate_shapes():
     z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device="cuda")
     rc, out = call("forward", z(2, 4, 0, 128), z(2, 4, 16, 128), z(2, 4, 16, 128))

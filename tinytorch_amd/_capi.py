@@ -41,6 +41,7 @@ class Params(ctypes.Structure):
         ("causal", ctypes.c_int32),
         ("mask_kind", ctypes.c_int32),
         ("mask", ctypes.c_void_p),
+        ("mask_stride", ctypes.c_int64 * 4),
     ]
 
 
@@ -76,7 +77,7 @@ def lib():
         L.ttsdpa_decode.restype = ctypes.c_int
         L.ttsdpa_general.argtypes = [P, ctypes.c_void_p]
         L.ttsdpa_general.restype = ctypes.c_int
-        if L.ttsdpa_abi_version() != 1:
+        if L.ttsdpa_abi_version() != 2:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L
     return _lib

@@ -19,6 +19,7 @@ struct KArgs {
   int mask_kind;
   float scale;
   long long qs[3], ks[3], vs[3], os[3];  // element strides: batch, head, sequence
+  long long ms[4];                       // mask element strides: batch, head, query row, key (0 = broadcast)
 };
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));

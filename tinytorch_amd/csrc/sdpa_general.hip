@@ -46,6 +46,7 @@ __global__ __launch_bounds__(256) void general_kernel(KArgs a) {
   const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1] + rowc * a.qs[2];
   const T* kp = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
   const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
+  const long long mrow = b * a.ms[0] + h * a.ms[1] + rowc * a.ms[2];  // a stride of 0 broadcasts that axis
 
   float qreg[DQ], acc[DQ];
 #pragma unroll
@@ -92,9 +93,9 @@ __global__ __launch_bounds__(256) void general_kernel(KArgs a) {
         int key = k0 + c0 + j;
         bool hidden = key >= a.S || (a.causal && key > row);
         if (a.mask_kind == 1) {
-          if (key < a.S && ((const uint8_t*)a.mask)[(long long)rowc * a.S + key] == 0) hidden = true;
+          if (key < a.S && ((const uint8_t*)a.mask)[mrow + key * a.ms[3]] == 0) hidden = true;
         } else if (a.mask_kind == 2) {
-          if (key < a.S) x += load_as_float((const T*)a.mask + (long long)rowc * a.S + key);
+          if (key < a.S) x += load_as_float((const T*)a.mask + mrow + key * a.ms[3]);
         }
         if (hidden) x = -INFINITY;
         s[j] = x;

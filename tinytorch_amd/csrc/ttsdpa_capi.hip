@@ -40,6 +40,11 @@ int validate(const ttsdpa_params* p, KArgs* a) {
   const size_t esz = p->dtype == TTSDPA_F32 ? 4 : 2;
   if (!ptr_aligned(p->q, esz) || !ptr_aligned(p->k, esz) || !ptr_aligned(p->v, esz) || !ptr_aligned(p->out, esz))
     return TTSDPA_ERR_STRIDE;
+  for (int i = 0; i < 4; i++) {
+    if (p->mask_kind != TTSDPA_MASK_NONE && p->mask_stride[i] < 0) return TTSDPA_ERR_STRIDE;
+    a->ms[i] = p->mask_kind != TTSDPA_MASK_NONE ? p->mask_stride[i] : 0;
+  }
+  if (p->mask_kind == TTSDPA_MASK_ADD && !ptr_aligned(p->mask, esz)) return TTSDPA_ERR_STRIDE;
   a->q = p->q, a->k = p->k, a->v = p->v, a->out = p->out, a->mask = p->mask;
   a->B = p->B, a->Hq = p->Hq, a->Hkv = p->Hkv, a->L = p->L, a->S = p->S, a->D = p->D;
   a->G = p->Hq / p->Hkv;
@@ -119,6 +124,7 @@ void ttsdpa_params_init(ttsdpa_params* p, int dtype, int B, int Hq, int Hkv, int
   p->causal = 0;
   p->mask_kind = TTSDPA_MASK_NONE;
   p->mask = nullptr;
+  p->mask_stride[0] = 0, p->mask_stride[1] = 0, p->mask_stride[2] = S, p->mask_stride[3] = 1;
 }
 
 int ttsdpa_plan(const ttsdpa_params* p, int* route) {

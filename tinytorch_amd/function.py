@@ -53,8 +53,13 @@ def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=No
     if attnMask is not None:
         if isCausal:
             raise ValueError("sdpAttention: isCausal and attnMask are exclusive")  # reference FuncNNLayer.h:242
-        if tuple(attnMask.shape) != (L, S):
-            raise ValueError("sdpAttention: attnMask must be [L, S]")
+        if attnMask.dim() > 4:
+            raise ValueError("sdpAttention: attnMask must broadcast to [B, H, L, S]")
+        try:  # the reference adds the mask with a broadcasting add (FuncNNLayer.h:249-260)
+            full = attnMask.expand(B, Hq, L, S)  # a view: broadcast axes get stride 0
+        except RuntimeError:
+            raise ValueError("sdpAttention: attnMask %s does not broadcast to [%d, %d, %d, %d]"
+                             % (tuple(attnMask.shape), B, Hq, L, S))
         if attnMask.dtype == torch.bool:
             p.mask_kind = _capi.MASK_BOOL
         elif attnMask.dtype == query.dtype:
@@ -62,6 +67,8 @@ def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=No
         else:
             raise TypeError("sdpAttention: attnMask must be bool or of the query dtype")
         p.mask = attnMask.data_ptr()
+        for i in range(4):
+            p.mask_stride[i] = full.stride(i) if full.size(i) > 1 else 0
     return p
 
 
@@ -81,8 +88,6 @@ def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0,
         raise RuntimeError("sdpAttention: q, k, v must live on the same device")
     fix = lambda t: t if (t.stride(-1) == 1 or t.size(-1) == 1) else t.contiguous()
     query, key, value = fix(query), fix(key), fix(value)
-    if attnMask is not None:
-        attnMask = attnMask.contiguous()
     out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
     p = build_params(query, key, value, out, isCausal, attnMask, scale)
     L = _capi.lib()

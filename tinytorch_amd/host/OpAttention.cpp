@@ -45,10 +45,23 @@ Tensor sdpAttentionGpuImpl(const Tensor& query, const Tensor& key, const Tensor&
   p.scale = scale;
   p.causal = isCausal ? 1 : 0;
   if (attnMask.defined()) {
-    ASSERT(attnMask.dim() == 2 && attnMask.size(0) == L && attnMask.size(1) == S);
     ASSERT(attnMask.device() == query.device());
     ASSERT(attnMask.dtype() == DType::Bool || attnMask.dtype() == query.dtype());
-    if (attnMask.dim() != 2 || attnMask.size(0) != L || attnMask.size(1) != S) return {};
+    // Any shape that broadcasts to [B,Hq,L,S], as the reference's broadcasting add of the bias accepts
+    // (src/Function/FuncNNLayer.h:249-260): right-align the mask's axes, size-1 and missing axes get stride 0.
+    const int md = static_cast<int>(attnMask.dim());
+    ASSERT(md >= 1 && md <= 4);
+    if (md < 1 || md > 4) return {};
+    const int64_t target[4] = {B, Hq, L, S};
+    int64_t dense = 1;
+    for (int i = 3; i >= 0; i--) {
+      const int mi = i - (4 - md);
+      const int64_t n = mi >= 0 ? attnMask.size(mi) : 1;
+      ASSERT(n == target[i] || n == 1);
+      if (n != target[i] && n != 1) return {};
+      p.mask_stride[i] = n == 1 ? 0 : dense;
+      dense *= n;
+    }
     p.mask_kind = attnMask.dtype() == DType::Bool ? TTSDPA_MASK_BOOL : TTSDPA_MASK_ADD;
     p.mask = attnMask.rawPtr();
   }
