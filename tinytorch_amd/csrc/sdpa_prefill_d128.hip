@@ -24,14 +24,24 @@
 //                                                 load ds_read_b64_tr_b16; B = P^T straight from the S^T
 //                                                 accumulator registers (same permutation of the contraction
 //                                                 index on both sides)
-// Software pipeline: the S^T MFMAs of half h+1 are issued in the same straight-line block as the exponentials of
-// half h, and the row maximum of half h+1 is taken while the P.V MFMAs of half h run, so the matrix pipe works under
-// the vector work.  K and V tiles are requested three tiles before use (four stages each); one barrier per 64-key
-// tile.
-// The running maximum m is raised only when a half's maximum exceeds it by more than 2^8 in the exponent (the
-// probabilities stay <= 256), so the accumulator rescale is rare.
+// Software pipeline, three strands per step h: the matrix pipe forms S^T of half h+2 and accumulates P.V of half h
+// while the vector ALU turns the scores of half h+1 into P.  In the steady state the 16 MFMAs of a step are issued
+// in a fixed order that alternates the (dependent) S^T chain with the (independent) P.V products, each followed by
+// one score's scale/exp/sum, and every LDS operand is requested six MFMAs before its use into a ring of registers.
+// On this chip a wavefront's MFMA blocks the SIMD's vector issue port for about 16 of its 32 cycles and two
+// wavefronts of a SIMD overlap little (the older one is served first), so the order inside one wavefront is what
+// keeps the matrix pipe fed.
+// K is consumed one tile ahead of V, so K tiles are requested four tiles before their P.V step and V tiles three
+// (four stages each); one bare s_barrier per 64-key tile.  The global->LDS loads are issued as asm: the compiler
+// would otherwise order every later LDS read behind all outstanding loads.
+// The maximum m the exponentials are taken against is raised lazily: a lane's 16 probabilities of a half are summed
+// anyway, and only when such a sum leaves [0, 1024] (which includes the first half of a row, taken against -1e30)
+// is the true row maximum formed, sum and accumulator rescaled, and the half redone.  The scores of a half stay in
+// their accumulator registers until that check has passed.
 // Causal masking (key j visible to query i iff j <= i, reference src/Operation/OpTransformCpu.h:202-209) skips
 // halves above the diagonal and applies the predicate only on halves that straddle it.
+// Under a causal mask a workgroup takes a row tile and its mirror (equal work for every workgroup), and neighbouring
+// workgroups take the two in opposite order so their load/store bursts do not coincide.
 // Grouped-query attention: kv head = query head / (Hq/Hkv), resolved in the kernel; the workgroup order puts the
 // query heads and row tiles that share a KV head on the same XCD so its L2 holds that K/V once.
 
@@ -50,7 +60,7 @@ constexpr int ROW_BYTES = D * 2;
 constexpr int STAGE_BYTES = BN * ROW_BYTES;  // 16 KiB
 constexpr int KSTAGES = 4, VSTAGES = 4;     // K and V tiles are requested three tiles before use
 constexpr int LDS_BYTES = (KSTAGES + VSTAGES) * STAGE_BYTES;
-constexpr float kLazyExp = 8.f;
+constexpr float kSumLimit = 1024.f;  // a lane's 16 probabilities of a half may sum to this much before the maximum is raised
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -102,8 +112,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
 
   for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
-  const int rt = (CAUSAL && part == 0) ? ntile - 1 - slot_rt : slot_rt;  // the long tile first
-  if (part == 1 && slot_rt >= ntile - 1 - slot_rt) break;                  // odd count: the middle tile has no mirror
+  // Neighbouring workgroups take their two tiles in opposite order, so that the load / store bursts between the
+  // parts of one half of the workgroups fall into the steady loops of the other half.
+  const bool long_first = ((blockIdx.x >> 3) & 1) == 0;
+  const int rt = (CAUSAL && (part == 0) == long_first) ? ntile - 1 - slot_rt : slot_rt;
+  if (part == 1 && slot_rt >= ntile - 1 - slot_rt) break;  // odd count: the middle tile has no mirror
   const int q0 = rt * BM;
   const int qw0 = q0 + wave * WM;
 
@@ -115,16 +128,21 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }
   // 32-key halves this wavefront computes on: under a causal mask those that start at or before its last row
   int my_halves = 2 * ntiles_kv;
-  // tiles whose both halves need no mask for this wavefront and whose successor half exists: the fast path
-  int nfast = a.S / BN;
   if (CAUSAL) {
     int t = (qw0 + WM - 1) / 32 + 1;
     my_halves = t < my_halves ? t : my_halves;
-    int f = (qw0 + 1) / BN;  // tiles with 64j + 63 <= qw0
-    nfast = f < nfast ? f : nfast;
   }
-  if (nfast > ntiles_kv - 1) nfast = ntiles_kv - 1;
-  if (2 * nfast > my_halves - 2) nfast = (my_halves - 2) / 2;  // half 2j+2 must be one of ours
+  // Tiles j whose two steps take the fast form: halves up to 2j+3 are this wavefront's, tile j+1 is complete, and
+  // half 2j+2 (whose exponentials step 2j+1 takes) needs no mask.
+  int nfast = (my_halves - 2) / 2;
+  {
+    int f = a.S >= 96 ? (a.S - 32) / BN : 0;
+    nfast = f < nfast ? f : nfast;
+    if (CAUSAL) {
+      f = qw0 >= 95 ? (qw0 - 31) / BN : 0;
+      nfast = f < nfast ? f : nfast;
+    }
+  }
   if (nfast < 0) nfast = 0;
 
   // ---- global -> LDS: wavefront w moves rows 8w .. 8w+7 of a tile, 4 rows (1 KiB) per instruction --------------
@@ -134,30 +152,33 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   for (int i = 0; i < 2; i++) {
     int row = 8 * wave + 4 * i + (lane >> 4);
     int chunk = (lane & 15) ^ swz(row);
-    ld_koff[i] = (unsigned)(row * a.ks[2] + 8 * chunk) * 2u;
-    ld_voff[i] = (unsigned)(row * a.vs[2] + 8 * chunk) * 2u;
+    ld_koff[i] = ((unsigned)row * (unsigned)a.ks[2] + 8u * chunk) * 2u;  // the host checks that 64 rows fit 32 bits
+    ld_voff[i] = ((unsigned)row * (unsigned)a.vs[2] + 8u * chunk) * 2u;
   }
-  auto dma_tile = [&](const T* base, long long rstride, const unsigned (&off)[2], int kv0, char* stage) __attribute__((always_inline)) {
-    const char* src = (const char*)(base + kv0 * rstride);
+  // Issued as asm so that the compiler does not see a store to LDS: it would otherwise make every later LDS read
+  // wait for all outstanding loads (vmcnt(0)).  The waits are placed by hand in dma_wait_and_sync.
+  auto dma_issue = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
+  };
+  const unsigned smem_addr = (unsigned)(unsigned long)(lds_void*)smem;
+  auto dma_tile = [&](const T* base, long long rstride, const unsigned (&off)[2], int kv0, unsigned stage_addr) __attribute__((always_inline)) {
     if (kv0 + BN <= a.S) {
+      const char* src = (const char*)(base + kv0 * rstride);
 #pragma unroll
-      for (int i = 0; i < 2; i++)
-        __builtin_amdgcn_global_load_lds((gbl_void*)(src + off[i]), (lds_void*)(stage + (8 * wave + 4 * i) * ROW_BYTES),
-                                         16, 0, 0);
+      for (int i = 0; i < 2; i++) dma_issue(src, off[i], stage_addr + (8 * wave + 4 * i) * ROW_BYTES);
     } else {  // ragged last tile: rows past the end re-read the last valid row (their scores are masked)
 #pragma unroll
       for (int i = 0; i < 2; i++) {
         int row = 8 * wave + 4 * i + (lane >> 4);
-        int key = kv0 + row;
-        key = key < a.S ? key : a.S - 1;
         int chunk = (lane & 15) ^ swz(row);
-        __builtin_amdgcn_global_load_lds((gbl_void*)(base + key * rstride + 8 * chunk),
-                                         (lds_void*)(stage + (8 * wave + 4 * i) * ROW_BYTES), 16, 0, 0);
+        int rowc = row < a.S - kv0 ? row : a.S - 1 - kv0;
+        unsigned voff = ((unsigned)rowc * (unsigned)rstride + 8u * chunk) * 2u;
+        dma_issue((const char*)(base + kv0 * rstride), voff, stage_addr + (8 * wave + 4 * i) * ROW_BYTES);
       }
     }
   };
-  auto dma_k = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(kp, a.ks[2], ld_koff, tile * BN, smem + stage * STAGE_BYTES); };
-  auto dma_v = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(vp, a.vs[2], ld_voff, tile * BN, smem + (KSTAGES + stage) * STAGE_BYTES); };
+  auto dma_k = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(kp, a.ks[2], ld_koff, tile * BN, smem_addr + stage * STAGE_BYTES); };
+  auto dma_v = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(vp, a.vs[2], ld_voff, tile * BN, smem_addr + (KSTAGES + stage) * STAGE_BYTES); };
   // Wait until at most `keep` of this wavefront's global->LDS loads are still in flight (they complete in issue
   // order), then meet the other wavefronts: what was issued before the newest `keep` loads is visible to all.
   auto dma_wait_and_sync = [&](int keep) __attribute__((always_inline)) {
@@ -168,7 +189,9 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    __syncthreads();
+    // bare barrier: the loads above carry the ordering; __syncthreads() would also drain the LDS operand prefetch
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
   };
 
   // ---- LDS operand addresses (bytes), loop-invariant ---------------------------------------------------------------
@@ -197,14 +220,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     }
   }
 
-  // ---- prologue: first tiles on their way, Q into registers ---------------------------------------------------------
-  dma_k(0, 0);
-  dma_v(0, 0);
-  if (ntiles_kv > 1) dma_k(1, 1);
-  if (ntiles_kv > 1) dma_v(1, 1);
-  if (ntiles_kv > 2) dma_k(2, 2);
-  if (ntiles_kv > 2) dma_v(2, 2);
 
+  // ---- prologue: first tiles on their way, Q into registers ---------------------------------------------------------
+  // K runs one tile ahead of V in consumption (scores are formed two halves before their P.V), so K is requested
+  // four tiles ahead and V three: iteration j sends for K(j+4) (stage of K(j), last read in iteration j-1) and
+  // V(j+3) (stage of V(j-1)).
   vec8 qreg[8];
   {
     int row = qw0 + lq;
@@ -213,6 +233,16 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #pragma unroll
     for (int ks = 0; ks < 8; ks++) qreg[ks] = *(const vec8*)(qr + 16 * ks);
   }
+  // Order of need: K(0) for the first scores, then K(1), V(0), ...; with four tiles or more the waits below let the
+  // later ones land while the first scores are formed.
+  const bool staged_start = ntiles_kv >= 4;
+  dma_k(0, 0);
+  if (1 < ntiles_kv) dma_k(1, 1);
+  dma_v(0, 0);
+  if (2 < ntiles_kv) dma_k(2, 2);
+  if (1 < ntiles_kv) dma_v(1, 1);
+  if (3 < ntiles_kv) dma_k(3, 3);
+  if (2 < ntiles_kv) dma_v(2, 2);
 
   f32x16 oacc[4];
 #pragma unroll
@@ -220,7 +250,6 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
   const float c = a.scale * kLog2e;
-  const float lazy = kLazyExp / c;
   float m_use = -1e30f;  // maximum the exponentials are taken against (raw scores)
   float mc = -1e30f * c;
   float l_run = 0.f;
@@ -258,10 +287,30 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     return fmaxf(__builtin_bit_cast(float, lo), __builtin_bit_cast(float, hi));
   };
 
-  // raise the running maximum when some row needs it (rare), rescaling sum and accumulator
-  auto raise_max = [&](float mx) __attribute__((always_inline)) {
-    if (__builtin_amdgcn_ballot_w64(mx > m_use + lazy) != 0) {
-      const float m_new = fmaxf(m_use, mx);
+  // exponentials of one half against the current maximum -> P^T as MFMA B operands pb[k-step of 16 keys];
+  // returns this lane's sum of the 16 probabilities
+  auto exp_half = [&](const f32x16& s, vec8 (&pb)[2]) __attribute__((always_inline)) {
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      f32x8 x;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        x[i] = fast_exp2(fmaf(s[8 * t + i], c, -mc));
+        psum += x[i];
+      }
+      pb[t] = __builtin_convertvector(x, vec8);
+    }
+    return psum;
+  };
+
+  // The exponentials are taken against a maximum that is only raised when a lane's sum of probabilities shows that
+  // some probability left the range [0, kSumLimit] (which includes the first half of a row, taken against -1e30):
+  // then the true row maximum is formed, sum and accumulator are rescaled and the half is redone.  Every
+  // probability that reaches the matrix pipe is therefore at most kSumLimit.
+  auto settle_half = [&](const f32x16& s, vec8 (&pb)[2], float psum) __attribute__((always_inline)) {
+    if (__builtin_amdgcn_ballot_w64(!(psum <= kSumLimit)) != 0) {
+      const float m_new = fmaxf(m_use, row_max(s));
       const float alpha = fast_exp2((m_use - m_new) * c);
       m_use = m_new;
       mc = m_new * c;
@@ -270,26 +319,9 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       for (int db = 0; db < 4; db++)
 #pragma unroll
         for (int r = 0; r < 16; r++) oacc[db][r] *= alpha;
-    }
-  };
-
-  // exponentials of one half -> P^T as MFMA B operands pb[k-step of 16 keys]
-  auto exp_half = [&](f32x16& s, vec8 (&pb)[2]) __attribute__((always_inline)) {
-    float psum = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      float p = fast_exp2(fmaf(s[r], c, -mc));
-      s[r] = p;
-      psum += p;
+      psum = exp_half(s, pb);
     }
     l_run += psum;
-#pragma unroll
-    for (int t = 0; t < 2; t++) {
-      f32x8 x;
-#pragma unroll
-      for (int i = 0; i < 8; i++) x[i] = s[8 * t + i];
-      pb[t] = __builtin_convertvector(x, vec8);
-    }
   };
 
   // O^T += V_half^T . P^T; vh = LDS address of the half's first V row
@@ -305,71 +337,120 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       }
   };
 
-  // Pipeline step, fast form: half hb needs no mask and half hb+1 is wanted.
-  auto fast_step = [&](f32x16& cur, float& mcur, f32x16& nxt, float& mnxt, const char* kn, const char* vc) __attribute__((always_inline)) {
-    raise_max(mcur);
-    vec8 pb[2];
-    qk_half(nxt, kn);
-    exp_half(cur, pb);
-    pv_half(pb, vc);
-    mnxt = row_max(nxt);
-  };
-  // General form: half hb may be unwanted / masked, half hb+1 may be unwanted.
-  auto slow_step = [&](f32x16& cur, float& mcur, f32x16& nxt, float& mnxt, int hb, const char* kn, const char* vc,
-                       bool do_nxt) __attribute__((always_inline)) {
-    const int kv0 = 32 * hb;
-    if (do_nxt) qk_half(nxt, kn);
-    if (hb < my_halves) {
-      if ((CAUSAL && kv0 + 31 > qw0) || kv0 + 32 > a.S) {  // the half straddles the diagonal or the end of the keys
-        mask_half(cur, kv0);
-        mcur = row_max(cur);
-      }
-      raise_max(mcur);
-      vec8 pb[2];
-      exp_half(cur, pb);
-      pv_half(pb, vc);
-    }
-    if (do_nxt) mnxt = row_max(nxt);
+  // LDS address of the first K row of half h (v_addr carries the V region's base, so the same value serves V)
+  auto half_base = [&](int h) __attribute__((always_inline)) {
+    return smem + ((h >> 1) & 3) * STAGE_BYTES + (h & 1) * 32 * ROW_BYTES;
   };
 
-  f32x16 sP, sN;
-  float mP, mN = 0.f;
-  dma_wait_and_sync(0);
-  qk_half(sP, smem);
-  mP = row_max(sP);
-  // Tile t lives in stage t % 4 (K and V alike).  Iteration j reads K(j) (second half), K(j+1) (first half) and
-  // V(j), and sends for K(j+3) and V(j+3), whose stage was last read in iteration j-1.  Its closing barrier publishes
-  // tile j+2, requested one iteration earlier: only this iteration's own loads may still be in flight.
-  // The stage index is a compile-time constant in the unrolled fast loop, so every LDS address there is
-  // lane address + immediate.
-  auto tile_iter = [&](int j, const int st, const bool fast) __attribute__((always_inline)) {
+  // Pipeline state between steps: P of half h (ready for the matrix pipe) and the raw scores of half h+1.
+  // Step h:  matrix pipe: S^T(h+2) and O^T += V(h)^T . P(h);  vector ALU: P(h+1) = exp2(...) of the scores of h+1.
+  // General form of a step (any half may be masked or missing); the compiler orders it.
+  auto slow_step = [&](int h, const vec8 (&p_cur)[2], f32x16& s_nxt, f32x16& s_new, vec8 (&p_nxt)[2]) __attribute__((always_inline)) {
+    if (h + 2 < my_halves) qk_half(s_new, half_base(h + 2));
+    if (h < my_halves) pv_half(p_cur, half_base(h));
+    if (h + 1 < my_halves) {
+      const int kv0 = 32 * (h + 1);
+      if ((CAUSAL && kv0 + 31 > qw0) || kv0 + 32 > a.S) mask_half(s_nxt, kv0);
+      settle_half(s_nxt, p_nxt, exp_half(s_nxt, p_nxt));
+    }
+  };
+
+  // ---- fast form: hand-ordered, one MFMA per slot, operands fetched PD slots ahead -------------------------------------
+  // A tile iteration has 32 slots (two steps of 16).  Even slot 2i of a step is the S^T MFMA of k-step i, odd slot
+  // 2i+1 the P.V MFMA (t = i/4, db = i%4): the dependent S^T chain is spaced by independent P.V MFMAs.  Each slot
+  // also carries one score's scale/exp (and every second slot the pair's conversion), and requests the LDS operand
+  // of the slot PD places further on into a ring of RING operand registers.
+  constexpr int PD = 6, RING = 8;  // RING divides the 128 slots of the unrolled body
+  vec8 ring[RING];
+  auto fetch = [&](const int G) __attribute__((always_inline)) {  // G: slot index within the 4-tile unrolled body
+    const int u = (G >> 5) & 3, kind = (G >> 4) & 1, s = G & 15, i = s >> 1;
+    if ((s & 1) == 0) {
+      const char* base = smem + ((u + 1) & 3) * STAGE_BYTES + kind * 32 * ROW_BYTES;
+      ring[G % RING] = *(const vec8*)(base + k_addr[i]);
+    } else {
+      const int t = i >> 2, db = i & 3;
+      const char* base = smem + u * STAGE_BYTES + kind * 32 * ROW_BYTES + 16 * t * ROW_BYTES;
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + v_addr[db][0]));
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + v_addr[db][1]));
+      ring[G % RING] = __builtin_bit_cast(vec8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+  };
+  auto fast_step = [&](const int G0, f32x16& s_new, const f32x16& s_nxt, const vec8 (&p_cur)[2], vec8 (&p_nxt)[2]) __attribute__((always_inline)) {
+    float psum = 0.f;
+    f32x8 x;
+#pragma unroll
+    for (int s = 0; s < 16; s++) {
+      const int G = G0 + s, i = s >> 1;
+      fetch((G + PD) & 127);
+      if ((s & 1) == 0) {
+        if (i == 0) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) s_new[r] = 0.f;
+        }
+        s_new = TR::mfma32(ring[G % RING], qreg[i], s_new);
+      } else {
+        oacc[i & 3] = TR::mfma32(ring[G % RING], p_cur[i >> 2], oacc[i & 3]);
+      }
+      x[s & 7] = fast_exp2(fmaf(s_nxt[s], c, -mc));
+      psum += x[s & 7];
+      if ((s & 7) == 7) p_nxt[s >> 3] = __builtin_convertvector(x, vec8);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    settle_half(s_nxt, p_nxt, psum);
+  };
+
+  f32x16 sB, sC;
+  vec8 pA[2], pB[2];
+  if (staged_start) {
+    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // Q and K(0) are here; six tiles (12 loads) may be on their way
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  } else {
+    dma_wait_and_sync(0);
+  }
+  {  // P(0) and the scores of half 1
+    qk_half(sC, half_base(0));
+    if ((CAUSAL && 31 > qw0) || 32 > a.S) mask_half(sC, 0);
+    settle_half(sC, pA, exp_half(sC, pA));
+    if (1 < my_halves) qk_half(sB, half_base(1));
+  }
+  // Every wavefront has read K(0): iteration 0 may overwrite its stage.  K(1), V(0), K(2), V(1) must be visible
+  // before iteration 0; K(3) and V(2) (4 loads) are waited for at its end.
+  dma_wait_and_sync(staged_start ? 4 : 0);
+
+  auto tile_dma = [&](int j) __attribute__((always_inline)) {
     int keep = 0;
     if (j + 3 < ntiles_kv) {
-      dma_k(j + 3, (st + 3) & 3);
-      dma_v(j + 3, (st + 3) & 3);
-      keep = 4;
+      if (j + 4 < ntiles_kv) {
+        dma_k(j + 4, j & 3);
+        keep = 4;
+      } else {
+        keep = 2;
+      }
+      dma_v(j + 3, (j + 3) & 3);
     }
-    const char* kc1 = smem + st * STAGE_BYTES + 32 * ROW_BYTES;
-    const char* kn0 = smem + ((st + 1) & 3) * STAGE_BYTES;
-    const char* vc = smem + st * STAGE_BYTES;  // v_addr carries the V region's base
-    if (fast) {
-      fast_step(sP, mP, sN, mN, kc1, vc);
-      fast_step(sN, mN, sP, mP, kn0, vc + 32 * ROW_BYTES);
-    } else {
-      slow_step(sP, mP, sN, mN, 2 * j, kc1, vc, 2 * j + 1 < my_halves);
-      slow_step(sN, mN, sP, mP, 2 * j + 1, kn0, vc + 32 * ROW_BYTES, j + 1 < ntiles_kv && 2 * j + 2 < my_halves);
-    }
-    dma_wait_and_sync(keep);
+    return keep;
   };
   int j = 0;
-  for (; j + 4 <= nfast; j += 4) {  // tiles that need no mask and whose successor half is wanted
-    tile_iter(j, 0, true);
-    tile_iter(j + 1, 1, true);
-    tile_iter(j + 2, 2, true);
-    tile_iter(j + 3, 3, true);
+  if (nfast >= 4) {
+#pragma unroll
+    for (int g = 0; g < PD; g++) fetch(g);
+    for (; j + 4 <= nfast; j += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int keep = tile_dma(j + u);
+        fast_step(32 * u, sC, sB, pA, pB);
+        fast_step(32 * u + 16, sB, sC, pB, pA);
+        dma_wait_and_sync(keep);
+      }
+    }
   }
-  for (; j < ntiles_kv; j++)  // the rest: diagonal tiles, the ragged end of the keys, tiles this wavefront skips
-    tile_iter(j, j & 3, false);
+  for (; j < ntiles_kv; j++) {
+    const int keep = tile_dma(j);
+    slow_step(2 * j, pA, sB, sC, pB);
+    slow_step(2 * j + 1, pB, sC, sB, pA);
+    dma_wait_and_sync(keep);
+  }
 
   // ---- normalise and store ----------------------------------------------------------------------------------------------
   {

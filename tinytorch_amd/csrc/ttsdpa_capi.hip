@@ -159,8 +159,10 @@ int ttsdpa_prefill(const ttsdpa_params* p, void* stream) {
   if (p->B == 0 || p->L == 0) return TTSDPA_OK;
   if (!prefill_ok(p)) return TTSDPA_ERR_UNSUPPORTED;
   if ((rc = check_grid((long long)a.B * a.Hq * ((a.L + 127) / 128))) != TTSDPA_OK) return rc;
-  // head_dim 128 with enough rows to fill 256-row workgroups takes the software-pipelined kernel
-  if (a.D == 128 && a.L > 128) return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
+  // head_dim 128 with enough rows to fill 256-row workgroups takes the software-pipelined kernel (its tile loads
+  // address 64 rows with 32-bit byte offsets)
+  if (a.D == 128 && a.L > 128 && a.ks[2] < (1 << 24) && a.vs[2] < (1 << 24))
+    return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
   return launch_prefill(a, p->dtype, (hipStream_t)stream);
 }
 
