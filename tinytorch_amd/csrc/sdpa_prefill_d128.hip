@@ -452,23 +452,45 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     dma_wait_and_sync(keep);
   }
 
-  // ---- normalise and store ----------------------------------------------------------------------------------------------
+  // ---- normalise, transpose through LDS, store whole rows -----------------------------------------------------------------
+  // A lane holds 4 consecutive head_dim elements per register group of its query row: stored directly, every store
+  // instruction would touch 32 rows with 16 bytes each.  Instead each wavefront stages 8 of its rows at a time in its
+  // 2 KiB slice of the last V stage and writes them out as whole 256-byte rows.  That stage is free here: all
+  // wavefronts passed the closing barrier of the last tile, and the next part sends for V(3) only in its iteration 0,
+  // two barriers from now.  16-byte chunk c of staged row r sits at chunk slot c ^ r (no bank conflicts either way).
   {
     float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv = 1.f / l_tot;
-    const int qi = qw0 + lq;
-    if (qi < a.L) {
-      T* op = (T*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2];
+    typename TR::vec4 y[4][4];
 #pragma unroll
-      for (int db = 0; db < 4; db++)
+    for (int db = 0; db < 4; db++)
 #pragma unroll
-        for (int rg = 0; rg < 4; rg++) {
-          f32x4 x;
+      for (int rg = 0; rg < 4; rg++) {
+        f32x4 x;
 #pragma unroll
-          for (int i = 0; i < 4; i++) x[i] = oacc[db][4 * rg + i] * inv;
-          typename TR::vec4 y = __builtin_convertvector(x, typename TR::vec4);
-          *(typename TR::vec4*)(op + 32 * db + 8 * rg + 4 * lh) = y;
-        }
+        for (int i = 0; i < 4; i++) x[i] = oacc[db][4 * rg + i] * inv;
+        y[db][rg] = __builtin_convertvector(x, typename TR::vec4);
+      }
+    char* tbuf = smem + (KSTAGES + 3) * STAGE_BYTES + wave * 2048;
+    T* obase = (T*)a.out + b * a.os[0] + h * a.os[1];
+    const int rr = lq & 7;
+    const int cc = lane & 15;
+#pragma unroll
+    for (int r8 = 0; r8 < 4; r8++) {
+      if ((lq >> 3) == r8) {
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+          for (int rg = 0; rg < 4; rg++)
+            *(typename TR::vec4*)(tbuf + rr * ROW_BYTES + (((4 * db + rg) ^ rr) << 4) + 8 * lh) = y[db][rg];
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const int row = 4 * i + (lane >> 4);
+        vec8 v = *(const vec8*)(tbuf + row * ROW_BYTES + ((cc ^ row) << 4));
+        const int qi = qw0 + 8 * r8 + row;
+        if (qi < a.L) *(vec8*)(obase + qi * a.os[2] + 8 * cc) = v;
+      }
     }
   }
   }  // part
