@@ -158,7 +158,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   // Issued as asm so that the compiler does not see a store to LDS: it would otherwise make every later LDS read
   // wait for all outstanding loads (vmcnt(0)).  The waits are placed by hand in dma_wait_and_sync.
   auto dma_issue = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   const unsigned smem_addr = (unsigned)(unsigned long)(lds_void*)smem;
   auto dma_tile = [&](const T* base, long long rstride, const unsigned (&off)[2], int kv0, unsigned stage_addr) __attribute__((always_inline)) {
@@ -170,6 +170,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #pragma unroll
       for (int i = 0; i < 2; i++) {
         int row = 8 * wave + 4 * i + (lane >> 4);
+        asm volatile("" : "+v"(row));  // keeps this rarely taken path's address arithmetic inside the branch
         int chunk = (lane & 15) ^ swz(row);
         int rowc = row < a.S - kv0 ? row : a.S - 1 - kv0;
         unsigned voff = ((unsigned)rowc * (unsigned)rstride + 8u * chunk) * 2u;
@@ -432,16 +433,22 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     return keep;
   };
   int j = 0;
-  if (nfast >= 4) {
+  if (nfast >= 1) {
 #pragma unroll
     for (int g = 0; g < PD; g++) fetch(g);
-    for (; j + 4 <= nfast; j += 4) {
+    // Four tiles per trip so that the stage of a tile is a compile-time constant; the trip may end after any of them.
+    for (bool more = true; more;) {
 #pragma unroll
       for (int u = 0; u < 4; u++) {
-        const int keep = tile_dma(j + u);
+        if (j >= nfast) {
+          more = false;
+          break;
+        }
+        const int keep = tile_dma(j);
         fast_step(32 * u, sC, sB, pA, pB);
         fast_step(32 * u + 16, sB, sC, pB, pA);
         dma_wait_and_sync(keep);
+        j++;
       }
     }
   }
