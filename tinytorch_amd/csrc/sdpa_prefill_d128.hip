@@ -118,7 +118,10 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   const int rt = (CAUSAL && (part == 0) == long_first) ? ntile - 1 - slot_rt : slot_rt;
   if (part == 1 && slot_rt >= ntile - 1 - slot_rt) break;  // odd count: the middle tile has no mirror
   const int q0 = rt * BM;
-  const int qw0 = q0 + wave * WM;
+  // Wavefronts w and w+4 share a SIMD.  Under a causal mask the row group g of a tile has g+1 halves of work on the
+  // diagonal, so the second four wavefronts take the groups in reverse: every SIMD then carries groups g and 7-g.
+  const int rowgroup = (CAUSAL && wave >= 4) ? 11 - wave : wave;
+  const int qw0 = q0 + rowgroup * WM;
 
   int ntiles_kv = (a.S + BN - 1) / BN;
   if (CAUSAL) {
