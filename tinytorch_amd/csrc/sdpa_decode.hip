@@ -119,14 +119,14 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
       key = key < a.S ? key : a.S - 1;
       const T* kr = kp + key * a.ks[2] + 8 * lg;
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++) kreg[gi][ks] = *(const u32x4*)(kr + 32 * ks);
+      for (int ks = 0; ks < 4; ks++) kreg[gi][ks] = __builtin_nontemporal_load((const u32x4*)(kr + 32 * ks));  // read once: keep it out of the caches
     }
     u32x4 vreg[KB / 4];
 #pragma unroll
     for (int i = 0; i < KB / 4; i++) {
       int key = k0 + 4 * i + lg;
       key = key < a.S ? key : a.S - 1;
-      vreg[i] = *(const u32x4*)(vp + key * a.vs[2] + 8 * l16);
+      vreg[i] = __builtin_nontemporal_load((const u32x4*)(vp + key * a.vs[2] + 8 * l16));
     }
 
     // ---- scores --------------------------------------------------------------------------------------------------------
