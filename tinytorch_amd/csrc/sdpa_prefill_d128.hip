@@ -499,7 +499,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
         const int row = 4 * i + (lane >> 4);
         vec8 v = *(const vec8*)(tbuf + row * ROW_BYTES + ((cc ^ row) << 4));
         const int qi = qw0 + 8 * r8 + row;
-        if (qi < a.L) *(vec8*)(obase + qi * a.os[2] + 8 * cc) = v;
+        if (qi < a.L) __builtin_nontemporal_store(v, (vec8*)(obase + qi * a.os[2] + 8 * cc));  // written once, not read here
       }
     }
   }
