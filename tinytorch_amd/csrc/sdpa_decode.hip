@@ -245,29 +245,42 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
   }
 }
 
-// Combine the per-split records of one (batch, kv head): one workgroup, thread t handles (row, dim) pairs.
+// Combine the per-split records of one query row: one workgroup of 128 threads per (batch, kv head, row).  The first
+// wavefront turns the (max, sum) pairs of the up to 64 splits into weights (one split per lane, wave reductions);
+// then thread d accumulates head_dim element d over the splits with independent, coalesced loads.
+constexpr int kMaxSplits = 64;
 template <typename T>
-__global__ __launch_bounds__(256) void merge_kernel(KArgs a, int splits, const float* __restrict__ ws) {
-  const int pair = blockIdx.x;  // b * Hkv + hk
-  const int hk = pair % a.Hkv, b = pair / a.Hkv;
+__global__ __launch_bounds__(DD) void merge_kernel(KArgs a, int splits, const float* __restrict__ ws) {
+  __shared__ float weight[kMaxSplits];
+  __shared__ float total;
   const int rows = a.L * a.G;
+  const int pair = blockIdx.x / rows, x = blockIdx.x % rows;  // pair = b * Hkv + hk
+  const int hk = pair % a.Hkv, b = pair / a.Hkv;
   const float c = a.scale * kLog2e;
-  for (int e = threadIdx.x; e < rows * DD; e += 256) {
-    int x = e / DD, d = e % DD;
-    const float* rec0 = ws + ((long long)pair * splits * rows + x) * (DD + 2);
-    const long long step = (long long)rows * (DD + 2);
-    float mx = -1e30f;
-    for (int s = 0; s < splits; s++) mx = fmaxf(mx, rec0[s * step + DD]);
-    float lsum = 0.f, o = 0.f;
-    for (int s = 0; s < splits; s++) {
-      float f = fast_exp2((rec0[s * step + DD] - mx) * c);
-      lsum += f * rec0[s * step + DD + 1];
-      o += f * rec0[s * step + d];
-    }
-    int xl = x / a.G, xg = x % a.G;
-    T* op = (T*)a.out + b * a.os[0] + (hk * a.G + xg) * a.os[1] + xl * a.os[2];
-    store_from_float(op + d, o / lsum);
+  const float* rec0 = ws + ((long long)pair * splits * rows + x) * (DD + 2);
+  const long long step = (long long)rows * (DD + 2);
+  const int t = threadIdx.x;
+  if (t < 64) {
+    const bool have = t < splits;
+    const float m = have ? rec0[t * step + DD] : -1e30f;
+    const float l = have ? rec0[t * step + DD + 1] : 0.f;
+    float mx = m;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    const float f = have ? fast_exp2((m - mx) * c) : 0.f;
+    float lsum = f * l;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) lsum += __shfl_xor(lsum, off);
+    weight[t] = f;
+    if (t == 0) total = lsum;
   }
+  __syncthreads();
+  float o = 0.f;
+#pragma unroll 8
+  for (int s = 0; s < splits; s++) o = fmaf(weight[s], rec0[s * step + t], o);
+  const int xl = x / a.G, xg = x % a.G;
+  T* op = (T*)a.out + b * a.os[0] + (hk * a.G + xg) * a.os[1] + xl * a.os[2];
+  store_from_float(op + t, o / total);
 }
 
 template <typename TR>
@@ -283,7 +296,7 @@ int launch_decode_t(const KArgs& a, const DecodePlan& pl, float* ws, hipStream_t
   }
   int rc = (int)hipGetLastError();
   if (rc != 0 || pl.splits == 1) return rc;
-  hipLaunchKernelGGL((merge_kernel<T>), dim3((unsigned)(a.B * a.Hkv)), block, 0, stream, a, pl.splits, ws);
+  hipLaunchKernelGGL((merge_kernel<T>), dim3((unsigned)((long long)a.B * a.Hkv * pl.rows)), dim3(DD), 0, stream, a, pl.splits, ws);
   return (int)hipGetLastError();
 }
 
@@ -302,7 +315,7 @@ DecodePlan plan_decode(const KArgs& a) {
   long long want = (2 * 256 + pairs - 1) / pairs;  // aim for >= 2 workgroups per CU
   int splits = (int)(want < 1 ? 1 : want);
   if (splits > max_splits) splits = max_splits;
-  if (splits > 64) splits = 64;
+  if (splits > kMaxSplits) splits = kMaxSplits;
   int chunk = (a.S + splits - 1) / splits;
   chunk = (chunk + round - 1) / round * round;
   if (chunk < round) chunk = round;
