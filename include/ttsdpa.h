@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TTSDPA_ABI_VERSION 2
+#define TTSDPA_ABI_VERSION 3
 
 /* Element types; numbering is the reference's DType enum (reference src/Tensor/DType.h:20-28). */
 enum ttsdpa_dtype { TTSDPA_F32 = 0, TTSDPA_F16 = 1, TTSDPA_BF16 = 2 };
@@ -94,6 +94,12 @@ typedef struct ttsdpa_params {
   int32_t mask_kind; /* ttsdpa_mask_kind */
   const void* mask;
   int64_t mask_stride[4]; /* elements: batch, head, query row, key; 0 broadcasts the axis */
+  /* Per-batch number of valid keys, int32[B] in device memory, or NULL (all S keys valid).  With a preallocated cache
+   * [B,Hkv,Smax,D] pass S = Smax and the filled lengths here: batch b attends to keys 0 .. min(kv_len[b], S) - 1, the
+   * result the reference gives on K/V grown to that length with op::concat (reference
+   * src/Operation/OpTransform.cpp:306-357).  A length of 0 yields zeros (the reference's empty contraction).
+   * Served by the decode and general kernels. */
+  const int32_t* kv_len;
 } ttsdpa_params;
 
 /* Library identification.  No counterpart in the reference (its device ops are linked statically). */
@@ -124,6 +130,35 @@ int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_byt
 int ttsdpa_prefill(const ttsdpa_params* p, void* stream);
 int ttsdpa_decode(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream);
 int ttsdpa_general(const ttsdpa_params* p, void* stream);
+
+/*
+ * KV-cache append.  The reference has no KV cache: a caller that generates token by token grows K and V with
+ * op::concat on the sequence axis (reference src/Operation/OpTransform.cpp:306-357), an O(S) copy per token.  Here the
+ * caller preallocates k_cache / v_cache [B,Hkv,Smax,D] and this call writes the Lnew new rows of every (batch, kv head)
+ * at rows pos .. pos+Lnew-1, where pos = positions[b] (int32[B], device memory) or `position` when positions is NULL.
+ * Rows that would land at or beyond Smax are dropped.  Strides are in elements {batch, head, sequence}; head_dim stride
+ * is 1.  Enqueued on `stream`; no allocation, no synchronisation.  The matching attention call passes the caches with
+ * S = Smax and ttsdpa_params.kv_len = positions + Lnew.
+ */
+typedef struct ttsdpa_kv_append_params {
+  uint32_t struct_size; /* sizeof(ttsdpa_kv_append_params) */
+  int32_t dtype;        /* ttsdpa_dtype of all four tensors */
+  void* k_cache;
+  void* v_cache;
+  const void* k_new;
+  const void* v_new;
+  int32_t B, Hkv, Smax, Lnew, D;
+  int32_t position;
+  int64_t kc_stride[3];
+  int64_t vc_stride[3];
+  int64_t kn_stride[3];
+  int64_t vn_stride[3];
+  const int32_t* positions;
+} ttsdpa_kv_append_params;
+
+/* Fill *p for dense tensors (cache [B,Hkv,Smax,D], new rows [B,Hkv,Lnew,D]); pointers NULL, position 0. */
+void ttsdpa_kv_append_params_init(ttsdpa_kv_append_params* p, int dtype, int B, int Hkv, int Smax, int Lnew, int D);
+int ttsdpa_kv_append(const ttsdpa_kv_append_params* p, void* stream);
 
 #ifdef __cplusplus
 }

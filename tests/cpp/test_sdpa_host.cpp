@@ -176,6 +176,64 @@ static void test_broadcast_masks() {
   setAssertHandler(old);
 }
 
+static void test_kv_cache() {
+  std::printf("KV cache: append in place, attention over per-batch lengths\n");
+  const int B = 2, Hq = 8, Hkv = 2, D = 128, Smax = 400;
+  const Options gpu = options::device(DeviceType::GPU).dtype(DType::BFloat16);
+  const Options gpuInt = options::device(DeviceType::GPU).dtype(DType::Int32);
+  std::vector<float> kall = pseudoRandom(static_cast<size_t>(B) * Hkv * Smax * D, 7);
+  std::vector<float> vall = pseudoRandom(static_cast<size_t>(B) * Hkv * Smax * D, 8);
+  Tensor tk(kall, {B, Hkv, Smax, D}, gpu), tv(vall, {B, Hkv, Smax, D}, gpu);
+  kall = tk.toList<float>();  // the values the device holds (rounded to bf16)
+  vall = tv.toList<float>();
+  Tensor kc = Tensor::zeros({B, Hkv, Smax, D}, gpu), vc = Tensor::zeros({B, Hkv, Smax, D}, gpu);
+  auto rowsOf = [&](const std::vector<float>& all, int b, int from, int n) {  // [1?]: rows from..from+n-1 of batch b
+    std::vector<float> r(static_cast<size_t>(Hkv) * n * D);
+    for (int h = 0; h < Hkv; h++)
+      for (int j = 0; j < n; j++)
+        for (int d = 0; d < D; d++)
+          r[(static_cast<size_t>(h) * n + j) * D + d] = all[((static_cast<size_t>(b) * Hkv + h) * Smax + from + j) * D + d];
+    return r;
+  };
+  int lens[B] = {0, 0};
+  const int prompt[B] = {300, 41};
+  // prompts: one append per batch entry would need per-entry lengths; append the longer prompt for both at position 0
+  // and let the shorter entry report its own length (its extra rows are overwritten by later appends)
+  {
+    const int n = 300;
+    std::vector<float> kn(static_cast<size_t>(B) * Hkv * n * D), vn(kn.size());
+    for (int b = 0; b < B; b++) {
+      std::vector<float> kb = rowsOf(kall, b, 0, n), vb = rowsOf(vall, b, 0, n);
+      std::copy(kb.begin(), kb.end(), kn.begin() + static_cast<size_t>(b) * Hkv * n * D);
+      std::copy(vb.begin(), vb.end(), vn.begin() + static_cast<size_t>(b) * Hkv * n * D);
+    }
+    op::kvCacheAppend(kc, vc, Tensor(kn, {B, Hkv, n, D}, gpu), Tensor(vn, {B, Hkv, n, D}, gpu), Tensor{}, 0);
+    for (int b = 0; b < B; b++) lens[b] = prompt[b];
+  }
+  for (int step = 0; step < 3; step++) {
+    std::vector<float> kn(static_cast<size_t>(B) * Hkv * D), vn(kn.size());
+    for (int b = 0; b < B; b++) {
+      std::vector<float> kb = rowsOf(kall, b, lens[b], 1), vb = rowsOf(vall, b, lens[b], 1);
+      std::copy(kb.begin(), kb.end(), kn.begin() + static_cast<size_t>(b) * Hkv * D);
+      std::copy(vb.begin(), vb.end(), vn.begin() + static_cast<size_t>(b) * Hkv * D);
+    }
+    Tensor pos(std::vector<int>{lens[0], lens[1]}, {B}, gpuInt);
+    op::kvCacheAppend(kc, vc, Tensor(kn, {B, Hkv, 1, D}, gpu), Tensor(vn, {B, Hkv, 1, D}, gpu), pos, 0);
+    for (int b = 0; b < B; b++) lens[b]++;
+    std::vector<float> q = pseudoRandom(static_cast<size_t>(B) * Hq * D, 20 + step);
+    Tensor tq(q, {B, Hq, 1, D}, gpu);
+    q = tq.toList<float>();
+    Tensor kvLens(std::vector<int>{lens[0], lens[1]}, {B}, gpuInt);
+    std::vector<float> y = op::sdpAttentionCached(tq, kc, vc, kvLens, 1.f / std::sqrt(static_cast<float>(D))).toList<float>();
+    for (int b = 0; b < B; b++) {
+      std::vector<float> qb(q.begin() + static_cast<size_t>(b) * Hq * D, q.begin() + static_cast<size_t>(b + 1) * Hq * D);
+      std::vector<float> ref = closedForm(qb, rowsOf(kall, b, 0, lens[b]), rowsOf(vall, b, 0, lens[b]), 1, Hq, Hkv, 1, lens[b], D, false);
+      std::vector<float> yb(y.begin() + static_cast<size_t>(b) * Hq * D, y.begin() + static_cast<size_t>(b + 1) * Hq * D);
+      EXPECT_TRUE(vectorNear(yb, ref, 2e-2f));
+    }
+  }
+}
+
 static void test_grad_bookkeeping_and_errors() {
   std::printf("Function::apply bookkeeping, dispatcher failure, allocator reuse\n");
   const Options gpu = options::device(DeviceType::GPU).dtype(DType::BFloat16);
@@ -229,6 +287,7 @@ int main() {
   test_func_sdpAttention_reference_vectors();
   test_half_dtypes_and_gqa();
   test_broadcast_masks();
+  test_kv_cache();
   test_grad_bookkeeping_and_errors();
   std::printf(g_failures == 0 ? "ALL PASSED\n" : "%d FAILURES\n", g_failures);
   return g_failures == 0 ? 0 : 1;

@@ -38,14 +38,21 @@ def test_exports_match_header():
 
 
 def test_struct_layout_matches_header():
-    # 4+4, 4 pointers, 6 ints, 12 int64, float, 2 ints, (pad), pointer, 4 int64
-    assert ctypes.sizeof(_capi.Params) == 8 + 32 + 24 + 96 + 12 + 4 + 8 + 32
+    # 4+4, 4 pointers, 6 ints, 12 int64, float, 2 ints, (pad), pointer, 4 int64, pointer
+    assert ctypes.sizeof(_capi.Params) == 8 + 32 + 24 + 96 + 12 + 4 + 8 + 32 + 8
     p = _capi.make_params(_capi.BF16, 2, 32, 8, 4096, 4096, 128)
     assert p.struct_size == ctypes.sizeof(_capi.Params)
     assert list(p.q_stride) == [32 * 4096 * 128, 4096 * 128, 128]
     assert list(p.k_stride) == [8 * 4096 * 128, 4096 * 128, 128]
     assert abs(p.scale - 128 ** -0.5) < 1e-8 and p.causal == 0 and p.mask_kind == 0
     assert list(p.mask_stride) == [0, 0, 4096, 1]  # a dense [L,S] mask shared by every batch and head
+    assert p.kv_len is None
+    # 4+4, 4 pointers, 6 ints, 12 int64, pointer
+    assert ctypes.sizeof(_capi.KvAppendParams) == 8 + 32 + 24 + 96 + 8
+    kp = _capi.KvAppendParams()
+    _capi.lib().ttsdpa_kv_append_params_init(ctypes.byref(kp), _capi.BF16, 4, 8, 1024, 2, 128)
+    assert kp.struct_size == ctypes.sizeof(_capi.KvAppendParams)
+    assert list(kp.kc_stride) == [8 * 1024 * 128, 1024 * 128, 128] and list(kp.vn_stride) == [8 * 2 * 128, 2 * 128, 128]
 
 
 @pytest.mark.parametrize("args,route", [
@@ -108,6 +115,34 @@ def test_validation_errors(mutate, status):
     assert L.ttsdpa_prefill(ctypes.byref(p), None) == status
     assert L.ttsdpa_decode(ctypes.byref(p), None, 0, None) == status
     assert _capi.status_string(status) not in ("ok", "unknown status")
+
+
+def test_kv_len_routes_and_append_validation():
+    # per-batch key counts are served by the decode and general kernels, never by the prefill kernels
+    base = (_capi.BF16, 2, 32, 8, 4096, 4096, 128)
+    assert _capi.plan(params(*base, causal=1))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(*base, causal=1, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.BF16, 8, 32, 8, 1, 4096, 128, kv_len=FAKE))[1] == _capi.ROUTE_DECODE
+    assert _capi.plan(params(_capi.BF16, 8, 32, 8, 1, 4096, 128, kv_len=FAKE + 2))[0] == _capi.ERR_STRIDE
+    L = _capi.lib()
+    kp = _capi.KvAppendParams()
+    L.ttsdpa_kv_append_params_init(ctypes.byref(kp), _capi.BF16, 4, 8, 1024, 2, 128)
+    assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == _capi.ERR_NULL  # pointers missing
+    kp.k_cache = kp.v_cache = kp.k_new = kp.v_new = FAKE
+    kp.struct_size = 12
+    assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == _capi.ERR_ABI
+    kp.struct_size = ctypes.sizeof(_capi.KvAppendParams)
+    kp.dtype = 9
+    assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == _capi.ERR_DTYPE
+    kp.dtype = _capi.BF16
+    kp.kn_stride[2] = 64  # rows of the new tokens overlap
+    assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == _capi.ERR_STRIDE
+    kp.kn_stride[2] = 128
+    kp.positions = FAKE + 1
+    assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == _capi.ERR_STRIDE
+    kp.positions = None
+    kp.Lnew = 0  # nothing to append: accepted without touching the GPU
+    assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == 0
 
 
 def test_kernel_domains_and_workspace():

@@ -316,3 +316,83 @@ def test_host_wrapper_matches_capi():
     hostd, devd = make_inputs(62, 2, 8, 2, 1, 3000, 128, "bf16")
     y = sdpAttention(*devd)
     assert max_abs_err(y, oracle.sdpa_f32(*hostd)) <= TOL["bf16"]
+
+
+# ---- KV cache: append in place + per-batch key counts (what a token-by-token caller of the reference would get from
+# growing K/V with op::concat and calling sdpAttention on the grown tensors) -------------------------------------------
+
+def _cache_case(dtype, B, Hq, Hkv, D, Smax, seed):
+    kfull = oracle.randn(seed, 1, (B, Hkv, Smax, D))
+    vfull = oracle.randn(seed, 2, (B, Hkv, Smax, D))
+    kv, kb = oracle.round_to(kfull, dtype)
+    vv, vb = oracle.round_to(vfull, dtype)
+    return kv, vv, to_device(kv, kb, dtype), to_device(vv, vb, dtype)
+
+
+@pytest.mark.parametrize("dtype,B,Hq,Hkv,D,Smax,L", [
+    ("bf16", 3, 8, 2, 128, 700, 1),    # decode route, one row per head
+    ("f16", 2, 8, 8, 128, 300, 1),
+    ("bf16", 2, 8, 2, 128, 520, 3),    # three new tokens per step (12 rows per KV head)
+    ("f32", 2, 4, 2, 64, 90, 1),       # general route
+    ("bf16", 2, 4, 4, 64, 130, 2),     # general route, 16-bit, head_dim 64
+])
+def test_kv_cache_generation_matches_concat(dtype, B, Hq, Hkv, D, Smax, L):
+    from tinytorch_amd import kvCacheAppend, sdpAttention
+    kh, vh, kd, vd = _cache_case(dtype, B, Hq, Hkv, D, Smax, 70 + Smax)
+    kc = torch.zeros_like(kd)
+    vc = torch.zeros_like(vd)
+    # prompts of different lengths, appended in one call per batch entry count: position 0, Lnew = the longest prompt,
+    # then the shorter entries simply report a smaller length (their extra rows are overwritten later)
+    lens = np.array([(37 * (b + 1)) % (Smax // 2) + 5 for b in range(B)], np.int32)
+    pmax = int(lens.max())
+    kvCacheAppend(kc, vc, kd[:, :, :pmax], vd[:, :, :pmax], 0)
+    steps = 4
+    for step in range(steps):
+        pos = torch.from_numpy(lens).cuda()
+        # the new tokens of batch b are rows lens[b] .. lens[b]+L-1 of the full tensors: gather them per batch entry
+        knew = torch.stack([kd[b, :, lens[b]:lens[b] + L] for b in range(B)])
+        vnew = torch.stack([vd[b, :, lens[b]:lens[b] + L] for b in range(B)])
+        kvCacheAppend(kc, vc, knew, vnew, pos)
+        lens = lens + L
+        qh, qb = oracle.round_to(oracle.randn(900 + step, 0, (B, Hq, L, D)), dtype)
+        q = to_device(qh, qb, dtype)
+        out = sdpAttention(q, kc, vc, kvLens=torch.from_numpy(lens).cuda())
+        torch.cuda.synchronize()
+        for b in range(B):
+            exp = oracle.sdpa_f32(qh[b:b + 1], kh[b:b + 1, :, :lens[b]], vh[b:b + 1, :, :lens[b]])
+            assert max_abs_err(out[b:b + 1], exp) <= TOL[dtype], (step, b)
+    # the caches hold exactly the rows of the full tensors up to each length
+    for b in range(B):
+        assert torch.equal(kc[b, :, :lens[b]], kd[b, :, :lens[b]]) and torch.equal(vc[b, :, :lens[b]], vd[b, :, :lens[b]])
+
+
+def test_kv_len_edge_cases():
+    from tinytorch_amd import kvCacheAppend, sdpAttention
+    B, Hq, Hkv, D, Smax = 3, 4, 2, 128, 600
+    kh, vh, kd, vd = _cache_case("bf16", B, Hq, Hkv, D, Smax, 77)
+    qh, qb = oracle.round_to(oracle.randn(78, 0, (B, Hq, 1, D)), "bf16")
+    q = to_device(qh, qb, "bf16")
+    lens = torch.tensor([0, 1, 9999], dtype=torch.int32, device="cuda")  # empty, one key, more than the cache holds
+    for route_q, tol in ((q, TOL["bf16"]), (q.float(), TOL["f32"])):   # decode route, then general route (fp32)
+        k, v = (kd, vd) if route_q.dtype == torch.bfloat16 else (kd.float(), vd.float())
+        out = sdpAttention(route_q, k, v, kvLens=lens)
+        assert torch.count_nonzero(out[0]) == 0                       # no keys: zeros, the reference's empty contraction
+        assert max_abs_err(out[1:2], np.repeat(vh[1:2, :, 0:1, :], Hq // Hkv, axis=1)) <= tol  # one key: its value row
+        assert max_abs_err(out[2:3], oracle.sdpa_f32(qh[2:3], kh[2:3], vh[2:3])) <= tol
+    # rows that do not fit the cache are dropped, everything else is untouched
+    kc, vc = torch.zeros_like(kd), torch.zeros_like(vd)
+    kvCacheAppend(kc, vc, kd[:, :, :4], vd[:, :, :4], torch.tensor([Smax - 2, 10, Smax + 5], dtype=torch.int32, device="cuda"))
+    assert torch.equal(kc[0, :, Smax - 2:], kd[0, :, :2]) and torch.count_nonzero(kc[0, :, :Smax - 2]) == 0
+    assert torch.equal(kc[1, :, 10:14], kd[1, :, :4]) and torch.count_nonzero(kc[2]) == 0
+    # strided cache views and rows narrower than 16 bytes
+    big = torch.zeros(2, 2, 50, 2 * 20, dtype=torch.float16, device="cuda")
+    kc2, vc2 = big[..., :20], big[..., 20:]
+    kn = torch.randn(2, 2, 3, 20, device="cuda").half()
+    vn = torch.randn(2, 2, 3, 20, device="cuda").half()
+    kvCacheAppend(kc2, vc2, kn, vn, 7)
+    assert torch.equal(kc2[:, :, 7:10], kn) and torch.equal(vc2[:, :, 7:10], vn) and torch.count_nonzero(big[:, :, :7]) == 0
+    kc3 = torch.zeros(1, 1, 9, 3, dtype=torch.bfloat16, device="cuda")
+    vc3 = torch.zeros_like(kc3)
+    kn3 = torch.randn(1, 1, 2, 3, device="cuda").bfloat16()
+    kvCacheAppend(kc3, vc3, kn3, kn3, 5)
+    assert torch.equal(kc3[:, :, 5:7], kn3) and torch.equal(vc3[:, :, 5:7], kn3)

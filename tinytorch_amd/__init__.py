@@ -7,6 +7,6 @@ from . import _capi
 
 _capi.lib()  # fail loudly when the extension is missing
 
-from .function import sdpAttention, build_params  # noqa: E402
+from .function import sdpAttention, kvCacheAppend, build_params  # noqa: E402
 
-__all__ = ["sdpAttention", "build_params"]
+__all__ = ["sdpAttention", "kvCacheAppend", "build_params"]

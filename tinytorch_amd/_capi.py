@@ -19,6 +19,7 @@ ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_STRIDE, ERR_MASK, ERR_WORKSPACE, ERR_UNSUPPO
 EXPORTS = [
     "ttsdpa_abi_version", "ttsdpa_status_string", "ttsdpa_params_init", "ttsdpa_plan", "ttsdpa_workspace_bytes",
     "ttsdpa_forward", "ttsdpa_prefill", "ttsdpa_decode", "ttsdpa_general",
+    "ttsdpa_kv_append_params_init", "ttsdpa_kv_append",
 ]
 
 
@@ -42,6 +43,27 @@ class Params(ctypes.Structure):
         ("mask_kind", ctypes.c_int32),
         ("mask", ctypes.c_void_p),
         ("mask_stride", ctypes.c_int64 * 4),
+        ("kv_len", ctypes.c_void_p),
+    ]
+
+
+class KvAppendParams(ctypes.Structure):
+    """struct ttsdpa_kv_append_params"""
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("dtype", ctypes.c_int32),
+        ("k_cache", ctypes.c_void_p),
+        ("v_cache", ctypes.c_void_p),
+        ("k_new", ctypes.c_void_p),
+        ("v_new", ctypes.c_void_p),
+        ("B", ctypes.c_int32), ("Hkv", ctypes.c_int32), ("Smax", ctypes.c_int32),
+        ("Lnew", ctypes.c_int32), ("D", ctypes.c_int32),
+        ("position", ctypes.c_int32),
+        ("kc_stride", ctypes.c_int64 * 3),
+        ("vc_stride", ctypes.c_int64 * 3),
+        ("kn_stride", ctypes.c_int64 * 3),
+        ("vn_stride", ctypes.c_int64 * 3),
+        ("positions", ctypes.c_void_p),
     ]
 
 
@@ -77,7 +99,11 @@ def lib():
         L.ttsdpa_decode.restype = ctypes.c_int
         L.ttsdpa_general.argtypes = [P, ctypes.c_void_p]
         L.ttsdpa_general.restype = ctypes.c_int
-        if L.ttsdpa_abi_version() != 2:
+        L.ttsdpa_kv_append_params_init.argtypes = [ctypes.POINTER(KvAppendParams)] + [ctypes.c_int] * 6
+        L.ttsdpa_kv_append_params_init.restype = None
+        L.ttsdpa_kv_append.argtypes = [ctypes.POINTER(KvAppendParams), ctypes.c_void_p]
+        L.ttsdpa_kv_append.restype = ctypes.c_int
+        if L.ttsdpa_abi_version() != 3:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L
     return _lib

@@ -13,6 +13,7 @@ struct KArgs {
   const void* v;
   void* out;
   const void* mask;
+  const int* kv_len;  // per-batch valid key count (device), or nullptr
   int B, Hq, Hkv, L, S, D;
   int G;  // Hq / Hkv: query heads per KV head
   int causal;
@@ -83,6 +84,16 @@ int launch_prefill(const KArgs& a, int dtype, hipStream_t stream);       // 128-
 int launch_prefill_d128(const KArgs& a, int dtype, hipStream_t stream);  // 256-row workgroups, pipelined; head_dim 128
 int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream);
 int launch_zero(const KArgs& a, int dtype, hipStream_t stream);
+struct KvAppendArgs {
+  void* kc;
+  void* vc;
+  const void* kn;
+  const void* vn;
+  const int* positions;
+  int B, Hkv, Smax, Lnew, D, position, esz;
+  long long kcs[3], vcs[3], kns[3], vns[3];
+};
+int launch_kv_append(const KvAppendArgs& a, hipStream_t stream);
 
 // Decode tiling, shared by the workspace-size query and the launcher.
 struct DecodePlan {

@@ -75,6 +75,11 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
   const int hk = n % a.Hkv;
   const int b = n / a.Hkv;
   const int rows = a.L * a.G;  // query rows sharing this KV head, row x = (l, g) = (x / G, x % G)
+  int S = a.S;                 // keys of this batch entry: the whole cache, or its filled prefix
+  if (a.kv_len) {
+    int len = a.kv_len[b];
+    S = len < 0 ? 0 : (len < S ? len : S);
+  }
 
   const T* kp = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
   const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
@@ -107,7 +112,7 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
   const float c = a.scale * kLog2e;
 
   const int s_begin = split * chunk;
-  const int s_end = s_begin + chunk < a.S ? s_begin + chunk : a.S;
+  const int s_end = s_begin + chunk < S ? s_begin + chunk : S;
   float* pl = Pl[wave];
 
   for (int k0 = s_begin + wave * KB; k0 < s_end; k0 += NWAVE * KB) {
@@ -116,7 +121,7 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
 #pragma unroll
     for (int gi = 0; gi < 2; gi++) {
       int key = k0 + 16 * gi + l16;
-      key = key < a.S ? key : a.S - 1;
+      key = key < S ? key : S - 1;
       const T* kr = kp + key * a.ks[2] + 8 * lg;
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) kreg[gi][ks] = __builtin_nontemporal_load((const u32x4*)(kr + 32 * ks));  // read once: keep it out of the caches
@@ -125,7 +130,7 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
 #pragma unroll
     for (int i = 0; i < KB / 4; i++) {
       int key = k0 + 4 * i + lg;
-      key = key < a.S ? key : a.S - 1;
+      key = key < S ? key : S - 1;
       vreg[i] = __builtin_nontemporal_load((const u32x4*)(vp + key * a.vs[2] + 8 * l16));
     }
 
@@ -233,7 +238,7 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
     if (splits == 1) {
       int xl = x / a.G, xg = x % a.G;
       T* op = (T*)a.out + b * a.os[0] + (hk * a.G + xg) * a.os[1] + xl * a.os[2];
-      store_from_float(op + d, o / lsum);
+      store_from_float(op + d, lsum > 0.f ? o / lsum : 0.f);  // no keys at all: zeros, as the reference's empty contraction
     } else {
       float* rec = ws + ((long long)blockIdx.x * rows + x) * (DD + 2);
       rec[d] = o;
@@ -280,7 +285,7 @@ __global__ __launch_bounds__(DD) void merge_kernel(KArgs a, int splits, const fl
   for (int s = 0; s < splits; s++) o = fmaf(weight[s], rec0[s * step + t], o);
   const int xl = x / a.G, xg = x % a.G;
   T* op = (T*)a.out + b * a.os[0] + (hk * a.G + xg) * a.os[1] + xl * a.os[2];
-  store_from_float(op + t, o / total);
+  store_from_float(op + t, total > 0.f ? o / total : 0.f);
 }
 
 template <typename TR>

@@ -57,10 +57,15 @@ __global__ __launch_bounds__(256) void general_kernel(KArgs a) {
   }
   float m = -FLT_MAX, l = 0.f;
 
-  int send = a.S;
+  int S = a.S;  // keys of this batch entry: all of them, or the filled prefix of a cache
+  if (a.kv_len) {
+    int len = a.kv_len[b];
+    S = len < 0 ? 0 : (len < S ? len : S);
+  }
+  int send = S;
   if (a.causal) {
     int last = row0 + kRows - 1 < a.L - 1 ? row0 + kRows - 1 : a.L - 1;
-    send = last + 1 < a.S ? last + 1 : a.S;
+    send = last + 1 < S ? last + 1 : S;
   }
 
   for (int k0 = 0; k0 < send; k0 += kTileK) {
@@ -69,7 +74,7 @@ __global__ __launch_bounds__(256) void general_kernel(KArgs a) {
       int kk = e / DP, d = e % DP;
       int key = k0 + kk;
       float kv = 0.f, vv = 0.f;
-      if (key < a.S && d < a.D) {
+      if (key < S && d < a.D) {
         kv = load_as_float(kp + key * a.ks[2] + d);
         vv = load_as_float(vp + key * a.vs[2] + d);
       }
@@ -91,11 +96,11 @@ __global__ __launch_bounds__(256) void general_kernel(KArgs a) {
         part += __shfl_xor(part, 2);
         float x = part * a.scale;
         int key = k0 + c0 + j;
-        bool hidden = key >= a.S || (a.causal && key > row);
+        bool hidden = key >= S || (a.causal && key > row);
         if (a.mask_kind == 1) {
-          if (key < a.S && ((const uint8_t*)a.mask)[mrow + key * a.ms[3]] == 0) hidden = true;
+          if (key < S && ((const uint8_t*)a.mask)[mrow + key * a.ms[3]] == 0) hidden = true;
         } else if (a.mask_kind == 2) {
-          if (key < a.S) x += load_as_float((const T*)a.mask + mrow + key * a.ms[3]);
+          if (key < S) x += load_as_float((const T*)a.mask + mrow + key * a.ms[3]);
         }
         if (hidden) x = -INFINITY;
         s[j] = x;
@@ -123,7 +128,7 @@ __global__ __launch_bounds__(256) void general_kernel(KArgs a) {
 
   if (row < a.L) {
     T* op = (T*)a.out + b * a.os[0] + h * a.os[1] + row * a.os[2];
-    float inv = 1.f / l;
+    float inv = S == 0 ? 0.f : 1.f / l;  // no keys: zeros (the reference's empty contraction); hidden rows: NaN
 #pragma unroll
     for (int t = 0; t < DQ; t++) {
       int d = 4 * t + sub;

@@ -45,6 +45,8 @@ int validate(const ttsdpa_params* p, KArgs* a) {
     a->ms[i] = p->mask_kind != TTSDPA_MASK_NONE ? p->mask_stride[i] : 0;
   }
   if (p->mask_kind == TTSDPA_MASK_ADD && !ptr_aligned(p->mask, esz)) return TTSDPA_ERR_STRIDE;
+  if (p->kv_len && !ptr_aligned(p->kv_len, 4)) return TTSDPA_ERR_STRIDE;
+  a->kv_len = p->kv_len;
   a->q = p->q, a->k = p->k, a->v = p->v, a->out = p->out, a->mask = p->mask;
   a->B = p->B, a->Hq = p->Hq, a->Hkv = p->Hkv, a->L = p->L, a->S = p->S, a->D = p->D;
   a->G = p->Hq / p->Hkv;
@@ -69,6 +71,7 @@ bool fast_layout_ok(const ttsdpa_params* p) {
 }
 
 bool prefill_ok(const ttsdpa_params* p) {
+  if (p->kv_len) return false;  // per-batch key counts are served by the decode and general kernels
   return fast_layout_ok(p) && (p->D == 128 || p->D == 64) && p->S >= 1 && p->L >= 1;
 }
 
@@ -125,6 +128,7 @@ void ttsdpa_params_init(ttsdpa_params* p, int dtype, int B, int Hq, int Hkv, int
   p->mask_kind = TTSDPA_MASK_NONE;
   p->mask = nullptr;
   p->mask_stride[0] = 0, p->mask_stride[1] = 0, p->mask_stride[2] = S, p->mask_stride[3] = 1;
+  p->kv_len = nullptr;
 }
 
 int ttsdpa_plan(const ttsdpa_params* p, int* route) {
@@ -190,6 +194,39 @@ int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_byt
     case TTSDPA_ROUTE_PREFILL: return ttsdpa_prefill(p, stream);
     default: return ttsdpa_general(p, stream);
   }
+}
+
+void ttsdpa_kv_append_params_init(ttsdpa_kv_append_params* p, int dtype, int B, int Hkv, int Smax, int Lnew, int D) {
+  memset(p, 0, sizeof(*p));
+  p->struct_size = sizeof(*p);
+  p->dtype = dtype;
+  p->B = B, p->Hkv = Hkv, p->Smax = Smax, p->Lnew = Lnew, p->D = D;
+  p->kc_stride[0] = (int64_t)Hkv * Smax * D, p->kc_stride[1] = (int64_t)Smax * D, p->kc_stride[2] = D;
+  p->kn_stride[0] = (int64_t)Hkv * Lnew * D, p->kn_stride[1] = (int64_t)Lnew * D, p->kn_stride[2] = D;
+  for (int i = 0; i < 3; i++) p->vc_stride[i] = p->kc_stride[i], p->vn_stride[i] = p->kn_stride[i];
+}
+
+int ttsdpa_kv_append(const ttsdpa_kv_append_params* p, void* stream) {
+  if (!p) return TTSDPA_ERR_NULL;
+  if (p->struct_size != sizeof(ttsdpa_kv_append_params)) return TTSDPA_ERR_ABI;
+  if (p->dtype != TTSDPA_F32 && p->dtype != TTSDPA_F16 && p->dtype != TTSDPA_BF16) return TTSDPA_ERR_DTYPE;
+  if (p->B < 0 || p->Hkv < 1 || p->Smax < 0 || p->Lnew < 0 || p->D < 1) return TTSDPA_ERR_SHAPE;
+  if (p->B == 0 || p->Lnew == 0 || p->Smax == 0) return TTSDPA_OK;
+  if (!p->k_cache || !p->v_cache || !p->k_new || !p->v_new) return TTSDPA_ERR_NULL;
+  const size_t esz = p->dtype == TTSDPA_F32 ? 4 : 2;
+  if (!ptr_aligned(p->k_cache, esz) || !ptr_aligned(p->v_cache, esz) || !ptr_aligned(p->k_new, esz) ||
+      !ptr_aligned(p->v_new, esz) || (p->positions && !ptr_aligned(p->positions, 4)))
+    return TTSDPA_ERR_STRIDE;
+  KvAppendArgs a;
+  for (int i = 0; i < 3; i++) {
+    if (p->kc_stride[i] < 0 || p->vc_stride[i] < 0 || p->kn_stride[i] < 0 || p->vn_stride[i] < 0) return TTSDPA_ERR_STRIDE;
+    a.kcs[i] = p->kc_stride[i], a.vcs[i] = p->vc_stride[i], a.kns[i] = p->kn_stride[i], a.vns[i] = p->vn_stride[i];
+  }
+  if ((p->kc_stride[2] < p->D || p->vc_stride[2] < p->D) && p->Smax > 1) return TTSDPA_ERR_STRIDE;
+  if ((p->kn_stride[2] < p->D || p->vn_stride[2] < p->D) && p->Lnew > 1) return TTSDPA_ERR_STRIDE;
+  a.kc = p->k_cache, a.vc = p->v_cache, a.kn = p->k_new, a.vn = p->v_new, a.positions = p->positions;
+  a.B = p->B, a.Hkv = p->Hkv, a.Smax = p->Smax, a.Lnew = p->Lnew, a.D = p->D, a.position = p->position, a.esz = (int)esz;
+  return launch_kv_append(a, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -31,7 +31,7 @@ def _strides3(t):
     return (t.stride(0), t.stride(1), t.stride(2))
 
 
-def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=None):
+def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=None, kvLens=None):
     """Fill a ttsdpa_params for 4-D tensors [B,H,N,D]."""
     B, Hq, L, D = query.shape
     Bk, Hkv, S, Dk = key.shape
@@ -69,14 +69,22 @@ def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=No
         p.mask = attnMask.data_ptr()
         for i in range(4):
             p.mask_stride[i] = full.stride(i) if full.size(i) > 1 else 0
+    if kvLens is not None:
+        if kvLens.dtype != torch.int32 or kvLens.dim() != 1 or kvLens.numel() != B or not kvLens.is_contiguous():
+            raise ValueError("sdpAttention: kvLens must be a contiguous int32 tensor of B entries")
+        if kvLens.device != query.device:
+            raise RuntimeError("sdpAttention: kvLens must live on the device of the tensors")
+        p.kv_len = kvLens.data_ptr()
     return p
 
 
-def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0, scale=None):
+def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0, scale=None, kvLens=None):
     """out = softmax(query @ key^T * scale + bias) @ value on the GPU.
 
     query [B,Hq,L,D]; key/value [B,Hkv,S,D] with Hq a multiple of Hkv (query head h reads KV head h // (Hq//Hkv));
     returns [B,Hq,L,D] in the dtype of query.  isCausal is top-left aligned (key j visible iff j <= i).
+    kvLens (not in the reference, which has no KV cache): int32 [B] on the device; batch b attends to the first
+    kvLens[b] keys only, so key/value may be preallocated caches [B,Hkv,Smax,D] filled by kvCacheAppend.
     """
     if dropoutP != 0.0:
         raise NotImplementedError("sdpAttention: dropoutP must be 0 on this path")
@@ -89,7 +97,7 @@ def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0,
     fix = lambda t: t if (t.stride(-1) == 1 or t.size(-1) == 1) else t.contiguous()
     query, key, value = fix(query), fix(key), fix(value)
     out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
-    p = build_params(query, key, value, out, isCausal, attnMask, scale)
+    p = build_params(query, key, value, out, isCausal, attnMask, scale, kvLens)
     L = _capi.lib()
     with torch.cuda.device(query.device):
         nbytes = L.ttsdpa_workspace_bytes(ctypes.byref(p))
@@ -99,3 +107,42 @@ def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0,
     if rc != 0:
         raise RuntimeError("ttsdpa_forward failed: %d (%s)" % (rc, _capi.status_string(rc)))
     return out
+
+
+def kvCacheAppend(kCache, vCache, kNew, vNew, positions):
+    """Write kNew/vNew [B,Hkv,Lnew,D] into the caches [B,Hkv,Smax,D] at rows positions[b] .. positions[b]+Lnew-1.
+
+    positions: int32 [B] device tensor, or an int used for every batch entry.  In place, on the current stream; rows
+    that would land beyond Smax are dropped.  Replaces growing K/V with op::concat on the sequence axis (reference
+    src/Operation/OpTransform.cpp:306-357), which copies the whole history per generated token.
+    """
+    if kCache.dim() != 4 or kNew.dim() != 4 or vCache.shape != kCache.shape or vNew.shape != kNew.shape:
+        raise ValueError("kvCacheAppend: expected caches [B,Hkv,Smax,D] and new rows [B,Hkv,Lnew,D]")
+    B, Hkv, Smax, D = kCache.shape
+    if kNew.shape[0] != B or kNew.shape[1] != Hkv or kNew.shape[3] != D:
+        raise ValueError("kvCacheAppend: new rows %s do not match the cache %s" % (tuple(kNew.shape), tuple(kCache.shape)))
+    if kCache.dtype not in _DTYPES or any(t.dtype != kCache.dtype for t in (vCache, kNew, vNew)):
+        raise TypeError("kvCacheAppend: dtype must be one of float32/float16/bfloat16 and equal for all four tensors")
+    if not kCache.is_cuda or any(t.device != kCache.device for t in (vCache, kNew, vNew)):
+        raise RuntimeError("kvCacheAppend runs on the GPU only, all tensors on one device")
+    for t in (kCache, vCache, kNew, vNew):
+        if t.stride(-1) != 1 and t.size(-1) != 1:
+            raise ValueError("kvCacheAppend: head_dim must be contiguous")
+    p = _capi.KvAppendParams()
+    L = _capi.lib()
+    L.ttsdpa_kv_append_params_init(ctypes.byref(p), _DTYPES[kCache.dtype], B, Hkv, Smax, kNew.shape[2], D)
+    p.k_cache, p.v_cache, p.k_new, p.v_new = kCache.data_ptr(), vCache.data_ptr(), kNew.data_ptr(), vNew.data_ptr()
+    for name, t in (("kc_stride", kCache), ("vc_stride", vCache), ("kn_stride", kNew), ("vn_stride", vNew)):
+        for i in range(3):
+            getattr(p, name)[i] = t.stride(i)
+    if isinstance(positions, int):
+        p.position = positions
+    else:
+        if positions.dtype != torch.int32 or positions.numel() != B or not positions.is_contiguous() \
+                or positions.device != kCache.device:
+            raise ValueError("kvCacheAppend: positions must be a contiguous int32 device tensor of B entries")
+        p.positions = positions.data_ptr()
+    with torch.cuda.device(kCache.device):
+        rc = L.ttsdpa_kv_append(ctypes.byref(p), torch.cuda.current_stream().cuda_stream)
+    if rc != 0:
+        raise RuntimeError("ttsdpa_kv_append failed: %d (%s)" % (rc, _capi.status_string(rc)))

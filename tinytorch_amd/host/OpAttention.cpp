@@ -80,12 +80,81 @@ Tensor sdpAttentionGpuImpl(const Tensor& query, const Tensor& key, const Tensor&
   return out;
 }
 
+void kvCacheAppendGpuImpl(const Tensor& kCache, const Tensor& vCache, const Tensor& kNew, const Tensor& vNew,
+                          const Tensor& positions, int32_t position) {
+  ASSERT(kCache.defined() && vCache.defined() && kNew.defined() && vNew.defined());
+  ASSERT(kCache.dim() == 4 && kNew.dim() == 4 && kCache.shape() == vCache.shape() && kNew.shape() == vNew.shape());
+  ASSERT(kNew.size(0) == kCache.size(0) && kNew.size(1) == kCache.size(1) && kNew.size(3) == kCache.size(3));
+  ASSERT(vCache.dtype() == kCache.dtype() && kNew.dtype() == kCache.dtype() && vNew.dtype() == kCache.dtype());
+  ASSERT(vCache.device() == kCache.device() && kNew.device() == kCache.device() && vNew.device() == kCache.device());
+  if (kCache.dim() != 4 || kNew.dim() != 4 || kCache.shape() != vCache.shape() || kNew.shape() != vNew.shape()) return;
+  if (kNew.size(0) != kCache.size(0) || kNew.size(1) != kCache.size(1) || kNew.size(3) != kCache.size(3)) return;
+  ttsdpa_kv_append_params p;
+  ttsdpa_kv_append_params_init(&p, dtypeCode(kCache.dtype()), static_cast<int>(kCache.size(0)),
+                               static_cast<int>(kCache.size(1)), static_cast<int>(kCache.size(2)),
+                               static_cast<int>(kNew.size(2)), static_cast<int>(kCache.size(3)));
+  p.k_cache = kCache.rawPtr(), p.v_cache = vCache.rawPtr(), p.k_new = kNew.rawPtr(), p.v_new = vNew.rawPtr();
+  p.position = position;
+  if (positions.defined()) {
+    ASSERT(positions.dtype() == DType::Int32 && positions.numel() == kCache.size(0) &&
+           positions.device() == kCache.device());
+    if (positions.dtype() != DType::Int32 || positions.numel() != kCache.size(0)) return;
+    p.positions = static_cast<const int32_t*>(positions.rawPtr());
+  }
+  const DeviceIndex dev = kCache.device().index;
+  HIP_CHECK(hipSetDevice(dev));
+  const int rc = ttsdpa_kv_append(&p, getCurrentStream(dev));
+  if (rc != TTSDPA_OK) {
+    LOGE("ttsdpa_kv_append failed: %d (%s)", rc, ttsdpa_status_string(rc));
+    ASSERT(rc == TTSDPA_OK);
+  }
+}
+
+Tensor sdpAttentionCachedGpuImpl(const Tensor& query, const Tensor& kCache, const Tensor& vCache, const Tensor& kvLens,
+                                 float scale) {
+  ASSERT(query.defined() && kCache.defined() && vCache.defined() && kvLens.defined());
+  ASSERT(query.dim() == 4 && kCache.dim() == 4 && kCache.shape() == vCache.shape());
+  ASSERT(kCache.size(0) == query.size(0) && kCache.size(3) == query.size(3) && query.size(1) % kCache.size(1) == 0);
+  ASSERT(kCache.dtype() == query.dtype() && vCache.dtype() == query.dtype());
+  ASSERT(kvLens.dtype() == DType::Int32 && kvLens.numel() == query.size(0) && kvLens.device() == query.device());
+  if (query.dim() != 4 || kCache.dim() != 4 || kCache.shape() != vCache.shape() || kCache.size(0) != query.size(0) ||
+      kCache.size(3) != query.size(3) || query.size(1) % kCache.size(1) != 0 || kvLens.dtype() != DType::Int32 ||
+      kvLens.numel() != query.size(0))
+    return {};
+  ttsdpa_params p;
+  ttsdpa_params_init(&p, dtypeCode(query.dtype()), static_cast<int>(query.size(0)), static_cast<int>(query.size(1)),
+                     static_cast<int>(kCache.size(1)), static_cast<int>(query.size(2)),
+                     static_cast<int>(kCache.size(2)), static_cast<int>(query.size(3)));
+  Tensor out = Tensor::empty(query.shape(), query.options().noGrad());
+  p.q = query.rawPtr(), p.k = kCache.rawPtr(), p.v = vCache.rawPtr(), p.out = out.rawPtr();
+  p.scale = scale;
+  p.kv_len = static_cast<const int32_t*>(kvLens.rawPtr());
+  const DeviceIndex dev = query.device().index;
+  HIP_CHECK(hipSetDevice(dev));
+  const size_t wsBytes = ttsdpa_workspace_bytes(&p);
+  std::shared_ptr<Storage> ws;
+  if (wsBytes) ws = std::make_shared<Storage>(wsBytes, query.device());
+  const int rc = ttsdpa_forward(&p, ws ? ws->data() : nullptr, wsBytes, getCurrentStream(dev));
+  if (rc != TTSDPA_OK) {
+    LOGE("ttsdpa_forward failed: %d (%s)", rc, ttsdpa_status_string(rc));
+    ASSERT(rc == TTSDPA_OK);
+    return {};
+  }
+  return out;
+}
+
 }  // namespace
 
 void registerAttentionGpu() {
   REGISTER_OP_IMPL(sdpAttention, GPU, Float32, &sdpAttentionGpuImpl);
   REGISTER_OP_IMPL(sdpAttention, GPU, Float16, &sdpAttentionGpuImpl);
   REGISTER_OP_IMPL(sdpAttention, GPU, BFloat16, &sdpAttentionGpuImpl);
+  REGISTER_OP_IMPL(kvCacheAppend, GPU, Float32, &kvCacheAppendGpuImpl);
+  REGISTER_OP_IMPL(kvCacheAppend, GPU, Float16, &kvCacheAppendGpuImpl);
+  REGISTER_OP_IMPL(kvCacheAppend, GPU, BFloat16, &kvCacheAppendGpuImpl);
+  REGISTER_OP_IMPL(sdpAttentionCached, GPU, Float32, &sdpAttentionCachedGpuImpl);
+  REGISTER_OP_IMPL(sdpAttentionCached, GPU, Float16, &sdpAttentionCachedGpuImpl);
+  REGISTER_OP_IMPL(sdpAttentionCached, GPU, BFloat16, &sdpAttentionCachedGpuImpl);
 }
 
 }  // namespace tinytorch::op

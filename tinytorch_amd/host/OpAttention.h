@@ -19,6 +19,19 @@ using SdpAttentionOpFn = Tensor (*)(const Tensor& query, const Tensor& key, cons
 
 DEFINE_OP(sdpAttention, SdpAttentionOpFn)
 
+// KV cache (no counterpart in the reference, whose callers would grow K/V with op::concat on the sequence axis,
+// src/Operation/OpTransform.cpp:306-357, copying the whole history per generated token).
+// kvCacheAppend writes kNew/vNew [B,Hkv,Lnew,D] into the preallocated caches [B,Hkv,Smax,D] in place, at rows
+// positions[b] .. +Lnew-1 (positions: Int32 [B] on the device; undefined = `position` for every batch entry); rows
+// that do not fit are dropped.  sdpAttentionCached attends query [B,Hq,L,D] to the first kvLens[b] rows of the caches
+// (kvLens: Int32 [B] on the device), not causal, no mask.
+using KvCacheAppendOpFn = void (*)(const Tensor& kCache, const Tensor& vCache, const Tensor& kNew, const Tensor& vNew,
+                                   const Tensor& positions, int32_t position);
+using SdpAttentionCachedOpFn = Tensor (*)(const Tensor& query, const Tensor& kCache, const Tensor& vCache,
+                                          const Tensor& kvLens, float scale);
+DEFINE_OP(kvCacheAppend, KvCacheAppendOpFn)
+DEFINE_OP(sdpAttentionCached, SdpAttentionCachedOpFn)
+
 void registerAttentionGpu();
 STATIC_CALL(registerAttentionGpu);
 
