@@ -1,0 +1,67 @@
+"""Seeded random call shapes through ttsdpa_forward against the oracle: every route, ragged sizes, grouped heads,
+causal / masks / per-batch key counts.  The shapes are drawn once from a fixed seed, so a failure names its case."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import TOL, make_inputs, max_abs_err, route_of, to_device
+from tinytorch_amd import sdpAttention
+
+pytestmark = pytest.mark.gpu
+
+
+def _cases():
+    rng = np.random.RandomState(20240607)
+    out = []
+    for i in range(48):
+        dtype = ["bf16", "f16", "f32"][rng.randint(3)]
+        D = [128, 128, 128, 64, 32, 80][rng.randint(6)]
+        Hkv = int(rng.randint(1, 4))
+        G = [1, 1, 2, 4, 7][rng.randint(5)]
+        B = int(rng.randint(1, 4))
+        kind = ["prefill", "prefill", "decode", "short"][rng.randint(4)]
+        if kind == "prefill":
+            L = int(rng.randint(129, 700))
+            S = L if rng.rand() < 0.5 else int(rng.randint(1, 900))
+        elif kind == "decode":
+            L = int(rng.randint(1, 4))
+            S = int(rng.randint(1, 3000))
+            G = min(G, 16 // L)
+        else:
+            L = int(rng.randint(1, 129))
+            S = int(rng.randint(1, 400))
+        extra = ["none", "none", "causal", "causal", "boolmask", "addmask", "kvlen"][rng.randint(7)]
+        out.append((i, dtype, B, Hkv * G, Hkv, L, S, D, extra))
+    return out
+
+
+@pytest.mark.parametrize("case", _cases(), ids=lambda c: "%d-%s-B%d-H%d/%d-L%d-S%d-D%d-%s" % c)
+def test_random_shape(case):
+    i, dtype, B, Hq, Hkv, L, S, D, extra = case
+    host, dev = make_inputs(3000 + i, B, Hq, Hkv, L, S, D, dtype)
+    kw_dev, kw_host = {}, {}
+    if extra == "causal":
+        kw_dev["isCausal"] = True
+        kw_host["causal"] = True
+    elif extra == "boolmask":
+        m = (np.random.RandomState(i).rand(B, 1, L, S) > 0.4).astype(np.uint8)
+        m[..., 0] = 1  # no row without a visible key
+        kw_dev["attnMask"] = torch.from_numpy(m).cuda().bool()
+        kw_host["mask"] = m
+    elif extra == "addmask":
+        m, bits = oracle.round_to(oracle.randn(4000 + i, 5, (Hq, 1, S)), dtype)
+        kw_dev["attnMask"] = to_device(m, bits, dtype)
+        kw_host["mask"] = m
+    if extra == "kvlen":
+        lens = np.random.RandomState(i).randint(1, S + 1, size=B).astype(np.int32)
+        out = sdpAttention(*dev, kvLens=torch.from_numpy(lens).cuda())
+        torch.cuda.synchronize()
+        for b in range(B):
+            exp = oracle.sdpa_f32(host[0][b:b + 1], host[1][b:b + 1, :, :lens[b]], host[2][b:b + 1, :, :lens[b]])
+            assert max_abs_err(out[b:b + 1], exp) <= TOL[dtype], (route_of(*dev), b)
+        return
+    out = sdpAttention(*dev, **kw_dev)
+    torch.cuda.synchronize()
+    exp = oracle.sdpa_f32(*host, **kw_host)
+    assert max_abs_err(out, exp) <= TOL[dtype], route_of(*dev, causal=extra == "causal")
