@@ -78,7 +78,10 @@ def test_routes(args, route):
 def test_routes_depend_on_flags():
     base = (_capi.BF16, 2, 8, 2, 512, 512, 128)
     assert _capi.plan(params(*base, causal=1))[1] == _capi.ROUTE_PREFILL
-    assert _capi.plan(params(*base, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
+    # an attnMask is taken by the pipelined head_dim-128 kernel (L > 128); other masked shapes go to the general kernel
+    assert _capi.plan(params(*base, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 64, 512, 128, mask_kind=_capi.MASK_ADD, mask=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 512, 512, 64, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
     assert _capi.plan(params(*base, scale=-1.0))[1] == _capi.ROUTE_GENERAL
     p = params(*base)
     p.k_stride[2] = 132  # rows not 16-byte aligned

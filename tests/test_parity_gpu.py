@@ -396,3 +396,44 @@ def test_kv_len_edge_cases():
     kn3 = torch.randn(1, 1, 2, 3, device="cuda").bfloat16()
     kvCacheAppend(kc3, vc3, kn3, kn3, 5)
     assert torch.equal(kc3[:, :, 5:7], kn3) and torch.equal(vc3[:, :, 5:7], kn3)
+
+
+# ---- attnMask on the pipelined MFMA kernel (head_dim 128, more than 128 query rows) -------------------------------------
+
+@pytest.mark.parametrize("mshape,kind", [((2, 1, 1, 600), "bool"), ((300, 600), "bool"), ((2, 8, 300, 600), "float"),
+                                         ((8, 1, 600), "float"), ((2, 1, 300, 1), "float")])
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_masks_on_the_mfma_route(mshape, kind, dtype):
+    B, Hq, Hkv, L, S, D = 2, 8, 2, 300, 600, 128
+    host, dev = make_inputs(91, B, Hq, Hkv, L, S, D, dtype)
+    if kind == "bool":
+        m = (np.random.RandomState(len(mshape)).rand(*mshape) > 0.5).astype(np.uint8)
+        m[..., 5] = 1
+        md = torch.from_numpy(m).cuda().bool()
+    else:
+        m, bits = oracle.round_to(oracle.randn(92, 9, mshape, 2.0), dtype)
+        md = to_device(m, bits, dtype)
+    assert route_of(*dev, mask=md) == "prefill"
+    exp = oracle.sdpa_f32(*host, mask=m)
+    rc, out = call("forward", *dev, mask=md)
+    assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]
+    rc, out2 = call("general", *dev, mask=md)   # the vector-ALU kernel agrees
+    assert rc == 0 and max_abs_err(out2, exp) <= TOL[dtype]
+
+
+def test_fully_hidden_rows_on_the_mfma_route():
+    # rows whose mask hides every key are NaN in the reference (0 * inf); rows hidden only partly are not affected
+    B, Hq, Hkv, L, S, D = 1, 4, 2, 260, 200, 128
+    host, dev = make_inputs(93, B, Hq, Hkv, L, S, D, "bf16")
+    m = np.ones((L, S), np.uint8)
+    m[7] = 0
+    m[200:230] = 0
+    m[100, 50:] = 0
+    md = torch.from_numpy(m).cuda().bool()
+    assert route_of(*dev, mask=md) == "prefill"
+    exp = oracle.sdpa_f32(*host, mask=m)
+    rc, out = call("forward", *dev, mask=md)
+    y = to_host_f32(out)
+    assert rc == 0 and np.array_equal(np.isnan(y), np.isnan(exp)) and np.isnan(exp[0, :, 7]).all() and not np.isnan(exp[0, :, 100]).any()
+    ok = ~np.isnan(exp)
+    assert np.abs(y[ok] - exp[ok]).max() <= TOL["bf16"]

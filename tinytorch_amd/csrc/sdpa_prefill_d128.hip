@@ -147,6 +147,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     }
   }
   if (nfast < 0) nfast = 0;
+  if (a.mask_kind != 0) nfast = 0;  // an attnMask is applied in the general form of a step
 
   // ---- global -> LDS: wavefront w moves rows 8w .. 8w+7 of a tile, 4 rows (1 KiB) per instruction --------------
   // lane l fills slot (row 4i + l/16, chunk slot l%16) and therefore fetches chunk (l%16) ^ f(row)
@@ -279,6 +280,27 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     }
   };
 
+  // attnMask (reference src/Function/FuncNNLayer.h:249-260): Bool -> hidden keys get -inf; additive -> the bias is
+  // added to the scaled score, i.e. bias / scale to the raw score held here.  Element strides of 0 broadcast an axis.
+  auto user_mask_half = [&](f32x16& s, int kv0) __attribute__((always_inline)) {
+    int qi = qw0 + lq;
+    qi = qi < a.L ? qi : a.L - 1;
+    const long long mrow = b * a.ms[0] + h * a.ms[1] + qi * a.ms[2];
+    const float inv_scale = 1.f / a.scale;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+      if (key < a.S) {
+        const long long at = mrow + key * a.ms[3];
+        if (a.mask_kind == 1) {
+          if (((const uint8_t*)a.mask)[at] == 0) s[r] = -INFINITY;
+        } else {
+          s[r] += (float)((const T*)a.mask)[at] * inv_scale;
+        }
+      }
+    }
+  };
+
   auto row_max = [&](const f32x16& s) __attribute__((always_inline)) {
     float m = s[0];
 #pragma unroll
@@ -355,6 +377,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     if (h + 1 < my_halves) {
       const int kv0 = 32 * (h + 1);
       if ((CAUSAL && kv0 + 31 > qw0) || kv0 + 32 > a.S) mask_half(s_nxt, kv0);
+      if (!CAUSAL && a.mask_kind != 0) user_mask_half(s_nxt, kv0);
       settle_half(s_nxt, p_nxt, exp_half(s_nxt, p_nxt));
     }
   };
@@ -415,6 +438,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   {  // P(0) and the scores of half 1
     qk_half(sC, half_base(0));
     if ((CAUSAL && 31 > qw0) || 32 > a.S) mask_half(sC, 0);
+    if (!CAUSAL && a.mask_kind != 0) user_mask_half(sC, 0);
     settle_half(sC, pA, exp_half(sC, pA));
     if (1 < my_halves) qk_half(sB, half_base(1));
   }

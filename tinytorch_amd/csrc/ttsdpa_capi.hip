@@ -60,9 +60,9 @@ int validate(const ttsdpa_params* p, KArgs* a) {
 }
 
 // 16-bit tensors the MFMA kernels can read with 16-byte loads and write with 8-byte stores.
-bool fast_layout_ok(const ttsdpa_params* p) {
+bool fast_layout_ok(const ttsdpa_params* p, bool masks_ok = false) {
   if (p->dtype != TTSDPA_F16 && p->dtype != TTSDPA_BF16) return false;
-  if (p->mask_kind != TTSDPA_MASK_NONE) return false;
+  if (p->mask_kind != TTSDPA_MASK_NONE && !masks_ok) return false;
   if (!(p->scale > 0.f) || !isfinite(p->scale)) return false;  // the row maximum is taken on unscaled scores
   if (!dense_last_ok(p->q_stride, 8) || !dense_last_ok(p->k_stride, 8) || !dense_last_ok(p->v_stride, 8) ||
       !dense_last_ok(p->o_stride, 8))
@@ -72,7 +72,9 @@ bool fast_layout_ok(const ttsdpa_params* p) {
 
 bool prefill_ok(const ttsdpa_params* p) {
   if (p->kv_len) return false;  // per-batch key counts are served by the decode and general kernels
-  return fast_layout_ok(p) && (p->D == 128 || p->D == 64) && p->S >= 1 && p->L >= 1;
+  // an attnMask is taken by the pipelined head_dim-128 kernel only
+  const bool pipelined = p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
+  return fast_layout_ok(p, pipelined) && (p->D == 128 || p->D == 64) && p->S >= 1 && p->L >= 1;
 }
 
 bool decode_ok(const ttsdpa_params* p) {
