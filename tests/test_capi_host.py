@@ -63,7 +63,9 @@ def test_struct_layout_matches_header():
     ((_capi.BF16, 1, 28, 4, 16384, 16384, 128), _capi.ROUTE_PREFILL),  # config 5
     ((_capi.BF16, 1, 28, 4, 1, 4096, 128), _capi.ROUTE_DECODE),      # 7 heads per KV head
     ((_capi.BF16, 1, 8, 8, 300, 300, 64), _capi.ROUTE_PREFILL),
-    ((_capi.BF16, 1, 8, 8, 300, 300, 96), _capi.ROUTE_GENERAL),
+    ((_capi.BF16, 1, 8, 8, 300, 300, 96), _capi.ROUTE_PREFILL),
+    ((_capi.F16, 1, 8, 8, 300, 300, 256), _capi.ROUTE_PREFILL),
+    ((_capi.BF16, 1, 8, 8, 300, 300, 80), _capi.ROUTE_GENERAL),      # not one of the MFMA head sizes
     ((_capi.BF16, 1, 64, 2, 1, 4096, 128), _capi.ROUTE_PREFILL),     # 32 rows per KV head: too many for decode
     ((_capi.BF16, 1, 8, 8, 0, 16, 128), _capi.ROUTE_NONE),
     ((_capi.BF16, 0, 8, 8, 4, 16, 128), _capi.ROUTE_NONE),

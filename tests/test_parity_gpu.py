@@ -437,3 +437,14 @@ def test_fully_hidden_rows_on_the_mfma_route():
     assert rc == 0 and np.array_equal(np.isnan(y), np.isnan(exp)) and np.isnan(exp[0, :, 7]).all() and not np.isnan(exp[0, :, 100]).any()
     ok = ~np.isnan(exp)
     assert np.abs(y[ok] - exp[ok]).max() <= TOL["bf16"]
+
+
+@pytest.mark.parametrize("D", [32, 96, 256])
+@pytest.mark.parametrize("dtype,causal", [("bf16", True), ("f16", False)])
+def test_other_head_sizes_on_the_mfma_route(D, dtype, causal):
+    B, Hq, Hkv, L, S = 2, 6, 2, 333, 333 if causal else 411
+    host, dev = make_inputs(95 + D, B, Hq, Hkv, L, S, D, dtype, 0.7)
+    assert route_of(*dev, causal=causal) == "prefill"
+    exp = oracle.sdpa_f32(*host, causal=causal)
+    rc, out = call("forward", *dev, causal=causal)
+    assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]

@@ -60,7 +60,7 @@ __device__ __forceinline__ vec8 v_operand(const void* lane_base, int byte_off_lo
 }
 
 template <typename TR, int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void prefill_kernel(KArgs a) {
+__global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
   typedef PrefillLds<D> Lds;
@@ -315,11 +315,19 @@ int launch_prefill_t(const KArgs& a, hipStream_t stream) {
 
 }  // namespace
 
-int launch_prefill(const KArgs& a, int dtype, hipStream_t stream) {
-  if (dtype == 1) {
-    return a.D == 128 ? launch_prefill_t<F16, 128>(a, stream) : launch_prefill_t<F16, 64>(a, stream);
+template <typename TR>
+int launch_prefill_d(const KArgs& a, hipStream_t stream) {
+  switch (a.D) {
+    case 32: return launch_prefill_t<TR, 32>(a, stream);
+    case 64: return launch_prefill_t<TR, 64>(a, stream);
+    case 96: return launch_prefill_t<TR, 96>(a, stream);
+    case 128: return launch_prefill_t<TR, 128>(a, stream);
+    default: return launch_prefill_t<TR, 256>(a, stream);
   }
-  return a.D == 128 ? launch_prefill_t<BF16, 128>(a, stream) : launch_prefill_t<BF16, 64>(a, stream);
+}
+
+int launch_prefill(const KArgs& a, int dtype, hipStream_t stream) {
+  return dtype == 1 ? launch_prefill_d<F16>(a, stream) : launch_prefill_d<BF16>(a, stream);
 }
 
 }  // namespace ttsdpa

@@ -74,7 +74,8 @@ bool prefill_ok(const ttsdpa_params* p) {
   if (p->kv_len) return false;  // per-batch key counts are served by the decode and general kernels
   // an attnMask is taken by the pipelined head_dim-128 kernel only
   const bool pipelined = p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
-  return fast_layout_ok(p, pipelined) && (p->D == 128 || p->D == 64) && p->S >= 1 && p->L >= 1;
+  const bool mfma_head_dim = p->D == 32 || p->D == 64 || p->D == 96 || p->D == 128 || p->D == 256;
+  return fast_layout_ok(p, pipelined) && mfma_head_dim && p->S >= 1 && p->L >= 1;
 }
 
 bool decode_ok(const ttsdpa_params* p) {
