@@ -98,7 +98,7 @@ typedef struct ttsdpa_params {
    * [B,Hkv,Smax,D] pass S = Smax and the filled lengths here: batch b attends to keys 0 .. min(kv_len[b], S) - 1, the
    * result the reference gives on K/V grown to that length with op::concat (reference
    * src/Operation/OpTransform.cpp:306-357).  A length of 0 yields zeros (the reference's empty contraction).
-   * Served by the decode and general kernels. */
+   * Served by the decode kernel, the pipelined head_dim-128 prefill kernel and the general kernel. */
   const int32_t* kv_len;
 } ttsdpa_params;
 

@@ -123,10 +123,12 @@ def test_validation_errors(mutate, status):
 
 
 def test_kv_len_routes_and_append_validation():
-    # per-batch key counts are served by the decode and general kernels, never by the prefill kernels
+    # per-batch key counts: decode kernel, pipelined head_dim-128 prefill kernel, general kernel for the rest
     base = (_capi.BF16, 2, 32, 8, 4096, 4096, 128)
     assert _capi.plan(params(*base, causal=1))[1] == _capi.ROUTE_PREFILL
-    assert _capi.plan(params(*base, causal=1, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(*base, causal=1, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 4096, 4096, 64, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 100, 4096, 128, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
     assert _capi.plan(params(_capi.BF16, 8, 32, 8, 1, 4096, 128, kv_len=FAKE))[1] == _capi.ROUTE_DECODE
     assert _capi.plan(params(_capi.BF16, 8, 32, 8, 1, 4096, 128, kv_len=FAKE + 2))[0] == _capi.ERR_STRIDE
     L = _capi.lib()

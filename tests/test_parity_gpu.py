@@ -448,3 +448,25 @@ def test_other_head_sizes_on_the_mfma_route(D, dtype, causal):
     exp = oracle.sdpa_f32(*host, causal=causal)
     rc, out = call("forward", *dev, causal=causal)
     assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_per_batch_key_counts_on_the_mfma_route(causal, dtype):
+    # a padded batch: every entry has its own number of valid keys (0, 1, ragged, full)
+    B, Hq, Hkv, L, S, D = 5, 4, 2, 300, 520, 128
+    host, dev = make_inputs(97, B, Hq, Hkv, L, S, D, dtype)
+    lens = np.array([0, 1, 77, 333, 9999], np.int32)
+    ld = torch.from_numpy(lens).cuda()
+    out = torch.empty_like(dev[0])
+    from tinytorch_amd import _capi, build_params
+    rc, r = _capi.plan(build_params(*dev, out, causal, None, None, ld))
+    assert rc == 0 and _capi.ROUTE_NAMES[r] == "prefill"
+    from tinytorch_amd import sdpAttention
+    y = sdpAttention(*dev, isCausal=causal, kvLens=ld)
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(y[0]) == 0
+    for b in range(1, B):
+        n = min(int(lens[b]), S)
+        exp = oracle.sdpa_f32(host[0][b:b + 1], host[1][b:b + 1, :, :n], host[2][b:b + 1, :, :n], causal=causal)
+        assert max_abs_err(y[b:b + 1], exp) <= TOL[dtype], b

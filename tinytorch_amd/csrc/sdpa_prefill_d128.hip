@@ -110,6 +110,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
   const T* kp = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
   const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
+  int S = a.S;  // keys of this batch entry: all of them, or the filled prefix of a cache / the unpadded length
+  if (a.kv_len) {
+    int len = __builtin_amdgcn_readfirstlane(a.kv_len[b]);
+    S = len < 0 ? 0 : (len < S ? len : S);
+  }
 
   for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
   // Neighbouring workgroups take their two tiles in opposite order, so that the load / store bursts between the
@@ -122,11 +127,23 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   // diagonal, so the second four wavefronts take the groups in reverse: every SIMD then carries groups g and 7-g.
   const int rowgroup = (CAUSAL && wave >= 4) ? 11 - wave : wave;
   const int qw0 = q0 + rowgroup * WM;
+  if (S == 0) {  // no keys for this batch entry: zeros, the reference's empty contraction
+    T* obase = (T*)a.out + b * a.os[0] + h * a.os[1];
+    vec8 zero;
+#pragma unroll
+    for (int i = 0; i < 8; i++) zero[i] = (T)0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int qi = qw0 + 4 * i + (lane >> 4);
+      if (qi < a.L) *(vec8*)(obase + qi * a.os[2] + 8 * (lane & 15)) = zero;
+    }
+    continue;
+  }
 
-  int ntiles_kv = (a.S + BN - 1) / BN;
+  int ntiles_kv = (S + BN - 1) / BN;
   if (CAUSAL) {
     int last = q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1;
-    int lastkv = last < a.S - 1 ? last : a.S - 1;
+    int lastkv = last < S - 1 ? last : S - 1;
     ntiles_kv = lastkv / BN + 1;
   }
   // 32-key halves this wavefront computes on: under a causal mask those that start at or before its last row
@@ -139,7 +156,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   // half 2j+2 (whose exponentials step 2j+1 takes) needs no mask.
   int nfast = (my_halves - 2) / 2;
   {
-    int f = a.S >= 96 ? (a.S - 32) / BN : 0;
+    int f = S >= 96 ? (S - 32) / BN : 0;
     nfast = f < nfast ? f : nfast;
     if (CAUSAL) {
       f = qw0 >= 95 ? (qw0 - 31) / BN : 0;
@@ -166,7 +183,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
   const unsigned smem_addr = (unsigned)(unsigned long)(lds_void*)smem;
   auto dma_tile = [&](const T* base, long long rstride, const unsigned (&off)[2], int kv0, unsigned stage_addr) __attribute__((always_inline)) {
-    if (kv0 + BN <= a.S) {
+    if (kv0 + BN <= S) {
       const char* src = (const char*)(base + kv0 * rstride);
 #pragma unroll
       for (int i = 0; i < 2; i++) dma_issue(src, off[i], stage_addr + (8 * wave + 4 * i) * ROW_BYTES);
@@ -176,7 +193,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
         int row = 8 * wave + 4 * i + (lane >> 4);
         asm volatile("" : "+v"(row));  // keeps this rarely taken path's address arithmetic inside the branch
         int chunk = (lane & 15) ^ swz(row);
-        int rowc = row < a.S - kv0 ? row : a.S - 1 - kv0;
+        int rowc = row < S - kv0 ? row : S - 1 - kv0;
         unsigned voff = ((unsigned)rowc * (unsigned)rstride + 8u * chunk) * 2u;
         dma_issue((const char*)(base + kv0 * rstride), voff, stage_addr + (8 * wave + 4 * i) * ROW_BYTES);
       }
@@ -275,7 +292,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-      bool hidden = key >= a.S || (CAUSAL && key > qi);
+      bool hidden = key >= S || (CAUSAL && key > qi);
       if (hidden) s[r] = -INFINITY;
     }
   };
@@ -290,7 +307,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-      if (key < a.S) {
+      if (key < S) {
         const long long at = mrow + key * a.ms[3];
         if (a.mask_kind == 1) {
           if (((const uint8_t*)a.mask)[at] == 0) s[r] = -INFINITY;
@@ -376,7 +393,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     if (h < my_halves) pv_half(p_cur, half_base(h));
     if (h + 1 < my_halves) {
       const int kv0 = 32 * (h + 1);
-      if ((CAUSAL && kv0 + 31 > qw0) || kv0 + 32 > a.S) mask_half(s_nxt, kv0);
+      if ((CAUSAL && kv0 + 31 > qw0) || kv0 + 32 > S) mask_half(s_nxt, kv0);
       if (!CAUSAL && a.mask_kind != 0) user_mask_half(s_nxt, kv0);
       settle_half(s_nxt, p_nxt, exp_half(s_nxt, p_nxt));
     }
@@ -437,7 +454,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }
   {  // P(0) and the scores of half 1
     qk_half(sC, half_base(0));
-    if ((CAUSAL && 31 > qw0) || 32 > a.S) mask_half(sC, 0);
+    if ((CAUSAL && 31 > qw0) || 32 > S) mask_half(sC, 0);
     if (!CAUSAL && a.mask_kind != 0) user_mask_half(sC, 0);
     settle_half(sC, pA, exp_half(sC, pA));
     if (1 < my_halves) qk_half(sB, half_base(1));

@@ -71,9 +71,9 @@ bool fast_layout_ok(const ttsdpa_params* p, bool masks_ok = false) {
 }
 
 bool prefill_ok(const ttsdpa_params* p) {
-  if (p->kv_len) return false;  // per-batch key counts are served by the decode and general kernels
-  // an attnMask is taken by the pipelined head_dim-128 kernel only
+  // an attnMask or per-batch key counts are taken by the pipelined head_dim-128 kernel only
   const bool pipelined = p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
+  if (p->kv_len && !pipelined) return false;
   const bool mfma_head_dim = p->D == 32 || p->D == 64 || p->D == 96 || p->D == 128 || p->D == 256;
   return fast_layout_ok(p, pipelined) && mfma_head_dim && p->S >= 1 && p->L >= 1;
 }
