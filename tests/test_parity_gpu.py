@@ -470,3 +470,17 @@ def test_per_batch_key_counts_on_the_mfma_route(causal, dtype):
         n = min(int(lens[b]), S)
         exp = oracle.sdpa_f32(host[0][b:b + 1], host[1][b:b + 1, :, :n], host[2][b:b + 1, :, :n], causal=causal)
         assert max_abs_err(y[b:b + 1], exp) <= TOL[dtype], b
+
+
+@pytest.mark.parametrize("case", [(4, 32, 8, 1, 2048, "bf16"), (2, 8, 2, 1, 33, "f16"), (3, 28, 4, 1, 777, "bf16"),
+                                  (1, 16, 1, 1, 513, "bf16"), (2, 4, 1, 4, 640, "f16"), (1, 16, 2, 1, 9000, "bf16")],
+                         ids=lambda c: "B%dH%dk%dL%dS%d-%s" % c)
+def test_decode_head_dim_64(case):
+    B, Hq, Hkv, L, S, dtype = case
+    host, dev = make_inputs(99 + S, B, Hq, Hkv, L, S, 64, dtype)
+    assert route_of(*dev) == "decode"
+    exp = oracle.sdpa_f32(*host)
+    rc, out = call("forward", *dev)
+    assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]
+    rc, out2 = call("general", *dev)
+    assert rc == 0 and max_abs_err(out2, exp) <= TOL[dtype]

@@ -1,5 +1,5 @@
 // Split-KV attention for decode: a few query rows per KV head against a long, contiguous KV cache (fp16 / bf16,
-// head_dim 128).  Memory-bound: every K and V byte is read exactly once with 16-byte loads, whatever the number of
+// head_dim 128 or 64).  Memory-bound: every K and V byte is read exactly once with 16-byte loads, whatever the number of
 // query heads sharing the KV head, instead of the reference's GEMM -> scale -> softmax -> GEMM chain over a
 // materialised score tensor (reference src/Function/FuncNNLayer.h:237-265).
 //
@@ -10,11 +10,12 @@
 // Per 32-key block and wavefront:
 //   scores  v_mfma_f32_16x16x32: A = the query rows (16 x 32 slice of head_dim, zero rows where unused), B = K^T taken
 //           straight from global memory: lane l supplies key l%16 and the 8 head_dim elements of group l/16, i.e. one
-//           16-byte load; four MFMAs cover head_dim 128.  Query row x sits at MFMA row 4*(x%4) + x/4, so the
+//           16-byte load; head_dim/32 MFMAs cover the head.  Query row x sits at MFMA row 4*(x%4) + x/4, so the
 //           result lane (key l%16, group l/16) holds rows l/16, l/16+4, ... in registers 0, 1, ...
 //   softmax running max per row (reduced over the 16 key lanes with DPP row rotations), exp2 with scale*log2e folded
-//   P.V     on the vector ALUs: lane l owns head_dim elements 8*(l%16) .. +7 of keys l/16, l/16+4, ... (one 16-byte
-//           load per key, a wavefront load instruction covers 4 whole V rows = 1 KiB contiguous); the probabilities
+//   P.V     on the vector ALUs: with C = head_dim/8 chunks per row, lane l owns head_dim elements 8*(l%C) .. +7 of keys
+//           l/C, l/C + 64/C, ... (one 16-byte load per key, a wavefront load instruction covers 64/C whole V rows =
+//           1 KiB contiguous); the probabilities
 //           travel from the score lanes to the value lanes through a per-wavefront LDS patch.
 // Each wavefront ends with (max, sum, acc) per row; the workgroup merges its four, then either writes the final
 // output (splits == 1) or a partial (max, sum, acc) record that merge_kernel combines by log-sum-exp.
@@ -26,7 +27,6 @@ namespace ttsdpa {
 namespace {
 
 constexpr int KB = 32;       // keys per wavefront block
-constexpr int DD = 128;      // head_dim
 constexpr int NWAVE = 4;
 
 // max over the 16 lanes of a DPP row (lanes 16*i .. 16*i+15), result in every lane of the row
@@ -53,11 +53,14 @@ __device__ __forceinline__ void wave_lds_sync() {
 }
 
 // R = registers of query rows per score lane: rows handled = up to 4*R.
-template <typename TR, int R>
+template <typename TR, int R, int DD>
 __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int chunk, float* __restrict__ ws) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
-  constexpr int NR = 4 * R;  // row slots
+  constexpr int NR = 4 * R;    // row slots
+  constexpr int KS = DD / 32;  // MFMAs along head_dim per 16 keys
+  constexpr int CH = DD / 8;   // 16-byte chunks of a V row = value lanes per key
+  constexpr int PH = 64 / CH;  // keys a wavefront V load covers (key phases)
 
   // per-wavefront patch: probabilities [KB keys][NR rows] + rescale factors [NR]; reused for the final merge
   __shared__ __attribute__((aligned(16))) float Pl[NWAVE][KB * NR + NR];
@@ -66,8 +69,10 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int l16 = lane & 15;  // score lanes: key within a 16-key group | value lanes: 16-byte chunk of the row
-  const int lg = lane >> 4;   // score lanes: row group              | value lanes: key phase
+  const int l16 = lane & 15;  // score lanes: key within a 16-key group
+  const int lg = lane >> 4;   // score lanes: row group
+  const int vc = lane % CH;   // value lanes: 16-byte chunk of the row
+  const int vph = lane / CH;  // value lanes: key phase
 
   int n = blockIdx.x;
   const int split = n % splits;
@@ -85,7 +90,7 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
   const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
 
   // ---- query rows as MFMA A operands: lane l supplies MFMA row l%16, head_dim 32*ks + 8*(l/16) .. +7 --------------
-  vec8 qa[4];
+  vec8 qa[KS];
   {
     int mrow = l16;                       // MFMA row
     int x = (mrow & 3) * 4 + (mrow >> 2); // query row stored there: row x sits at 4*(x%4) + x/4
@@ -93,7 +98,7 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
     int xl = used ? x / a.G : 0, xg = used ? x % a.G : 0;
     const T* qr = (const T*)a.q + b * a.qs[0] + (hk * a.G + xg) * a.qs[1] + xl * a.qs[2] + 8 * lg;
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
+    for (int ks = 0; ks < KS; ks++) {
       vec8 t = *(const vec8*)(qr + 32 * ks);
 #pragma unroll
       for (int i = 0; i < 8; i++) qa[ks][i] = used ? t[i] : (T)0.f;
@@ -117,21 +122,21 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
 
   for (int k0 = s_begin + wave * KB; k0 < s_end; k0 += NWAVE * KB) {
     // ---- issue all loads of the block: K for the score MFMAs, V for the accumulation ----------------------------------
-    u32x4 kreg[2][4];
+    u32x4 kreg[2][KS];
 #pragma unroll
     for (int gi = 0; gi < 2; gi++) {
       int key = k0 + 16 * gi + l16;
       key = key < S ? key : S - 1;
       const T* kr = kp + key * a.ks[2] + 8 * lg;
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++) kreg[gi][ks] = __builtin_nontemporal_load((const u32x4*)(kr + 32 * ks));  // read once: keep it out of the caches
+      for (int ks = 0; ks < KS; ks++) kreg[gi][ks] = __builtin_nontemporal_load((const u32x4*)(kr + 32 * ks));  // read once: keep it out of the caches
     }
-    u32x4 vreg[KB / 4];
+    u32x4 vreg[KB / PH];
 #pragma unroll
-    for (int i = 0; i < KB / 4; i++) {
-      int key = k0 + 4 * i + lg;
+    for (int i = 0; i < KB / PH; i++) {
+      int key = k0 + PH * i + vph;
       key = key < S ? key : S - 1;
-      vreg[i] = __builtin_nontemporal_load((const u32x4*)(vp + key * a.vs[2] + 8 * l16));
+      vreg[i] = __builtin_nontemporal_load((const u32x4*)(vp + key * a.vs[2] + 8 * vc));
     }
 
     // ---- scores --------------------------------------------------------------------------------------------------------
@@ -140,7 +145,7 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
     for (int gi = 0; gi < 2; gi++) {
       sc[gi] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++)
+      for (int ks = 0; ks < KS; ks++)
         sc[gi] = TR::mfma16(qa[ks], __builtin_bit_cast(vec8, kreg[gi][ks]), sc[gi]);
       if (k0 + 16 * gi + l16 >= s_end) {
 #pragma unroll
@@ -175,7 +180,7 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
         for (int i = 0; i < 8; i++) acc[4 * r + j][i] *= al[j];
     }
 #pragma unroll
-    for (int i = 0; i < KB / 4; i++) {
+    for (int i = 0; i < KB / PH; i++) {
       float vf[8];
 #pragma unroll
       for (int w = 0; w < 4; w++) {
@@ -184,7 +189,7 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
       }
 #pragma unroll
       for (int r = 0; r < R; r++) {
-        f32x4 p = *(const f32x4*)(pl + (4 * i + lg) * NR + 4 * r);
+        f32x4 p = *(const f32x4*)(pl + (PH * i + vph) * NR + 4 * r);
 #pragma unroll
         for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -202,15 +207,16 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       float t = acc[x][i];
+      if (CH <= 8) t += __shfl_xor(t, 8);
       t += __shfl_xor(t, 16);
       t += __shfl_xor(t, 32);
       acc[x][i] = t;
     }
-  if (lg == 0) {
+  if (vph == 0) {
 #pragma unroll
     for (int x = 0; x < NR; x++)
 #pragma unroll
-      for (int i = 0; i < 8; i++) Om[wave][x][8 * l16 + i] = acc[x][i];
+      for (int i = 0; i < 8; i++) Om[wave][x][8 * vc + i] = acc[x][i];
   }
   if (l16 == 0) {
 #pragma unroll
@@ -250,11 +256,11 @@ __global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int ch
   }
 }
 
-// Combine the per-split records of one query row: one workgroup of 128 threads per (batch, kv head, row).  The first
+// Combine the per-split records of one query row: one workgroup of head_dim threads per (batch, kv head, row).  The first
 // wavefront turns the (max, sum) pairs of the up to 64 splits into weights (one split per lane, wave reductions);
 // then thread d accumulates head_dim element d over the splits with independent, coalesced loads.
 constexpr int kMaxSplits = 64;
-template <typename T>
+template <typename T, int DD>
 __global__ __launch_bounds__(DD) void merge_kernel(KArgs a, int splits, const float* __restrict__ ws) {
   __shared__ float weight[kMaxSplits];
   __shared__ float total;
@@ -288,28 +294,25 @@ __global__ __launch_bounds__(DD) void merge_kernel(KArgs a, int splits, const fl
   store_from_float(op + t, total > 0.f ? o / total : 0.f);
 }
 
-template <typename TR>
+template <typename TR, int DD>
 int launch_decode_t(const KArgs& a, const DecodePlan& pl, float* ws, hipStream_t stream) {
   typedef typename TR::elem T;
   dim3 grid((unsigned)((long long)a.B * a.Hkv * pl.splits)), block(256);
   int R = (pl.rows + 3) / 4;
   switch (R) {
-    case 1: hipLaunchKernelGGL((decode_kernel<TR, 1>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
-    case 2: hipLaunchKernelGGL((decode_kernel<TR, 2>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
-    case 3: hipLaunchKernelGGL((decode_kernel<TR, 3>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
-    default: hipLaunchKernelGGL((decode_kernel<TR, 4>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
+    case 1: hipLaunchKernelGGL((decode_kernel<TR, 1, DD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
+    case 2: hipLaunchKernelGGL((decode_kernel<TR, 2, DD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
+    case 3: hipLaunchKernelGGL((decode_kernel<TR, 3, DD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
+    default: hipLaunchKernelGGL((decode_kernel<TR, 4, DD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
   }
   int rc = (int)hipGetLastError();
   if (rc != 0 || pl.splits == 1) return rc;
-  hipLaunchKernelGGL((merge_kernel<T>), dim3((unsigned)((long long)a.B * a.Hkv * pl.rows)), dim3(DD), 0, stream, a, pl.splits, ws);
+  hipLaunchKernelGGL((merge_kernel<T, DD>), dim3((unsigned)((long long)a.B * a.Hkv * pl.rows)), dim3(DD), 0, stream, a, pl.splits, ws);
   return (int)hipGetLastError();
 }
 
 }  // namespace
 
-// Splits: two workgroups per CU are enough to keep HBM busy (measured on config 4: 1 split = 512 workgroups is the
-// fastest, more splits only add partial records and the merge launch), so split only while (batch x kv heads) alone
-// gives fewer than that; each split at least 256 keys, chunk a multiple of the 128 keys a workgroup consumes per round.
 DecodePlan plan_decode(const KArgs& a) {
   DecodePlan p;
   p.rows = a.L * a.G;
@@ -328,14 +331,17 @@ DecodePlan plan_decode(const KArgs& a) {
   if (splits < 1) splits = 1;
   p.splits = splits;
   p.chunk = chunk;
-  p.ws_bytes = splits > 1 ? (size_t)pairs * splits * p.rows * (DD + 2) * sizeof(float) : 0;
+  p.ws_bytes = splits > 1 ? (size_t)pairs * splits * p.rows * (a.D + 2) * sizeof(float) : 0;
   return p;
 }
 
 int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream) {
   DecodePlan pl = plan_decode(a);
-  if (dtype == 1) return launch_decode_t<F16>(a, pl, (float*)workspace, stream);
-  return launch_decode_t<BF16>(a, pl, (float*)workspace, stream);
+  if (a.D == 64)
+    return dtype == 1 ? launch_decode_t<F16, 64>(a, pl, (float*)workspace, stream)
+                      : launch_decode_t<BF16, 64>(a, pl, (float*)workspace, stream);
+  return dtype == 1 ? launch_decode_t<F16, 128>(a, pl, (float*)workspace, stream)
+                    : launch_decode_t<BF16, 128>(a, pl, (float*)workspace, stream);
 }
 
 }  // namespace ttsdpa

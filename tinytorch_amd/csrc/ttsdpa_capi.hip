@@ -79,7 +79,7 @@ bool prefill_ok(const ttsdpa_params* p) {
 }
 
 bool decode_ok(const ttsdpa_params* p) {
-  if (!fast_layout_ok(p) || p->D != 128 || p->causal || p->S < 1 || p->L < 1) return false;
+  if (!fast_layout_ok(p) || (p->D != 128 && p->D != 64) || p->causal || p->S < 1 || p->L < 1) return false;
   return (long long)p->L * (p->Hq / p->Hkv) <= kDecodeMaxRows;
 }
 
