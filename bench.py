@@ -118,6 +118,42 @@ def run_gpu(name, steps, warmup):
     return res, (q, k, v, out)
 
 
+def run_probes():
+    """What this GPU sustains on the two bounding resources, measured with the library's probe kernels (ttsdpa_probe):
+    a register-only MFMA loop and a streaming read of 1 GiB, plain and nontemporal.  HIP events on the launch stream."""
+    import torch
+    from tinytorch_amd import _capi
+
+    lib = _capi.lib()
+    stream = torch.cuda.current_stream()
+    buf = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+    out = {}
+    for key, kind, iters, reps, unit in (("mfma_loop", 0, 20000, 300, 1e12), ("read_plain", 1, 1, 300, 1e9),
+                                         ("read_nontemporal", 2, 1, 300, 1e9)):
+        work = ctypes.c_double(0.0)
+
+        def go():
+            rc = lib.ttsdpa_probe(kind, buf.data_ptr(), buf.numel(), iters, stream.cuda_stream, ctypes.byref(work))
+            if rc != 0:
+                raise RuntimeError("ttsdpa_probe: %s" % _capi.status_string(rc))
+        for _ in range(reps):
+            go()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            go()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        out[key] = round(work.value / (ms * 1e-3) / unit, 1)
+    del buf
+    torch.cuda.empty_cache()
+    return {"mfma_loop_tflops": out["mfma_loop"], "read_plain_gbs": out["read_plain"],
+            "read_nontemporal_gbs": out["read_nontemporal"],
+            "note": "sustained by ttsdpa_probe kernels in this run: bf16 32x32x16 MFMA loop, 1 GiB streaming reads"}
+
+
 def run_cpu_baseline(name, tensors, budget_s=20.0):
     """The reference CPU path (compiled reference if oracle/_ref is present, else this repository's C restatement)
     on one host core, over as many (batch, head) slices of the same inputs as fit the time budget."""
@@ -167,6 +203,7 @@ def main():
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--no-probes", action="store_true", help="skip the hardware ceiling probes")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one device-to-device copy of 1 GiB (a kernel of known traffic that calibrates "
                          "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc)")
@@ -185,6 +222,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     main_res, tensors = run_gpu(args.workload, args.steps, args.warmup)
+    ceilings = None if args.no_probes else run_probes()
     cpu = None if args.no_cpu else run_cpu_baseline(args.workload, tensors, args.cpu_seconds)
     del tensors
     torch.cuda.empty_cache()
@@ -196,6 +234,8 @@ def main():
         "config": {"workload": "%s: %s" % (args.workload, main_res["description"]), "route": main_res["route"]},
         "roofline": main_res["roofline"], "cpu_baseline": cpu,
     }
+    if ceilings:
+        line["measured_ceilings"] = ceilings
     if not args.no_secondary and args.secondary != args.workload:
         sec, tensors = run_gpu(args.secondary, args.steps, args.warmup)
         sec["cpu_baseline"] = None if args.no_cpu else run_cpu_baseline(args.secondary, tensors, args.cpu_seconds)

@@ -152,6 +152,16 @@ def test_kv_len_routes_and_append_validation():
     assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == 0
 
 
+def test_probe_argument_checks():
+    L = _capi.lib()
+    w = ctypes.c_double(0.0)
+    assert L.ttsdpa_probe(0, None, 64, 10, None, ctypes.byref(w)) == _capi.ERR_NULL
+    assert L.ttsdpa_probe(0, FAKE, 64, 10, None, None) == _capi.ERR_NULL
+    assert L.ttsdpa_probe(7, FAKE, 64, 10, None, ctypes.byref(w)) == _capi.ERR_UNSUPPORTED
+    assert L.ttsdpa_probe(1, FAKE + 4, 1 << 26, 1, None, ctypes.byref(w)) == _capi.ERR_UNSUPPORTED  # not 16-byte aligned
+    assert L.ttsdpa_probe(1, FAKE, 1024, 1, None, ctypes.byref(w)) == _capi.ERR_SHAPE                 # buffer too small
+
+
 def test_kernel_domains_and_workspace():
     L = _capi.lib()
     fp32 = params(_capi.F32, 1, 4, 4, 128, 128, 64)

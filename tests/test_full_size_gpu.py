@@ -95,3 +95,26 @@ def test_config4_decode_split_invariance():
     w1 = 1.0 / (1.0 + np.exp(l2 - l1))
     merged = o1 * w1 + o2 * (1 - w1)
     assert np.abs(merged - full).max() <= 2e-2
+
+
+def test_probes_report_plausible_ceilings():
+    # the measurement probes of the library run and land between a tenth of the published peak and the peak itself
+    import ctypes
+    from tinytorch_amd import _capi
+    lib = _capi.lib()
+    buf = torch.empty(1 << 28, dtype=torch.uint8, device="cuda").fill_(3)
+    stream = torch.cuda.current_stream()
+    for kind, iters, lo, hi in ((0, 4000, 250e12, 2.6e15), (1, 1, 0.8e12, 8.2e12), (2, 1, 0.8e12, 8.2e12)):
+        work = ctypes.c_double(0.0)
+        for _ in range(3):
+            assert lib.ttsdpa_probe(kind, buf.data_ptr(), buf.numel(), iters, stream.cuda_stream, ctypes.byref(work)) == 0
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(10):
+            assert lib.ttsdpa_probe(kind, buf.data_ptr(), buf.numel(), iters, stream.cuda_stream, ctypes.byref(work)) == 0
+        e1.record(stream)
+        torch.cuda.synchronize()
+        rate = work.value / (e0.elapsed_time(e1) / 10 * 1e-3)
+        assert lo < rate < hi, (kind, rate)
+    assert torch.all(buf[4096:] == 3)  # the read probes leave the buffer alone (their sink is never written)

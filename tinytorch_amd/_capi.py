@@ -19,7 +19,7 @@ ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_STRIDE, ERR_MASK, ERR_WORKSPACE, ERR_UNSUPPO
 EXPORTS = [
     "ttsdpa_abi_version", "ttsdpa_status_string", "ttsdpa_params_init", "ttsdpa_plan", "ttsdpa_workspace_bytes",
     "ttsdpa_forward", "ttsdpa_prefill", "ttsdpa_decode", "ttsdpa_general",
-    "ttsdpa_kv_append_params_init", "ttsdpa_kv_append",
+    "ttsdpa_kv_append_params_init", "ttsdpa_kv_append", "ttsdpa_probe",
 ]
 
 
@@ -103,6 +103,9 @@ def lib():
         L.ttsdpa_kv_append_params_init.restype = None
         L.ttsdpa_kv_append.argtypes = [ctypes.POINTER(KvAppendParams), ctypes.c_void_p]
         L.ttsdpa_kv_append.restype = ctypes.c_int
+        L.ttsdpa_probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
+                                   ctypes.POINTER(ctypes.c_double)]
+        L.ttsdpa_probe.restype = ctypes.c_int
         if L.ttsdpa_abi_version() != 3:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L
