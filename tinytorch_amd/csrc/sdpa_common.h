@@ -35,6 +35,22 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// Kernels that use more than 64 KiB of dynamic LDS need that granted per kernel and per device.  Done on the first
+// launch on a device (the device is the current one of the calling thread) and remembered; safe from several host
+// threads (the worst case is granting twice).
+constexpr int kMaxDevices = 64;
+inline hipError_t grant_dynamic_lds(const void* kernel, int bytes, hipError_t (&state)[kMaxDevices], bool (&done)[kMaxDevices]) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (!__atomic_load_n(&done[dev], __ATOMIC_ACQUIRE)) {
+    state[dev] = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    __atomic_store_n(&done[dev], true, __ATOMIC_RELEASE);
+  }
+  return state[dev];
+}
+
 // Element-type traits: storage is 16-bit (or fp32 for the general kernel), arithmetic is fp32.
 struct BF16 {
   typedef __bf16 elem;

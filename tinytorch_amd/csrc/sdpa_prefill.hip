@@ -298,9 +298,9 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
 
 template <typename TR, int D, bool CAUSAL>
 int launch_prefill_k(const KArgs& a, dim3 grid, hipStream_t stream) {
-  // more than 64 KiB of dynamic LDS has to be granted per kernel once
-  static const hipError_t granted = hipFuncSetAttribute((const void*)prefill_kernel<TR, D, CAUSAL>,
-                                                        hipFuncAttributeMaxDynamicSharedMemorySize, PrefillLds<D>::BYTES);
+  static hipError_t state[kMaxDevices];
+  static bool done[kMaxDevices];
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill_kernel<TR, D, CAUSAL>, PrefillLds<D>::BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
   hipLaunchKernelGGL((prefill_kernel<TR, D, CAUSAL>), grid, dim3(256), PrefillLds<D>::BYTES, stream, a);
   return (int)hipGetLastError();

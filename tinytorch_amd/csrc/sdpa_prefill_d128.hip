@@ -549,8 +549,9 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 
 template <typename TR, bool CAUSAL>
 int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
-  static const hipError_t granted = hipFuncSetAttribute((const void*)prefill128_kernel<TR, CAUSAL>,
-                                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+  static hipError_t state[kMaxDevices];
+  static bool done[kMaxDevices];
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill128_kernel<TR, CAUSAL>, LDS_BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
   hipLaunchKernelGGL((prefill128_kernel<TR, CAUSAL>), grid, dim3(NW * 64), LDS_BYTES, stream, a);
   return (int)hipGetLastError();
