@@ -54,7 +54,7 @@ __device__ __forceinline__ void wave_lds_sync() {
 
 // R = registers of query rows per score lane: rows handled = up to 4*R.
 template <typename TR, int R, int DD>
-__global__ __launch_bounds__(256) void decode_kernel(KArgs a, int splits, int chunk, float* __restrict__ ws) {
+__global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int chunk, float* __restrict__ ws) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
   constexpr int NR = 4 * R;    // row slots
