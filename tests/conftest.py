@@ -15,6 +15,16 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """The tests load what is built; only when nothing is built (a fresh checkout) they build it first."""
+    lib = os.path.join(ROOT, "tinytorch_amd", "lib")
+    built = [os.path.join(lib, "libttsdpa.so"), os.path.join(lib, "libtinytorch_host.so"),
+             os.path.join(lib, "test_sdpa_host")]
+    if not any(os.path.exists(f) for f in built):
+        import __graft_entry__
+        __graft_entry__.build()
+
+
 def load_golden(name):
     z = np.load(os.path.join(GOLDEN, name + ".npz"), allow_pickle=False)
     d = {k: z[k] for k in z.files}
