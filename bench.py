@@ -6,7 +6,8 @@
 A step is one call of the hot path (ttsdpa_forward through the C ABI) over one batch of synthetic input already
 resident in HBM.  The headline workload is BASELINE.json's configs[2] (bf16 causal GQA prefill, B2 32q/8kv S4096
 D128: the shape the prefill target is quoted on); the decode workload configs[3] (bf16, B64 32q/8kv KV 8192) is
-measured in the same run and reported under "secondary".  One JSON line is printed.
+measured in the same run and reported under "secondary", and config 3's shape in fp32 (the reference's default dtype,
+on the fp32 MFMA kernel, against the 157.3 TFLOP/s fp32 peak) under "fp32".  One JSON line is printed.
 
 Algorithmic work per launch (what "achieved" divides by the measured launch time):
   prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)
@@ -33,6 +34,7 @@ WORKLOADS = {
     "config3": (2, 32, 8, 4096, 4096, 128, "bf16", True, 1.0, "mfma"),
     "config4": (64, 32, 8, 1, 8192, 128, "bf16", False, 1.0, "hbm"),
     "config5": (1, 28, 4, 16384, 16384, 128, "bf16", True, 1.0, "mfma"),
+    "config3_f32": (2, 32, 8, 4096, 4096, 128, "f32", True, 1.0, "mfma"),  # config 3's shape in the reference's default dtype
 }
 DESCR = {
     "config1": "fp32 causal SDPA B1 H4 S128 D64",
@@ -40,6 +42,7 @@ DESCR = {
     "config3": "bf16 causal GQA prefill B2 32q/8kv S4096 D128",
     "config4": "bf16 decode B64 32q/8kv L1 KV8192 D128 (isCausal=false)",
     "config5": "bf16 causal GQA prefill B1 28q/4kv S16384 D128",
+    "config3_f32": "fp32 causal GQA prefill B2 32q/8kv S4096 D128",
 }
 
 
@@ -241,6 +244,10 @@ def main():
         sec["cpu_baseline"] = None if args.no_cpu else run_cpu_baseline(args.secondary, tensors, args.cpu_seconds)
         del tensors
         line["secondary"] = sec
+        if args.workload == "config3":  # the same shape in fp32, against the fp32 MFMA peak (no CPU leg: same arithmetic as config 3's)
+            f32, tensors = run_gpu("config3_f32", max(1, min(args.steps, 100)), min(args.warmup, 20))
+            del tensors
+            line["fp32"] = f32
     print(json.dumps(line), flush=True)
 
 

@@ -61,8 +61,9 @@ def call(entry, q, k, v, causal=False, mask=None, scale=None, out=None):
     return rc, out
 
 
-def route_of(q, k, v, causal=False, mask=None, scale=None):
-    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+def route_of(q, k, v, causal=False, mask=None, scale=None, out=None):
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     rc, r = _capi.plan(build_params(q, k, v, out, causal, mask, scale))
     assert rc == 0
     return _capi.ROUTE_NAMES[r]

@@ -56,7 +56,9 @@ def test_struct_layout_matches_header():
 
 
 @pytest.mark.parametrize("args,route", [
-    ((_capi.F32, 1, 4, 4, 128, 128, 64), _capi.ROUTE_GENERAL),       # config 1
+    ((_capi.F32, 1, 4, 4, 128, 128, 64), _capi.ROUTE_PREFILL),       # config 1: fp32 MFMA kernel
+    ((_capi.F32, 2, 8, 2, 300, 300, 128), _capi.ROUTE_PREFILL),
+    ((_capi.F32, 2, 8, 2, 300, 300, 96), _capi.ROUTE_GENERAL),       # fp32 MFMA kernel: head_dim 64 and 128 only
     ((_capi.F16, 4, 32, 32, 2048, 2048, 128), _capi.ROUTE_PREFILL),  # config 2
     ((_capi.BF16, 2, 32, 8, 4096, 4096, 128), _capi.ROUTE_PREFILL),  # config 3
     ((_capi.BF16, 64, 32, 8, 1, 8192, 128), _capi.ROUTE_DECODE),     # config 4
@@ -90,6 +92,14 @@ def test_routes_depend_on_flags():
     assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL
     p = params(*base)
     p.q = FAKE + 2
+    assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL
+    # fp32: the MFMA kernel takes no attnMask and needs 16-byte aligned rows
+    f32 = (_capi.F32, 2, 8, 2, 512, 512, 128)
+    assert _capi.plan(params(*f32, causal=1))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(*f32, mask_kind=_capi.MASK_ADD, mask=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(*f32, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
+    p = params(*f32)
+    p.v_stride[2] = 130
     assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL
     # decode with causal set is the top-left triangle (only key 0 visible): not the streaming kernel's case
     assert _capi.plan(params(_capi.BF16, 4, 8, 2, 1, 1024, 128, causal=1))[1] == _capi.ROUTE_PREFILL
@@ -164,7 +174,7 @@ def test_probe_argument_checks():
 
 def test_kernel_domains_and_workspace():
     L = _capi.lib()
-    fp32 = params(_capi.F32, 1, 4, 4, 128, 128, 64)
+    fp32 = params(_capi.F32, 1, 4, 4, 128, 128, 96)  # the fp32 MFMA kernel covers head_dim 64 and 128
     assert L.ttsdpa_prefill(ctypes.byref(fp32), None) == _capi.ERR_UNSUPPORTED
     assert L.ttsdpa_decode(ctypes.byref(fp32), None, 0, None) == _capi.ERR_UNSUPPORTED
     # config 4 has 512 (batch, kv head) pairs: enough workgroups without splitting the cache, hence no scratch

@@ -238,7 +238,7 @@ def test_general_against_oracle(case):
     assert rc == 0
     assert max_abs_err(out, exp) <= TOL[dtype]
     if dtype == "f32":
-        assert route_of(*dev, causal=causal) == "general"
+        assert route_of(*dev, causal=causal) == ("prefill" if D in (64, 128) else "general")
 
 
 def test_general_masks_large():
@@ -484,3 +484,67 @@ def test_decode_head_dim_64(case):
     assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]
     rc, out2 = call("general", *dev)
     assert rc == 0 and max_abs_err(out2, exp) <= TOL[dtype]
+
+
+# ---- fp32 tensors on the fp32 matrix cores -----------------------------------------------------------------------
+
+F32_PREFILL_CASES = [
+    # B, Hq, Hkv, L, S, D, causal
+    (1, 4, 4, 128, 128, 64, False),    # config 1's shape, unmasked
+    (1, 8, 2, 512, 512, 128, True),    # config 3's grouping, scaled down
+    (1, 7, 1, 300, 300, 128, True),    # 7 heads per KV head
+    (2, 4, 2, 130, 257, 128, False),   # ragged in both directions
+    (1, 2, 2, 200, 77, 64, True),      # L > S, top-left causal
+    (1, 2, 2, 77, 200, 64, True),      # L < S
+    (1, 3, 3, 33, 31, 128, False),     # less than one key tile
+    (1, 2, 1, 1, 40, 64, False),       # a single query row
+    (1, 2, 2, 5, 1, 128, True),        # a single key
+    (8, 8, 8, 160, 160, 64, True),     # (batch x kv heads) multiple of 8: the XCD-aware order
+]
+
+
+@pytest.mark.parametrize("case", F32_PREFILL_CASES, ids=lambda c: "B%dH%dk%dL%dS%dD%d-c%d" % c)
+def test_fp32_mfma_prefill_against_oracle(case):
+    B, Hq, Hkv, L, S, D, causal = case
+    say("fp32 prefill", case)
+    host, dev = make_inputs(5000 + L + S, B, Hq, Hkv, L, S, D, "f32")
+    exp = oracle.sdpa_f32(*host, causal=causal)
+    assert route_of(*dev, causal=causal) == "prefill"
+    rc, out = call("prefill", *dev, causal=causal)
+    assert rc == 0
+    err = max_abs_err(out, exp)
+    say("   max-abs-err", err)
+    assert err <= TOL["f32"]
+    rc, out2 = call("forward", *dev, causal=causal)
+    assert rc == 0 and np.array_equal(to_host_f32(out2), to_host_f32(out))
+    rc, out3 = call("general", *dev, causal=causal)    # the vector-ALU kernel agrees
+    assert rc == 0 and max_abs_err(out3, exp) <= TOL["f32"]
+
+
+def test_fp32_mfma_large_scores_views_and_scale():
+    """Scores spread over hundreds of units (the running maximum has to follow every tile), a custom scale, q as a
+    transposed view of a [B, L, H, D] buffer, k/v as the leading rows of a longer cache, out into a padded buffer."""
+    B, Hq, Hkv, L, S, D = 2, 4, 2, 200, 333, 128
+    host, dev = make_inputs(99, B, Hq, Hkv, L, S, D, "f32", mul=5.0)
+    exp = oracle.sdpa_f32(*host, causal=True, scale=0.11)
+    qv = dev[0].permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    kc = torch.zeros(B, Hkv, S + 50, D, device="cuda")
+    vc = torch.full((B, Hkv, S + 50, D), float("nan"), device="cuda")
+    kc[:, :, :S], vc[:, :, :S] = dev[1], dev[2]
+    obuf = torch.full((B, Hq, L, D + 4), -7.0, device="cuda")
+    ov = obuf[..., :D]
+    assert route_of(qv, kc[:, :, :S], vc[:, :, :S], causal=True, scale=0.11, out=ov) == "prefill"
+    rc, out = call("forward", qv, kc[:, :, :S], vc[:, :, :S], causal=True, scale=0.11, out=ov)
+    assert rc == 0
+    assert max_abs_err(ov, exp) <= 5.0 * TOL["f32"]     # values are 5x larger than unit-variance inputs
+    assert bool((obuf[..., D:] == -7.0).all())           # nothing written outside the rows
+
+
+def test_fp32_mfma_gqa_equals_repeated_kv_bitwise():
+    B, Hq, Hkv, L, S, D = 1, 8, 2, 150, 150, 64
+    host, dev = make_inputs(31, B, Hq, Hkv, L, S, D, "f32")
+    rc, a = call("prefill", *dev, causal=True)
+    G = Hq // Hkv
+    rc2, b = call("prefill", dev[0], dev[1].repeat_interleave(G, 1), dev[2].repeat_interleave(G, 1), causal=True)
+    assert rc == 0 and rc2 == 0
+    assert torch.equal(a, b)

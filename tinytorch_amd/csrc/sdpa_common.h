@@ -98,6 +98,7 @@ __device__ __forceinline__ void store_from_float(_Float16* p, float x) { *p = (_
 int launch_general(const KArgs& a, int dtype, hipStream_t stream);
 int launch_prefill(const KArgs& a, int dtype, hipStream_t stream);       // 128-row workgroups; head_dim 64 or 128
 int launch_prefill_d128(const KArgs& a, int dtype, hipStream_t stream);  // 256-row workgroups, pipelined; head_dim 128
+int launch_prefill_f32(const KArgs& a, hipStream_t stream);              // fp32 tensors on the fp32 matrix cores; head_dim 64 or 128
 int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream);
 int launch_zero(const KArgs& a, int dtype, hipStream_t stream);
 struct KvAppendArgs {

@@ -1,0 +1,264 @@
+// Flash-attention forward for fp32 tensors on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32, full fp32 products
+// and sums): fp32 is the reference's default dtype, and its fp32 path is what the 1e-4 parity bar is stated against.
+// Replaces the same device chain as the 16-bit kernels (reference src/Function/FuncNNLayer.h:237-265): the score
+// matrix never leaves registers.  head_dim 64 or 128, no attnMask (those calls take the vector-ALU kernel).
+//
+// A workgroup of 4 wavefronts owns 128 query rows of one (batch, query head), 32 rows per wavefront; keys/values come
+// in tiles of 32, staged global -> registers -> LDS, double-buffered.
+// Per wavefront and tile, with v_mfma_f32_32x32x2 (A: 32 rows x 2, B: 2 x 32 cols, lane l supplies row/col l%32 and
+// contraction element l/32; C: lane l holds column l%32 and rows 8*(r/4) + 4*(l/32) + r%4):
+//   S^T[32 keys x 32 queries] = K . Q^T   MFMA ks contracts head_dim elements ks (lanes 0-31) and ks + D/2 (lanes 32-63),
+//                                         so a lane's Q operands are one contiguous half of its query row (registers)
+//                                         and K comes from LDS rows padded by one float (conflict-free columns);
+//                                         two accumulators take alternate ks so the chain never waits on itself
+//   P^T = exp2((S^T - m) * scale*log2e)   a query is one lane column; its other 16 keys sit in lane l^32
+//   O^T[D x 32 queries] += V^T . P^T      MFMA t contracts the two keys that the lane halves hold in accumulator
+//                                         register t, so P^T feeds the pipe straight from those registers and
+//                                         V^T[d][key] is a plain row-major LDS read along d
+// The running maximum is raised only when exceeded by 2^8 in the exponent.  Causal masking as in the 16-bit kernels
+// (top-left aligned, reference src/Operation/OpTransformCpu.h:202-209): tiles above the diagonal are skipped.
+
+#include "sdpa_common.h"
+
+namespace ttsdpa {
+
+namespace {
+
+constexpr int BM = 128;  // query rows per workgroup
+constexpr int BN = 32;   // keys per tile
+constexpr float kLazyExp = 8.f;
+
+template <int D>
+struct F32Lds {
+  static constexpr int K_PITCH = D + 1;   // floats; a column of 32 keys falls into 32 different banks
+  static constexpr int V_PITCH = D + 32;  // floats; rows stay 16-byte aligned, the two lane halves use disjoint banks
+  static constexpr int STAGE = BN * (K_PITCH + V_PITCH);
+  static constexpr int BYTES = 2 * STAGE * 4;
+};
+
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
+  typedef F32Lds<D> Lds;
+  constexpr int K_PITCH = Lds::K_PITCH, V_PITCH = Lds::V_PITCH;
+  constexpr int KSTEPS = D / 2;   // MFMAs along head_dim for S^T
+  constexpr int DBLK = D / 32;    // 32-row blocks of O^T
+  constexpr int NLD = BN * D / 4 / 256;  // 16-byte chunks per thread per tile, for K and for V
+
+  extern __shared__ __attribute__((aligned(16))) float smem_f32[];
+  float* smem = smem_f32;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31;
+  const int lh = lane >> 5;
+
+  // ---- workgroup -> (batch, kv head, query head in group, row tile); workgroup n runs on XCD n % 8 -------------
+  const int ntile = (a.L + BM - 1) / BM;
+  const int inner = a.G * ntile;
+  const int npair = a.B * a.Hkv;
+  int pair, in;
+  {
+    int n = blockIdx.x;
+    if ((npair & 7) == 0) {
+      int xcd = n & 7, slot = n >> 3;
+      pair = (slot / inner) * 8 + xcd;
+      in = slot % inner;
+    } else {
+      pair = n / inner;
+      in = n % inner;
+    }
+  }
+  const int b = pair / a.Hkv, hk = pair % a.Hkv;
+  const int g = in % a.G;
+  const int rt = CAUSAL ? ntile - 1 - in / a.G : in / a.G;  // longest rows first
+  const int h = hk * a.G + g;
+  const int q0 = rt * BM;
+  const int qw0 = q0 + wave * 32;
+
+  const float* qp = (const float*)a.q + b * a.qs[0] + h * a.qs[1];
+  const float* kp = (const float*)a.k + b * a.ks[0] + hk * a.ks[1];
+  const float* vp = (const float*)a.v + b * a.vs[0] + hk * a.vs[1];
+
+  // ---- Q: this lane's half of its query row, the B operands of the S^T MFMAs ---------------------------------------
+  float qreg[KSTEPS];
+  {
+    int row = qw0 + lq;
+    row = row < a.L ? row : a.L - 1;
+    const float* qr = qp + row * a.qs[2] + lh * (D / 2);
+#pragma unroll
+    for (int i = 0; i < KSTEPS / 4; i++) {
+      f32x4 t = *(const f32x4*)(qr + 4 * i);
+#pragma unroll
+      for (int e = 0; e < 4; e++) qreg[4 * i + e] = t[e];
+    }
+  }
+
+  f32x16 oacc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
+  const float c = a.scale * kLog2e;
+  const float lazy = kLazyExp / c;
+  float m_use = -1e30f;
+  float mc = m_use * c;
+  float l_run = 0.f;
+
+  int ntiles_kv = (a.S + BN - 1) / BN;
+  if (CAUSAL) {
+    int last = q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1;
+    int lastkv = last < a.S - 1 ? last : a.S - 1;
+    ntiles_kv = lastkv / BN + 1;
+  }
+
+  // ---- global -> register -> LDS staging: thread t moves 16-byte chunks t, t+256, ... of a tile ----------------------
+  f32x4 kst[NLD], vst[NLD];
+  int lrow[NLD], lcol[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; i++) {
+    int cidx = tid + 256 * i;
+    lrow[i] = cidx / (D / 4);
+    lcol[i] = cidx % (D / 4);
+  }
+  auto load_tile = [&](int kv0) {
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+      int key = kv0 + lrow[i];
+      key = key < a.S ? key : a.S - 1;  // rows past the end re-read the last valid row (masked later)
+      kst[i] = *(const f32x4*)(kp + key * a.ks[2] + 4 * lcol[i]);
+      vst[i] = *(const f32x4*)(vp + key * a.vs[2] + 4 * lcol[i]);
+    }
+  };
+  auto store_tile = [&](int stage) {
+    float* Ks = smem + stage * Lds::STAGE;
+    float* Vs = Ks + BN * K_PITCH;
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) Ks[lrow[i] * K_PITCH + 4 * lcol[i] + e] = kst[i][e];  // rows are not 16-byte aligned
+      *(f32x4*)(Vs + lrow[i] * V_PITCH + 4 * lcol[i]) = vst[i];
+    }
+  };
+
+  const int k_lane = lq * K_PITCH + lh * (D / 2);  // floats
+  const int v_lane = 4 * lh * V_PITCH + lq;        // floats; + (8*(t/4) + t%4) * V_PITCH + 32*db
+
+  load_tile(0);
+  store_tile(0);
+  if (ntiles_kv > 1) load_tile(BN);
+  __syncthreads();
+
+  for (int jt = 0; jt < ntiles_kv; jt++) {
+    const int kv0 = jt * BN;
+    const int cur = jt & 1;
+    if (jt + 1 < ntiles_kv) {
+      store_tile(cur ^ 1);  // stage cur^1 was last read before the barrier that ended the previous iteration
+      if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BN);
+    }
+
+    if (!CAUSAL || kv0 <= qw0 + 31) {  // else: the whole tile is above this wavefront's diagonal
+      const float* Ks = smem + cur * Lds::STAGE;
+      const float* Vs = Ks + BN * K_PITCH;
+
+      // ---- S^T = K . Q^T, two accumulators over alternate k-steps ----------------------------------------------------
+      f32x16 s0, s1;
+#pragma unroll
+      for (int r = 0; r < 16; r++) s0[r] = 0.f, s1[r] = 0.f;
+      const float* krow = Ks + k_lane;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks += 2) {
+        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[ks], qreg[ks], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[ks + 1], qreg[ks + 1], s1, 0, 0, 0);
+      }
+      f32x16 s;
+#pragma unroll
+      for (int r = 0; r < 16; r++) s[r] = s0[r] + s1[r];
+
+      // ---- mask the diagonal / ragged tile -----------------------------------------------------------------------------
+      if ((CAUSAL && kv0 + BN - 1 > qw0) || (kv0 + BN > a.S)) {
+        const int qi = qw0 + lq;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          bool hidden = key >= a.S || (CAUSAL && key > qi);
+          if (hidden) s[r] = -INFINITY;
+        }
+      }
+
+      // ---- online softmax with a lazily raised maximum -----------------------------------------------------------------
+      float mloc = s[0];
+#pragma unroll
+      for (int r = 1; r < 16; r++) mloc = fmaxf(mloc, s[r]);
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+      if (__builtin_amdgcn_ballot_w64(mloc > m_use + lazy) != 0) {
+        const float m_new = fmaxf(m_use, mloc);
+        const float alpha = fast_exp2((m_use - m_new) * c);
+        m_use = m_new;
+        mc = m_new * c;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DBLK; i++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+      }
+      float psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        s[r] = fast_exp2(fmaf(s[r], c, -mc));
+        psum += s[r];
+      }
+      l_run += psum;
+
+      // ---- O^T += V^T . P^T: MFMA t contracts the keys held in accumulator register t of the two lane halves -------------
+      const float* vl = Vs + v_lane;
+#pragma unroll
+      for (int t = 0; t < 16; t++) {
+#pragma unroll
+        for (int db = 0; db < DBLK; db++) {
+          float va = vl[(8 * (t >> 2) + (t & 3)) * V_PITCH + 32 * db];
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va, s[t], oacc[db], 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- normalise and store ----------------------------------------------------------------------------------------------
+  float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = 1.f / l_tot;
+  const int qi = qw0 + lq;
+  if (qi < a.L) {
+    float* op = (float*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2];
+#pragma unroll
+    for (int db = 0; db < DBLK; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        f32x4 x;
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = oacc[db][4 * rg + i] * inv;
+        *(f32x4*)(op + 32 * db + 8 * rg + 4 * lh) = x;
+      }
+  }
+}
+
+template <int D, bool CAUSAL>
+int launch_f32_k(const KArgs& a, dim3 grid, hipStream_t stream) {
+  static hipError_t state[kMaxDevices];
+  static bool done[kMaxDevices];
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill_f32_kernel<D, CAUSAL>, F32Lds<D>::BYTES, state, done);
+  if (granted != hipSuccess) return (int)granted;
+  hipLaunchKernelGGL((prefill_f32_kernel<D, CAUSAL>), grid, dim3(256), F32Lds<D>::BYTES, stream, a);
+  return (int)hipGetLastError();
+}
+
+}  // namespace
+
+int launch_prefill_f32(const KArgs& a, hipStream_t stream) {
+  long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM);
+  dim3 grid((unsigned)nwg);
+  if (a.D == 128) return a.causal ? launch_f32_k<128, true>(a, grid, stream) : launch_f32_k<128, false>(a, grid, stream);
+  return a.causal ? launch_f32_k<64, true>(a, grid, stream) : launch_f32_k<64, false>(a, grid, stream);
+}
+
+}  // namespace ttsdpa

@@ -70,7 +70,19 @@ bool fast_layout_ok(const ttsdpa_params* p, bool masks_ok = false) {
   return ptr_aligned(p->q, 16) && ptr_aligned(p->k, 16) && ptr_aligned(p->v, 16) && ptr_aligned(p->out, 16);
 }
 
+// fp32 tensors the fp32 MFMA kernel can read and write with 16-byte accesses.
+bool f32_prefill_ok(const ttsdpa_params* p) {
+  if (p->dtype != TTSDPA_F32 || p->mask_kind != TTSDPA_MASK_NONE || p->kv_len) return false;
+  if (p->D != 128 && p->D != 64) return false;
+  if (!(p->scale > 0.f) || !isfinite(p->scale) || p->S < 1 || p->L < 1) return false;
+  if (!dense_last_ok(p->q_stride, 4) || !dense_last_ok(p->k_stride, 4) || !dense_last_ok(p->v_stride, 4) ||
+      !dense_last_ok(p->o_stride, 4))
+    return false;
+  return ptr_aligned(p->q, 16) && ptr_aligned(p->k, 16) && ptr_aligned(p->v, 16) && ptr_aligned(p->out, 16);
+}
+
 bool prefill_ok(const ttsdpa_params* p) {
+  if (f32_prefill_ok(p)) return true;
   // an attnMask or per-batch key counts are taken by the pipelined head_dim-128 kernel only
   const bool pipelined = p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
   if (p->kv_len && !pipelined) return false;
@@ -166,6 +178,7 @@ int ttsdpa_prefill(const ttsdpa_params* p, void* stream) {
   if (p->B == 0 || p->L == 0) return TTSDPA_OK;
   if (!prefill_ok(p)) return TTSDPA_ERR_UNSUPPORTED;
   if ((rc = check_grid((long long)a.B * a.Hq * ((a.L + 127) / 128))) != TTSDPA_OK) return rc;
+  if (p->dtype == TTSDPA_F32) return launch_prefill_f32(a, (hipStream_t)stream);
   // head_dim 128 with enough rows to fill 256-row workgroups takes the software-pipelined kernel (its tile loads
   // address 64 rows with 32-bit byte offsets)
   if (a.D == 128 && a.L > 128 && a.ks[2] < (1 << 24) && a.vs[2] < (1 << 24))
