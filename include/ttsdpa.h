@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TTSDPA_ABI_VERSION 3
+#define TTSDPA_ABI_VERSION 4
 
 /* Element types; numbering is the reference's DType enum (reference src/Tensor/DType.h:20-28). */
 enum ttsdpa_dtype { TTSDPA_F32 = 0, TTSDPA_F16 = 1, TTSDPA_BF16 = 2 };
@@ -54,6 +54,12 @@ enum ttsdpa_status {
 };
 
 /* Which kernel a call maps to (ttsdpa_plan). */
+enum ttsdpa_causal {
+  TTSDPA_CAUSAL_NONE = 0,
+  TTSDPA_CAUSAL_TOP_LEFT = 1,    /* the reference's isCausal */
+  TTSDPA_CAUSAL_BOTTOM_RIGHT = 2 /* queries are the last L positions of the key sequence */
+};
+
 enum ttsdpa_route {
   TTSDPA_ROUTE_NONE = 0,    /* nothing to launch (an empty output) */
   TTSDPA_ROUTE_GENERAL = 1, /* any dtype / head_dim / mask / per-batch key counts; fp32 arithmetic on the vector ALUs */
@@ -69,8 +75,12 @@ enum ttsdpa_route {
  * the reference; Hkv == Hq is plain multi-head attention.
  * Strides are in elements: {batch, head, sequence}; the head_dim stride is 1.  A dense tensor [B,H,N,D] has
  * {H*N*D, N*D, D}.
- * causal: key j is visible to query i iff j <= i (top-left aligned, tril(ones(L,S),0), reference
- * src/Function/FuncNNLayer.h:241-247) — a decode step with L == 1 must therefore pass causal = 0.
+ * causal (ttsdpa_causal): TTSDPA_CAUSAL_TOP_LEFT is the reference's isCausal — key j is visible to query i iff
+ * j <= i (tril(ones(L,S),0), reference src/Function/FuncNNLayer.h:241-247); a decode step with L == 1 must therefore
+ * not pass it.  TTSDPA_CAUSAL_BOTTOM_RIGHT aligns the diagonal with the end of the keys instead: the L queries are the
+ * last L positions of a sequence of S_b keys (S_b = kv_len[b] when given, else S), key j is visible to query i iff
+ * j <= i + max(0, S_b - L).  It is what the reference computes when handed the Bool mask tril(ones(L,S), S-L), and
+ * what a chunked prefill or a multi-token decode step against a KV cache needs; for L == S the two coincide.
  * mask: NULL, or an attnMask of any shape that broadcasts to [B,Hq,L,S] — the reference adds it to the scores with
  * a broadcasting add (src/Function/FuncNNLayer.h:249-260).  mask_stride gives its element strides along
  * {batch, head, query row, key}; an axis the mask does not have, or has with size 1, gets stride 0.  A dense
@@ -90,7 +100,7 @@ typedef struct ttsdpa_params {
   int64_t v_stride[3];
   int64_t o_stride[3];
   float scale;
-  int32_t causal;
+  int32_t causal;    /* ttsdpa_causal */
   int32_t mask_kind; /* ttsdpa_mask_kind */
   const void* mask;
   int64_t mask_stride[4]; /* elements: batch, head, query row, key; 0 broadcasts the axis */
@@ -124,9 +134,10 @@ size_t ttsdpa_workspace_bytes(const ttsdpa_params* p);
 int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The three kernels individually (same contract; TTSDPA_ERR_UNSUPPORTED when *p is outside the kernel's domain).
- * ttsdpa_prefill replaces the reference's GEMM -> scale -> bias -> softmax -> GEMM chain for training/prefill shapes;
+ * ttsdpa_prefill replaces the reference's GEMM -> scale -> bias -> softmax -> GEMM chain for training/prefill shapes
+ * (16-bit tensors on the 16-bit matrix cores with fp32 accumulation, fp32 tensors on the fp32 matrix cores);
  * ttsdpa_decode replaces it for one (or a few) query rows against a long contiguous KV cache;
- * ttsdpa_general covers everything else the reference op accepts (masks, fp32, other head sizes). */
+ * ttsdpa_general covers everything else the reference op accepts (other head sizes, unaligned rows, masks on fp32 or short inputs). */
 int ttsdpa_prefill(const ttsdpa_params* p, void* stream);
 int ttsdpa_decode(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream);
 int ttsdpa_general(const ttsdpa_params* p, void* stream);

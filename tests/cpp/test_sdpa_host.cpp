@@ -224,7 +224,7 @@ static void test_kv_cache() {
     Tensor tq(q, {B, Hq, 1, D}, gpu);
     q = tq.toList<float>();
     Tensor kvLens(std::vector<int>{lens[0], lens[1]}, {B}, gpuInt);
-    std::vector<float> y = op::sdpAttentionCached(tq, kc, vc, kvLens, 1.f / std::sqrt(static_cast<float>(D))).toList<float>();
+    std::vector<float> y = op::sdpAttentionCached(tq, kc, vc, kvLens, false, 1.f / std::sqrt(static_cast<float>(D))).toList<float>();
     for (int b = 0; b < B; b++) {
       std::vector<float> qb(q.begin() + static_cast<size_t>(b) * Hq * D, q.begin() + static_cast<size_t>(b + 1) * Hq * D);
       std::vector<float> ref = closedForm(qb, rowsOf(kall, b, 0, lens[b]), rowsOf(vall, b, 0, lens[b]), 1, Hq, Hkv, 1, lens[b], D, false);

@@ -101,6 +101,12 @@ def test_routes_depend_on_flags():
     p = params(*f32)
     p.v_stride[2] = 130
     assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL
+    # bottom-right aligned causal: a few new rows against a long cache stream it; one new row hides nothing
+    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 4, 1024, 128, causal=2))[1] == _capi.ROUTE_DECODE
+    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 1, 1024, 128, causal=2))[1] == _capi.ROUTE_DECODE
+    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 512, 1024, 128, causal=2))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.F32, 4, 8, 2, 512, 1024, 128, causal=2))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 4, 1024, 128, causal=2, kv_len=FAKE))[1] == _capi.ROUTE_DECODE
     # decode with causal set is the top-left triangle (only key 0 visible): not the streaming kernel's case
     assert _capi.plan(params(_capi.BF16, 4, 8, 2, 1, 1024, 128, causal=1))[1] == _capi.ROUTE_PREFILL
 
@@ -115,6 +121,9 @@ def test_routes_depend_on_flags():
     (dict(D=512), _capi.ERR_SHAPE),
     (dict(L=-1), _capi.ERR_SHAPE),
     (dict(mask_kind=7), _capi.ERR_MASK),
+    (dict(causal=3), _capi.ERR_MASK),                                        # not a causal mode
+    (dict(causal=-1), _capi.ERR_MASK),
+    (dict(mask_kind=_capi.MASK_BOOL, mask=FAKE, causal=2), _capi.ERR_MASK),
     (dict(mask_kind=_capi.MASK_BOOL), _capi.ERR_NULL),                      # mask kind without a mask
     (dict(mask_kind=_capi.MASK_BOOL, mask=FAKE, causal=1), _capi.ERR_MASK),  # reference asserts on this
     (dict(mask_kind=_capi.MASK_BOOL, mask=FAKE, mask_stride=(0, 0, -64, 1)), _capi.ERR_STRIDE),

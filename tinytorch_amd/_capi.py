@@ -10,6 +10,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libttsdpa.so")
 
 F32, F16, BF16 = 0, 1, 2
 MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
+CAUSAL_NONE, CAUSAL_TOP_LEFT, CAUSAL_BOTTOM_RIGHT = 0, 1, 2
 ROUTE_NONE, ROUTE_GENERAL, ROUTE_PREFILL, ROUTE_DECODE, ROUTE_ZERO = 0, 1, 2, 3, 4
 ROUTE_NAMES = {0: "none", 1: "general", 2: "prefill", 3: "decode", 4: "zero"}
 
@@ -106,7 +107,7 @@ def lib():
         L.ttsdpa_probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
                                    ctypes.POINTER(ctypes.c_double)]
         L.ttsdpa_probe.restype = ctypes.c_int
-        if L.ttsdpa_abi_version() != 3:
+        if L.ttsdpa_abi_version() != 4:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L
     return _lib

@@ -16,12 +16,19 @@ struct KArgs {
   const int* kv_len;  // per-batch valid key count (device), or nullptr
   int B, Hq, Hkv, L, S, D;
   int G;  // Hq / Hkv: query heads per KV head
-  int causal;
+  int causal;     // key j is visible to query i iff j <= i + offset
+  int causal_br;  // offset: 0 (top-left aligned, the reference's mask) or max(0, keys of the batch entry - L) (bottom-right)
   int mask_kind;
   float scale;
   long long qs[3], ks[3], vs[3], os[3];  // element strides: batch, head, sequence
   long long ms[4];                       // mask element strides: batch, head, query row, key (0 = broadcast)
 };
+
+// Offset of the causal diagonal in key coordinates for a batch entry with S keys.
+__device__ __forceinline__ int causal_offset(const KArgs& a, int S) {
+  const int d = S - a.L;
+  return (a.causal_br && d > 0) ? d : 0;
+}
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));

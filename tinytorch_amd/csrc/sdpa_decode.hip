@@ -119,6 +119,18 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int
   const int s_begin = split * chunk;
   const int s_end = s_begin + chunk < S ? s_begin + chunk : S;
   float* pl = Pl[wave];
+  // First hidden key per row of this score lane: the end of the split, or under a (bottom-right aligned) causal mask
+  // the key after the row's own position S - L + l.
+  int klim[R], klim_min = s_end;
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    klim[r] = s_end;
+    if (a.causal) {
+      int own = causal_offset(a, S) + (lg + 4 * r) / a.G + 1;
+      klim[r] = own < s_end ? own : s_end;
+    }
+    klim_min = klim[r] < klim_min ? klim[r] : klim_min;
+  }
 
   for (int k0 = s_begin + wave * KB; k0 < s_end; k0 += NWAVE * KB) {
     // ---- issue all loads of the block: K for the score MFMAs, V for the accumulation ----------------------------------
@@ -147,9 +159,10 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int
 #pragma unroll
       for (int ks = 0; ks < KS; ks++)
         sc[gi] = TR::mfma16(qa[ks], __builtin_bit_cast(vec8, kreg[gi][ks]), sc[gi]);
-      if (k0 + 16 * gi + l16 >= s_end) {
+      if (k0 + 16 * gi + l16 >= klim_min) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) sc[gi][r] = -INFINITY;
+        for (int r = 0; r < 4; r++)
+          if (r >= R || k0 + 16 * gi + l16 >= klim[r < R ? r : 0]) sc[gi][r] = -INFINITY;
       }
     }
 

@@ -63,8 +63,9 @@ __global__ __launch_bounds__(256) void general_kernel(KArgs a) {
     S = len < 0 ? 0 : (len < S ? len : S);
   }
   int send = S;
+  const int coff = causal_offset(a, S);
   if (a.causal) {
-    int last = row0 + kRows - 1 < a.L - 1 ? row0 + kRows - 1 : a.L - 1;
+    int last = (row0 + kRows - 1 < a.L - 1 ? row0 + kRows - 1 : a.L - 1) + coff;
     send = last + 1 < S ? last + 1 : S;
   }
 
@@ -96,7 +97,7 @@ __global__ __launch_bounds__(256) void general_kernel(KArgs a) {
         part += __shfl_xor(part, 2);
         float x = part * a.scale;
         int key = k0 + c0 + j;
-        bool hidden = key >= S || (a.causal && key > row);
+        bool hidden = key >= S || (a.causal && key > row + coff);
         if (a.mask_kind == 1) {
           if (key < S && ((const uint8_t*)a.mask)[mrow + key * a.ms[3]] == 0) hidden = true;
         } else if (a.mask_kind == 2) {

@@ -127,8 +127,9 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
   float l_run = 0.f;     // this lane's share of the running row sum
 
   int ntiles_kv = (a.S + BN - 1) / BN;
+  const int coff = CAUSAL ? causal_offset(a, a.S) : 0;  // query row i sees keys up to i + coff
   if (CAUSAL) {
-    int last = q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1;  // last query row of the workgroup
+    int last = (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1) + coff;  // last key of the workgroup's last query row
     int lastkv = last < a.S - 1 ? last : a.S - 1;
     ntiles_kv = lastkv / BN + 1;
   }
@@ -192,7 +193,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
       if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BN);
     }
 
-    if (!CAUSAL || kv0 <= qw0 + 31) {  // else: the whole tile is above this wavefront's diagonal
+    if (!CAUSAL || kv0 <= qw0 + 31 + coff) {  // else: the whole tile is above this wavefront's diagonal
       const T* Ks = smem + cur * Lds::STAGE;
       const T* Vs = Ks + BN * K_PITCH;
 
@@ -211,9 +212,9 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
       }
 
       // ---- mask the diagonal / ragged tile -----------------------------------------------------------------------
-      const bool need_mask = (CAUSAL && kv0 + BN - 1 > qw0) || (kv0 + BN > a.S);
+      const bool need_mask = (CAUSAL && kv0 + BN - 1 > qw0 + coff) || (kv0 + BN > a.S);
       if (need_mask) {
-        const int qi = qw0 + lq;
+        const int qi = qw0 + lq + coff;
 #pragma unroll
         for (int blk = 0; blk < 2; blk++)
 #pragma unroll

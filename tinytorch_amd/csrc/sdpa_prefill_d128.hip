@@ -140,16 +140,20 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     continue;
   }
 
+  // Query row i sees keys up to i + coff (coff = 0: the reference's top-left aligned mask); qc0 is this wavefront's
+  // first row in key coordinates.
+  const int coff = CAUSAL ? causal_offset(a, S) : 0;
+  const int qc0 = qw0 + coff;
   int ntiles_kv = (S + BN - 1) / BN;
   if (CAUSAL) {
-    int last = q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1;
+    int last = (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1) + coff;
     int lastkv = last < S - 1 ? last : S - 1;
     ntiles_kv = lastkv / BN + 1;
   }
   // 32-key halves this wavefront computes on: under a causal mask those that start at or before its last row
   int my_halves = 2 * ntiles_kv;
   if (CAUSAL) {
-    int t = (qw0 + WM - 1) / 32 + 1;
+    int t = (qc0 + WM - 1) / 32 + 1;
     my_halves = t < my_halves ? t : my_halves;
   }
   // Tiles j whose two steps take the fast form: halves up to 2j+3 are this wavefront's, tile j+1 is complete, and
@@ -159,7 +163,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     int f = S >= 96 ? (S - 32) / BN : 0;
     nfast = f < nfast ? f : nfast;
     if (CAUSAL) {
-      f = qw0 >= 95 ? (qw0 - 31) / BN : 0;
+      f = qc0 >= 95 ? (qc0 - 31) / BN : 0;
       nfast = f < nfast ? f : nfast;
     }
   }
@@ -288,7 +292,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
 
   auto mask_half = [&](f32x16& s, int kv0) __attribute__((always_inline)) {
-    const int qi = qw0 + lq;
+    const int qi = qc0 + lq;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
@@ -393,7 +397,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     if (h < my_halves) pv_half(p_cur, half_base(h));
     if (h + 1 < my_halves) {
       const int kv0 = 32 * (h + 1);
-      if ((CAUSAL && kv0 + 31 > qw0) || kv0 + 32 > S) mask_half(s_nxt, kv0);
+      if ((CAUSAL && kv0 + 31 > qc0) || kv0 + 32 > S) mask_half(s_nxt, kv0);
       if (!CAUSAL && a.mask_kind != 0) user_mask_half(s_nxt, kv0);
       settle_half(s_nxt, p_nxt, exp_half(s_nxt, p_nxt));
     }
@@ -454,7 +458,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }
   {  // P(0) and the scores of half 1
     qk_half(sC, half_base(0));
-    if ((CAUSAL && 31 > qw0) || 32 > S) mask_half(sC, 0);
+    if ((CAUSAL && 31 > qc0) || 32 > S) mask_half(sC, 0);
     if (!CAUSAL && a.mask_kind != 0) user_mask_half(sC, 0);
     settle_half(sC, pA, exp_half(sC, pA));
     if (1 < my_halves) qk_half(sB, half_base(1));

@@ -106,8 +106,9 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
   float l_run = 0.f;
 
   int ntiles_kv = (a.S + BN - 1) / BN;
+  const int coff = CAUSAL ? causal_offset(a, a.S) : 0;  // query row i sees keys up to i + coff
   if (CAUSAL) {
-    int last = q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1;
+    int last = (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1) + coff;
     int lastkv = last < a.S - 1 ? last : a.S - 1;
     ntiles_kv = lastkv / BN + 1;
   }
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
       if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BN);
     }
 
-    if (!CAUSAL || kv0 <= qw0 + 31) {  // else: the whole tile is above this wavefront's diagonal
+    if (!CAUSAL || kv0 <= qw0 + 31 + coff) {  // else: the whole tile is above this wavefront's diagonal
       const float* Ks = smem + cur * Lds::STAGE;
       const float* Vs = Ks + BN * K_PITCH;
 
@@ -176,8 +177,8 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
       for (int r = 0; r < 16; r++) s[r] = s0[r] + s1[r];
 
       // ---- mask the diagonal / ragged tile -----------------------------------------------------------------------------
-      if ((CAUSAL && kv0 + BN - 1 > qw0) || (kv0 + BN > a.S)) {
-        const int qi = qw0 + lq;
+      if ((CAUSAL && kv0 + BN - 1 > qw0 + coff) || (kv0 + BN > a.S)) {
+        const int qi = qw0 + lq + coff;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);

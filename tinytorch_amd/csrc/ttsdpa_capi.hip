@@ -16,6 +16,15 @@ bool dense_last_ok(const int64_t* st, int align) { return st[0] % align == 0 && 
 
 bool ptr_aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
+// The causal mode a call reduces to.  Bottom-right alignment with one query row hides nothing; without per-batch key
+// counts and with S <= L its offset is 0, which is the top-left aligned mask.
+int effective_causal(const ttsdpa_params* p) {
+  if (p->causal != TTSDPA_CAUSAL_BOTTOM_RIGHT) return p->causal;
+  if (p->L == 1) return TTSDPA_CAUSAL_NONE;
+  if (!p->kv_len && p->S <= p->L) return TTSDPA_CAUSAL_TOP_LEFT;
+  return TTSDPA_CAUSAL_BOTTOM_RIGHT;
+}
+
 // Validation shared by every entry point; fills the kernel argument block.
 int validate(const ttsdpa_params* p, KArgs* a) {
   if (!p) return TTSDPA_ERR_NULL;
@@ -24,6 +33,7 @@ int validate(const ttsdpa_params* p, KArgs* a) {
   if (p->B < 0 || p->Hq < 1 || p->Hkv < 1 || p->L < 0 || p->S < 0 || p->D < 1 || p->D > 256) return TTSDPA_ERR_SHAPE;
   if (p->Hq % p->Hkv != 0) return TTSDPA_ERR_SHAPE;
   if (p->mask_kind < TTSDPA_MASK_NONE || p->mask_kind > TTSDPA_MASK_ADD) return TTSDPA_ERR_MASK;
+  if (p->causal < TTSDPA_CAUSAL_NONE || p->causal > TTSDPA_CAUSAL_BOTTOM_RIGHT) return TTSDPA_ERR_MASK;
   if (p->mask_kind != TTSDPA_MASK_NONE && p->causal) return TTSDPA_ERR_MASK;  // reference FuncNNLayer.h:242
   const bool empty_out = p->B == 0 || p->L == 0;
   if (!empty_out) {
@@ -50,7 +60,8 @@ int validate(const ttsdpa_params* p, KArgs* a) {
   a->q = p->q, a->k = p->k, a->v = p->v, a->out = p->out, a->mask = p->mask;
   a->B = p->B, a->Hq = p->Hq, a->Hkv = p->Hkv, a->L = p->L, a->S = p->S, a->D = p->D;
   a->G = p->Hq / p->Hkv;
-  a->causal = p->causal ? 1 : 0;
+  a->causal = effective_causal(p) != TTSDPA_CAUSAL_NONE ? 1 : 0;
+  a->causal_br = effective_causal(p) == TTSDPA_CAUSAL_BOTTOM_RIGHT ? 1 : 0;
   a->mask_kind = p->mask_kind;
   a->scale = p->scale;
   for (int i = 0; i < 3; i++) {
@@ -91,7 +102,9 @@ bool prefill_ok(const ttsdpa_params* p) {
 }
 
 bool decode_ok(const ttsdpa_params* p) {
-  if (!fast_layout_ok(p) || (p->D != 128 && p->D != 64) || p->causal || p->S < 1 || p->L < 1) return false;
+  // a top-left aligned causal mask leaves a few keys per row: not the streaming kernel's case
+  if (!fast_layout_ok(p) || (p->D != 128 && p->D != 64) || effective_causal(p) == TTSDPA_CAUSAL_TOP_LEFT || p->S < 1 || p->L < 1)
+    return false;
   return (long long)p->L * (p->Hq / p->Hkv) <= kDecodeMaxRows;
 }
 

@@ -31,7 +31,10 @@ def _strides3(t):
     return (t.stride(0), t.stride(1), t.stride(2))
 
 
-def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=None, kvLens=None):
+_CAUSAL_ALIGN = {"top-left": _capi.CAUSAL_TOP_LEFT, "bottom-right": _capi.CAUSAL_BOTTOM_RIGHT}
+
+
+def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=None, kvLens=None, causalAlign="top-left"):
     """Fill a ttsdpa_params for 4-D tensors [B,H,N,D]."""
     B, Hq, L, D = query.shape
     Bk, Hkv, S, Dk = key.shape
@@ -49,7 +52,9 @@ def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=No
         for i in range(3):
             getattr(p, name)[i] = st[i]
     p.scale = float(scale) if scale is not None else 1.0 / math.sqrt(float(D))
-    p.causal = 1 if isCausal else 0
+    if causalAlign not in _CAUSAL_ALIGN:
+        raise ValueError("sdpAttention: causalAlign must be 'top-left' or 'bottom-right'")
+    p.causal = _CAUSAL_ALIGN[causalAlign] if isCausal else _capi.CAUSAL_NONE
     if attnMask is not None:
         if isCausal:
             raise ValueError("sdpAttention: isCausal and attnMask are exclusive")  # reference FuncNNLayer.h:242
@@ -78,11 +83,14 @@ def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=No
     return p
 
 
-def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0, scale=None, kvLens=None):
+def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0, scale=None, kvLens=None,
+                 causalAlign="top-left"):
     """out = softmax(query @ key^T * scale + bias) @ value on the GPU.
 
     query [B,Hq,L,D]; key/value [B,Hkv,S,D] with Hq a multiple of Hkv (query head h reads KV head h // (Hq//Hkv));
-    returns [B,Hq,L,D] in the dtype of query.  isCausal is top-left aligned (key j visible iff j <= i).
+    returns [B,Hq,L,D] in the dtype of query.  isCausal is top-left aligned (key j visible iff j <= i), as in the
+    reference; causalAlign="bottom-right" makes the L queries the last L positions of the keys instead (key j visible
+    iff j <= i + S_b - L with S_b = kvLens[b] or S): a prompt chunk or several new tokens against a KV cache.
     kvLens (not in the reference, which has no KV cache): int32 [B] on the device; batch b attends to the first
     kvLens[b] keys only, so key/value may be preallocated caches [B,Hkv,Smax,D] filled by kvCacheAppend.
     """
@@ -97,7 +105,7 @@ def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0,
     fix = lambda t: t if (t.stride(-1) == 1 or t.size(-1) == 1) else t.contiguous()
     query, key, value = fix(query), fix(key), fix(value)
     out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
-    p = build_params(query, key, value, out, isCausal, attnMask, scale, kvLens)
+    p = build_params(query, key, value, out, isCausal, attnMask, scale, kvLens, causalAlign)
     L = _capi.lib()
     with torch.cuda.device(query.device):
         nbytes = L.ttsdpa_workspace_bytes(ctypes.byref(p))

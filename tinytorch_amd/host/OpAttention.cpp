@@ -43,7 +43,7 @@ Tensor sdpAttentionGpuImpl(const Tensor& query, const Tensor& key, const Tensor&
   Tensor out = Tensor::empty(query.shape(), query.options().noGrad());
   p.q = query.rawPtr(), p.k = key.rawPtr(), p.v = value.rawPtr(), p.out = out.rawPtr();
   p.scale = scale;
-  p.causal = isCausal ? 1 : 0;
+  p.causal = isCausal ? TTSDPA_CAUSAL_TOP_LEFT : TTSDPA_CAUSAL_NONE;  // the reference's alignment
   if (attnMask.defined()) {
     ASSERT(attnMask.device() == query.device());
     ASSERT(attnMask.dtype() == DType::Bool || attnMask.dtype() == query.dtype());
@@ -111,7 +111,7 @@ void kvCacheAppendGpuImpl(const Tensor& kCache, const Tensor& vCache, const Tens
 }
 
 Tensor sdpAttentionCachedGpuImpl(const Tensor& query, const Tensor& kCache, const Tensor& vCache, const Tensor& kvLens,
-                                 float scale) {
+                                 bool isCausal, float scale) {
   ASSERT(query.defined() && kCache.defined() && vCache.defined() && kvLens.defined());
   ASSERT(query.dim() == 4 && kCache.dim() == 4 && kCache.shape() == vCache.shape());
   ASSERT(kCache.size(0) == query.size(0) && kCache.size(3) == query.size(3) && query.size(1) % kCache.size(1) == 0);
@@ -128,6 +128,7 @@ Tensor sdpAttentionCachedGpuImpl(const Tensor& query, const Tensor& kCache, cons
   Tensor out = Tensor::empty(query.shape(), query.options().noGrad());
   p.q = query.rawPtr(), p.k = kCache.rawPtr(), p.v = vCache.rawPtr(), p.out = out.rawPtr();
   p.scale = scale;
+  p.causal = isCausal ? TTSDPA_CAUSAL_BOTTOM_RIGHT : TTSDPA_CAUSAL_NONE;
   p.kv_len = static_cast<const int32_t*>(kvLens.rawPtr());
   const DeviceIndex dev = query.device().index;
   HIP_CHECK(hipSetDevice(dev));

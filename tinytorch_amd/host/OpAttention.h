@@ -24,11 +24,13 @@ DEFINE_OP(sdpAttention, SdpAttentionOpFn)
 // kvCacheAppend writes kNew/vNew [B,Hkv,Lnew,D] into the preallocated caches [B,Hkv,Smax,D] in place, at rows
 // positions[b] .. +Lnew-1 (positions: Int32 [B] on the device; undefined = `position` for every batch entry); rows
 // that do not fit are dropped.  sdpAttentionCached attends query [B,Hq,L,D] to the first kvLens[b] rows of the caches
-// (kvLens: Int32 [B] on the device), not causal, no mask.
+// (kvLens: Int32 [B] on the device), no mask.  isCausal here means: the L query rows are the last L positions of each
+// batch entry's kvLens[b] keys (their K/V already appended) and row i sees the keys up to its own position,
+// kvLens[b] - L + i — a chunk of a prompt, or several speculated tokens; one new token (L == 1) sees every key either way.
 using KvCacheAppendOpFn = void (*)(const Tensor& kCache, const Tensor& vCache, const Tensor& kNew, const Tensor& vNew,
                                    const Tensor& positions, int32_t position);
 using SdpAttentionCachedOpFn = Tensor (*)(const Tensor& query, const Tensor& kCache, const Tensor& vCache,
-                                          const Tensor& kvLens, float scale);
+                                          const Tensor& kvLens, bool isCausal, float scale);
 DEFINE_OP(kvCacheAppend, KvCacheAppendOpFn)
 DEFINE_OP(sdpAttentionCached, SdpAttentionCachedOpFn)
 
