@@ -232,6 +232,37 @@ static void test_kv_cache() {
       EXPECT_TRUE(vectorNear(yb, ref, 2e-2f));
     }
   }
+  // three new tokens at once: row i of the step sees the cache up to its own position (bottom-right aligned causal)
+  {
+    const int n = 3;
+    std::vector<float> kn(static_cast<size_t>(B) * Hkv * n * D), vn(kn.size());
+    for (int b = 0; b < B; b++) {
+      std::vector<float> kb = rowsOf(kall, b, lens[b], n), vb = rowsOf(vall, b, lens[b], n);
+      std::copy(kb.begin(), kb.end(), kn.begin() + static_cast<size_t>(b) * Hkv * n * D);
+      std::copy(vb.begin(), vb.end(), vn.begin() + static_cast<size_t>(b) * Hkv * n * D);
+    }
+    Tensor pos(std::vector<int>{lens[0], lens[1]}, {B}, gpuInt);
+    op::kvCacheAppend(kc, vc, Tensor(kn, {B, Hkv, n, D}, gpu), Tensor(vn, {B, Hkv, n, D}, gpu), pos, 0);
+    for (int b = 0; b < B; b++) lens[b] += n;
+    std::vector<float> q = pseudoRandom(static_cast<size_t>(B) * Hq * n * D, 40);
+    Tensor tq(q, {B, Hq, n, D}, gpu);
+    q = tq.toList<float>();
+    Tensor kvLens(std::vector<int>{lens[0], lens[1]}, {B}, gpuInt);
+    std::vector<float> y = op::sdpAttentionCached(tq, kc, vc, kvLens, true, 1.f / std::sqrt(static_cast<float>(D))).toList<float>();
+    for (int b = 0; b < B; b++)
+      for (int i = 0; i < n; i++) {
+        const int visible = lens[b] - n + i + 1;
+        std::vector<float> qi(static_cast<size_t>(Hq) * D), yi(qi.size());
+        for (int h = 0; h < Hq; h++)
+          for (int d = 0; d < D; d++) {
+            const size_t at = ((static_cast<size_t>(b) * Hq + h) * n + i) * D + d;
+            qi[static_cast<size_t>(h) * D + d] = q[at];
+            yi[static_cast<size_t>(h) * D + d] = y[at];
+          }
+        std::vector<float> ref = closedForm(qi, rowsOf(kall, b, 0, visible), rowsOf(vall, b, 0, visible), 1, Hq, Hkv, 1, visible, D, false);
+        EXPECT_TRUE(vectorNear(yi, ref, 2e-2f));
+      }
+  }
 }
 
 static void test_grad_bookkeeping_and_errors() {
