@@ -53,6 +53,14 @@ def lib():
         L.oracle_sdpa_rows_f32.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p] + [_i64] * 6 + [
             ctypes.c_int, ctypes.c_float, _c_i64p, _i64, ctypes.c_int]
         L.oracle_sdpa_rows_f32.restype = ctypes.c_int
+        L.oracle_rms_norm.argtypes = [_c_f32p, _c_f32p, _c_f32p, _i64, _i64, ctypes.c_float, ctypes.c_int]
+        L.oracle_rms_norm.restype = None
+        L.oracle_fused_add_rms_norm.argtypes = [_c_f32p, _c_f32p, _c_f32p, _i64, _i64, ctypes.c_float, ctypes.c_int]
+        L.oracle_fused_add_rms_norm.restype = None
+        L.oracle_silu_mul.argtypes = [_c_f32p, _c_f32p, _i64, _i64, ctypes.c_int]
+        L.oracle_silu_mul.restype = None
+        L.oracle_softmax.argtypes = [_c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int]
+        L.oracle_softmax.restype = None
         _lib = L
     return _lib
 
@@ -73,6 +81,14 @@ def ref():
         R.tt_ref_sdpa_f32.restype = ctypes.c_int
         R.tt_ref_sdpa_f32_gqa5d.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p] + [_i64] * 6 + [ctypes.c_int]
         R.tt_ref_sdpa_f32_gqa5d.restype = ctypes.c_int
+        R.tt_ref_rms_norm.argtypes = [_c_f32p, _c_f32p, _c_f32p, _i64, _i64, ctypes.c_float]
+        R.tt_ref_rms_norm.restype = ctypes.c_int
+        R.tt_ref_fused_add_rms_norm.argtypes = [_c_f32p, _c_f32p, _c_f32p, _i64, _i64, ctypes.c_float]
+        R.tt_ref_fused_add_rms_norm.restype = ctypes.c_int
+        R.tt_ref_silu_mul.argtypes = [_c_f32p, _c_f32p, _i64, _i64]
+        R.tt_ref_silu_mul.restype = ctypes.c_int
+        R.tt_ref_softmax.argtypes = [_c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int]
+        R.tt_ref_softmax.restype = ctypes.c_int
         _ref = R
     return _ref
 
@@ -206,4 +222,87 @@ def ref_round_trip(x, dtype):
     x = _f32(x).reshape(-1)
     out = np.empty_like(x)
     ref().tt_ref_round_trip(_p(x), _p(out), x.size, d)
+    return out
+
+
+# ---- row-wise neighbour ops (oracle/fused_oracle.c) ---------------------------------------------------------------
+
+def _dt(dtype):
+    return _DTYPES[dtype] if isinstance(dtype, str) else dtype
+
+
+def _softmax_dims(shape, dim):
+    dim = dim % len(shape)
+    outer = int(np.prod(shape[:dim], dtype=np.int64))
+    inner = int(np.prod(shape[dim + 1:], dtype=np.int64))
+    return outer, int(shape[dim]), inner
+
+
+def rms_norm(x, w=None, eps=1e-8, dtype="f32"):
+    """rmsNorm over the last axis; x holds values representable in dtype, the result is rounded to dtype."""
+    x = _f32(x)
+    w = _f32(w) if w is not None else None
+    out = np.empty_like(x)
+    dim = x.shape[-1]
+    lib().oracle_rms_norm(_p(x), _p(w) if w is not None else None, _p(out), x.size // dim, dim, eps, _dt(dtype))
+    return out
+
+
+def fused_add_rms_norm(inp, residual, w, eps, dtype="f32"):
+    """-> (input after, residual after): residual <- input + residual, input <- rmsNorm(residual) * w."""
+    a, r, w = _f32(inp).copy(), _f32(residual).copy(), _f32(w)
+    dim = a.shape[-1]
+    lib().oracle_fused_add_rms_norm(_p(a), _p(r), _p(w), a.size // dim, dim, eps, _dt(dtype))
+    return a, r
+
+
+def silu_mul(x, dtype="f32"):
+    x = _f32(x)
+    d = x.shape[-1] // 2
+    out = np.empty(x.shape[:-1] + (d,), dtype=np.float32)
+    lib().oracle_silu_mul(_p(x), _p(out), x.size // (2 * d) if d else 0, d, _dt(dtype))
+    return out
+
+
+def softmax(x, dim=-1, log=False, dtype="f32"):
+    x = _f32(x)
+    out = np.empty_like(x)
+    outer, n, inner = _softmax_dims(x.shape, dim)
+    lib().oracle_softmax(_p(x), _p(out), outer, n, inner, int(log), _dt(dtype))
+    return out
+
+
+def ref_rms_norm(x, w=None, eps=1e-8):
+    x = _f32(x)
+    w = _f32(w) if w is not None else None
+    out = np.empty_like(x)
+    dim = x.shape[-1]
+    rc = ref().tt_ref_rms_norm(_p(x), _p(w) if w is not None else None, _p(out), x.size // dim, dim, eps)
+    assert rc == 0
+    return out
+
+
+def ref_fused_add_rms_norm(inp, residual, w, eps):
+    a, r, w = _f32(inp).copy(), _f32(residual).copy(), _f32(w)
+    dim = a.shape[-1]
+    rc = ref().tt_ref_fused_add_rms_norm(_p(a), _p(r), _p(w), a.size // dim, dim, eps)
+    assert rc == 0
+    return a, r
+
+
+def ref_silu_mul(x):
+    x = _f32(x)
+    d = x.shape[-1] // 2
+    out = np.empty(x.shape[:-1] + (d,), dtype=np.float32)
+    rc = ref().tt_ref_silu_mul(_p(x), _p(out), x.size // (2 * d), d)
+    assert rc == 0
+    return out
+
+
+def ref_softmax(x, dim=-1, log=False):
+    x = _f32(x)
+    out = np.empty_like(x)
+    outer, n, inner = _softmax_dims(x.shape, dim)
+    rc = ref().tt_ref_softmax(_p(x), _p(out), outer, n, inner, int(log))
+    assert rc == 0
     return out

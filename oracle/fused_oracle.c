@@ -1,0 +1,107 @@
+/*
+ * TEST INFRASTRUCTURE — not part of the product.  Nothing under tinytorch_amd/ may call this.
+ *
+ * CPU restatement of the row-wise inference ops that sit next to attention in the reference: rmsNorm,
+ * fusedAddRmsNorm, siluMul and softmax / logSoftmax.  All tensors are fp32 arrays here; `dtype` (0 fp32, 1 fp16,
+ * 2 bf16) says where the reference rounds to its element type T: inputs are expected to hold T-representable values,
+ * intermediate stores to T tensors and the results are rounded with the same casts as the attention oracle.
+ * Arithmetic between those points is fp32 — the reference's CPU path for fp32 tensors, and its device kernels
+ * (which convert every element to float) for 16-bit tensors.
+ *
+ * Pinning:
+ *   oracle_rms_norm            reference KAT test/test_function.cpp:385-391; oracle/_ref (function::rmsNorm) bit-exact
+ *                              in fp32 on random rows
+ *   oracle_fused_add_rms_norm  no KAT in the reference; oracle/_ref (op::fusedAddRmsNorm) bit-exact in fp32; the
+ *                              identity fusedAddRmsNorm(x, r, w) == rmsNorm(x + r, w) with residual == x + r
+ *   oracle_silu_mul            reference KAT for silu test/test_function.cpp:139-143 (up = 1); oracle/_ref
+ *                              (op::siluMul) bit-exact in fp32
+ *   oracle_softmax             reference KATs test/test_function.cpp:147-176; oracle/_ref (function::softmax /
+ *                              logSoftmax, every axis) bit-exact in fp32; rows sum to 1
+ */
+#include <math.h>
+#include <stdint.h>
+
+#include "sdpa_oracle.h"
+
+static float round_t(float x, int dtype) {
+  if (dtype == 1) return oracle_f16_bits_to_f32(oracle_f32_to_f16_bits(x));
+  if (dtype == 2) return oracle_bf16_bits_to_f32(oracle_f32_to_bf16_bits(x));
+  return x;
+}
+
+/* reference src/Operation/OpNNLayerCpu.h:219-233 (normOpCpuImplDetail, RMSNorm branch): sequential sum of squares,
+ * divided by dim, invRms = 1 / sqrt(meanSquare + eps), normed = x * invRms, then *= weight when given.
+ * 16-bit: float accumulation and one rounding of the result (device kernel, src/Operation/OpNNLayerCuda.cuh:253-299). */
+void oracle_rms_norm(const float* x, const float* w, float* out, int64_t rows, int64_t dim, float eps, int dtype) {
+  for (int64_t i = 0; i < rows; i++) {
+    const float* src = x + i * dim;
+    float* dst = out + i * dim;
+    float ms = 0.f;
+    for (int64_t j = 0; j < dim; j++) ms += src[j] * src[j];
+    ms /= (float)dim;
+    const float inv = 1.f / sqrtf(ms + eps);
+    for (int64_t j = 0; j < dim; j++) {
+      float normed = src[j] * inv;
+      if (w) normed *= w[j];
+      dst[j] = round_t(normed, dtype);
+    }
+  }
+}
+
+/* reference src/Operation/OpFusedCpu.h:44-74 (fusedAddRmsNormOpCpuImpl), in place on both tensors:
+ * r = input + residual in float; residual <- T(r); sumSq += r * r (the unrounded r);
+ * invRms = 1 / sqrt(sumSq / dim + eps); input <- T(float(residual) * invRms * float(weight)). */
+void oracle_fused_add_rms_norm(float* input, float* residual, const float* w, int64_t rows, int64_t dim, float eps,
+                               int dtype) {
+  for (int64_t row = 0; row < rows; row++) {
+    float* in = input + row * dim;
+    float* res = residual + row * dim;
+    float sum_sq = 0.f;
+    for (int64_t i = 0; i < dim; i++) {
+      float r = in[i] + res[i];
+      res[i] = round_t(r, dtype);
+      sum_sq += r * r;
+    }
+    const float inv = 1.f / sqrtf(sum_sq / (float)dim + eps);
+    for (int64_t i = 0; i < dim; i++) in[i] = round_t(res[i] * inv * w[i], dtype);
+  }
+}
+
+/* reference src/Operation/OpFusedCpu.h:16-42 (siluMulOpCpuImpl): rows of 2*d elements, gate = first half, up = second
+ * half, out = silu(gate) * up with silu(a) = a / (1 + exp(-a)) (src/Operation/OpElemWiseCpu.h:123-128). */
+void oracle_silu_mul(const float* x, float* out, int64_t rows, int64_t d, int dtype) {
+  for (int64_t i = 0; i < rows; i++)
+    for (int64_t j = 0; j < d; j++) {
+      const float g = x[i * 2 * d + j], u = x[i * 2 * d + d + j];
+      const float s = g / (1.0f + expf(-g));
+      out[i * d + j] = round_t(s * u, dtype);
+    }
+}
+
+/* reference src/Operation/OpNNLayerCpu.h:16-65 (softmaxForwardCpuImpl): for every (outer, inner) column of the axis,
+ * maximum from -FLT_MAX, e = exp(x - max) stored and summed in order, then softmax: e * (float)(1.0 / sum);
+ * logSoftmax: x - max - log(sum). */
+void oracle_softmax(const float* x, float* out, int64_t outer, int64_t dim, int64_t inner, int log_form, int dtype) {
+  for (int64_t o = 0; o < outer; o++)
+    for (int64_t i = 0; i < inner; i++) {
+      const int64_t base = o * dim * inner + i;
+      float mx = -3.402823466e+38f;
+      for (int64_t d = 0; d < dim; d++) {
+        float v = x[base + d * inner];
+        if (v > mx) mx = v;
+      }
+      float sum = 0.f;
+      for (int64_t d = 0; d < dim; d++) {
+        float e = expf(x[base + d * inner] - mx);
+        out[base + d * inner] = e;
+        sum += e;
+      }
+      if (!log_form) {
+        const float inv = (float)(1.0 / (double)sum);
+        for (int64_t d = 0; d < dim; d++) out[base + d * inner] = round_t(out[base + d * inner] * inv, dtype);
+      } else {
+        const float ls = logf(sum);
+        for (int64_t d = 0; d < dim; d++) out[base + d * inner] = round_t(x[base + d * inner] - mx - ls, dtype);
+      }
+    }
+}

@@ -2,7 +2,8 @@
 //
 // C-ABI shim over the *real* TinyTorch CPU library (compiled by oracle/Makefile from the sources where they lie
 // under /root/reference; nothing of the reference is copied into this repository).  It calls
-// tinytorch::function::sdpAttention (reference src/Function/FuncNNLayer.h:298-302) on CPU fp32 tensors and hands
+// tinytorch::function::sdpAttention (reference src/Function/FuncNNLayer.h:298-302) and the row-wise neighbour ops
+// (rmsNorm, fusedAddRmsNorm, siluMul, softmax) on CPU fp32 tensors and hands
 // the result back through plain pointers, so the tests can pin oracle/sdpa_oracle.c against the reference itself
 // and write the golden fixtures under tests/golden/.
 //
@@ -106,6 +107,59 @@ int tt_ref_sdpa_f32_gqa5d(const float* q, const float* k, const float* v, float*
   Tensor y = function::sdpAttention(tq, tk, tv, causal != 0);
   auto r = y.toList<float>();
   if (static_cast<int64_t>(r.size()) != B * Hq * L * D) return -2;
+  std::memcpy(out, r.data(), sizeof(float) * r.size());
+  return 0;
+}
+
+// function::rmsNorm over the last axis of [rows, dim] (reference src/Function/FuncNNLayer.h:294); w may be NULL.
+int tt_ref_rms_norm(const float* x, const float* w, float* out, int64_t rows, int64_t dim, float eps) {
+  ensureCpu();
+  NoGradGuard guard;
+  Tensor tx = fromF32(x, {rows, dim});
+  Tensor tw;
+  if (w) tw = fromF32(w, {dim});
+  Tensor y = function::rmsNorm(tx, {dim}, tw, eps);
+  auto r = y.toList<float>();
+  if (static_cast<int64_t>(r.size()) != rows * dim) return -2;
+  std::memcpy(out, r.data(), sizeof(float) * r.size());
+  return 0;
+}
+
+// function::fusedAddRmsNorm (reference src/Function/FuncFused.h:32), in place: input and residual are overwritten.
+int tt_ref_fused_add_rms_norm(float* input, float* residual, const float* w, int64_t rows, int64_t dim, float eps) {
+  ensureCpu();
+  NoGradGuard guard;
+  Tensor ti = fromF32(input, {rows, dim});
+  Tensor tr = fromF32(residual, {rows, dim});
+  Tensor tw = fromF32(w, {dim});
+  function::fusedAddRmsNorm(ti, tr, tw, eps);
+  auto a = ti.toList<float>();
+  auto b = tr.toList<float>();
+  if (static_cast<int64_t>(a.size()) != rows * dim || a.size() != b.size()) return -2;
+  std::memcpy(input, a.data(), sizeof(float) * a.size());
+  std::memcpy(residual, b.data(), sizeof(float) * b.size());
+  return 0;
+}
+
+// function::siluMul (reference src/Function/FuncFused.h:30) on [rows, 2*d] -> [rows, d].
+int tt_ref_silu_mul(const float* x, float* out, int64_t rows, int64_t d) {
+  ensureCpu();
+  NoGradGuard guard;
+  Tensor y = function::siluMul(fromF32(x, {rows, 2 * d}));
+  auto r = y.toList<float>();
+  if (static_cast<int64_t>(r.size()) != rows * d) return -2;
+  std::memcpy(out, r.data(), sizeof(float) * r.size());
+  return 0;
+}
+
+// function::softmax / logSoftmax (reference src/Function/FuncActivation.h:91-92) along axis 1 of [outer, dim, inner].
+int tt_ref_softmax(const float* x, float* out, int64_t outer, int64_t dim, int64_t inner, int log_form) {
+  ensureCpu();
+  NoGradGuard guard;
+  Tensor tx = fromF32(x, {outer, dim, inner});
+  Tensor y = log_form ? function::logSoftmax(tx, 1) : function::softmax(tx, 1);
+  auto r = y.toList<float>();
+  if (static_cast<int64_t>(r.size()) != outer * dim * inner) return -2;
   std::memcpy(out, r.data(), sizeof(float) * r.size());
   return 0;
 }

@@ -56,6 +56,14 @@ int oracle_sdpa_rows_f32(const float* q, const float* k, const float* v, float* 
                          int64_t Hkv, int64_t L, int64_t S, int64_t D, int causal, float scale, const int64_t* rows,
                          int64_t nrows, int nthreads);
 
+/* Row-wise neighbour ops (fused_oracle.c): rmsNorm, fusedAddRmsNorm (in place), siluMul, softmax / logSoftmax over
+ * [outer, dim, inner].  dtype: 0 fp32, 1 fp16, 2 bf16 = the element type the reference would store in. */
+void oracle_rms_norm(const float* x, const float* w, float* out, int64_t rows, int64_t dim, float eps, int dtype);
+void oracle_fused_add_rms_norm(float* input, float* residual, const float* w, int64_t rows, int64_t dim, float eps,
+                               int dtype);
+void oracle_silu_mul(const float* x, float* out, int64_t rows, int64_t d, int dtype);
+void oracle_softmax(const float* x, float* out, int64_t outer, int64_t dim, int64_t inner, int log_form, int dtype);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,9 +26,9 @@ def params(*dims, **kw):
 
 
 def test_exports_match_header():
-    text = open(os.path.join(ROOT, "include", "ttsdpa.h")).read()
+    text = open(os.path.join(ROOT, "include", "ttsdpa.h")).read() + open(os.path.join(ROOT, "include", "ttfused.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    declared = sorted(set(re.findall(r"\b(ttsdpa_[a-z_]+)\s*\(", text)))
+    declared = sorted(set(re.findall(r"\b(tt(?:sdpa|fused)_[a-z_]+)\s*\(", text)))
     assert declared == sorted(_capi.EXPORTS)
     L = _capi.lib()
     for name in declared:
@@ -211,3 +211,19 @@ def test_host_wrapper_argument_errors():
         sdpAttention(q, q, q, dropoutP=0.1)
     with pytest.raises(ValueError):
         sdpAttention(q[0], q[0], q[0])
+
+
+def test_fused_ops_argument_checks_without_a_gpu():
+    """include/ttfused.h: empty problems return before any launch; bad arguments are refused the same way."""
+    L = _capi.lib()
+    assert L.ttfused_rms_norm(_capi.BF16, None, None, None, 0, 4096, 1e-6, None) == 0
+    assert L.ttfused_rms_norm(_capi.BF16, FAKE, None, None, 4, 4096, 1e-6, None) == _capi.ERR_NULL
+    assert L.ttfused_rms_norm(9, FAKE, None, FAKE, 4, 4096, 1e-6, None) == _capi.ERR_DTYPE
+    assert L.ttfused_rms_norm(_capi.F32, FAKE, None, FAKE, -4, 4096, 1e-6, None) == _capi.ERR_SHAPE
+    assert L.ttfused_rms_norm(_capi.F32, FAKE, None, FAKE, 4, 1 << 31, 1e-6, None) == _capi.ERR_SHAPE
+    assert L.ttfused_add_rms_norm(_capi.F16, FAKE, FAKE, None, 4, 128, 1e-6, None) == _capi.ERR_NULL   # weight is required
+    assert L.ttfused_add_rms_norm(_capi.F16, FAKE, FAKE, FAKE, 0, 128, 1e-6, None) == 0
+    assert L.ttfused_silu_mul(_capi.F32, FAKE, None, 4, 128, None) == _capi.ERR_NULL
+    assert L.ttfused_silu_mul(_capi.F32, None, None, 4, 0, None) == 0
+    assert L.ttfused_softmax(_capi.F32, FAKE, FAKE, 4, 8, -1, 0, None) == _capi.ERR_SHAPE
+    assert L.ttfused_softmax(_capi.F32, None, None, 4, 0, 1, 1, None) == 0

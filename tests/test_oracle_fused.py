@@ -1,0 +1,104 @@
+"""Pins oracle/fused_oracle.c (rmsNorm, fusedAddRmsNorm, siluMul, softmax / logSoftmax) before anything is checked
+against it: the reference's own known answers (reference test/test_function.cpp:139-176, 385-391), the compiled
+reference when oracle/_ref is present (bit for bit in fp32), fp64 closed forms, and identities a wrong index, a
+dropped term or a swapped half would break."""
+import numpy as np
+import pytest
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def test_reference_known_answers(oracle_mod):
+    o = oracle_mod
+    # func_rmsNorm, reference test/test_function.cpp:385-391 (default eps 1e-8, src/Function/FuncNNLayer.h:294)
+    x = np.array([[1.4176, 0.1874, 0.8367], [-0.1203, 2.5638, -1.2554]], np.float32)
+    w = np.array([1.4072, -0.4768, -0.6006], np.float32)
+    assert np.abs(o.rms_norm(x, w, 1e-8).ravel() - [2.0855, -0.0934, -0.5254, -0.1026, -0.7410, 0.4571]).max() < 1e-3
+    # func_softmax / func_logSoftmax, reference test/test_function.cpp:147-176
+    v = np.array([1.1, 1.2, 1.3, 1.6], np.float32)
+    assert np.abs(o.softmax(v, 0) - [0.2010, 0.2221, 0.2455, 0.3314]).max() < 1e-3
+    assert np.abs(o.softmax(v, 0, log=True) - [-1.6045, -1.5045, -1.4045, -1.1045]).max() < 1e-3
+    m = np.array([[1, 2], [3, 4]], np.float32)
+    assert np.abs(o.softmax(m, 0, log=True).ravel() - [-2.1269, -2.1269, -0.1269, -0.1269]).max() < 1e-3
+    assert np.abs(o.softmax(m, 1, log=True).ravel() - [-1.3133, -0.3133, -1.3133, -0.3133]).max() < 1e-3
+    # func_silu, reference test/test_function.cpp:139-143: siluMul with up == 1 is silu
+    g = np.array([-1.0, -0.5, 0.5, 1.0], np.float32)
+    assert np.abs(o.silu_mul(np.concatenate([g, np.ones(4, np.float32)])[None, :]).ravel()
+                  - [-0.2689, -0.1888, 0.3112, 0.7311]).max() < 1e-3
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 1), (3, 7), (5, 128), (2, 4096), (4, 1000)])
+def test_against_compiled_reference_bitwise(oracle_mod, rows, dim):
+    o = oracle_mod
+    if not o.have_ref():
+        pytest.skip("oracle/_ref not built")
+    r = rng(rows * 1000 + dim)
+    x = r.standard_normal((rows, dim)).astype(np.float32) * 2
+    res = r.standard_normal((rows, dim)).astype(np.float32)
+    w = r.standard_normal(dim).astype(np.float32)
+    assert np.array_equal(o.rms_norm(x, w, 1e-6), o.ref_rms_norm(x, w, 1e-6))
+    assert np.array_equal(o.rms_norm(x, None, 1e-5), o.ref_rms_norm(x, None, 1e-5))
+    a, b = o.fused_add_rms_norm(x, res, w, 1e-6)
+    ra, rb = o.ref_fused_add_rms_norm(x, res, w, 1e-6)
+    assert np.array_equal(a, ra) and np.array_equal(b, rb)
+    if dim % 2 == 0:
+        assert np.array_equal(o.silu_mul(x), o.ref_silu_mul(x))
+    for log in (False, True):
+        assert np.array_equal(o.softmax(x, -1, log), o.ref_softmax(x, -1, log))
+        assert np.array_equal(o.softmax(x, 0, log), o.ref_softmax(x, 0, log))
+    x3 = r.standard_normal((3, max(dim // 4, 1), 5)).astype(np.float32)
+    assert np.array_equal(o.softmax(x3, 1), o.ref_softmax(x3, 1))
+
+
+def test_closed_forms_and_identities(oracle_mod):
+    o = oracle_mod
+    r = rng(7)
+    x = r.standard_normal((6, 320)).astype(np.float32) * 3
+    res = r.standard_normal((6, 320)).astype(np.float32)
+    w = r.standard_normal(320).astype(np.float32)
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)
+    ref = x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + 1e-6) * w64
+    assert np.abs(o.rms_norm(x, w, 1e-6) - ref).max() < 1e-5
+    # scale invariance (eps = 0): rmsNorm(c x) == rmsNorm(x); unit mean square of the unweighted result
+    assert np.abs(o.rms_norm(4 * x, w, 0.0) - o.rms_norm(x, w, 0.0)).max() < 1e-5
+    assert np.abs((o.rms_norm(x, None, 0.0).astype(np.float64) ** 2).mean(-1) - 1).max() < 1e-5
+    # fusedAddRmsNorm(x, r, w) == rmsNorm(x + r, w), and its residual output is x + r
+    a, b = o.fused_add_rms_norm(x, res, w, 1e-6)
+    assert np.array_equal(b, x + res)
+    assert np.abs(a - o.rms_norm(x + res, w, 1e-6)).max() < 1e-5
+    # siluMul: gate is the FIRST half, up the second; against the fp64 closed form
+    g, u = x[:, :160].astype(np.float64), x[:, 160:].astype(np.float64)
+    assert np.abs(o.silu_mul(x) - g / (1 + np.exp(-g)) * u).max() < 1e-5
+    assert np.abs(o.silu_mul(x) - o.silu_mul(np.concatenate([x[:, 160:], x[:, :160]], -1))).max() > 0.1
+    # softmax: rows sum to one, shift invariance, log form is the log, an axis in the middle equals a transposed last axis
+    p = o.softmax(x, -1)
+    assert np.abs(p.sum(-1) - 1).max() < 1e-5 and (p >= 0).all()
+    assert np.abs(o.softmax(x + 5, -1) - p).max() < 1e-6
+    assert np.abs(np.exp(o.softmax(x, -1, log=True)) - p).max() < 1e-6
+    x3 = r.standard_normal((4, 9, 6)).astype(np.float32)
+    assert np.array_equal(o.softmax(x3, 1), np.swapaxes(o.softmax(np.swapaxes(x3, 1, 2).copy(), -1), 1, 2))
+    e = np.exp(x3.astype(np.float64) - x3.max(1, keepdims=True))
+    assert np.abs(o.softmax(x3, 1) - e / e.sum(1, keepdims=True)).max() < 1e-6
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_16bit_results_are_representable_and_close(oracle_mod, dtype):
+    """16-bit form: float arithmetic on the rounded inputs, every stored tensor rounded once (the reference's device
+    kernels, src/Operation/OpFusedCuda.cuh:104-127, OpNNLayerCuda.cuh:253-299)."""
+    o = oracle_mod
+    r = rng(3)
+    x, _ = o.round_to(r.standard_normal((4, 256)).astype(np.float32), dtype)
+    res, _ = o.round_to(r.standard_normal((4, 256)).astype(np.float32), dtype)
+    w, _ = o.round_to(r.standard_normal(256).astype(np.float32), dtype)
+    outs = [o.rms_norm(x, w, 1e-6, dtype), *o.fused_add_rms_norm(x, res, w, 1e-6, dtype), o.silu_mul(x, dtype),
+            o.softmax(x, -1, False, dtype)]
+    fp32 = [o.rms_norm(x, w, 1e-6), *o.fused_add_rms_norm(x, res, w, 1e-6), o.silu_mul(x), o.softmax(x, -1)]
+    ulp = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    for y, y32 in zip(outs, fp32):
+        assert np.array_equal(o.round_to(y, dtype)[0], y)              # representable
+        assert (np.abs(y - y32) <= 2 * ulp * np.abs(y32) + 1e-7).all()  # one or two roundings away from fp32
+    # the normalised row is computed from the ROUNDED residual (what the reference stores and re-reads)
+    a, b = o.fused_add_rms_norm(x, res, w, 1e-6, dtype)
+    assert np.array_equal(b, o.round_to(x + res, dtype)[0])

@@ -21,6 +21,8 @@ EXPORTS = [
     "ttsdpa_abi_version", "ttsdpa_status_string", "ttsdpa_params_init", "ttsdpa_plan", "ttsdpa_workspace_bytes",
     "ttsdpa_forward", "ttsdpa_prefill", "ttsdpa_decode", "ttsdpa_general",
     "ttsdpa_kv_append_params_init", "ttsdpa_kv_append", "ttsdpa_probe",
+    # include/ttfused.h
+    "ttfused_rms_norm", "ttfused_add_rms_norm", "ttfused_silu_mul", "ttfused_softmax",
 ]
 
 
@@ -107,6 +109,15 @@ def lib():
         L.ttsdpa_probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
                                    ctypes.POINTER(ctypes.c_double)]
         L.ttsdpa_probe.restype = ctypes.c_int
+        vp, i64 = ctypes.c_void_p, ctypes.c_int64
+        L.ttfused_rms_norm.argtypes = [ctypes.c_int, vp, vp, vp, i64, i64, ctypes.c_float, vp]
+        L.ttfused_rms_norm.restype = ctypes.c_int
+        L.ttfused_add_rms_norm.argtypes = [ctypes.c_int, vp, vp, vp, i64, i64, ctypes.c_float, vp]
+        L.ttfused_add_rms_norm.restype = ctypes.c_int
+        L.ttfused_silu_mul.argtypes = [ctypes.c_int, vp, vp, i64, i64, vp]
+        L.ttfused_silu_mul.restype = ctypes.c_int
+        L.ttfused_softmax.argtypes = [ctypes.c_int, vp, vp, i64, i64, i64, ctypes.c_int, vp]
+        L.ttfused_softmax.restype = ctypes.c_int
         if L.ttsdpa_abi_version() != 4:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L

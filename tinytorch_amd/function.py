@@ -154,3 +154,97 @@ def kvCacheAppend(kCache, vCache, kNew, vNew, positions):
         rc = L.ttsdpa_kv_append(ctypes.byref(p), torch.cuda.current_stream().cuda_stream)
     if rc != 0:
         raise RuntimeError("ttsdpa_kv_append failed: %d (%s)" % (rc, _capi.status_string(rc)))
+
+
+# ---- the row-wise ops next to attention (include/ttfused.h) ---------------------------------------------------------
+
+def _check_rowwise(name, *tensors):
+    t0 = tensors[0]
+    if t0.dtype not in _DTYPES:
+        raise TypeError("%s: dtype must be one of float32/float16/bfloat16" % name)
+    if not t0.is_cuda:
+        raise RuntimeError("tinytorch_amd.%s runs on the GPU only; got a %s tensor" % (name, t0.device))
+    for t in tensors[1:]:
+        if t is not None and (t.dtype != t0.dtype or t.device != t0.device):
+            raise TypeError("%s: all tensors must share dtype and device" % name)
+
+
+def _launch(name, fn, device, *args):
+    with torch.cuda.device(device):
+        rc = fn(*args, torch.cuda.current_stream().cuda_stream)
+    if rc != 0:
+        raise RuntimeError("%s failed: %d (%s)" % (name, rc, _capi.status_string(rc)))
+
+
+def rmsNorm(input, normalizedShape, weight=None, eps=1e-8):
+    """input / sqrt(mean(input^2) + eps) * weight over the last axis (reference src/Function/FuncNNLayer.h:294-296;
+    normalizedShape must be [input.shape[-1]] as in src/Operation/OpNNLayerCpu.h:183-184)."""
+    _check_rowwise("rmsNorm", input, weight)
+    dim = input.shape[-1]
+    if list(normalizedShape) != [dim]:
+        raise ValueError("rmsNorm: normalizedShape must be [%d]" % dim)
+    if weight is not None and tuple(weight.shape) != (dim,):
+        raise ValueError("rmsNorm: weight must have shape [%d]" % dim)
+    x = input.contiguous()
+    w = weight.contiguous() if weight is not None else None
+    out = torch.empty_like(x)
+    rows = x.numel() // dim if dim else 0
+    _launch("ttfused_rms_norm", _capi.lib().ttfused_rms_norm, x.device, _DTYPES[x.dtype], x.data_ptr(),
+            w.data_ptr() if w is not None else None, out.data_ptr(), rows, dim, float(eps))
+    return out
+
+
+def fusedAddRmsNorm(input, residual, weight, eps):
+    """In place: residual += input; input = rmsNorm(residual) * weight (reference src/Function/FuncFused.h:32-34)."""
+    _check_rowwise("fusedAddRmsNorm", input, residual, weight)
+    if input.shape != residual.shape or not input.is_contiguous() or not residual.is_contiguous():
+        raise ValueError("fusedAddRmsNorm: input and residual must be contiguous tensors of one shape")
+    dim = input.shape[-1]
+    if tuple(weight.shape) != (dim,):
+        raise ValueError("fusedAddRmsNorm: weight must have shape [%d]" % dim)
+    w = weight.contiguous()
+    rows = input.numel() // dim if dim else 0
+    _launch("ttfused_add_rms_norm", _capi.lib().ttfused_add_rms_norm, input.device, _DTYPES[input.dtype],
+            input.data_ptr(), residual.data_ptr(), w.data_ptr(), rows, dim, float(eps))
+
+
+def siluMul(x):
+    """silu(x[..., :d]) * x[..., d:] with d = x.shape[-1] / 2 (reference src/Function/FuncFused.h:30)."""
+    _check_rowwise("siluMul", x)
+    if x.shape[-1] % 2 != 0:
+        raise ValueError("siluMul: the last axis must be even")  # reference ASSERT, src/Operation/OpFusedCpu.h:17
+    x = x.contiguous()
+    d = x.shape[-1] // 2
+    out = torch.empty(x.shape[:-1] + (d,), dtype=x.dtype, device=x.device)
+    rows = x.numel() // (2 * d) if d else 0
+    _launch("ttfused_silu_mul", _capi.lib().ttfused_silu_mul, x.device, _DTYPES[x.dtype], x.data_ptr(), out.data_ptr(),
+            rows, d)
+    return out
+
+
+def _softmax(name, x, dim, log):
+    _check_rowwise(name, x)
+    if x.dim() == 0:
+        raise ValueError("%s: expected at least one axis" % name)
+    dim = dim % x.dim()
+    x = x.contiguous()
+    out = torch.empty_like(x)
+    outer = 1
+    for n in x.shape[:dim]:
+        outer *= n
+    inner = 1
+    for n in x.shape[dim + 1:]:
+        inner *= n
+    _launch("ttfused_softmax", _capi.lib().ttfused_softmax, x.device, _DTYPES[x.dtype], x.data_ptr(), out.data_ptr(),
+            outer, x.shape[dim], inner, int(log))
+    return out
+
+
+def softmax(x, dim=-1):
+    """softmax along `dim` (reference src/Function/FuncActivation.h:91)."""
+    return _softmax("softmax", x, dim, False)
+
+
+def logSoftmax(x, dim=-1):
+    """logSoftmax along `dim` (reference src/Function/FuncActivation.h:92)."""
+    return _softmax("logSoftmax", x, dim, True)
