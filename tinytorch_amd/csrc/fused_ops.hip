@@ -55,10 +55,11 @@ __device__ __forceinline__ typename Pack<T, VEC>::type load_plain(const T* p) {
 template <typename T, int VEC>
 __device__ __forceinline__ void store_pack(T* p, const typename Pack<T, VEC>::type& v) {
   typedef typename Pack<T, VEC>::type V;
+  // written once, not read again here: keep it from displacing the cached input
   if constexpr (VEC == 1) {
-    *p = v.x;
+    __builtin_nontemporal_store(v.x, p);
   } else {
-    *(V*)p = v;
+    __builtin_nontemporal_store(v, (V*)p);
   }
 }
 
@@ -86,13 +87,27 @@ __device__ __forceinline__ float row_reduce(float v, float* lds, int slot) {
   return v;
 }
 
+// Walk the part of a row that a lane does not keep in registers (vectors lr + CACHE*LPR, + LPR, ...), four loads in
+// flight: `load(i)` fetches vector i, `use(i, v)` consumes it.
+template <int LPR, typename Load, typename Use>
+__device__ __forceinline__ void walk_rest(int lr, int nvec, Load load, Use use) {
+  for (int i0 = lr + CACHE * LPR; i0 < nvec; i0 += 4 * LPR) {
+    decltype(load(0)) v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (i0 + u * LPR < nvec) v[u] = load(i0 + u * LPR);
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (i0 + u * LPR < nvec) use(i0 + u * LPR, v[u]);
+  }
+}
+
 // ---- rmsNorm and fusedAddRmsNorm ---------------------------------------------------------------------------------
 // FUSED: r = input + residual, residual <- T(r), sum of squares over the unrounded r, input <- T(float(T(r)) * inv * w).
 // else:  out <- T(x * inv [* w]).
 template <typename T, int VEC, int LPR, bool FUSED>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const T* x, T* res, const T* __restrict__ w, T* out,  // out may be x
-                                                       long long rows,
-                                                       int dim, float eps) {
+                                                       long long rows, int dim, float eps) {
   typedef typename Pack<T, VEC>::type V;
   __shared__ float lds[8];
   constexpr int RPB = 256 / LPR;
@@ -106,13 +121,23 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const T* x, T* res, const
 
   V keep[CACHE];
   float ss = 0.f;
-  auto take = [&](int i) __attribute__((always_inline)) {
-    V a = load_stream<T, VEC>(xr + (long long)i * VEC);
+  // input vector i (FUSED: both operands, packed side by side)
+  struct In {
+    V a, b;
+  };
+  auto fetch = [&](int i) __attribute__((always_inline)) {
+    In v;
+    v.a = load_stream<T, VEC>(xr + (long long)i * VEC);
+    if constexpr (FUSED) v.b = load_stream<T, VEC>(rr + (long long)i * VEC);
+    return v;
+  };
+  // -> the vector the second phase normalises; adds its squares to ss
+  auto absorb = [&](int i, const In& v) __attribute__((always_inline)) {
+    V a = v.a;
     if constexpr (FUSED) {
-      V b = load_stream<T, VEC>(rr + (long long)i * VEC);
 #pragma unroll
       for (int e = 0; e < VEC; e++) {
-        float r = (float)a[e] + (float)b[e];
+        float r = (float)v.a[e] + (float)v.b[e];
         a[e] = (T)r;
         ss = fmaf(r, r, ss);
       }
@@ -124,12 +149,14 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const T* x, T* res, const
     return a;
   };
   if (live) {
+    In first[CACHE];
 #pragma unroll
-    for (int c = 0; c < CACHE; c++) {
-      int i = lr + c * LPR;
-      if (i < nvec) keep[c] = take(i);
-    }
-    for (int i = lr + CACHE * LPR; i < nvec; i += LPR) take(i);
+    for (int c = 0; c < CACHE; c++)
+      if (lr + c * LPR < nvec) first[c] = fetch(lr + c * LPR);
+#pragma unroll
+    for (int c = 0; c < CACHE; c++)
+      if (lr + c * LPR < nvec) keep[c] = absorb(lr + c * LPR, first[c]);
+    walk_rest<LPR>(lr, nvec, fetch, [&](int i, const In& v) __attribute__((always_inline)) { absorb(i, v); });
   }
   ss = row_reduce<LPR, SumOp>(ss, lds, 0);
   const float inv = 1.f / sqrtf(ss / (float)dim + eps);
@@ -147,15 +174,18 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const T* x, T* res, const
     store_pack<T, VEC>(orow + (long long)i * VEC, o);
   };
 #pragma unroll
-  for (int c = 0; c < CACHE; c++) {
-    int i = lr + c * LPR;
-    if (i < nvec) give(i, keep[c]);
-  }
-  for (int i = lr + CACHE * LPR; i < nvec; i += LPR)  // the part of a very long row that was not kept
-    give(i, load_plain<T, VEC>((FUSED ? rr : xr) + (long long)i * VEC));
+  for (int c = 0; c < CACHE; c++)
+    if (lr + c * LPR < nvec) give(lr + c * LPR, keep[c]);
+  // the part of a very long row that was not kept is read again (FUSED: the residual just stored)
+  walk_rest<LPR>(
+      lr, nvec, [&](int i) __attribute__((always_inline)) { return load_plain<T, VEC>((FUSED ? rr : xr) + (long long)i * VEC); },
+      give);
 }
 
 // ---- softmax / logSoftmax over the last axis ---------------------------------------------------------------------------
+// One reading pass: every lane keeps a running maximum and the sum of exponentials relative to it (rescaled when the
+// maximum grows), the lanes' pairs are merged after the row maximum is known, then the row is written from the
+// registers (and from a second read for the part of a very long row that was not kept).
 template <typename T, int VEC, int LPR, bool LOG>
 __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* out, long long rows, int dim) {  // out may be x
   typedef typename Pack<T, VEC>::type V;
@@ -170,40 +200,28 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* out, l
 
   V keep[CACHE];
   float mx = -3.402823466e+38f;  // the reference starts from the lowest finite float
-  if (live) {
-#pragma unroll
-    for (int c = 0; c < CACHE; c++) {
-      int i = lr + c * LPR;
-      if (i < nvec) {
-        keep[c] = load_stream<T, VEC>(xr + (long long)i * VEC);
-#pragma unroll
-        for (int e = 0; e < VEC; e++) mx = fmaxf(mx, (float)keep[c][e]);
-      }
-    }
-    for (int i = lr + CACHE * LPR; i < nvec; i += LPR) {
-      V a = load_plain<T, VEC>(xr + (long long)i * VEC);
-#pragma unroll
-      for (int e = 0; e < VEC; e++) mx = fmaxf(mx, (float)a[e]);
-    }
-  }
-  mx = row_reduce<LPR, MaxOp>(mx, lds, 0);
   float sum = 0.f;
+  auto absorb = [&](int, const V& a) __attribute__((always_inline)) {
+    float vm = (float)a[0];
+#pragma unroll
+    for (int e = 1; e < VEC; e++) vm = fmaxf(vm, (float)a[e]);
+    const float mn = fmaxf(mx, vm);
+    sum *= __expf(mx - mn);
+#pragma unroll
+    for (int e = 0; e < VEC; e++) sum += __expf((float)a[e] - mn);
+    mx = mn;
+  };
   if (live) {
 #pragma unroll
-    for (int c = 0; c < CACHE; c++) {
-      int i = lr + c * LPR;
-      if (i < nvec) {
+    for (int c = 0; c < CACHE; c++)
+      if (lr + c * LPR < nvec) keep[c] = load_stream<T, VEC>(xr + (long long)(lr + c * LPR) * VEC);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) sum += __expf((float)keep[c][e] - mx);
-      }
-    }
-    for (int i = lr + CACHE * LPR; i < nvec; i += LPR) {
-      V a = load_plain<T, VEC>(xr + (long long)i * VEC);
-#pragma unroll
-      for (int e = 0; e < VEC; e++) sum += __expf((float)a[e] - mx);
-    }
+    for (int c = 0; c < CACHE; c++)
+      if (lr + c * LPR < nvec) absorb(0, keep[c]);
+    walk_rest<LPR>(lr, nvec, [&](int i) __attribute__((always_inline)) { return load_plain<T, VEC>(xr + (long long)i * VEC); }, absorb);
   }
-  sum = row_reduce<LPR, SumOp>(sum, lds, 1);
+  const float rmax = row_reduce<LPR, MaxOp>(mx, lds, 0);
+  sum = row_reduce<LPR, SumOp>(sum * __expf(mx - rmax), lds, 1);
   if (!live) return;
   const float inv = 1.f / sum;
   const float lsum = LOG ? __logf(sum) : 0.f;
@@ -211,60 +229,110 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* out, l
     V o;
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
-      float v = (float)a[e] - mx;
+      float v = (float)a[e] - rmax;
       o[e] = (T)(LOG ? v - lsum : __expf(v) * inv);
     }
     store_pack<T, VEC>(orow + (long long)i * VEC, o);
   };
 #pragma unroll
-  for (int c = 0; c < CACHE; c++) {
-    int i = lr + c * LPR;
-    if (i < nvec) give(i, keep[c]);
-  }
-  for (int i = lr + CACHE * LPR; i < nvec; i += LPR) give(i, load_plain<T, VEC>(xr + (long long)i * VEC));
+  for (int c = 0; c < CACHE; c++)
+    if (lr + c * LPR < nvec) give(lr + c * LPR, keep[c]);
+  walk_rest<LPR>(lr, nvec, [&](int i) __attribute__((always_inline)) { return load_plain<T, VEC>(xr + (long long)i * VEC); }, give);
 }
 
-// ---- softmax / logSoftmax over an inner axis: one lane per (outer, inner) column, lanes along the contiguous axis --------
-template <typename T, bool LOG>
+// ---- softmax / logSoftmax over an inner axis: a lane owns VEC neighbouring (outer, inner) columns, lanes run along the
+// contiguous axis, four steps of the softmax axis are in flight ----------------------------------------------------------------
+template <typename T, int VEC, bool LOG>
 __global__ __launch_bounds__(256) void softmax_strided_kernel(const T* x, T* out, long long outer, int dim,  // out may be x
                                                               long long inner) {
-  const long long col = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (col >= outer * inner) return;
-  const long long base = (col / inner) * dim * inner + col % inner;
-  float mx = -3.402823466e+38f, sum = 0.f;
-  for (int d = 0; d < dim; d++) {  // one pass: running maximum and rescaled sum
-    float v = (float)x[base + d * inner];
-    float mn = fmaxf(mx, v);
-    sum = sum * __expf(mx - mn) + __expf(v - mn);
-    mx = mn;
+  typedef typename Pack<T, VEC>::type V;
+  const long long ivec = inner / VEC;  // column groups per outer index
+  const long long cg = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (cg >= outer * ivec) return;
+  const long long base = (cg / ivec) * dim * inner + (cg % ivec) * VEC;
+  float mx[VEC], sum[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; e++) mx[e] = -3.402823466e+38f, sum[e] = 0.f;
+  for (int d0 = 0; d0 < dim; d0 += 4) {  // running maximum and rescaled sum per column
+    V v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (d0 + u < dim) v[u] = load_plain<T, VEC>(x + base + (d0 + u) * inner);
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      float mn = mx[e];
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        if (d0 + u < dim) mn = fmaxf(mn, (float)v[u][e]);
+      float acc = sum[e] * __expf(mx[e] - mn);
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        if (d0 + u < dim) acc += __expf((float)v[u][e] - mn);
+      sum[e] = acc, mx[e] = mn;
+    }
   }
-  const float inv = 1.f / sum;
-  const float lsum = LOG ? __logf(sum) : 0.f;
-  for (int d = 0; d < dim; d++) {
-    float v = (float)x[base + d * inner] - mx;
-    out[base + d * inner] = (T)(LOG ? v - lsum : __expf(v) * inv);
+  float inv[VEC], lsum[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; e++) inv[e] = 1.f / sum[e], lsum[e] = LOG ? __logf(sum[e]) : 0.f;
+  for (int d0 = 0; d0 < dim; d0 += 4) {
+    V v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (d0 + u < dim) v[u] = load_plain<T, VEC>(x + base + (d0 + u) * inner);
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (d0 + u < dim) {
+        V o;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+          float t = (float)v[u][e] - mx[e];
+          o[e] = (T)(LOG ? t - lsum[e] : __expf(t) * inv[e]);
+        }
+        store_pack<T, VEC>(out + base + (d0 + u) * inner, o);
+      }
   }
 }
 
 // ---- siluMul --------------------------------------------------------------------------------------------------------------
+// A workgroup is 2^txshift lanes along the row by 256 >> txshift rows and takes UNR consecutive row groups of one
+// column chunk; workgroups are numbered with the chunk running fastest, so the launch walks memory front to back and
+// no lane divides.
+constexpr int kSiluUnroll = 4;
+
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ out, long long rows, int d) {
+__global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ out, long long rows, int d,
+                                                       int txshift, unsigned nchunk) {
   typedef typename Pack<T, VEC>::type V;
+  constexpr int UNR = kSiluUnroll;
   const int vpr = d / VEC;  // vectors per output row
-  const long long total = rows * vpr;
-  for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256) {
-    const long long row = idx / vpr;
-    const int col = (int)(idx % vpr) * VEC;
-    const T* g = x + row * 2 * d + col;
-    V gv = load_stream<T, VEC>(g);
-    V uv = load_stream<T, VEC>(g + d);
-    V o;
+  const int tx = threadIdx.x & ((1 << txshift) - 1), ty = threadIdx.x >> txshift;
+  const unsigned chunk = blockIdx.x % nchunk, group = blockIdx.x / nchunk;
+  const int col = (int)(chunk << txshift) + tx;
+  if (col >= vpr) return;
+  const int rpb = 256 >> txshift;
+  const long long row0 = (long long)group * UNR * rpb + ty;
+  V gv[UNR], uv[UNR];
 #pragma unroll
-    for (int e = 0; e < VEC; e++) {
-      float gf = (float)gv[e];
-      o[e] = (T)(gf / (1.f + __expf(-gf)) * (float)uv[e]);
+  for (int u = 0; u < UNR; u++) {
+    const long long row = row0 + u * rpb;
+    if (row < rows) {
+      const T* g = x + row * 2 * d + (long long)col * VEC;
+      gv[u] = load_stream<T, VEC>(g);
+      uv[u] = load_stream<T, VEC>(g + d);
     }
-    store_pack<T, VEC>(out + row * d + col, o);
+  }
+#pragma unroll
+  for (int u = 0; u < UNR; u++) {
+    const long long row = row0 + u * rpb;
+    if (row < rows) {
+      V o;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        float gf = (float)gv[u][e];
+        o[e] = (T)(gf / (1.f + __expf(-gf)) * (float)uv[u][e]);
+      }
+      store_pack<T, VEC>(out + row * d + (long long)col * VEC, o);
+    }
   }
 }
 
@@ -341,12 +409,18 @@ int softmax_dispatch(const void* x, void* out, long long outer, int dim, long lo
     if (log_form) return vec ? launch_softmax_rows<T, VEC, true>(x, out, outer, dim, s) : launch_softmax_rows<T, 1, true>(x, out, outer, dim, s);
     return vec ? launch_softmax_rows<T, VEC, false>(x, out, outer, dim, s) : launch_softmax_rows<T, 1, false>(x, out, outer, dim, s);
   }
-  const long long cols = outer * inner;
-  const unsigned grid = (unsigned)((cols + 255) / 256);
-  if (log_form)
-    hipLaunchKernelGGL((softmax_strided_kernel<T, true>), dim3(grid), dim3(256), 0, s, (const T*)x, (T*)out, outer, dim, inner);
-  else
-    hipLaunchKernelGGL((softmax_strided_kernel<T, false>), dim3(grid), dim3(256), 0, s, (const T*)x, (T*)out, outer, dim, inner);
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const bool vec = inner % VEC == 0 && aligned16(x) && aligned16(out);
+  const long long groups = outer * (vec ? inner / VEC : inner);
+  const unsigned grid = (unsigned)((groups + 255) / 256);
+#define TT_SMS(V_, LOG_) \
+  hipLaunchKernelGGL((softmax_strided_kernel<T, V_, LOG_>), dim3(grid), dim3(256), 0, s, (const T*)x, (T*)out, outer, dim, inner)
+  if (vec) {
+    if (log_form) TT_SMS(VEC, true); else TT_SMS(VEC, false);
+  } else {
+    if (log_form) TT_SMS(1, true); else TT_SMS(1, false);
+  }
+#undef TT_SMS
   return (int)hipGetLastError();
 }
 
@@ -354,14 +428,17 @@ template <typename T>
 int silu_dispatch(const void* x, void* out, long long rows, int d, hipStream_t s) {
   constexpr int VEC = 16 / (int)sizeof(T);
   const bool vec = d % VEC == 0 && aligned16(x) && aligned16(out);
-  const long long total = rows * (vec ? d / VEC : d);
-  long long blocks = (total + 255) / 256;
-  const long long cap = 256LL * 32;  // grid-stride beyond 32 workgroups per CU
-  if (blocks > cap) blocks = cap;
+  const int vpr = vec ? d / VEC : d;
+  int txshift = 0;
+  while (txshift < 8 && (1 << txshift) < vpr) txshift++;
+  const long long rows_per_wg = (long long)(256 >> txshift) * kSiluUnroll;
+  const unsigned nchunk = (unsigned)((vpr + (1 << txshift) - 1) >> txshift);
+  const long long blocks = (rows + rows_per_wg - 1) / rows_per_wg * nchunk;
+  if (!grid_ok(blocks)) return TTSDPA_ERR_SHAPE;
   if (vec)
-    hipLaunchKernelGGL((silu_mul_kernel<T, VEC>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)x, (T*)out, rows, d);
+    hipLaunchKernelGGL((silu_mul_kernel<T, VEC>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)x, (T*)out, rows, d, txshift, nchunk);
   else
-    hipLaunchKernelGGL((silu_mul_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)x, (T*)out, rows, d);
+    hipLaunchKernelGGL((silu_mul_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)x, (T*)out, rows, d, txshift, nchunk);
   return (int)hipGetLastError();
 }
 
