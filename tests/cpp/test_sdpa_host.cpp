@@ -3,6 +3,7 @@
 // test/test.h:17-30) with the tensors on the accelerator; the others cover what the drop-in adds or must keep:
 // fp16/bf16 dispatch, grouped-query heads, a decode-shaped call, grad bookkeeping of Function::apply, and the loud
 // failure when a CPU tensor reaches an op that has no CPU slot.
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -309,6 +310,77 @@ static void test_grad_bookkeeping_and_errors() {
   EXPECT_TRUE(deviceAllocatorLiveBytes(0) == live0);
 }
 
+// The reference's own vectors for the row-wise ops (reference test/test_function.cpp:139-152, 385-391) and fp64 closed
+// forms on longer rows, through function:: on the GPU.
+static void test_row_wise_ops() {
+  std::printf("row-wise ops: rmsNorm, fusedAddRmsNorm, siluMul, softmax, logSoftmax\n");
+  const Options gpu = options::device(DeviceType::GPU);
+  {
+    Tensor input(std::vector<float>{1.4176f, 0.1874f, 0.8367f, -0.1203f, 2.5638f, -1.2554f}, {2, 3}, gpu);
+    Tensor w(std::vector<float>{1.4072f, -0.4768f, -0.6006f}, {3}, gpu);
+    Tensor y = function::rmsNorm(input, {3}, w);
+    EXPECT_TRUE(y.shape() == input.shape());
+    EXPECT_TRUE(vectorNear(y.toList<float>(), {2.0855f, -0.0934f, -0.5254f, -0.1026f, -0.7410f, 0.4571f}));
+    Tensor v(std::vector<float>{1.1f, 1.2f, 1.3f, 1.6f}, {4}, gpu);
+    EXPECT_TRUE(vectorNear(function::softmax(v, 0).toList<float>(), {0.2010f, 0.2221f, 0.2455f, 0.3314f}));
+    EXPECT_TRUE(vectorNear(function::logSoftmax(v, 0).toList<float>(), {-1.6045f, -1.5045f, -1.4045f, -1.1045f}));
+    Tensor m(std::vector<float>{1.f, 2.f, 3.f, 4.f}, {2, 2}, gpu);
+    EXPECT_TRUE(vectorNear(function::logSoftmax(m, 0).toList<float>(), {-2.1269f, -2.1269f, -0.1269f, -0.1269f}));
+    EXPECT_TRUE(vectorNear(function::logSoftmax(m, 1).toList<float>(), {-1.3133f, -0.3133f, -1.3133f, -0.3133f}));
+    // silu(x) * 1 with the reference's silu vector
+    Tensor g(std::vector<float>{-1.f, -0.5f, 0.5f, 1.f, 1.f, 1.f, 1.f, 1.f}, {1, 8}, gpu);
+    EXPECT_TRUE(vectorNear(function::siluMul(g).toList<float>(), {-0.2689f, -0.1888f, 0.3112f, 0.7311f}));
+  }
+  for (DType dt : {DType::Float32, DType::BFloat16, DType::Float16}) {
+    const Options o = options::device(DeviceType::GPU).dtype(dt);
+    const float tol = dt == DType::Float32 ? 1e-4f : 3e-2f;
+    const int rows = 5, dim = 1024;
+    Tensor x(pseudoRandom(static_cast<size_t>(rows) * dim, 51), {rows, dim}, o);
+    Tensor r(pseudoRandom(static_cast<size_t>(rows) * dim, 52), {rows, dim}, o);
+    Tensor w(pseudoRandom(dim, 53), {dim}, o);
+    const std::vector<float> xs = x.toList<float>(), rs = r.toList<float>(), ws = w.toList<float>();
+    std::vector<float> sum(xs.size()), normed(xs.size()), gated(static_cast<size_t>(rows) * dim / 2), probs(xs.size());
+    for (int i = 0; i < rows; i++) {
+      double ss = 0, mx = -1e30, den = 0;
+      for (int j = 0; j < dim; j++) {
+        sum[i * dim + j] = xs[i * dim + j] + rs[i * dim + j];
+        ss += static_cast<double>(sum[i * dim + j]) * sum[i * dim + j];
+        mx = std::max(mx, static_cast<double>(xs[i * dim + j]));
+      }
+      const double inv = 1.0 / std::sqrt(ss / dim + 1e-6);
+      for (int j = 0; j < dim; j++) {
+        normed[i * dim + j] = static_cast<float>(sum[i * dim + j] * inv * ws[j]);
+        den += std::exp(xs[i * dim + j] - mx);
+      }
+      for (int j = 0; j < dim; j++) probs[i * dim + j] = static_cast<float>(std::exp(xs[i * dim + j] - mx) / den);
+      for (int j = 0; j < dim / 2; j++) {
+        const double gt = xs[i * dim + j];
+        gated[i * (dim / 2) + j] = static_cast<float>(gt / (1.0 + std::exp(-gt)) * xs[i * dim + dim / 2 + j]);
+      }
+    }
+    EXPECT_TRUE(vectorNear(function::softmax(x, -1).toList<float>(), probs, tol));
+    Tensor sg = function::siluMul(x);
+    EXPECT_TRUE(sg.size(-1) == dim / 2 && vectorNear(sg.toList<float>(), gated, tol));
+    Tensor xin = x.clone(), res = r.clone();
+    function::fusedAddRmsNorm(xin, res, w, 1e-6f);
+    EXPECT_TRUE(vectorNear(res.toList<float>(), sum, tol));
+    EXPECT_TRUE(vectorNear(xin.toList<float>(), normed, 2 * tol));
+    // rmsNorm of the summed rows gives the same normalised rows; no weight = weight of ones
+    Tensor rn = function::rmsNorm(res, {dim}, w, 1e-6f);
+    EXPECT_TRUE(vectorNear(rn.toList<float>(), xin.toList<float>(), 2 * tol));
+    Tensor ones = Tensor::ones({dim}, o);
+    EXPECT_TRUE(vectorNear(function::rmsNorm(x, {dim}, Tensor{}, 1e-6f).toList<float>(),
+                           function::rmsNorm(x, {dim}, ones, 1e-6f).toList<float>(), 1e-6f));
+  }
+  // failed preconditions are loud, like the reference's ASSERTs
+  AssertHandler old = setAssertHandler(countingAssertHandler);
+  int before = g_asserts;
+  Tensor odd = function::siluMul(Tensor::ones({2, 3}, gpu));            // odd last axis
+  Tensor bad = function::rmsNorm(Tensor::ones({2, 4}, gpu), {2, 4}, Tensor{});  // normalizedShape must be the last axis
+  EXPECT_TRUE(g_asserts >= before + 2 && !odd.defined() && !bad.defined());
+  setAssertHandler(old);
+}
+
 int main() {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
@@ -319,6 +391,7 @@ int main() {
   test_half_dtypes_and_gqa();
   test_broadcast_masks();
   test_kv_cache();
+  test_row_wise_ops();
   test_grad_bookkeeping_and_errors();
   std::printf(g_failures == 0 ? "ALL PASSED\n" : "%d FAILURES\n", g_failures);
   return g_failures == 0 ? 0 : 1;

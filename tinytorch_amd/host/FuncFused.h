@@ -1,0 +1,68 @@
+// function::siluMul / fusedAddRmsNorm / rmsNorm / softmax / logSoftmax with the reference's signatures and defaults
+// (src/Function/FuncFused.h:14-34, src/Function/FuncNNLayer.h:219-227,294-296, src/Function/FuncActivation.h:42-92).
+// Forward only: the reference's backward of siluMul, fusedAddRmsNorm and rmsNorm is NOT_IMPLEMENTED as well; the
+// softmax backward of the reference is not part of this inference path and fails the same loud way here.
+#pragma once
+
+#include <vector>
+
+#include "Function.h"
+#include "OpFused.h"
+
+namespace tinytorch::function {
+
+class FuncSiluMul : public Function<FuncSiluMul> {
+ public:
+  static Tensor forward(AutogradContext* ctx, const Tensor& x) {
+    (void)ctx;
+    return op::siluMul(x);
+  }
+  static void backward(AutogradContext* ctx, const Tensor& grad) {
+    (void)ctx, (void)grad;
+    NOT_IMPLEMENTED();
+  }
+};
+
+class FuncRMSNorm : public Function<FuncRMSNorm> {
+ public:
+  static Tensor forward(AutogradContext* ctx, const Tensor& input, const std::vector<int64_t>& normalizedShape,
+                        const Tensor& weight, float eps) {
+    (void)ctx;
+    return op::rmsNorm(input, normalizedShape, weight, eps);
+  }
+  static void backward(AutogradContext* ctx, const Tensor& grad) {
+    (void)ctx, (void)grad;
+    NOT_IMPLEMENTED();
+  }
+};
+
+template <bool LOG>
+class FuncSoftmaxT : public Function<FuncSoftmaxT<LOG>> {
+ public:
+  static Tensor forward(AutogradContext* ctx, const Tensor& self, int64_t dim) {
+    (void)ctx;
+    return LOG ? op::logSoftmax(self, dim) : op::softmax(self, dim);
+  }
+  static void backward(AutogradContext* ctx, const Tensor& grad) {
+    (void)ctx, (void)grad;
+    NOT_IMPLEMENTED();
+  }
+};
+
+inline Tensor siluMul(const Tensor& x) { return FuncSiluMul::apply(x); }
+
+// In place on input and residual; no autograd node (the reference's wrapper has none to offer either: its backward is
+// NOT_IMPLEMENTED, src/Function/FuncFused.h:27).
+inline void fusedAddRmsNorm(Tensor& input, Tensor& residual, const Tensor& weight, float eps) {
+  op::fusedAddRmsNorm(input, residual, weight, eps);
+}
+
+inline Tensor rmsNorm(const Tensor& input, const std::vector<int64_t>& normalizedShape, const Tensor& weight,
+                      float eps = 1e-8f) {
+  return FuncRMSNorm::apply(input, normalizedShape, weight, eps);
+}
+
+inline Tensor softmax(const Tensor& self, int64_t dim = -1) { return FuncSoftmaxT<false>::apply(self, dim); }
+inline Tensor logSoftmax(const Tensor& self, int64_t dim = -1) { return FuncSoftmaxT<true>::apply(self, dim); }
+
+}  // namespace tinytorch::function
