@@ -7,7 +7,8 @@ A step is one call of the hot path (ttsdpa_forward through the C ABI) over one b
 resident in HBM.  The headline workload is BASELINE.json's configs[2] (bf16 causal GQA prefill, B2 32q/8kv S4096
 D128: the shape the prefill target is quoted on); the decode workload configs[3] (bf16, B64 32q/8kv KV 8192) is
 measured in the same run and reported under "secondary", and config 3's shape in fp32 (the reference's default dtype,
-on the fp32 MFMA kernel, against the 157.3 TFLOP/s fp32 peak) under "fp32".  One JSON line is printed.
+on the fp32 MFMA kernel, against the 157.3 TFLOP/s fp32 peak) under "fp32", and the row-wise neighbour ops (rmsNorm,
+fusedAddRmsNorm, siluMul, softmax; HBM-bound) under "fused_ops".  One JSON line is printed.
 
 Algorithmic work per launch (what "achieved" divides by the measured launch time):
   prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)
@@ -157,6 +158,105 @@ def run_probes():
             "note": "sustained by ttsdpa_probe kernels in this run: bf16 32x32x16 MFMA loop, 1 GiB streaming reads"}
 
 
+FUSED_WORKLOADS = {
+    # name: (op, rows, dim) — bf16, sized well beyond the 256 MB last-level cache so that the figure is HBM traffic
+    "rms_norm": ("rms_norm", 65536, 4096),            # [B16 x S4096 tokens, hidden 4096]
+    "fused_add_rms_norm": ("add_rms_norm", 65536, 4096),
+    "silu_mul": ("silu_mul", 32768, 14336),           # gate/up rows of 2 x 14336
+    "softmax": ("softmax", 8192, 32000),              # logits rows
+}
+
+
+def run_fused(name, steps, warmup, cpu=True):
+    """One row-wise neighbour op (include/ttfused.h) on bf16 rows resident in HBM: algorithmic bytes per launch / HIP-event
+    time per launch against the 8 TB/s HBM peak, with the compiled reference (one core) on the first rows beside it.
+    Algorithmic bytes: rms_norm and softmax read and write every element once (2 n e), fused_add_rms_norm reads and
+    writes two tensors (4 n e), silu_mul reads two halves and writes one (3 n e); e = 2 bytes."""
+    import numpy as np
+    import torch
+    from tinytorch_amd import _capi
+
+    op, rows, dim = FUSED_WORKLOADS[name]
+    lib = _capi.lib()
+    stream = torch.cuda.current_stream()
+    st = stream.cuda_stream
+    gen = torch.Generator(device="cuda").manual_seed(0x5EED)
+    cols = 2 * dim if op == "silu_mul" else dim
+    x = torch.randn(rows, cols, device="cuda", generator=gen).bfloat16()
+    w = torch.randn(dim, device="cuda", generator=gen).bfloat16()
+    n = rows * dim
+    if op == "rms_norm":
+        out = torch.empty_like(x)
+        step = lambda: lib.ttfused_rms_norm(_capi.BF16, x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, dim, 1e-6, st)
+        abytes = 2 * n * 2
+    elif op == "add_rms_norm":
+        res = torch.randn(rows, dim, device="cuda", generator=gen).bfloat16()
+        x0, r0 = x[:64].clone(), res[:64].clone()
+        step = lambda: lib.ttfused_add_rms_norm(_capi.BF16, x.data_ptr(), res.data_ptr(), w.data_ptr(), rows, dim, 1e-6, st)
+        abytes = 4 * n * 2
+    elif op == "silu_mul":
+        out = torch.empty(rows, dim, device="cuda", dtype=torch.bfloat16)
+        step = lambda: lib.ttfused_silu_mul(_capi.BF16, x.data_ptr(), out.data_ptr(), rows, dim, st)
+        abytes = 3 * n * 2
+    else:
+        out = torch.empty_like(x)
+        step = lambda: lib.ttfused_softmax(_capi.BF16, x.data_ptr(), out.data_ptr(), rows, dim, 1, 0, st)
+        abytes = 2 * n * 2
+    rc = step()
+    if rc != 0:
+        raise RuntimeError("%s: %s" % (name, _capi.status_string(rc)))
+    torch.cuda.synchronize()
+    first = None
+    if op == "add_rms_norm":
+        first = (x[:64].float().cpu().numpy(), res[:64].float().cpu().numpy())  # before further in-place passes
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    res_line = {"workload": "%s bf16 [%d, %d]" % (name, rows, cols), "dtype": "bf16", "ms_per_step": round(ms, 5),
+                "roofline": {"bound": "hbm", "achieved": round(abytes / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                             "unit": "GB/s", "frac": round(abytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                             "traffic": measured_traffic(name), "algorithmic_bytes": abytes}}
+    if cpu:
+        import oracle
+        kind = "reference" if oracle.have_ref() else "port"
+        take = 64
+        xh = (x0 if op == "add_rms_norm" else x[:take]).float().cpu().numpy()
+        wh = w.float().cpu().numpy()
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            if op == "rms_norm":
+                ref = (oracle.ref_rms_norm if kind == "reference" else oracle.rms_norm)(xh, wh, 1e-6)
+                got = out[:take].float().cpu().numpy()
+            elif op == "add_rms_norm":
+                rh = r0.float().cpu().numpy()
+                ref = (oracle.ref_fused_add_rms_norm if kind == "reference" else oracle.fused_add_rms_norm)(xh, rh, wh, 1e-6)[0]
+                got = first[0]
+            elif op == "silu_mul":
+                ref = (oracle.ref_silu_mul if kind == "reference" else oracle.silu_mul)(xh)
+                got = out[:take].float().cpu().numpy()
+            else:
+                ref = (oracle.ref_softmax if kind == "reference" else oracle.softmax)(xh, -1)
+                got = out[:take].float().cpu().numpy()
+            reps += 1
+            spent = time.perf_counter() - t0
+            if spent > 1.0:
+                break
+        frac_bytes = abytes * take / rows
+        res_line["cpu_baseline"] = {"value": float("%.4g" % (frac_bytes * reps / spent / 1e9)), "unit": "GB/s", "cores": 1,
+                                    "kind": kind, "sample": "the first %d rows, %d passes in %.1f s, one thread (fp32 on the bf16 values)"
+                                    % (take, reps, spent),
+                                    "max_abs_err_gpu_vs_cpu": float("%.3g" % float(np.abs(ref - got).max()))}
+    return res_line
+
+
 def run_cpu_baseline(name, tensors, budget_s=20.0):
     """The reference CPU path (compiled reference if oracle/_ref is present, else this repository's C restatement)
     on one host core, over as many (batch, head) slices of the same inputs as fit the time budget."""
@@ -207,6 +307,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-probes", action="store_true", help="skip the hardware ceiling probes")
+    ap.add_argument("--no-fused", action="store_true", help="skip the row-wise neighbour ops (rmsNorm, siluMul, ...)")
+    ap.add_argument("--fused-only", default=None, choices=sorted(FUSED_WORKLOADS),
+                    help="measure one row-wise op only and print its line (for profiling)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one device-to-device copy of 1 GiB (a kernel of known traffic that calibrates "
                          "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc)")
@@ -224,6 +327,9 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.fused_only:
+        print(json.dumps(run_fused(args.fused_only, args.steps, args.warmup, cpu=not args.no_cpu)), flush=True)
+        return
     main_res, tensors = run_gpu(args.workload, args.steps, args.warmup)
     ceilings = None if args.no_probes else run_probes()
     cpu = None if args.no_cpu else run_cpu_baseline(args.workload, tensors, args.cpu_seconds)
@@ -248,6 +354,10 @@ def main():
             f32, tensors = run_gpu("config3_f32", max(1, min(args.steps, 100)), min(args.warmup, 20))
             del tensors
             line["fp32"] = f32
+    if not args.no_fused:
+        torch.cuda.empty_cache()
+        line["fused_ops"] = [run_fused(n, max(1, min(args.steps, 100)), min(args.warmup, 20), cpu=not args.no_cpu)
+                             for n in ("rms_norm", "fused_add_rms_norm", "silu_mul", "softmax")]
     print(json.dumps(line), flush=True)
 
 

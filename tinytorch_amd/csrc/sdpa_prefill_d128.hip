@@ -116,29 +116,34 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     S = len < 0 ? 0 : (len < S ? len : S);
   }
 
-  for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
   // Neighbouring workgroups take their two tiles in opposite order, so that the load / store bursts between the
   // parts of one half of the workgroups fall into the steady loops of the other half.
   const bool long_first = ((blockIdx.x >> 3) & 1) == 0;
-  const int rt = (CAUSAL && (part == 0) == long_first) ? ntile - 1 - slot_rt : slot_rt;
-  if (part == 1 && slot_rt >= ntile - 1 - slot_rt) break;  // odd count: the middle tile has no mirror
-  const int q0 = rt * BM;
   // Wavefronts w and w+4 share a SIMD.  Under a causal mask the row group g of a tile has g+1 halves of work on the
   // diagonal, so the second four wavefronts take the groups in reverse: every SIMD then carries groups g and 7-g.
   const int rowgroup = (CAUSAL && wave >= 4) ? 11 - wave : wave;
-  const int qw0 = q0 + rowgroup * WM;
-  if (S == 0) {  // no keys for this batch entry: zeros, the reference's empty contraction
+
+  if (S == 0) {  // no keys for this batch entry: zeros, the reference's empty contraction (kept out of the main loop)
     T* obase = (T*)a.out + b * a.os[0] + h * a.os[1];
     vec8 zero;
 #pragma unroll
     for (int i = 0; i < 8; i++) zero[i] = (T)0.f;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int qi = qw0 + 4 * i + (lane >> 4);
-      if (qi < a.L) *(vec8*)(obase + qi * a.os[2] + 8 * (lane & 15)) = zero;
+    for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
+      if (part == 1 && slot_rt >= ntile - 1 - slot_rt) break;
+      const int rt = (CAUSAL && part == 0) ? ntile - 1 - slot_rt : slot_rt;
+      for (int i = 0; i < 8; i++) {
+        const int qi = rt * BM + rowgroup * WM + 4 * i + (lane >> 4);
+        if (qi < a.L) *(vec8*)(obase + qi * a.os[2] + 8 * (lane & 15)) = zero;
+      }
     }
-    continue;
+    return;
   }
+
+  for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
+  const int rt = (CAUSAL && (part == 0) == long_first) ? ntile - 1 - slot_rt : slot_rt;
+  if (part == 1 && slot_rt >= ntile - 1 - slot_rt) break;  // odd count: the middle tile has no mirror
+  const int q0 = rt * BM;
+  const int qw0 = q0 + rowgroup * WM;
 
   // Query row i sees keys up to i + coff (coff = 0: the reference's top-left aligned mask); qc0 is this wavefront's
   // first row in key coordinates.
