@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TTSDPA_ABI_VERSION 4
+#define TTSDPA_ABI_VERSION 5
 
 /* Element types; numbering is the reference's DType enum (reference src/Tensor/DType.h:20-28). */
 enum ttsdpa_dtype { TTSDPA_F32 = 0, TTSDPA_F16 = 1, TTSDPA_BF16 = 2 };
@@ -110,6 +110,15 @@ typedef struct ttsdpa_params {
    * src/Operation/OpTransform.cpp:306-357).  A length of 0 yields zeros (the reference's empty contraction).
    * Served by the decode kernel, the pipelined head_dim-128 prefill kernel and the general kernel. */
   const int32_t* kv_len;
+  /* Paged KV cache (optional; no counterpart in the reference).  block_table != NULL: k and v point to page pools
+   * [num_pages, Hkv, page_size, D] and k_stride / v_stride are {page, head, row} strides; key j of batch b is row
+   * j % page_size of page block_table[b * block_table_stride + j / page_size] (int32, device memory).  S is the
+   * logical capacity: the table holds at least ceil(S / page_size) entries per batch entry, of which those below
+   * ceil(kv_len[b] / page_size) are read.  page_size must be a power of two; the decode kernel takes pages of 32 rows
+   * or more, anything else paged goes to the general kernel. */
+  const int32_t* block_table;
+  int32_t page_size;
+  int32_t block_table_stride;
 } ttsdpa_params;
 
 /* Library identification.  No counterpart in the reference (its device ops are linked statically). */
@@ -165,6 +174,12 @@ typedef struct ttsdpa_kv_append_params {
   int64_t kn_stride[3];
   int64_t vn_stride[3];
   const int32_t* positions;
+  /* Paged caches: block_table != NULL makes k_cache / v_cache page pools [num_pages, Hkv, page_size, D] with
+   * kc_stride / vc_stride = {page, head, row}; row pos of batch b goes to row pos % page_size of page
+   * block_table[b * block_table_stride + pos / page_size].  Smax is the logical capacity per batch entry. */
+  const int32_t* block_table;
+  int32_t page_size;
+  int32_t block_table_stride;
 } ttsdpa_kv_append_params;
 
 /* Fill *p for dense tensors (cache [B,Hkv,Smax,D], new rows [B,Hkv,Lnew,D]); pointers NULL, position 0. */

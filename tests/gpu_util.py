@@ -36,11 +36,11 @@ def to_host_f32(t):
     return t.detach().float().cpu().numpy()
 
 
-def call(entry, q, k, v, causal=False, mask=None, scale=None, out=None, kv_lens=None, align="top-left"):
+def call(entry, q, k, v, causal=False, mask=None, scale=None, out=None, kv_lens=None, align="top-left", block_table=None):
     """Run one C ABI entry point ("forward" | "prefill" | "decode" | "general") -> (status, out tensor)."""
     if out is None:
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    p = build_params(q, k, v, out, causal, mask, scale, kv_lens, align)
+    p = build_params(q, k, v, out, causal, mask, scale, kv_lens, align, block_table)
     L = _capi.lib()
     stream = torch.cuda.current_stream().cuda_stream
     ws, nbytes = None, 0
@@ -61,10 +61,10 @@ def call(entry, q, k, v, causal=False, mask=None, scale=None, out=None, kv_lens=
     return rc, out
 
 
-def route_of(q, k, v, causal=False, mask=None, scale=None, out=None, kv_lens=None, align="top-left"):
+def route_of(q, k, v, causal=False, mask=None, scale=None, out=None, kv_lens=None, align="top-left", block_table=None):
     if out is None:
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    rc, r = _capi.plan(build_params(q, k, v, out, causal, mask, scale, kv_lens, align))
+    rc, r = _capi.plan(build_params(q, k, v, out, causal, mask, scale, kv_lens, align, block_table))
     assert rc == 0
     return _capi.ROUTE_NAMES[r]
 

@@ -38,8 +38,8 @@ def test_exports_match_header():
 
 
 def test_struct_layout_matches_header():
-    # 4+4, 4 pointers, 6 ints, 12 int64, float, 2 ints, (pad), pointer, 4 int64, pointer
-    assert ctypes.sizeof(_capi.Params) == 8 + 32 + 24 + 96 + 12 + 4 + 8 + 32 + 8
+    # 4+4, 4 pointers, 6 ints, 12 int64, float, 2 ints, (pad), pointer, 4 int64, pointer, pointer, 2 ints
+    assert ctypes.sizeof(_capi.Params) == 8 + 32 + 24 + 96 + 12 + 4 + 8 + 32 + 8 + 8 + 8
     p = _capi.make_params(_capi.BF16, 2, 32, 8, 4096, 4096, 128)
     assert p.struct_size == ctypes.sizeof(_capi.Params)
     assert list(p.q_stride) == [32 * 4096 * 128, 4096 * 128, 128]
@@ -47,8 +47,8 @@ def test_struct_layout_matches_header():
     assert abs(p.scale - 128 ** -0.5) < 1e-8 and p.causal == 0 and p.mask_kind == 0
     assert list(p.mask_stride) == [0, 0, 4096, 1]  # a dense [L,S] mask shared by every batch and head
     assert p.kv_len is None
-    # 4+4, 4 pointers, 6 ints, 12 int64, pointer
-    assert ctypes.sizeof(_capi.KvAppendParams) == 8 + 32 + 24 + 96 + 8
+    # 4+4, 4 pointers, 6 ints, 12 int64, pointer, pointer, 2 ints
+    assert ctypes.sizeof(_capi.KvAppendParams) == 8 + 32 + 24 + 96 + 8 + 8 + 8
     kp = _capi.KvAppendParams()
     _capi.lib().ttsdpa_kv_append_params_init(ctypes.byref(kp), _capi.BF16, 4, 8, 1024, 2, 128)
     assert kp.struct_size == ctypes.sizeof(_capi.KvAppendParams)
@@ -227,3 +227,26 @@ def test_fused_ops_argument_checks_without_a_gpu():
     assert L.ttfused_silu_mul(_capi.F32, None, None, 4, 0, None) == 0
     assert L.ttfused_softmax(_capi.F32, FAKE, FAKE, 4, 8, -1, 0, None) == _capi.ERR_SHAPE
     assert L.ttfused_softmax(_capi.F32, None, None, 4, 0, 1, 1, None) == 0
+
+
+def test_paged_cache_routes_and_validation():
+    """block_table: decode kernel for pages of 32 rows or more, general kernel otherwise; page sizes are powers of two."""
+    dec = (_capi.BF16, 4, 32, 8, 1, 4096, 128)
+    paged = dict(block_table=FAKE, page_size=64, block_table_stride=64)
+    assert _capi.plan(params(*dec, **paged))[1] == _capi.ROUTE_DECODE
+    assert _capi.plan(params(*dec, **paged, kv_len=FAKE))[1] == _capi.ROUTE_DECODE
+    assert _capi.plan(params(*dec, block_table=FAKE, page_size=16, block_table_stride=256))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.BF16, 4, 32, 8, 512, 4096, 128, causal=2, **paged))[1] == _capi.ROUTE_GENERAL  # prefill kernels read contiguous K/V
+    assert _capi.plan(params(_capi.F32, 4, 32, 8, 1, 4096, 128, **paged))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(*dec, block_table=FAKE, page_size=48, block_table_stride=128))[0] == _capi.ERR_SHAPE
+    assert _capi.plan(params(*dec, block_table=FAKE, page_size=0, block_table_stride=128))[0] == _capi.ERR_SHAPE
+    assert _capi.plan(params(*dec, block_table=FAKE + 2, page_size=64, block_table_stride=64))[0] == _capi.ERR_STRIDE
+    assert _capi.plan(params(*dec, block_table=FAKE, page_size=64, block_table_stride=8))[0] == _capi.ERR_STRIDE  # rows of the table overlap
+    L = _capi.lib()
+    kp = _capi.KvAppendParams()
+    L.ttsdpa_kv_append_params_init(ctypes.byref(kp), _capi.BF16, 4, 8, 4096, 1, 128)
+    kp.k_cache = kp.v_cache = kp.k_new = kp.v_new = FAKE
+    kp.block_table, kp.page_size, kp.block_table_stride = FAKE, 24, 64
+    assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == _capi.ERR_SHAPE
+    kp.block_table, kp.page_size = FAKE + 1, 64
+    assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == _capi.ERR_STRIDE

@@ -47,6 +47,9 @@ class Params(ctypes.Structure):
         ("mask", ctypes.c_void_p),
         ("mask_stride", ctypes.c_int64 * 4),
         ("kv_len", ctypes.c_void_p),
+        ("block_table", ctypes.c_void_p),
+        ("page_size", ctypes.c_int32),
+        ("block_table_stride", ctypes.c_int32),
     ]
 
 
@@ -67,6 +70,9 @@ class KvAppendParams(ctypes.Structure):
         ("kn_stride", ctypes.c_int64 * 3),
         ("vn_stride", ctypes.c_int64 * 3),
         ("positions", ctypes.c_void_p),
+        ("block_table", ctypes.c_void_p),
+        ("page_size", ctypes.c_int32),
+        ("block_table_stride", ctypes.c_int32),
     ]
 
 
@@ -118,7 +124,7 @@ def lib():
         L.ttfused_silu_mul.restype = ctypes.c_int
         L.ttfused_softmax.argtypes = [ctypes.c_int, vp, vp, i64, i64, i64, ctypes.c_int, vp]
         L.ttfused_softmax.restype = ctypes.c_int
-        if L.ttsdpa_abi_version() != 4:
+        if L.ttsdpa_abi_version() != 5:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L
     return _lib

@@ -1,4 +1,5 @@
-// KV-cache append: writes the new tokens' K and V rows into preallocated caches [B,Hkv,Smax,D] at per-batch positions.
+// KV-cache append: writes the new tokens' K and V rows into preallocated caches [B,Hkv,Smax,D] (or page pools
+// [pages,Hkv,page_size,D] addressed through a block table) at per-batch positions.
 // The reference grows K/V with op::concat on the sequence axis (reference src/Operation/OpTransform.cpp:306-357), which
 // copies the whole history for every generated token; here only the new rows move.  HBM-bound by construction:
 // 2 * B*Hkv*Lnew*D elements read and written once, 16 bytes per lane when rows allow it.
@@ -26,8 +27,14 @@ __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
     if (pos < 0 || pos >= a.Smax) continue;  // no room: the row is dropped
     const char* ksrc = (const char*)a.kn + (b * a.kns[0] + hk * a.kns[1] + l * a.kns[2]) * a.esz + piece * VEC;
     const char* vsrc = (const char*)a.vn + (b * a.vns[0] + hk * a.vns[1] + l * a.vns[2]) * a.esz + piece * VEC;
-    char* kdst = (char*)a.kc + (b * a.kcs[0] + hk * a.kcs[1] + pos * a.kcs[2]) * a.esz + piece * VEC;
-    char* vdst = (char*)a.vc + (b * a.vcs[0] + hk * a.vcs[1] + pos * a.vcs[2]) * a.esz + piece * VEC;
+    long long slab = b;  // contiguous cache: the batch entry; paged cache: the page that holds row pos
+    int row = pos;
+    if (a.block_table) {
+      slab = a.block_table[(long long)b * a.bt_stride + (pos >> a.page_shift)];
+      row = pos & ((1 << a.page_shift) - 1);
+    }
+    char* kdst = (char*)a.kc + (slab * a.kcs[0] + hk * a.kcs[1] + row * a.kcs[2]) * a.esz + piece * VEC;
+    char* vdst = (char*)a.vc + (slab * a.vcs[0] + hk * a.vcs[1] + row * a.vcs[2]) * a.esz + piece * VEC;
     if (VEC == 16) {
       *(u32x4*)kdst = *(const u32x4*)ksrc;
       *(u32x4*)vdst = *(const u32x4*)vsrc;

@@ -14,6 +14,8 @@ struct KArgs {
   void* out;
   const void* mask;
   const int* kv_len;  // per-batch valid key count (device), or nullptr
+  const int* block_table;  // paged cache: page of key j of batch b = block_table[b * bt_stride + (j >> page_shift)], or nullptr
+  int page_shift, bt_stride;
   int B, Hq, Hkv, L, S, D;
   int G;  // Hq / Hkv: query heads per KV head
   int causal;     // key j is visible to query i iff j <= i + offset
@@ -114,6 +116,8 @@ struct KvAppendArgs {
   const void* kn;
   const void* vn;
   const int* positions;
+  const int* block_table;  // paged caches, as in KArgs
+  int page_shift, bt_stride;
   int B, Hkv, Smax, Lnew, D, position, esz;
   long long kcs[3], vcs[3], kns[3], vns[3];
 };

@@ -53,7 +53,9 @@ __device__ __forceinline__ void wave_lds_sync() {
 }
 
 // R = registers of query rows per score lane: rows handled = up to 4*R.
-template <typename TR, int R, int DD>
+// PAGED: K/V are page pools addressed through a block table (a variant of its own, so that the contiguous kernel
+// carries none of the lookups).
+template <typename TR, int R, int DD, bool PAGED>
 __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int chunk, float* __restrict__ ws) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
@@ -68,7 +70,7 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = tid >> 6;  // (forcing it scalar measured slower, also for the page lookups)
   const int l16 = lane & 15;  // score lanes: key within a 16-key group
   const int lg = lane >> 4;   // score lanes: row group
   const int vc = lane % CH;   // value lanes: 16-byte chunk of the row
@@ -132,14 +134,29 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int
     klim_min = klim[r] < klim_min ? klim[r] : klim_min;
   }
 
+  // Paged cache: the 32 keys of a block lie in one page (pages hold a power of two >= 32 rows and blocks start at
+  // multiples of 32); its number is read one block ahead.
+  const int* table = PAGED ? a.block_table + (long long)b * a.bt_stride : nullptr;
+  int page_next = 0;
+  if (PAGED && s_begin + wave * KB < s_end) page_next = table[(s_begin + wave * KB) >> a.page_shift];
+
   for (int k0 = s_begin + wave * KB; k0 < s_end; k0 += NWAVE * KB) {
+    const T* kpb = kp;
+    const T* vpb = vp;
+    int key0 = 0;  // first key of the memory region kpb / vpb point to
+    if (PAGED) {
+      kpb = (const T*)a.k + (long long)page_next * a.ks[0] + hk * a.ks[1];
+      vpb = (const T*)a.v + (long long)page_next * a.vs[0] + hk * a.vs[1];
+      key0 = (k0 >> a.page_shift) << a.page_shift;
+      if (k0 + NWAVE * KB < s_end) page_next = table[(k0 + NWAVE * KB) >> a.page_shift];
+    }
     // ---- issue all loads of the block: K for the score MFMAs, V for the accumulation ----------------------------------
     u32x4 kreg[2][KS];
 #pragma unroll
     for (int gi = 0; gi < 2; gi++) {
       int key = k0 + 16 * gi + l16;
-      key = key < S ? key : S - 1;
-      const T* kr = kp + key * a.ks[2] + 8 * lg;
+      key = (key < S ? key : S - 1) - key0;
+      const T* kr = kpb + key * a.ks[2] + 8 * lg;
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) kreg[gi][ks] = __builtin_nontemporal_load((const u32x4*)(kr + 32 * ks));  // read once: keep it out of the caches
     }
@@ -147,8 +164,8 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int
 #pragma unroll
     for (int i = 0; i < KB / PH; i++) {
       int key = k0 + PH * i + vph;
-      key = key < S ? key : S - 1;
-      vreg[i] = __builtin_nontemporal_load((const u32x4*)(vp + key * a.vs[2] + 8 * vc));
+      key = (key < S ? key : S - 1) - key0;
+      vreg[i] = __builtin_nontemporal_load((const u32x4*)(vpb + key * a.vs[2] + 8 * vc));
     }
 
     // ---- scores --------------------------------------------------------------------------------------------------------
@@ -312,12 +329,18 @@ int launch_decode_t(const KArgs& a, const DecodePlan& pl, float* ws, hipStream_t
   typedef typename TR::elem T;
   dim3 grid((unsigned)((long long)a.B * a.Hkv * pl.splits)), block(256);
   int R = (pl.rows + 3) / 4;
+#define TT_DECODE(R_)                                                                                                      \
+  if (a.block_table)                                                                                                       \
+    hipLaunchKernelGGL((decode_kernel<TR, R_, DD, true>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws);            \
+  else                                                                                                                     \
+    hipLaunchKernelGGL((decode_kernel<TR, R_, DD, false>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws)
   switch (R) {
-    case 1: hipLaunchKernelGGL((decode_kernel<TR, 1, DD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
-    case 2: hipLaunchKernelGGL((decode_kernel<TR, 2, DD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
-    case 3: hipLaunchKernelGGL((decode_kernel<TR, 3, DD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
-    default: hipLaunchKernelGGL((decode_kernel<TR, 4, DD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws); break;
+    case 1: TT_DECODE(1); break;
+    case 2: TT_DECODE(2); break;
+    case 3: TT_DECODE(3); break;
+    default: TT_DECODE(4); break;
   }
+#undef TT_DECODE
   int rc = (int)hipGetLastError();
   if (rc != 0 || pl.splits == 1) return rc;
   hipLaunchKernelGGL((merge_kernel<T, DD>), dim3((unsigned)((long long)a.B * a.Hkv * pl.rows)), dim3(DD), 0, stream, a, pl.splits, ws);

@@ -76,8 +76,15 @@ __global__ __launch_bounds__(256) void general_kernel(KArgs a) {
       int key = k0 + kk;
       float kv = 0.f, vv = 0.f;
       if (key < S && d < a.D) {
-        kv = load_as_float(kp + key * a.ks[2] + d);
-        vv = load_as_float(vp + key * a.vs[2] + d);
+        if (a.block_table) {  // paged cache: page pools [pages, Hkv, page_size, D]
+          const long long page = a.block_table[(long long)b * a.bt_stride + (key >> a.page_shift)];
+          const int row = key & ((1 << a.page_shift) - 1);
+          kv = load_as_float((const T*)a.k + page * a.ks[0] + hk * a.ks[1] + row * a.ks[2] + d);
+          vv = load_as_float((const T*)a.v + page * a.vs[0] + hk * a.vs[1] + row * a.vs[2] + d);
+        } else {
+          kv = load_as_float(kp + key * a.ks[2] + d);
+          vv = load_as_float(vp + key * a.vs[2] + d);
+        }
       }
       Ks[kk][d] = kv;
       Vs[kk][d] = vv;

@@ -57,6 +57,13 @@ int validate(const ttsdpa_params* p, KArgs* a) {
   if (p->mask_kind == TTSDPA_MASK_ADD && !ptr_aligned(p->mask, esz)) return TTSDPA_ERR_STRIDE;
   if (p->kv_len && !ptr_aligned(p->kv_len, 4)) return TTSDPA_ERR_STRIDE;
   a->kv_len = p->kv_len;
+  a->block_table = p->block_table, a->page_shift = 0, a->bt_stride = p->block_table_stride;
+  if (p->block_table) {
+    if (!ptr_aligned(p->block_table, 4) || p->block_table_stride < 0) return TTSDPA_ERR_STRIDE;
+    if (p->page_size < 1 || (p->page_size & (p->page_size - 1)) != 0) return TTSDPA_ERR_SHAPE;
+    while ((1 << a->page_shift) < p->page_size) a->page_shift++;
+    if ((long long)p->block_table_stride * p->page_size < p->S && p->B > 1) return TTSDPA_ERR_STRIDE;  // tables would overlap
+  }
   a->q = p->q, a->k = p->k, a->v = p->v, a->out = p->out, a->mask = p->mask;
   a->B = p->B, a->Hq = p->Hq, a->Hkv = p->Hkv, a->L = p->L, a->S = p->S, a->D = p->D;
   a->G = p->Hq / p->Hkv;
@@ -71,7 +78,8 @@ int validate(const ttsdpa_params* p, KArgs* a) {
 }
 
 // 16-bit tensors the MFMA kernels can read with 16-byte loads and write with 8-byte stores.
-bool fast_layout_ok(const ttsdpa_params* p, bool masks_ok = false) {
+bool fast_layout_ok(const ttsdpa_params* p, bool masks_ok = false, bool pages_ok = false) {
+  if (p->block_table && !pages_ok) return false;
   if (p->dtype != TTSDPA_F16 && p->dtype != TTSDPA_BF16) return false;
   if (p->mask_kind != TTSDPA_MASK_NONE && !masks_ok) return false;
   if (!(p->scale > 0.f) || !isfinite(p->scale)) return false;  // the row maximum is taken on unscaled scores
@@ -83,7 +91,7 @@ bool fast_layout_ok(const ttsdpa_params* p, bool masks_ok = false) {
 
 // fp32 tensors the fp32 MFMA kernel can read and write with 16-byte accesses.
 bool f32_prefill_ok(const ttsdpa_params* p) {
-  if (p->dtype != TTSDPA_F32 || p->mask_kind != TTSDPA_MASK_NONE || p->kv_len) return false;
+  if (p->dtype != TTSDPA_F32 || p->mask_kind != TTSDPA_MASK_NONE || p->kv_len || p->block_table) return false;
   if (p->D != 128 && p->D != 64) return false;
   if (!(p->scale > 0.f) || !isfinite(p->scale) || p->S < 1 || p->L < 1) return false;
   if (!dense_last_ok(p->q_stride, 4) || !dense_last_ok(p->k_stride, 4) || !dense_last_ok(p->v_stride, 4) ||
@@ -103,8 +111,10 @@ bool prefill_ok(const ttsdpa_params* p) {
 
 bool decode_ok(const ttsdpa_params* p) {
   // a top-left aligned causal mask leaves a few keys per row: not the streaming kernel's case
-  if (!fast_layout_ok(p) || (p->D != 128 && p->D != 64) || effective_causal(p) == TTSDPA_CAUSAL_TOP_LEFT || p->S < 1 || p->L < 1)
+  if (!fast_layout_ok(p, false, true) || (p->D != 128 && p->D != 64) || effective_causal(p) == TTSDPA_CAUSAL_TOP_LEFT ||
+      p->S < 1 || p->L < 1)
     return false;
+  if (p->block_table && p->page_size < 32) return false;  // a 32-key block of a wavefront must lie in one page
   return (long long)p->L * (p->Hq / p->Hkv) <= kDecodeMaxRows;
 }
 
@@ -157,6 +167,7 @@ void ttsdpa_params_init(ttsdpa_params* p, int dtype, int B, int Hq, int Hkv, int
   p->mask = nullptr;
   p->mask_stride[0] = 0, p->mask_stride[1] = 0, p->mask_stride[2] = S, p->mask_stride[3] = 1;
   p->kv_len = nullptr;
+  p->block_table = nullptr, p->page_size = 0, p->block_table_stride = 0;
 }
 
 int ttsdpa_plan(const ttsdpa_params* p, int* route) {
@@ -254,6 +265,12 @@ int ttsdpa_kv_append(const ttsdpa_kv_append_params* p, void* stream) {
   if ((p->kc_stride[2] < p->D || p->vc_stride[2] < p->D) && p->Smax > 1) return TTSDPA_ERR_STRIDE;
   if ((p->kn_stride[2] < p->D || p->vn_stride[2] < p->D) && p->Lnew > 1) return TTSDPA_ERR_STRIDE;
   a.kc = p->k_cache, a.vc = p->v_cache, a.kn = p->k_new, a.vn = p->v_new, a.positions = p->positions;
+  a.block_table = p->block_table, a.page_shift = 0, a.bt_stride = p->block_table_stride;
+  if (p->block_table) {
+    if (!ptr_aligned(p->block_table, 4) || p->block_table_stride < 0) return TTSDPA_ERR_STRIDE;
+    if (p->page_size < 1 || (p->page_size & (p->page_size - 1)) != 0) return TTSDPA_ERR_SHAPE;
+    while ((1 << a.page_shift) < p->page_size) a.page_shift++;
+  }
   a.B = p->B, a.Hkv = p->Hkv, a.Smax = p->Smax, a.Lnew = p->Lnew, a.D = p->D, a.position = p->position, a.esz = (int)esz;
   return launch_kv_append(a, (hipStream_t)stream);
 }

@@ -34,10 +34,23 @@ def _strides3(t):
 _CAUSAL_ALIGN = {"top-left": _capi.CAUSAL_TOP_LEFT, "bottom-right": _capi.CAUSAL_BOTTOM_RIGHT}
 
 
-def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=None, kvLens=None, causalAlign="top-left"):
-    """Fill a ttsdpa_params for 4-D tensors [B,H,N,D]."""
+def _check_block_table(name, blockTable, B, device):
+    if blockTable.dtype != torch.int32 or blockTable.dim() != 2 or blockTable.shape[0] != B \
+            or blockTable.stride(1) != 1 or blockTable.device != device:
+        raise ValueError("%s: blockTable must be an int32 [B, pages per entry] tensor on the device of the tensors" % name)
+
+
+def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=None, kvLens=None, causalAlign="top-left",
+                 blockTable=None):
+    """Fill a ttsdpa_params for 4-D tensors [B,H,N,D] (with blockTable: key/value are page pools [pages,Hkv,page,D])."""
     B, Hq, L, D = query.shape
     Bk, Hkv, S, Dk = key.shape
+    if blockTable is not None:
+        _check_block_table("sdpAttention", blockTable, B, query.device)
+        page = S
+        if page < 1 or page & (page - 1):
+            raise ValueError("sdpAttention: the page size (%d rows) must be a power of two" % page)
+        Bk, S = B, blockTable.shape[1] * page  # logical capacity per batch entry
     if value.shape != key.shape or Bk != B or Dk != D:
         raise ValueError("sdpAttention: key/value shape %s / %s do not match query %s"
                          % (tuple(key.shape), tuple(value.shape), tuple(query.shape)))
@@ -80,11 +93,15 @@ def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=No
         if kvLens.device != query.device:
             raise RuntimeError("sdpAttention: kvLens must live on the device of the tensors")
         p.kv_len = kvLens.data_ptr()
+    if blockTable is not None:
+        p.block_table = blockTable.data_ptr()
+        p.page_size = key.shape[2]
+        p.block_table_stride = blockTable.stride(0)
     return p
 
 
 def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0, scale=None, kvLens=None,
-                 causalAlign="top-left"):
+                 causalAlign="top-left", blockTable=None):
     """out = softmax(query @ key^T * scale + bias) @ value on the GPU.
 
     query [B,Hq,L,D]; key/value [B,Hkv,S,D] with Hq a multiple of Hkv (query head h reads KV head h // (Hq//Hkv));
@@ -93,6 +110,8 @@ def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0,
     iff j <= i + S_b - L with S_b = kvLens[b] or S): a prompt chunk or several new tokens against a KV cache.
     kvLens (not in the reference, which has no KV cache): int32 [B] on the device; batch b attends to the first
     kvLens[b] keys only, so key/value may be preallocated caches [B,Hkv,Smax,D] filled by kvCacheAppend.
+    blockTable (likewise not in the reference): int32 [B, n] on the device makes key/value page pools
+    [pages,Hkv,pageSize,D]; key j of batch b is row j % pageSize of page blockTable[b, j // pageSize].
     """
     if dropoutP != 0.0:
         raise NotImplementedError("sdpAttention: dropoutP must be 0 on this path")
@@ -105,7 +124,7 @@ def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0,
     fix = lambda t: t if (t.stride(-1) == 1 or t.size(-1) == 1) else t.contiguous()
     query, key, value = fix(query), fix(key), fix(value)
     out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
-    p = build_params(query, key, value, out, isCausal, attnMask, scale, kvLens, causalAlign)
+    p = build_params(query, key, value, out, isCausal, attnMask, scale, kvLens, causalAlign, blockTable)
     L = _capi.lib()
     with torch.cuda.device(query.device):
         nbytes = L.ttsdpa_workspace_bytes(ctypes.byref(p))
@@ -117,16 +136,25 @@ def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0,
     return out
 
 
-def kvCacheAppend(kCache, vCache, kNew, vNew, positions):
+def kvCacheAppend(kCache, vCache, kNew, vNew, positions, blockTable=None):
     """Write kNew/vNew [B,Hkv,Lnew,D] into the caches [B,Hkv,Smax,D] at rows positions[b] .. positions[b]+Lnew-1.
 
     positions: int32 [B] device tensor, or an int used for every batch entry.  In place, on the current stream; rows
     that would land beyond Smax are dropped.  Replaces growing K/V with op::concat on the sequence axis (reference
     src/Operation/OpTransform.cpp:306-357), which copies the whole history per generated token.
+    blockTable: int32 [B, n] makes the caches page pools [pages,Hkv,pageSize,D]; row pos of batch b lands in row
+    pos % pageSize of page blockTable[b, pos // pageSize], and the capacity per batch entry is n * pageSize.
     """
     if kCache.dim() != 4 or kNew.dim() != 4 or vCache.shape != kCache.shape or vNew.shape != kNew.shape:
         raise ValueError("kvCacheAppend: expected caches [B,Hkv,Smax,D] and new rows [B,Hkv,Lnew,D]")
     B, Hkv, Smax, D = kCache.shape
+    if blockTable is not None:
+        B = kNew.shape[0]
+        _check_block_table("kvCacheAppend", blockTable, B, kCache.device)
+        page = Smax
+        if page < 1 or page & (page - 1):
+            raise ValueError("kvCacheAppend: the page size (%d rows) must be a power of two" % page)
+        Smax = blockTable.shape[1] * page
     if kNew.shape[0] != B or kNew.shape[1] != Hkv or kNew.shape[3] != D:
         raise ValueError("kvCacheAppend: new rows %s do not match the cache %s" % (tuple(kNew.shape), tuple(kCache.shape)))
     if kCache.dtype not in _DTYPES or any(t.dtype != kCache.dtype for t in (vCache, kNew, vNew)):
@@ -150,6 +178,10 @@ def kvCacheAppend(kCache, vCache, kNew, vNew, positions):
                 or positions.device != kCache.device:
             raise ValueError("kvCacheAppend: positions must be a contiguous int32 device tensor of B entries")
         p.positions = positions.data_ptr()
+    if blockTable is not None:
+        p.block_table = blockTable.data_ptr()
+        p.page_size = kCache.shape[2]
+        p.block_table_stride = blockTable.stride(0)
     with torch.cuda.device(kCache.device):
         rc = L.ttsdpa_kv_append(ctypes.byref(p), torch.cuda.current_stream().cuda_stream)
     if rc != 0:
