@@ -208,7 +208,7 @@ static void test_kv_cache() {
       std::copy(kb.begin(), kb.end(), kn.begin() + static_cast<size_t>(b) * Hkv * n * D);
       std::copy(vb.begin(), vb.end(), vn.begin() + static_cast<size_t>(b) * Hkv * n * D);
     }
-    op::kvCacheAppend(kc, vc, Tensor(kn, {B, Hkv, n, D}, gpu), Tensor(vn, {B, Hkv, n, D}, gpu), Tensor{}, 0);
+    op::kvCacheAppend(kc, vc, Tensor(kn, {B, Hkv, n, D}, gpu), Tensor(vn, {B, Hkv, n, D}, gpu), Tensor{}, 0, Tensor{});
     for (int b = 0; b < B; b++) lens[b] = prompt[b];
   }
   for (int step = 0; step < 3; step++) {
@@ -219,13 +219,13 @@ static void test_kv_cache() {
       std::copy(vb.begin(), vb.end(), vn.begin() + static_cast<size_t>(b) * Hkv * D);
     }
     Tensor pos(std::vector<int>{lens[0], lens[1]}, {B}, gpuInt);
-    op::kvCacheAppend(kc, vc, Tensor(kn, {B, Hkv, 1, D}, gpu), Tensor(vn, {B, Hkv, 1, D}, gpu), pos, 0);
+    op::kvCacheAppend(kc, vc, Tensor(kn, {B, Hkv, 1, D}, gpu), Tensor(vn, {B, Hkv, 1, D}, gpu), pos, 0, Tensor{});
     for (int b = 0; b < B; b++) lens[b]++;
     std::vector<float> q = pseudoRandom(static_cast<size_t>(B) * Hq * D, 20 + step);
     Tensor tq(q, {B, Hq, 1, D}, gpu);
     q = tq.toList<float>();
     Tensor kvLens(std::vector<int>{lens[0], lens[1]}, {B}, gpuInt);
-    std::vector<float> y = op::sdpAttentionCached(tq, kc, vc, kvLens, false, 1.f / std::sqrt(static_cast<float>(D))).toList<float>();
+    std::vector<float> y = op::sdpAttentionCached(tq, kc, vc, kvLens, false, 1.f / std::sqrt(static_cast<float>(D)), Tensor{}).toList<float>();
     for (int b = 0; b < B; b++) {
       std::vector<float> qb(q.begin() + static_cast<size_t>(b) * Hq * D, q.begin() + static_cast<size_t>(b + 1) * Hq * D);
       std::vector<float> ref = closedForm(qb, rowsOf(kall, b, 0, lens[b]), rowsOf(vall, b, 0, lens[b]), 1, Hq, Hkv, 1, lens[b], D, false);
@@ -243,13 +243,13 @@ static void test_kv_cache() {
       std::copy(vb.begin(), vb.end(), vn.begin() + static_cast<size_t>(b) * Hkv * n * D);
     }
     Tensor pos(std::vector<int>{lens[0], lens[1]}, {B}, gpuInt);
-    op::kvCacheAppend(kc, vc, Tensor(kn, {B, Hkv, n, D}, gpu), Tensor(vn, {B, Hkv, n, D}, gpu), pos, 0);
+    op::kvCacheAppend(kc, vc, Tensor(kn, {B, Hkv, n, D}, gpu), Tensor(vn, {B, Hkv, n, D}, gpu), pos, 0, Tensor{});
     for (int b = 0; b < B; b++) lens[b] += n;
     std::vector<float> q = pseudoRandom(static_cast<size_t>(B) * Hq * n * D, 40);
     Tensor tq(q, {B, Hq, n, D}, gpu);
     q = tq.toList<float>();
     Tensor kvLens(std::vector<int>{lens[0], lens[1]}, {B}, gpuInt);
-    std::vector<float> y = op::sdpAttentionCached(tq, kc, vc, kvLens, true, 1.f / std::sqrt(static_cast<float>(D))).toList<float>();
+    std::vector<float> y = op::sdpAttentionCached(tq, kc, vc, kvLens, true, 1.f / std::sqrt(static_cast<float>(D)), Tensor{}).toList<float>();
     for (int b = 0; b < B; b++)
       for (int i = 0; i < n; i++) {
         const int visible = lens[b] - n + i + 1;
@@ -263,6 +263,30 @@ static void test_kv_cache() {
         std::vector<float> ref = closedForm(qi, rowsOf(kall, b, 0, visible), rowsOf(vall, b, 0, visible), 1, Hq, Hkv, 1, visible, D, false);
         EXPECT_TRUE(vectorNear(yi, ref, 2e-2f));
       }
+  }
+  // the same history in pages of 32 rows placed in reverse order through a pool: appended through the block table, then
+  // attended to — the result equals the contiguous cache's
+  {
+    const int page = 32, perSeq = (Smax + page - 1) / page, pages = B * perSeq;
+    std::vector<int> table(static_cast<size_t>(B) * perSeq);
+    for (int i = 0; i < B * perSeq; i++) table[i] = pages - 1 - i;
+    Tensor blockTable(table, {B, perSeq}, gpuInt);
+    Tensor kPool = Tensor::zeros({pages, Hkv, page, D}, gpu), vPool = Tensor::zeros({pages, Hkv, page, D}, gpu);
+    const int n = std::min(lens[0], lens[1]);
+    std::vector<float> kn(static_cast<size_t>(B) * Hkv * n * D), vn(kn.size());
+    for (int b = 0; b < B; b++) {
+      std::vector<float> kb = rowsOf(kall, b, 0, n), vb = rowsOf(vall, b, 0, n);
+      std::copy(kb.begin(), kb.end(), kn.begin() + static_cast<size_t>(b) * Hkv * n * D);
+      std::copy(vb.begin(), vb.end(), vn.begin() + static_cast<size_t>(b) * Hkv * n * D);
+    }
+    op::kvCacheAppend(kPool, vPool, Tensor(kn, {B, Hkv, n, D}, gpu), Tensor(vn, {B, Hkv, n, D}, gpu), Tensor{}, 0, blockTable);
+    std::vector<float> q = pseudoRandom(static_cast<size_t>(B) * Hq * D, 60);
+    Tensor tq(q, {B, Hq, 1, D}, gpu);
+    Tensor kvLens(std::vector<int>{n, n}, {B}, gpuInt);
+    const float sc = 1.f / std::sqrt(static_cast<float>(D));
+    std::vector<float> paged = op::sdpAttentionCached(tq, kPool, vPool, kvLens, false, sc, blockTable).toList<float>();
+    std::vector<float> flat = op::sdpAttentionCached(tq, kc, vc, kvLens, false, sc, Tensor{}).toList<float>();
+    EXPECT_TRUE(vectorNear(paged, flat, 1e-6f));
   }
 }
 

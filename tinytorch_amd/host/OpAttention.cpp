@@ -80,25 +80,44 @@ Tensor sdpAttentionGpuImpl(const Tensor& query, const Tensor& key, const Tensor&
   return out;
 }
 
+// Fills the block-table fields of a parameter struct; false after a failed precondition.
+template <typename P>
+bool setBlockTable(P& p, const Tensor& blockTable, const Tensor& pool, int64_t B) {
+  ASSERT(blockTable.dtype() == DType::Int32 && blockTable.dim() == 2 && blockTable.size(0) == B &&
+         blockTable.device() == pool.device());
+  if (blockTable.dtype() != DType::Int32 || blockTable.dim() != 2 || blockTable.size(0) != B) return false;
+  p.block_table = static_cast<const int32_t*>(blockTable.rawPtr());
+  p.page_size = static_cast<int32_t>(pool.size(2));
+  p.block_table_stride = static_cast<int32_t>(blockTable.size(1));
+  return true;
+}
+
 void kvCacheAppendGpuImpl(const Tensor& kCache, const Tensor& vCache, const Tensor& kNew, const Tensor& vNew,
-                          const Tensor& positions, int32_t position) {
+                          const Tensor& positions, int32_t position, const Tensor& blockTable) {
   ASSERT(kCache.defined() && vCache.defined() && kNew.defined() && vNew.defined());
   ASSERT(kCache.dim() == 4 && kNew.dim() == 4 && kCache.shape() == vCache.shape() && kNew.shape() == vNew.shape());
-  ASSERT(kNew.size(0) == kCache.size(0) && kNew.size(1) == kCache.size(1) && kNew.size(3) == kCache.size(3));
+  const bool paged = blockTable.defined();
+  ASSERT((paged || kNew.size(0) == kCache.size(0)) && kNew.size(1) == kCache.size(1) && kNew.size(3) == kCache.size(3));
   ASSERT(vCache.dtype() == kCache.dtype() && kNew.dtype() == kCache.dtype() && vNew.dtype() == kCache.dtype());
   ASSERT(vCache.device() == kCache.device() && kNew.device() == kCache.device() && vNew.device() == kCache.device());
   if (kCache.dim() != 4 || kNew.dim() != 4 || kCache.shape() != vCache.shape() || kNew.shape() != vNew.shape()) return;
-  if (kNew.size(0) != kCache.size(0) || kNew.size(1) != kCache.size(1) || kNew.size(3) != kCache.size(3)) return;
+  if ((!paged && kNew.size(0) != kCache.size(0)) || kNew.size(1) != kCache.size(1) || kNew.size(3) != kCache.size(3)) return;
+  const int64_t B = kNew.size(0);
+  const int64_t capacity = paged && blockTable.dim() == 2 ? blockTable.size(1) * kCache.size(2) : kCache.size(2);
   ttsdpa_kv_append_params p;
-  ttsdpa_kv_append_params_init(&p, dtypeCode(kCache.dtype()), static_cast<int>(kCache.size(0)),
-                               static_cast<int>(kCache.size(1)), static_cast<int>(kCache.size(2)),
-                               static_cast<int>(kNew.size(2)), static_cast<int>(kCache.size(3)));
+  ttsdpa_kv_append_params_init(&p, dtypeCode(kCache.dtype()), static_cast<int>(B), static_cast<int>(kCache.size(1)),
+                               static_cast<int>(capacity), static_cast<int>(kNew.size(2)),
+                               static_cast<int>(kCache.size(3)));
+  if (paged) {  // the pool's strides are {page, head, row}
+    p.kc_stride[0] = p.vc_stride[0] = kCache.size(1) * kCache.size(2) * kCache.size(3);
+    p.kc_stride[1] = p.vc_stride[1] = kCache.size(2) * kCache.size(3);
+    if (!setBlockTable(p, blockTable, kCache, B)) return;
+  }
   p.k_cache = kCache.rawPtr(), p.v_cache = vCache.rawPtr(), p.k_new = kNew.rawPtr(), p.v_new = vNew.rawPtr();
   p.position = position;
   if (positions.defined()) {
-    ASSERT(positions.dtype() == DType::Int32 && positions.numel() == kCache.size(0) &&
-           positions.device() == kCache.device());
-    if (positions.dtype() != DType::Int32 || positions.numel() != kCache.size(0)) return;
+    ASSERT(positions.dtype() == DType::Int32 && positions.numel() == B && positions.device() == kCache.device());
+    if (positions.dtype() != DType::Int32 || positions.numel() != B) return;
     p.positions = static_cast<const int32_t*>(positions.rawPtr());
   }
   const DeviceIndex dev = kCache.device().index;
@@ -111,20 +130,27 @@ void kvCacheAppendGpuImpl(const Tensor& kCache, const Tensor& vCache, const Tens
 }
 
 Tensor sdpAttentionCachedGpuImpl(const Tensor& query, const Tensor& kCache, const Tensor& vCache, const Tensor& kvLens,
-                                 bool isCausal, float scale) {
+                                 bool isCausal, float scale, const Tensor& blockTable) {
+  const bool paged = blockTable.defined();
   ASSERT(query.defined() && kCache.defined() && vCache.defined() && kvLens.defined());
   ASSERT(query.dim() == 4 && kCache.dim() == 4 && kCache.shape() == vCache.shape());
-  ASSERT(kCache.size(0) == query.size(0) && kCache.size(3) == query.size(3) && query.size(1) % kCache.size(1) == 0);
+  ASSERT((paged || kCache.size(0) == query.size(0)) && kCache.size(3) == query.size(3) && query.size(1) % kCache.size(1) == 0);
   ASSERT(kCache.dtype() == query.dtype() && vCache.dtype() == query.dtype());
   ASSERT(kvLens.dtype() == DType::Int32 && kvLens.numel() == query.size(0) && kvLens.device() == query.device());
-  if (query.dim() != 4 || kCache.dim() != 4 || kCache.shape() != vCache.shape() || kCache.size(0) != query.size(0) ||
+  if (query.dim() != 4 || kCache.dim() != 4 || kCache.shape() != vCache.shape() || (!paged && kCache.size(0) != query.size(0)) ||
       kCache.size(3) != query.size(3) || query.size(1) % kCache.size(1) != 0 || kvLens.dtype() != DType::Int32 ||
       kvLens.numel() != query.size(0))
     return {};
   ttsdpa_params p;
   ttsdpa_params_init(&p, dtypeCode(query.dtype()), static_cast<int>(query.size(0)), static_cast<int>(query.size(1)),
                      static_cast<int>(kCache.size(1)), static_cast<int>(query.size(2)),
-                     static_cast<int>(kCache.size(2)), static_cast<int>(query.size(3)));
+                     static_cast<int>(paged && blockTable.dim() == 2 ? blockTable.size(1) * kCache.size(2) : kCache.size(2)),
+                     static_cast<int>(query.size(3)));
+  if (paged) {  // the pool's strides are {page, head, row}
+    p.k_stride[0] = p.v_stride[0] = kCache.size(1) * kCache.size(2) * kCache.size(3);
+    p.k_stride[1] = p.v_stride[1] = kCache.size(2) * kCache.size(3);
+    if (!setBlockTable(p, blockTable, kCache, query.size(0))) return {};
+  }
   Tensor out = Tensor::empty(query.shape(), query.options().noGrad());
   p.q = query.rawPtr(), p.k = kCache.rawPtr(), p.v = vCache.rawPtr(), p.out = out.rawPtr();
   p.scale = scale;

@@ -27,10 +27,12 @@ DEFINE_OP(sdpAttention, SdpAttentionOpFn)
 // (kvLens: Int32 [B] on the device), no mask.  isCausal here means: the L query rows are the last L positions of each
 // batch entry's kvLens[b] keys (their K/V already appended) and row i sees the keys up to its own position,
 // kvLens[b] - L + i — a chunk of a prompt, or several speculated tokens; one new token (L == 1) sees every key either way.
+// blockTable (Int32 [B, n] on the device, or undefined): the caches are page pools [pages,Hkv,pageSize,D] and key j of
+// batch entry b is row j % pageSize of page blockTable[b][j / pageSize]; pageSize is a power of two.
 using KvCacheAppendOpFn = void (*)(const Tensor& kCache, const Tensor& vCache, const Tensor& kNew, const Tensor& vNew,
-                                   const Tensor& positions, int32_t position);
+                                   const Tensor& positions, int32_t position, const Tensor& blockTable);
 using SdpAttentionCachedOpFn = Tensor (*)(const Tensor& query, const Tensor& kCache, const Tensor& vCache,
-                                          const Tensor& kvLens, bool isCausal, float scale);
+                                          const Tensor& kvLens, bool isCausal, float scale, const Tensor& blockTable);
 DEFINE_OP(kvCacheAppend, KvCacheAppendOpFn)
 DEFINE_OP(sdpAttentionCached, SdpAttentionCachedOpFn)
 
