@@ -1,0 +1,45 @@
+/*
+ * ttlinear — the linear layer y = x . w^T + bias for MI355X (gfx950) behind a plain C ABI, in the same library as
+ * ttsdpa (libttsdpa.so): the projections on either side of attention (QKV, output, MLP).
+ *
+ * Replaces, for this call shape, the reference's op::matmul(input, weight, false, true, bias) behind
+ * function::linear (reference src/Function/FuncNNLayer.h:14-19, 270-272; host side src/Operation/OpLinalg.cpp:244-276;
+ * its device GEMM is a cuBLAS call, src/Operation/OpLinalgCuda.cuh:239-293; CPU loop src/Operation/OpLinalgCpu.h:119-150).
+ * The op implementation passes raw device pointers, sizes, leading dimensions and its current stream.
+ */
+#ifndef TTLINEAR_H_
+#define TTLINEAR_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "ttsdpa.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum ttlinear_route {
+  TTLINEAR_ROUTE_NONE = 0,   /* empty output */
+  TTLINEAR_ROUTE_MFMA = 1,   /* fp16/bf16, K a multiple of 64, 16-byte aligned rows: MFMA kernel, fp32 accumulation */
+  TTLINEAR_ROUTE_GENERAL = 2 /* everything else (fp32, other K, unaligned rows): fp32 arithmetic on the vector ALUs */
+};
+
+/* out[m, n] = bias[n] + sum_k x[m, k] * w[n, k]   (m < M, n < N, k < K)
+ * x: [M, K] with row stride ldx elements; w: [N, K] (the layout of a Linear layer's weight) with row stride ldw;
+ * bias: [N] or NULL; out: [M, N] with row stride ldo.  dtype is a ttsdpa_dtype shared by all four tensors.
+ * Accumulation is fp32 starting from the bias (the reference writes the bias into C and accumulates onto it), one
+ * rounding to the element type at the end.  K == 0 yields the bias (or zeros).
+ * Enqueues on `stream` (a hipStream_t; NULL = the default stream); no allocation, no synchronisation.
+ * Returns a ttsdpa_status code, or a positive hipError_t. */
+int ttlinear_forward(int dtype, const void* x, const void* w, const void* bias, void* out, int64_t M, int64_t N,
+                     int64_t K, int64_t ldx, int64_t ldw, int64_t ldo, void* stream);
+
+/* Validate the arguments and report the kernel ttlinear_forward would pick (enum ttlinear_route).  Launches nothing. */
+int ttlinear_plan(int dtype, const void* x, const void* w, const void* bias, const void* out, int64_t M, int64_t N,
+                  int64_t K, int64_t ldx, int64_t ldw, int64_t ldo, int* route);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTLINEAR_H_ */

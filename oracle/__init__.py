@@ -61,6 +61,8 @@ def lib():
         L.oracle_silu_mul.restype = None
         L.oracle_softmax.argtypes = [_c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int]
         L.oracle_softmax.restype = None
+        L.oracle_linear.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int]
+        L.oracle_linear.restype = None
         _lib = L
     return _lib
 
@@ -89,6 +91,8 @@ def ref():
         R.tt_ref_silu_mul.restype = ctypes.c_int
         R.tt_ref_softmax.argtypes = [_c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int]
         R.tt_ref_softmax.restype = ctypes.c_int
+        R.tt_ref_linear.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64]
+        R.tt_ref_linear.restype = ctypes.c_int
         _ref = R
     return _ref
 
@@ -304,5 +308,27 @@ def ref_softmax(x, dim=-1, log=False):
     out = np.empty_like(x)
     outer, n, inner = _softmax_dims(x.shape, dim)
     rc = ref().tt_ref_softmax(_p(x), _p(out), outer, n, inner, int(log))
+    assert rc == 0
+    return out
+
+
+def linear(x, w, bias=None, dtype="f32"):
+    """x [M,K] . w [N,K]^T + bias [N] in the reference's loop order; the result rounded to dtype."""
+    x, w = _f32(x), _f32(w)
+    b = _f32(bias) if bias is not None else None
+    M, K = x.shape
+    N = w.shape[0]
+    out = np.empty((M, N), dtype=np.float32)
+    lib().oracle_linear(_p(x), _p(w), _p(b) if b is not None else None, _p(out), M, N, K, _dt(dtype))
+    return out
+
+
+def ref_linear(x, w, bias=None):
+    x, w = _f32(x), _f32(w)
+    b = _f32(bias) if bias is not None else None
+    M, K = x.shape
+    N = w.shape[0]
+    out = np.empty((M, N), dtype=np.float32)
+    rc = ref().tt_ref_linear(_p(x), _p(w), _p(b) if b is not None else None, _p(out), M, N, K)
     assert rc == 0
     return out

@@ -2,7 +2,7 @@
  * TEST INFRASTRUCTURE — not part of the product.  Nothing under tinytorch_amd/ may call this.
  *
  * CPU restatement of the row-wise inference ops that sit next to attention in the reference: rmsNorm,
- * fusedAddRmsNorm, siluMul and softmax / logSoftmax.  All tensors are fp32 arrays here; `dtype` (0 fp32, 1 fp16,
+ * fusedAddRmsNorm, siluMul, softmax / logSoftmax, and the linear layer.  All tensors are fp32 arrays here; `dtype` (0 fp32, 1 fp16,
  * 2 bf16) says where the reference rounds to its element type T: inputs are expected to hold T-representable values,
  * intermediate stores to T tensors and the results are rounded with the same casts as the attention oracle.
  * Arithmetic between those points is fp32 — the reference's CPU path for fp32 tensors, and its device kernels
@@ -15,6 +15,8 @@
  *                              identity fusedAddRmsNorm(x, r, w) == rmsNorm(x + r, w) with residual == x + r
  *   oracle_silu_mul            reference KAT for silu test/test_function.cpp:139-143 (up = 1); oracle/_ref
  *                              (op::siluMul) bit-exact in fp32
+ *   oracle_linear              reference KAT test/test_function.cpp:234-241; oracle/_ref (function::linear) bit-exact
+ *                              in fp32; fp64 closed form
  *   oracle_softmax             reference KATs test/test_function.cpp:147-176; oracle/_ref (function::softmax /
  *                              logSoftmax, every axis) bit-exact in fp32; rows sum to 1
  */
@@ -104,4 +106,22 @@ void oracle_softmax(const float* x, float* out, int64_t outer, int64_t dim, int6
         for (int64_t d = 0; d < dim; d++) out[base + d * inner] = round_t(x[base + d * inner] - mx - ls, dtype);
       }
     }
+}
+
+/* reference src/Operation/OpLinalgCpu.h:119-150 (gemmCpuImpl with transA = false, transB = true, as function::linear
+ * calls it, src/Function/FuncNNLayer.h:14-19): C starts as the bias broadcast over the rows (or zeros), then
+ * c[i][j] += a[i][p] * b[j][p] in i, p, j order, all in fp32; `dtype` rounds the result once (16-bit tensors: fp32
+ * accumulation as in the device GEMM).  Pinned by the reference KAT test/test_function.cpp:234-241, bit-exact against
+ * oracle/_ref (function::linear) in fp32, and the fp64 closed form. */
+void oracle_linear(const float* x, const float* w, const float* bias, float* out, int64_t M, int64_t N, int64_t K,
+                   int dtype) {
+  for (int64_t i = 0; i < M; i++)
+    for (int64_t j = 0; j < N; j++) out[i * N + j] = bias ? bias[j] : 0.f;
+  for (int64_t i = 0; i < M; i++)
+    for (int64_t p = 0; p < K; p++) {
+      const float av = x[i * K + p];
+      for (int64_t j = 0; j < N; j++) out[i * N + j] += av * w[j * K + p];
+    }
+  if (dtype != 0)
+    for (int64_t e = 0; e < M * N; e++) out[e] = round_t(out[e], dtype);
 }

@@ -164,4 +164,17 @@ int tt_ref_softmax(const float* x, float* out, int64_t outer, int64_t dim, int64
   return 0;
 }
 
+// function::linear (reference src/Function/FuncNNLayer.h:270-272): x [M,K], w [N,K], bias [N] or NULL -> out [M,N].
+int tt_ref_linear(const float* x, const float* w, const float* bias, float* out, int64_t M, int64_t N, int64_t K) {
+  ensureCpu();
+  NoGradGuard guard;
+  Tensor tb;
+  if (bias) tb = fromF32(bias, {N});
+  Tensor y = function::linear(fromF32(x, {M, K}), fromF32(w, {N, K}), tb);
+  auto r = y.toList<float>();
+  if (static_cast<int64_t>(r.size()) != M * N) return -2;
+  std::memcpy(out, r.data(), sizeof(float) * r.size());
+  return 0;
+}
+
 }  // extern "C"

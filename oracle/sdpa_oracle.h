@@ -63,6 +63,9 @@ void oracle_fused_add_rms_norm(float* input, float* residual, const float* w, in
                                int dtype);
 void oracle_silu_mul(const float* x, float* out, int64_t rows, int64_t d, int dtype);
 void oracle_softmax(const float* x, float* out, int64_t outer, int64_t dim, int64_t inner, int log_form, int dtype);
+/* out[M,N] = bias[N] (or 0) + x[M,K] . w[N,K]^T, the reference's gemm loop order. */
+void oracle_linear(const float* x, const float* w, const float* bias, float* out, int64_t M, int64_t N, int64_t K,
+                   int dtype);
 
 #ifdef __cplusplus
 }

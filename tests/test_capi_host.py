@@ -26,9 +26,9 @@ def params(*dims, **kw):
 
 
 def test_exports_match_header():
-    text = open(os.path.join(ROOT, "include", "ttsdpa.h")).read() + open(os.path.join(ROOT, "include", "ttfused.h")).read()
+    text = "".join(open(os.path.join(ROOT, "include", h)).read() for h in ("ttsdpa.h", "ttfused.h", "ttlinear.h"))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    declared = sorted(set(re.findall(r"\b(tt(?:sdpa|fused)_[a-z_]+)\s*\(", text)))
+    declared = sorted(set(re.findall(r"\b(tt(?:sdpa|fused|linear)_[a-z_]+)\s*\(", text)))
     assert declared == sorted(_capi.EXPORTS)
     L = _capi.lib()
     for name in declared:
@@ -250,3 +250,27 @@ def test_paged_cache_routes_and_validation():
     assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == _capi.ERR_SHAPE
     kp.block_table, kp.page_size = FAKE + 1, 64
     assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == _capi.ERR_STRIDE
+
+
+def test_linear_routes_and_validation():
+    L = _capi.lib()
+    r = ctypes.c_int(-1)
+
+    def plan(dtype, M, N, K, ldx=None, ldw=None, ldo=None, x=FAKE, w=FAKE, out=FAKE):
+        rc = L.ttlinear_plan(dtype, x, w, None, out, M, N, K, ldx or K, ldw or K, ldo or N, ctypes.byref(r))
+        return rc, _capi.LINEAR_ROUTE_NAMES.get(r.value)
+
+    assert plan(_capi.BF16, 8192, 4096, 4096) == (0, "mfma")
+    assert plan(_capi.F16, 100, 12, 64) == (0, "mfma")
+    assert plan(_capi.F32, 8192, 4096, 4096) == (0, "general")       # fp32: vector ALUs
+    assert plan(_capi.BF16, 8192, 4096, 4000) == (0, "general")      # K not a multiple of 64
+    assert plan(_capi.BF16, 8192, 4095, 4096) == (0, "general")      # N not a multiple of 4
+    assert plan(_capi.BF16, 64, 64, 64, x=FAKE + 2) == (0, "general")  # rows not 16-byte aligned
+    assert plan(_capi.BF16, 0, 64, 64) == (0, "none")
+    assert plan(_capi.BF16, 64, 64, 0) == (0, "general")             # K == 0: the bias
+    assert plan(7, 64, 64, 64)[0] == _capi.ERR_DTYPE
+    assert plan(_capi.BF16, -1, 64, 64)[0] == _capi.ERR_SHAPE
+    assert plan(_capi.BF16, 64, 64, 64, ldx=32)[0] == _capi.ERR_STRIDE
+    assert plan(_capi.BF16, 64, 64, 64, x=None)[0] == _capi.ERR_NULL
+    assert L.ttlinear_forward(_capi.BF16, None, None, None, None, 0, 64, 64, 64, 64, 64, None) == 0
+    assert L.ttlinear_forward(_capi.BF16, FAKE, FAKE, None, None, 8, 64, 64, 64, 64, 64, None) == _capi.ERR_NULL

@@ -1,0 +1,113 @@
+"""GPU parity of the linear layer (include/ttlinear.h) against the CPU oracle (the reference's gemm loop with the bias
+as the starting value, oracle/fused_oracle.c) on identical seeded inputs.  Bars: fp32 max-abs-error <= 1e-4 * sqrt(K)
+(sums of K unit-variance products; the summation order differs), fp16/bf16 <= 2e-2 relative to the result's scale
+sqrt(K) (fp32 accumulation, one rounding)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import to_device, to_host_f32
+from tinytorch_amd import _capi, linear
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def inputs(seed, stream, shape, dtype, mul=1.0):
+    vals, bits = oracle.round_to(oracle.randn(seed, stream, shape, mul), dtype)
+    return vals, to_device(vals, bits, dtype)
+
+
+def route(xd, wd, od):
+    r = ctypes.c_int(-1)
+    M, K = xd.shape
+    rc = _capi.lib().ttlinear_plan(_capi.BF16 if xd.dtype == torch.bfloat16 else _capi.F16 if xd.dtype == torch.float16 else _capi.F32,
+                                   xd.data_ptr(), wd.data_ptr(), None, od.data_ptr(), M, wd.shape[0], K,
+                                   xd.stride(0), wd.stride(0), od.stride(0), ctypes.byref(r))
+    assert rc == 0
+    return _capi.LINEAR_ROUTE_NAMES[r.value]
+
+
+CASES = [
+    # M, N, K, dtype, bias, route
+    (256, 256, 64, "bf16", True, "mfma"),        # one tile, one k step
+    (256, 512, 256, "f16", False, "mfma"),
+    (300, 260, 192, "bf16", True, "mfma"),       # ragged in M and N
+    (1, 4, 64, "bf16", True, "mfma"),            # a single row
+    (1100, 2300, 128, "f16", True, "mfma"),      # more than one 4 x 8 block of tiles
+    (64, 768, 1024, "bf16", False, "mfma"),
+    (2, 3, 5, "f32", True, "general"),
+    (70, 90, 100, "f32", True, "general"),
+    (129, 65, 200, "bf16", True, "general"),     # K not a multiple of 64
+    (64, 66, 128, "f16", False, "general"),      # N not a multiple of 4
+    (33, 40, 0, "f32", True, "general"),         # empty contraction: the bias
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "M%dN%dK%d-%s-b%d-%s" % c)
+def test_linear_against_oracle(case):
+    M, N, K, dtype, has_bias, want = case
+    say("linear", case)
+    xh, xd = inputs(600 + M + K, 0, (M, K), dtype)
+    wh, wd = inputs(600 + M + K, 1, (N, K), dtype)
+    bh, bd = inputs(600 + M + K, 2, (N,), dtype) if has_bias else (None, None)
+    exp = oracle.linear(xh, wh, bh, dtype)
+    out = linear(xd, wd, bd)
+    assert route(xd, wd, out) == want
+    y = to_host_f32(out)
+    assert y.shape == exp.shape and np.isfinite(y).all()
+    scale = max(1.0, np.sqrt(K))
+    tol = 1e-4 * scale if dtype == "f32" else 2e-2 * scale
+    err = float(np.abs(y.astype(np.float64) - exp).max()) if y.size else 0.0
+    say("   max-abs-err", err, "tol", tol)
+    assert err <= tol
+
+
+def test_reference_known_answer_and_views():
+    """reference test/test_function.cpp:234-241 through the GPU; leading batch axes; strided views of x, w and out."""
+    x = torch.tensor([[-0.3089, 0.5301, -0.0245], [1.5852, 0.8954, 0.7485]], device="cuda")
+    w = torch.tensor([[0.8397, 1.7990, -0.2738], [-0.8910, -0.6746, 0.3419]], device="cuda")
+    b = torch.tensor([-0.9601, -1.4163], device="cuda")
+    assert abs(float(linear(x, w, b).sum()) - (-3.1661377)) < 1e-5
+    xh, xd = inputs(1, 0, (2, 5, 70, 128), "bf16")
+    wh, wd = inputs(1, 1, (96, 128), "bf16")
+    exp = oracle.linear(xh.reshape(-1, 128), wh, None, "bf16").reshape(2, 5, 70, 96)
+    assert np.abs(to_host_f32(linear(xd, wd)) - exp).max() <= 2e-2 * np.sqrt(128)
+    # rows taken out of wider buffers (leading dimensions larger than K / N), through the C ABI
+    xbuf = torch.zeros(300, 192 + 64, dtype=torch.bfloat16, device="cuda")
+    wbuf = torch.zeros(260, 192 + 8, dtype=torch.bfloat16, device="cuda")
+    obuf = torch.full((300, 260 + 12), -3.0, dtype=torch.bfloat16, device="cuda")
+    xh, xd = inputs(2, 0, (300, 192), "bf16")
+    wh, wd = inputs(2, 1, (260, 192), "bf16")
+    xbuf[:, :192], wbuf[:, :192] = xd, wd
+    rc = _capi.lib().ttlinear_forward(_capi.BF16, xbuf.data_ptr(), wbuf.data_ptr(), None, obuf.data_ptr(), 300, 260, 192,
+                                      xbuf.stride(0), wbuf.stride(0), obuf.stride(0), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0
+    assert np.abs(to_host_f32(obuf[:, :260]) - oracle.linear(xh, wh, None, "bf16")).max() <= 2e-2 * np.sqrt(192)
+    assert bool((obuf[:, 260:] == -3.0).all())   # nothing written beyond N
+
+
+def test_full_size_projection_properties():
+    """The QKV projection of config 3's token batch (8192 tokens, hidden 4096 -> 6144): sampled outputs against fp64
+    dot products, linearity in x, and the bias entering exactly once."""
+    M, N, K = 8192, 6144, 4096
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(M, K, device="cuda", generator=gen).bfloat16()
+    w = (torch.randn(N, K, device="cuda", generator=gen) * K ** -0.5).bfloat16()
+    b = torch.randn(N, device="cuda", generator=gen).bfloat16()
+    y = linear(x, w, b)
+    rows = torch.randint(0, M, (64,), device="cuda", generator=gen)
+    cols = torch.randint(0, N, (64,), device="cuda", generator=gen)
+    exact = (x[rows].double() * w[cols].double()).sum(-1) + b[cols].double()
+    assert float((y[rows, cols].double() - exact).abs().max()) <= 2e-2
+    y0 = linear(x, w)
+    assert float((y.float() - y0.float() - b.float()[None, :]).abs().max()) <= 3e-2   # two roundings apart
+    y2 = linear(x * 2, w)   # doubling x is exact in bf16
+    assert torch.equal(y2.float(), y0.float() * 2)

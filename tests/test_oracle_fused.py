@@ -102,3 +102,32 @@ def test_16bit_results_are_representable_and_close(oracle_mod, dtype):
     # the normalised row is computed from the ROUNDED residual (what the reference stores and re-reads)
     a, b = o.fused_add_rms_norm(x, res, w, 1e-6, dtype)
     assert np.array_equal(b, o.round_to(x + res, dtype)[0])
+
+
+def test_linear_known_answer_reference_and_closed_form(oracle_mod):
+    o = oracle_mod
+    # func_linear, reference test/test_function.cpp:234-241: the sum of linear(x, w, b)
+    x = np.array([[-0.3089, 0.5301, -0.0245], [1.5852, 0.8954, 0.7485]], np.float32)
+    w = np.array([[0.8397, 1.7990, -0.2738], [-0.8910, -0.6746, 0.3419]], np.float32)
+    b = np.array([-0.9601, -1.4163], np.float32)
+    assert abs(float(o.linear(x, w, b).sum()) - (-3.1661377)) < 1e-5
+    r = rng(21)
+    for M, N, K in ((1, 1, 1), (5, 7, 3), (8, 16, 16), (33, 65, 129), (64, 128, 256)):
+        x = r.standard_normal((M, K)).astype(np.float32)
+        w = r.standard_normal((N, K)).astype(np.float32)
+        b = r.standard_normal(N).astype(np.float32)
+        y = o.linear(x, w, b)
+        ref64 = x.astype(np.float64) @ w.astype(np.float64).T + b
+        assert np.abs(y - ref64).max() < 1e-4 * max(1.0, np.sqrt(K))
+        assert np.abs(o.linear(x, w) - (ref64 - b)).max() < 1e-4 * max(1.0, np.sqrt(K))
+        # w is [N, K] (not [K, N]): transposing the operand must change the answer for a non-symmetric case
+        if N == K and N > 1:
+            assert np.abs(o.linear(x, w) - o.linear(x, w.T.copy())).max() > 0.1
+        if o.have_ref():
+            assert np.array_equal(y, o.ref_linear(x, w, b))
+            assert np.array_equal(o.linear(x, w), o.ref_linear(x, w))
+    # 16-bit: one rounding of the fp32 result
+    xb, _ = o.round_to(x, "bf16")
+    wb, _ = o.round_to(w, "bf16")
+    y16 = o.linear(xb, wb, None, "bf16")
+    assert np.array_equal(y16, o.round_to(o.linear(xb, wb), "bf16")[0])

@@ -23,7 +23,10 @@ EXPORTS = [
     "ttsdpa_kv_append_params_init", "ttsdpa_kv_append", "ttsdpa_probe",
     # include/ttfused.h
     "ttfused_rms_norm", "ttfused_add_rms_norm", "ttfused_silu_mul", "ttfused_softmax",
+    # include/ttlinear.h
+    "ttlinear_forward", "ttlinear_plan",
 ]
+LINEAR_ROUTE_NAMES = {0: "none", 1: "mfma", 2: "general"}
 
 
 class Params(ctypes.Structure):
@@ -124,6 +127,10 @@ def lib():
         L.ttfused_silu_mul.restype = ctypes.c_int
         L.ttfused_softmax.argtypes = [ctypes.c_int, vp, vp, i64, i64, i64, ctypes.c_int, vp]
         L.ttfused_softmax.restype = ctypes.c_int
+        L.ttlinear_forward.argtypes = [ctypes.c_int, vp, vp, vp, vp] + [i64] * 6 + [vp]
+        L.ttlinear_forward.restype = ctypes.c_int
+        L.ttlinear_plan.argtypes = [ctypes.c_int, vp, vp, vp, vp] + [i64] * 6 + [ctypes.POINTER(ctypes.c_int)]
+        L.ttlinear_plan.restype = ctypes.c_int
         if L.ttsdpa_abi_version() != 5:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L

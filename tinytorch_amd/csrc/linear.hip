@@ -1,0 +1,283 @@
+// The linear layer y = x . w^T + bias on gfx950 (reference: op::matmul(input, weight, false, true, bias) behind
+// function::linear, src/Function/FuncNNLayer.h:14-19; device GEMM src/Operation/OpLinalgCuda.cuh:239-293).
+//
+// linear_mfma_kernel (fp16 / bf16): a workgroup of 8 wavefronts owns a 256 x 256 tile of the output and walks K in
+// steps of 64.  Both operands have K contiguous ("NT"), which is the layout v_mfma_f32_32x32x16 wants for both inputs:
+// a lane supplies 8 consecutive k of one row, so operand fragments are plain 16-byte LDS reads, no transposes.
+//   global -> LDS   global_load_lds_dwordx4, two stages of 64 KB (x tile 256 x 64, w tile 256 x 64); the 16-byte chunks
+//                   of a 128-byte LDS row are XOR-swizzled with the row number so that the 32 rows a fragment read
+//                   touches spread over the banks; the loads for tile t+1 are in flight while tile t is multiplied
+//   MFMA            the wavefront's 64 (n) x 128 (m) part is computed transposed, A = w rows, B = x rows, so that an
+//                   accumulator register group holds 4 consecutive n of one m: the output is stored as 8-byte pieces
+//                   along its contiguous axis without a transpose
+//   accumulators    start from the bias (the reference writes the bias into C and accumulates onto it), fp32
+// Workgroups are numbered so that the 32 that run together on one XCD (workgroup i runs on XCD i % 8) form a 4 x 8
+// block of tiles: they share their x and w panels through that XCD's L2.
+//
+// linear_general_kernel: any element type and shape, fp32 arithmetic on the vector ALUs (64 x 64 tiles).
+
+#include "../../include/ttlinear.h"
+#include "sdpa_common.h"
+
+namespace ttsdpa {
+namespace {
+
+struct LinArgs {
+  const void* x;
+  const void* w;
+  const void* bias;
+  void* out;
+  long long M, N, K, ldx, ldw, ldo;
+};
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+constexpr int TM = 256, TN = 256, BK = 64;
+constexpr int ROWB = BK * 2;                 // bytes of an LDS row
+constexpr int XTILE = TM * ROWB;             // 32 KB
+constexpr int STAGE = (TM + TN) * ROWB;      // 64 KB
+constexpr int LIN_LDS = 2 * STAGE;
+
+template <typename TR>
+__global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
+  typedef typename TR::elem T;
+  typedef typename TR::vec8 vec8;
+  typedef typename TR::vec4 vec4;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, lh = lane >> 5;
+
+  // ---- workgroup -> tile: 4 x 8 tile blocks per XCD ---------------------------------------------------------------
+  const int tiles_m = (int)((a.M + TM - 1) / TM), tiles_n = (int)((a.N + TN - 1) / TN);
+  const int super_n = (tiles_n + 7) / 8;
+  const int nsuper = ((tiles_m + 3) / 4) * super_n;
+  const int slot = blockIdx.x >> 3;
+  const int super = (slot >> 5) * 8 + (blockIdx.x & 7);
+  if (super >= nsuper) return;
+  const int tm = (super / super_n) * 4 + ((slot & 31) >> 3);
+  const int tn = (super % super_n) * 8 + (slot & 7);
+  if (tm >= tiles_m || tn >= tiles_n) return;
+  const long long m0 = (long long)tm * TM, n0 = (long long)tn * TN;
+
+  // ---- global -> LDS: wavefront w moves rows 32w .. 32w+31 of both tiles, 8 rows (1 KB) per instruction ----------------
+  // lane l fills (row l/8, chunk slot l%8) and therefore fetches chunk (l%8) ^ (row % 8); rows past the end of the
+  // matrix re-read its last row (their products land in outputs that are not stored)
+  unsigned xoff[4], woff[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int row = 32 * wave + 8 * i + (lane >> 3);
+    const int chunk = (lane & 7) ^ (lane >> 3);
+    long long mr = m0 + row < a.M ? row : a.M - 1 - m0;
+    long long nr = n0 + row < a.N ? row : a.N - 1 - n0;
+    xoff[i] = (unsigned)((mr * a.ldx + 8 * chunk) * 2);
+    woff[i] = (unsigned)((nr * a.ldw + 8 * chunk) * 2);
+  }
+  const char* xbase = (const char*)((const T*)a.x + m0 * a.ldx);
+  const char* wbase = (const char*)((const T*)a.w + n0 * a.ldw);
+  const unsigned smem_addr = (unsigned)(unsigned long)(lds_void_t*)smem;
+  // issued as asm so that the compiler does not treat it as an LDS store it must order every later LDS read behind
+  auto dma_issue = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+  };
+  auto dma_tile = [&](int t, int stage) __attribute__((always_inline)) {
+    const char* xs = xbase + (long long)t * BK * 2;
+    const char* ws = wbase + (long long)t * BK * 2;
+    const unsigned dst = smem_addr + stage * STAGE + (32 * wave) * ROWB;
+#pragma unroll
+    for (int i = 0; i < 4; i++) dma_issue(xs, xoff[i], dst + 8 * i * ROWB);
+#pragma unroll
+    for (int i = 0; i < 4; i++) dma_issue(ws, woff[i], dst + XTILE + 8 * i * ROWB);
+  };
+
+  // ---- this wavefront's part: n rows 64*wn .. +63 of the w tile (A operand), m rows 128*wm .. +127 of the x tile (B) -----
+  const int wn = wave & 3, wm = wave >> 2;
+  // fragment (block, ks): row 32*block + lq, chunk 2*ks + lh at row*128 + 16 * (chunk ^ (row % 8)); row % 8 == lq % 8
+  const unsigned frag = (unsigned)(lq * ROWB + 16 * (lh ^ (lq & 7)));
+  const unsigned wfrag = XTILE + (64 * wn) * ROWB + frag;
+  const unsigned xfrag = (128 * wm) * ROWB + frag;
+
+  f32x16 acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const long long n = n0 + 64 * wn + 32 * i + 8 * (r >> 2) + 4 * lh + (r & 3);
+      const float b = (a.bias && n < a.N) ? (float)((const T*)a.bias)[n] : 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[i][j][r] = b;
+    }
+
+  const int ntk = (int)(a.K / BK);
+  if (ntk > 0) dma_tile(0, 0);
+  for (int t = 0; t < ntk; t++) {
+    // tile t has landed (this wavefront's loads; the barrier extends that to everyone's) and every wavefront is done
+    // reading the other stage, which tile t+1 now overwrites
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (t + 1 < ntk) dma_tile(t + 1, (t + 1) & 1);
+    const char* st = smem + (t & 1) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      vec8 wf[2], xf[4];
+#pragma unroll
+      for (int i = 0; i < 2; i++) wf[i] = *(const vec8*)(st + ((wfrag + 32 * i * ROWB) ^ (unsigned)(32 * ks)));
+#pragma unroll
+      for (int j = 0; j < 4; j++) xf[j] = *(const vec8*)(st + ((xfrag + 32 * j * ROWB) ^ (unsigned)(32 * ks)));
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = TR::mfma32(wf[i], xf[j], acc[i][j]);
+    }
+  }
+
+  // ---- store: register group rg of acc[i][j] is out[m = .. + 32j + lq][n = .. + 32i + 8rg + 4lh .. +3] ----------------------
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const long long m = m0 + 128 * wm + 32 * j + lq;
+    if (m >= a.M) continue;
+    T* orow = (T*)a.out + m * a.ldo;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        const long long n = n0 + 64 * wn + 32 * i + 8 * rg + 4 * lh;
+        if (n < a.N) {  // N is a multiple of 4 on this route
+          f32x4 v;
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * rg + e];
+          *(vec4*)(orow + n) = __builtin_convertvector(v, vec4);
+        }
+      }
+  }
+}
+
+// Any element type and shape: 64 x 64 output tile per workgroup, 4 x 4 outputs per lane, K in steps of 16 through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void linear_general_kernel(LinArgs a) {
+  __shared__ float Xs[16][64 + 1], Ws[16][64 + 1];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const long long m0 = (long long)blockIdx.y * 64, n0 = (long long)blockIdx.x * 64;
+  const T* x = (const T*)a.x;
+  const T* w = (const T*)a.w;
+  float acc[4][4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const long long n = n0 + 4 * tx + j;
+    const float b = (a.bias && n < a.N) ? load_as_float((const T*)a.bias + n) : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i][j] = b;
+  }
+  for (long long k0 = 0; k0 < a.K; k0 += 16) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int e = tid + 256 * i;
+      const int row = e >> 4, kk = e & 15;
+      const bool kin = k0 + kk < a.K;
+      Xs[kk][row] = (kin && m0 + row < a.M) ? load_as_float(x + (m0 + row) * a.ldx + k0 + kk) : 0.f;
+      Ws[kk][row] = (kin && n0 + row < a.N) ? load_as_float(w + (n0 + row) * a.ldw + k0 + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; kk++) {
+      float xv[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) xv[i] = Xs[kk][4 * ty + i], wv[i] = Ws[kk][4 * tx + i];
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = fmaf(xv[i], wv[j], acc[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const long long m = m0 + 4 * ty + i;
+    if (m >= a.M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const long long n = n0 + 4 * tx + j;
+      if (n < a.N) store_from_float((T*)a.out + m * a.ldo + n, acc[i][j]);
+    }
+  }
+}
+
+bool aligned(const void* p, size_t n) { return ((uintptr_t)p % n) == 0; }
+
+int check(int dtype, const void* x, const void* w, const void* out, long long M, long long N, long long K, long long ldx,
+          long long ldw, long long ldo, int* route) {
+  if (dtype != TTSDPA_F32 && dtype != TTSDPA_F16 && dtype != TTSDPA_BF16) return TTSDPA_ERR_DTYPE;
+  if (M < 0 || N < 0 || K < 0) return TTSDPA_ERR_SHAPE;
+  *route = TTLINEAR_ROUTE_NONE;
+  if (M == 0 || N == 0) return TTSDPA_OK;
+  if (!out || (K > 0 && (!x || !w))) return TTSDPA_ERR_NULL;
+  if (ldx < K || ldw < K || ldo < N) return TTSDPA_ERR_STRIDE;
+  const size_t esz = dtype == TTSDPA_F32 ? 4 : 2;
+  if (!aligned(x, esz) || !aligned(w, esz) || !aligned(out, esz)) return TTSDPA_ERR_STRIDE;
+  if ((M + 63) / 64 > 65535 || (N + 63) / 64 > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
+  const bool mfma = dtype != TTSDPA_F32 && K > 0 && K % BK == 0 && N % 4 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldo % 4 == 0 &&
+                    aligned(x, 16) && aligned(w, 16) && aligned(out, 8) &&
+                    ldx < (1 << 22) && ldw < (1 << 22);  // 256 rows are addressed with 32-bit byte offsets
+  *route = mfma ? TTLINEAR_ROUTE_MFMA : TTLINEAR_ROUTE_GENERAL;
+  return TTSDPA_OK;
+}
+
+template <typename TR>
+int launch_mfma(const LinArgs& a, hipStream_t stream) {
+  static hipError_t state[kMaxDevices];
+  static bool done[kMaxDevices];
+  const hipError_t granted = grant_dynamic_lds((const void*)linear_mfma_kernel<TR>, LIN_LDS, state, done);
+  if (granted != hipSuccess) return (int)granted;
+  const long long tiles_m = (a.M + TM - 1) / TM, tiles_n = (a.N + TN - 1) / TN;
+  const long long nsuper = ((tiles_m + 3) / 4) * ((tiles_n + 7) / 8);
+  const long long nwg = (nsuper + 7) / 8 * 8 * 32;
+  if (nwg > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
+  hipLaunchKernelGGL((linear_mfma_kernel<TR>), dim3((unsigned)nwg), dim3(512), LIN_LDS, stream, a);
+  return (int)hipGetLastError();
+}
+
+template <typename T>
+int launch_general_linear(const LinArgs& a, hipStream_t stream) {
+  dim3 grid((unsigned)((a.N + 63) / 64), (unsigned)((a.M + 63) / 64));
+  hipLaunchKernelGGL((linear_general_kernel<T>), grid, dim3(256), 0, stream, a);
+  return (int)hipGetLastError();
+}
+
+}  // namespace
+}  // namespace ttsdpa
+
+using namespace ttsdpa;
+
+extern "C" {
+
+int ttlinear_plan(int dtype, const void* x, const void* w, const void* bias, const void* out, int64_t M, int64_t N,
+                  int64_t K, int64_t ldx, int64_t ldw, int64_t ldo, int* route) {
+  (void)bias;
+  int r = TTLINEAR_ROUTE_NONE;
+  const int rc = check(dtype, x, w, out, M, N, K, ldx, ldw, ldo, &r);
+  if (rc == TTSDPA_OK && route) *route = r;
+  return rc;
+}
+
+int ttlinear_forward(int dtype, const void* x, const void* w, const void* bias, void* out, int64_t M, int64_t N,
+                     int64_t K, int64_t ldx, int64_t ldw, int64_t ldo, void* stream) {
+  int route = TTLINEAR_ROUTE_NONE;
+  const int rc = check(dtype, x, w, out, M, N, K, ldx, ldw, ldo, &route);
+  if (rc != TTSDPA_OK || route == TTLINEAR_ROUTE_NONE) return rc;
+  const size_t esz = dtype == TTSDPA_F32 ? 4 : 2;
+  if (bias && !aligned(bias, esz)) return TTSDPA_ERR_STRIDE;
+  LinArgs a{x, w, bias, out, M, N, K, ldx, ldw, ldo};
+  hipStream_t s = (hipStream_t)stream;
+  if (route == TTLINEAR_ROUTE_MFMA) return dtype == TTSDPA_F16 ? launch_mfma<F16>(a, s) : launch_mfma<BF16>(a, s);
+  switch (dtype) {
+    case TTSDPA_F32: return launch_general_linear<float>(a, s);
+    case TTSDPA_F16: return launch_general_linear<_Float16>(a, s);
+    default: return launch_general_linear<__bf16>(a, s);
+  }
+}
+
+}  // extern "C"

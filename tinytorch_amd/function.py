@@ -280,3 +280,30 @@ def softmax(x, dim=-1):
 def logSoftmax(x, dim=-1):
     """logSoftmax along `dim` (reference src/Function/FuncActivation.h:92)."""
     return _softmax("logSoftmax", x, dim, True)
+
+
+# ---- the linear layer (include/ttlinear.h) ------------------------------------------------------------------------------
+
+def linear(input, weight, bias=None):
+    """input [..., K] . weight [N, K]^T + bias [N] (reference src/Function/FuncNNLayer.h:270-272): fp32 accumulation
+    starting from the bias, one rounding to the dtype of input."""
+    _check_rowwise("linear", input, weight, bias)
+    if weight.dim() != 2 or input.dim() < 1 or input.shape[-1] != weight.shape[1]:
+        raise ValueError("linear: input [..., K] and weight [N, K] do not match: %s, %s"
+                         % (tuple(input.shape), tuple(weight.shape)))
+    N, K = weight.shape
+    if bias is not None and tuple(bias.shape) != (N,):
+        raise ValueError("linear: bias must have shape [%d]" % N)
+    M = 1
+    for n in input.shape[:-1]:
+        M *= n
+    x = input.reshape(M, K)
+    if x.stride(-1) != 1 and K > 1:
+        x = x.contiguous()
+    w = weight if (weight.stride(-1) == 1 or K == 1) else weight.contiguous()
+    b = bias.contiguous() if bias is not None else None
+    out = torch.empty(M, N, dtype=input.dtype, device=input.device)
+    _launch("ttlinear_forward", _capi.lib().ttlinear_forward, x.device, _DTYPES[x.dtype], x.data_ptr(), w.data_ptr(),
+            b.data_ptr() if b is not None else None, out.data_ptr(), M, N, K,
+            x.stride(0) if M > 1 else max(K, 1), w.stride(0) if N > 1 else max(K, 1), N)
+    return out.reshape(input.shape[:-1] + (N,))
