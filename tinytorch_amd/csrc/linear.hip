@@ -5,8 +5,9 @@
 // steps of 64.  Both operands have K contiguous ("NT"), which is the layout v_mfma_f32_32x32x16 wants for both inputs:
 // a lane supplies 8 consecutive k of one row, so operand fragments are plain 16-byte LDS reads, no transposes.
 //   global -> LDS   global_load_lds_dwordx4, two stages of 64 KB (x tile 256 x 64, w tile 256 x 64); the 16-byte chunks
-//                   of a 128-byte LDS row are XOR-swizzled with the row number so that the 32 rows a fragment read
-//                   touches spread over the banks; the loads for tile t+1 are in flight while tile t is multiplied
+//                   of a 128-byte LDS row are XOR-swizzled with half the row number so that the 32 rows a fragment read
+//                   touches spread over the banks; the loads for tile t+2 are requested while tile t's last k-step
+//                   runs, one barrier per tile
 //   MFMA            the wavefront's 64 (n) x 128 (m) part is computed transposed, A = w rows, B = x rows, so that an
 //                   accumulator register group holds 4 consecutive n of one m: the output is stored as 8-byte pieces
 //                   along its contiguous axis without a transpose
@@ -32,14 +33,17 @@ struct LinArgs {
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 
-constexpr int TM = 256, TN = 256, BK = 64;
-constexpr int ROWB = BK * 2;                 // bytes of an LDS row
-constexpr int XTILE = TM * ROWB;             // 32 KB
-constexpr int STAGE = (TM + TN) * ROWB;      // 64 KB
-constexpr int LIN_LDS = 2 * STAGE;
+constexpr int BK = 64;
+constexpr int ROWB = BK * 2;  // bytes of an LDS row
 
-template <typename TR>
+// TM x TN: the workgroup's output tile, 256 x 256 (two stages of 64 KB) or 128 x 128 for problems with too few large
+// tiles to fill the chip.
+template <typename TR, int TM, int TN>
 __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
+  constexpr int XTILE = TM * ROWB;
+  constexpr int STAGE = (TM + TN) * ROWB;
+  constexpr int XI = TM / 64, WI = TN / 64;  // load instructions per wavefront and tile
+  constexpr int NI = TN / 128, MJ = TM / 64;  // 32 x 32 blocks of a wavefront's part: (TN/4 n) x (TM/2 m)
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
   typedef typename TR::vec4 vec4;
@@ -62,17 +66,23 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
   if (tm >= tiles_m || tn >= tiles_n) return;
   const long long m0 = (long long)tm * TM, n0 = (long long)tn * TN;
 
-  // ---- global -> LDS: wavefront w moves rows 32w .. 32w+31 of both tiles, 8 rows (1 KB) per instruction ----------------
-  // lane l fills (row l/8, chunk slot l%8) and therefore fetches chunk (l%8) ^ (row % 8); rows past the end of the
+  // ---- global -> LDS: wavefront w moves rows (TM/8)w .. of the x tile and (TN/8)w .. of the w tile, 8 rows (1 KB) per instruction
+  // lane l fills (row l/8, chunk slot l%8) and therefore fetches chunk (l%8) ^ ((row / 2) % 8) — two rows share 256
+  // bytes of LDS, so 16 consecutive rows of one logical chunk land in 16 different bank groups; rows past the end of the
   // matrix re-read its last row (their products land in outputs that are not stored)
-  unsigned xoff[4], woff[4];
+  unsigned xoff[XI], woff[WI];
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int row = 32 * wave + 8 * i + (lane >> 3);
-    const int chunk = (lane & 7) ^ (lane >> 3);
+  for (int i = 0; i < XI; i++) {
+    const int row = (TM / 8) * wave + 8 * i + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     long long mr = m0 + row < a.M ? row : a.M - 1 - m0;
-    long long nr = n0 + row < a.N ? row : a.N - 1 - n0;
     xoff[i] = (unsigned)((mr * a.ldx + 8 * chunk) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < WI; i++) {
+    const int row = (TN / 8) * wave + 8 * i + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    long long nr = n0 + row < a.N ? row : a.N - 1 - n0;
     woff[i] = (unsigned)((nr * a.ldw + 8 * chunk) * 2);
   }
   const char* xbase = (const char*)((const T*)a.x + m0 * a.ldx);
@@ -85,66 +95,96 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
   auto dma_tile = [&](int t, int stage) __attribute__((always_inline)) {
     const char* xs = xbase + (long long)t * BK * 2;
     const char* ws = wbase + (long long)t * BK * 2;
-    const unsigned dst = smem_addr + stage * STAGE + (32 * wave) * ROWB;
+    const unsigned dst = smem_addr + stage * STAGE;
 #pragma unroll
-    for (int i = 0; i < 4; i++) dma_issue(xs, xoff[i], dst + 8 * i * ROWB);
+    for (int i = 0; i < XI; i++) dma_issue(xs, xoff[i], dst + ((TM / 8) * wave + 8 * i) * ROWB);
 #pragma unroll
-    for (int i = 0; i < 4; i++) dma_issue(ws, woff[i], dst + XTILE + 8 * i * ROWB);
+    for (int i = 0; i < WI; i++) dma_issue(ws, woff[i], dst + XTILE + ((TN / 8) * wave + 8 * i) * ROWB);
   };
 
-  // ---- this wavefront's part: n rows 64*wn .. +63 of the w tile (A operand), m rows 128*wm .. +127 of the x tile (B) -----
+  // ---- this wavefront's part: n rows (TN/4)*wn .. of the w tile (A operand), m rows (TM/2)*wm .. of the x tile (B) ---------
   const int wn = wave & 3, wm = wave >> 2;
-  // fragment (block, ks): row 32*block + lq, chunk 2*ks + lh at row*128 + 16 * (chunk ^ (row % 8)); row % 8 == lq % 8
-  const unsigned frag = (unsigned)(lq * ROWB + 16 * (lh ^ (lq & 7)));
-  const unsigned wfrag = XTILE + (64 * wn) * ROWB + frag;
-  const unsigned xfrag = (128 * wm) * ROWB + frag;
+  // fragment (block, ks): row 32*block + lq, chunk 2*ks + lh at row*128 + 16 * (chunk ^ ((row/2) % 8)); (row/2) % 8 == (lq/2) % 8
+  const unsigned frag = (unsigned)(lq * ROWB + 16 * (lh ^ ((lq >> 1) & 7)));
+  const unsigned wfrag = XTILE + ((TN / 4) * wn) * ROWB + frag;
+  const unsigned xfrag = ((TM / 2) * wm) * ROWB + frag;
 
-  f32x16 acc[2][4];
+  f32x16 acc[NI][MJ];
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < NI; i++)
 #pragma unroll
     for (int r = 0; r < 16; r++) {
-      const long long n = n0 + 64 * wn + 32 * i + 8 * (r >> 2) + 4 * lh + (r & 3);
+      const long long n = n0 + (TN / 4) * wn + 32 * i + 8 * (r >> 2) + 4 * lh + (r & 3);
       const float b = (a.bias && n < a.N) ? (float)((const T*)a.bias)[n] : 0.f;
 #pragma unroll
-      for (int j = 0; j < 4; j++) acc[i][j][r] = b;
+      for (int j = 0; j < MJ; j++) acc[i][j][r] = b;
     }
 
+  // Operand fragments are double-buffered in registers: while the MFMAs of k-step ks run, the fragments of ks+1 are
+  // on their way from LDS.  The one barrier per tile sits before the MFMAs of a tile's last k-step: by then every
+  // wavefront has taken its last fragment of tile t (its stage may be overwritten: tile t+2 is requested) and its own
+  // loads of tile t+1 have landed (requested a tile earlier), so right after the barrier the first fragments of tile
+  // t+1 are requested and arrive while the last 8 MFMAs of tile t run.
+  vec8 fw[2][NI], fx[2][MJ];
+  auto load_frag = [&](int buf, const char* st, int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NI; i++) fw[buf][i] = *(const vec8*)(st + ((wfrag + 32 * i * ROWB) ^ (unsigned)(32 * ks)));
+#pragma unroll
+    for (int j = 0; j < MJ; j++) fx[buf][j] = *(const vec8*)(st + ((xfrag + 32 * j * ROWB) ^ (unsigned)(32 * ks)));
+  };
+  auto mma = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NI; i++)
+#pragma unroll
+      for (int j = 0; j < MJ; j++) acc[i][j] = TR::mfma32(fw[buf][i], fx[buf][j], acc[i][j]);
+  };
+
   const int ntk = (int)(a.K / BK);
-  if (ntk > 0) dma_tile(0, 0);
-  for (int t = 0; t < ntk; t++) {
-    // tile t has landed (this wavefront's loads; the barrier extends that to everyone's) and every wavefront is done
-    // reading the other stage, which tile t+1 now overwrites
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (ntk > 0) {
+    dma_tile(0, 0);
+    if (ntk > 1) {
+      dma_tile(1, 1);
+      // tile 0's loads; tile 1's XI + WI may still be in flight
+      if constexpr (XI + WI == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (t + 1 < ntk) dma_tile(t + 1, (t + 1) & 1);
+    load_frag(0, smem, 0);
+  }
+  for (int t = 0; t < ntk; t++) {
     const char* st = smem + (t & 1) * STAGE;
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      vec8 wf[2], xf[4];
-#pragma unroll
-      for (int i = 0; i < 2; i++) wf[i] = *(const vec8*)(st + ((wfrag + 32 * i * ROWB) ^ (unsigned)(32 * ks)));
-#pragma unroll
-      for (int j = 0; j < 4; j++) xf[j] = *(const vec8*)(st + ((xfrag + 32 * j * ROWB) ^ (unsigned)(32 * ks)));
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = TR::mfma32(wf[i], xf[j], acc[i][j]);
-    }
+    load_frag(1, st, 1);
+    mma(0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frag(0, st, 2);
+    mma(1);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frag(1, st, 3);
+    mma(0);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (t + 2 < ntk) dma_tile(t + 2, t & 1);
+    if (t + 1 < ntk) load_frag(0, smem + ((t + 1) & 1) * STAGE, 0);
+    mma(1);
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // ---- store: register group rg of acc[i][j] is out[m = .. + 32j + lq][n = .. + 32i + 8rg + 4lh .. +3] ----------------------
 #pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const long long m = m0 + 128 * wm + 32 * j + lq;
+  for (int j = 0; j < MJ; j++) {
+    const long long m = m0 + (TM / 2) * wm + 32 * j + lq;
     if (m >= a.M) continue;
     T* orow = (T*)a.out + m * a.ldo;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < NI; i++)
 #pragma unroll
       for (int rg = 0; rg < 4; rg++) {
-        const long long n = n0 + 64 * wn + 32 * i + 8 * rg + 4 * lh;
+        const long long n = n0 + (TN / 4) * wn + 32 * i + 8 * rg + 4 * lh;
         if (n < a.N) {  // N is a multiple of 4 on this route
           f32x4 v;
 #pragma unroll
@@ -226,18 +266,26 @@ int check(int dtype, const void* x, const void* w, const void* out, long long M,
   return TTSDPA_OK;
 }
 
-template <typename TR>
-int launch_mfma(const LinArgs& a, hipStream_t stream) {
+template <typename TR, int TM, int TN>
+int launch_mfma_tile(const LinArgs& a, hipStream_t stream) {
+  constexpr int lds = 2 * (TM + TN) * ROWB;
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)linear_mfma_kernel<TR>, LIN_LDS, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)linear_mfma_kernel<TR, TM, TN>, lds, state, done);
   if (granted != hipSuccess) return (int)granted;
   const long long tiles_m = (a.M + TM - 1) / TM, tiles_n = (a.N + TN - 1) / TN;
   const long long nsuper = ((tiles_m + 3) / 4) * ((tiles_n + 7) / 8);
   const long long nwg = (nsuper + 7) / 8 * 8 * 32;
   if (nwg > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
-  hipLaunchKernelGGL((linear_mfma_kernel<TR>), dim3((unsigned)nwg), dim3(512), LIN_LDS, stream, a);
+  hipLaunchKernelGGL((linear_mfma_kernel<TR, TM, TN>), dim3((unsigned)nwg), dim3(512), lds, stream, a);
   return (int)hipGetLastError();
+}
+
+template <typename TR>
+int launch_mfma(const LinArgs& a, hipStream_t stream) {
+  // 256 x 256 tiles once they fill the 256 CUs; smaller problems get four times as many 128 x 128 tiles
+  const long long big = ((a.M + 255) / 256) * ((a.N + 255) / 256);
+  return big >= 256 ? launch_mfma_tile<TR, 256, 256>(a, stream) : launch_mfma_tile<TR, 128, 128>(a, stream);
 }
 
 template <typename T>
