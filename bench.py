@@ -8,7 +8,8 @@ resident in HBM.  The headline workload is BASELINE.json's configs[2] (bf16 caus
 D128: the shape the prefill target is quoted on); the decode workload configs[3] (bf16, B64 32q/8kv KV 8192) is
 measured in the same run and reported under "secondary", and config 3's shape in fp32 (the reference's default dtype,
 on the fp32 MFMA kernel, against the 157.3 TFLOP/s fp32 peak) under "fp32", and the row-wise neighbour ops (rmsNorm,
-fusedAddRmsNorm, siluMul, softmax; HBM-bound) under "fused_ops".  One JSON line is printed.
+fusedAddRmsNorm, siluMul, softmax; HBM-bound) under "fused_ops" and the linear layer (QKV projection of the same
+token batch; MFMA-bound) under "linear".  One JSON line is printed.
 
 Algorithmic work per launch (what "achieved" divides by the measured launch time):
   prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)
@@ -257,6 +258,71 @@ def run_fused(name, steps, warmup, cpu=True):
     return res_line
 
 
+LINEAR_WORKLOAD = (8192, 6144, 4096)  # config 3's token batch through the fused QKV projection: [B2 x S4096, 4096] -> 6144
+
+
+def run_linear(steps, warmup, cpu=True):
+    """The linear layer (include/ttlinear.h) at the QKV projection of config 3's token batch, bf16: 2*M*N*K flop per
+    launch / HIP-event time per launch against the bf16 MFMA peak, the compiled reference (one core) on a slice beside it."""
+    import numpy as np
+    import torch
+    from tinytorch_amd import _capi
+
+    M, N, K = LINEAR_WORKLOAD
+    lib = _capi.lib()
+    stream = torch.cuda.current_stream()
+    gen = torch.Generator(device="cuda").manual_seed(0x5EED)
+    x = torch.randn(M, K, device="cuda", generator=gen).bfloat16()
+    w = (torch.randn(N, K, device="cuda", generator=gen) * K ** -0.5).bfloat16()
+    b = torch.randn(N, device="cuda", generator=gen).bfloat16()
+    out = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+
+    def step():
+        rc = lib.ttlinear_forward(_capi.BF16, x.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(), M, N, K, K, K, N,
+                                  stream.cuda_stream)
+        if rc != 0:
+            raise RuntimeError("ttlinear_forward: %s" % _capi.status_string(rc))
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    flops = 2 * M * N * K
+    res = {"workload": "linear bf16 x[%d,%d] . w[%d,%d]^T + bias" % (M, K, N, K), "dtype": "bf16", "ms_per_step": round(ms, 5),
+           "roofline": {"bound": "mfma", "achieved": round(flops / (ms * 1e-3) / 1e12, 1), "peak": PEAK_TFLOPS["bf16"],
+                        "unit": "TFLOP/s", "frac": round(flops / (ms * 1e-3) / 1e12 / PEAK_TFLOPS["bf16"], 4),
+                        "traffic": measured_traffic("linear"), "algorithmic_flops": flops,
+                        "algorithmic_bytes": 2 * (M * K + N * K + M * N + N)}}
+    if cpu:
+        import oracle
+        kind = "reference" if oracle.have_ref() else "port"
+        rows, cols = 16, 256
+        xh = x[:rows].float().cpu().numpy()
+        wh = w[:cols].float().cpu().numpy()
+        bh = b[:cols].float().cpu().numpy()
+        fn = oracle.ref_linear if kind == "reference" else oracle.linear
+        fn(xh[:1], wh[:1], bh[:1])  # the library's one-time set-up stays out of the timing
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            ref = fn(xh, wh, bh)
+            reps += 1
+            spent = time.perf_counter() - t0
+            if spent > 1.0:
+                break
+        got = out[:rows, :cols].float().cpu().numpy()
+        res["cpu_baseline"] = {"value": float("%.4g" % (2.0 * rows * cols * K * reps / spent / 1e12)), "unit": "TFLOP/s", "cores": 1,
+                               "kind": kind, "sample": "a [%d, %d] corner of the output, %d passes in %.1f s, one thread (fp32 on the bf16 values)"
+                               % (rows, cols, reps, spent),
+                               "max_abs_err_gpu_vs_cpu": float("%.3g" % float(np.abs(ref - got).max()))}
+    return res
+
+
 def run_cpu_baseline(name, tensors, budget_s=20.0):
     """The reference CPU path (compiled reference if oracle/_ref is present, else this repository's C restatement)
     on one host core, over as many (batch, head) slices of the same inputs as fit the time budget."""
@@ -310,6 +376,7 @@ def main():
     ap.add_argument("--no-fused", action="store_true", help="skip the row-wise neighbour ops (rmsNorm, siluMul, ...)")
     ap.add_argument("--fused-only", default=None, choices=sorted(FUSED_WORKLOADS),
                     help="measure one row-wise op only and print its line (for profiling)")
+    ap.add_argument("--linear-only", action="store_true", help="measure the linear layer only and print its line (for profiling)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one device-to-device copy of 1 GiB (a kernel of known traffic that calibrates "
                          "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc)")
@@ -329,6 +396,9 @@ def main():
         del src, dst
     if args.fused_only:
         print(json.dumps(run_fused(args.fused_only, args.steps, args.warmup, cpu=not args.no_cpu)), flush=True)
+        return
+    if args.linear_only:
+        print(json.dumps(run_linear(args.steps, args.warmup, cpu=not args.no_cpu)), flush=True)
         return
     main_res, tensors = run_gpu(args.workload, args.steps, args.warmup)
     ceilings = None if args.no_probes else run_probes()
@@ -358,6 +428,8 @@ def main():
         torch.cuda.empty_cache()
         line["fused_ops"] = [run_fused(n, max(1, min(args.steps, 100)), min(args.warmup, 20), cpu=not args.no_cpu)
                              for n in ("rms_norm", "fused_add_rms_norm", "silu_mul", "softmax")]
+        torch.cuda.empty_cache()
+        line["linear"] = run_linear(max(1, min(args.steps, 100)), min(args.warmup, 50), cpu=not args.no_cpu)
     print(json.dumps(line), flush=True)
 
 

@@ -337,7 +337,7 @@ static void test_grad_bookkeeping_and_errors() {
 // The reference's own vectors for the row-wise ops (reference test/test_function.cpp:139-152, 385-391) and fp64 closed
 // forms on longer rows, through function:: on the GPU.
 static void test_row_wise_ops() {
-  std::printf("row-wise ops: rmsNorm, fusedAddRmsNorm, siluMul, softmax, logSoftmax\n");
+  std::printf("row-wise ops and linear: rmsNorm, fusedAddRmsNorm, siluMul, softmax, logSoftmax, linear\n");
   const Options gpu = options::device(DeviceType::GPU);
   {
     Tensor input(std::vector<float>{1.4176f, 0.1874f, 0.8367f, -0.1203f, 2.5638f, -1.2554f}, {2, 3}, gpu);
@@ -395,6 +395,31 @@ static void test_row_wise_ops() {
     Tensor ones = Tensor::ones({dim}, o);
     EXPECT_TRUE(vectorNear(function::rmsNorm(x, {dim}, Tensor{}, 1e-6f).toList<float>(),
                            function::rmsNorm(x, {dim}, ones, 1e-6f).toList<float>(), 1e-6f));
+  }
+  // function::linear: the reference's vector (test/test_function.cpp:234-241) and a bf16 projection against fp64 sums
+  {
+    Tensor x(std::vector<float>{-0.3089f, 0.5301f, -0.0245f, 1.5852f, 0.8954f, 0.7485f}, {2, 3}, gpu);
+    Tensor w(std::vector<float>{0.8397f, 1.7990f, -0.2738f, -0.8910f, -0.6746f, 0.3419f}, {2, 3}, gpu);
+    Tensor b(std::vector<float>{-0.9601f, -1.4163f}, {2}, gpu);
+    std::vector<float> y = function::linear(x, w, b).toList<float>();
+    float total = 0.f;
+    for (float f : y) total += f;
+    EXPECT_TRUE(y.size() == 4 && std::fabs(total - (-3.1661377f)) < 1e-5f);
+    const Options o = options::device(DeviceType::GPU).dtype(DType::BFloat16);
+    const int M = 70, N = 96, K = 128;
+    Tensor xb(pseudoRandom(static_cast<size_t>(3) * M * K, 71), {3, M, K}, o), wb(pseudoRandom(static_cast<size_t>(N) * K, 72), {N, K}, o);
+    Tensor bb(pseudoRandom(N, 73), {N}, o);
+    const std::vector<float> xs = xb.toList<float>(), ws = wb.toList<float>(), bs = bb.toList<float>();
+    std::vector<float> ref(static_cast<size_t>(3) * M * N);
+    for (int m = 0; m < 3 * M; m++)
+      for (int n = 0; n < N; n++) {
+        double s = bs[n];
+        for (int k = 0; k < K; k++) s += static_cast<double>(xs[static_cast<size_t>(m) * K + k]) * ws[static_cast<size_t>(n) * K + k];
+        ref[static_cast<size_t>(m) * N + n] = static_cast<float>(s);
+      }
+    Tensor yb = function::linear(xb, wb, bb);
+    EXPECT_TRUE(yb.dim() == 3 && yb.size(0) == 3 && yb.size(1) == M && yb.size(2) == N);
+    EXPECT_TRUE(vectorNear(yb.toList<float>(), ref, 2e-2f * std::sqrt(static_cast<float>(K))));
   }
   // failed preconditions are loud, like the reference's ASSERTs
   AssertHandler old = setAssertHandler(countingAssertHandler);

@@ -8,6 +8,7 @@
 
 #include "Function.h"
 #include "OpFused.h"
+#include "OpLinalg.h"
 
 namespace tinytorch::function {
 
@@ -48,6 +49,24 @@ class FuncSoftmaxT : public Function<FuncSoftmaxT<LOG>> {
     NOT_IMPLEMENTED();
   }
 };
+
+// function::linear (reference src/Function/FuncNNLayer.h:14-36, 270-272): forward is the reference's single op call;
+// the backward (three more matmul forms) is not part of this inference path.
+class FuncLinear : public Function<FuncLinear> {
+ public:
+  static Tensor forward(AutogradContext* ctx, const Tensor& input, const Tensor& weight, const Tensor& bias) {
+    (void)ctx;
+    return op::matmul(input, weight, false, true, bias);
+  }
+  static void backward(AutogradContext* ctx, const Tensor& grad) {
+    (void)ctx, (void)grad;
+    NOT_IMPLEMENTED();
+  }
+};
+
+inline Tensor linear(const Tensor& input, const Tensor& weight, const Tensor& bias = {}) {
+  return FuncLinear::apply(input, weight, bias);
+}
 
 inline Tensor siluMul(const Tensor& x) { return FuncSiluMul::apply(x); }
 

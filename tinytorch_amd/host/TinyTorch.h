@@ -9,4 +9,5 @@
 #include "Macros.h"
 #include "OpAttention.h"
 #include "OpFused.h"
+#include "OpLinalg.h"
 #include "Tensor.h"
