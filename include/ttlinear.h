@@ -21,8 +21,9 @@ extern "C" {
 
 enum ttlinear_route {
   TTLINEAR_ROUTE_NONE = 0,   /* empty output */
-  TTLINEAR_ROUTE_MFMA = 1,   /* fp16/bf16, K a multiple of 64, 16-byte aligned rows: MFMA kernel, fp32 accumulation */
-  TTLINEAR_ROUTE_GENERAL = 2 /* everything else (fp32, other K, unaligned rows): fp32 arithmetic on the vector ALUs */
+  TTLINEAR_ROUTE_MFMA = 1,   /* K a multiple of 64 (fp16/bf16) or 32 (fp32), 16-byte aligned rows, N a multiple of 4:
+                                MFMA kernel, fp32 accumulation (fp32 tensors: full fp32 products) */
+  TTLINEAR_ROUTE_GENERAL = 2 /* everything else (other K, unaligned rows): fp32 arithmetic on the vector ALUs */
 };
 
 /* out[m, n] = bias[n] + sum_k x[m, k] * w[n, k]   (m < M, n < N, k < K)

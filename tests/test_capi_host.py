@@ -262,7 +262,9 @@ def test_linear_routes_and_validation():
 
     assert plan(_capi.BF16, 8192, 4096, 4096) == (0, "mfma")
     assert plan(_capi.F16, 100, 12, 64) == (0, "mfma")
-    assert plan(_capi.F32, 8192, 4096, 4096) == (0, "general")       # fp32: vector ALUs
+    assert plan(_capi.F32, 8192, 4096, 4096) == (0, "mfma")          # fp32 on the fp32 matrix cores
+    assert plan(_capi.F32, 8192, 4096, 4000) == (0, "mfma")          # K a multiple of 32 suffices in fp32
+    assert plan(_capi.F32, 8192, 4096, 4008) == (0, "general")
     assert plan(_capi.BF16, 8192, 4096, 4000) == (0, "general")      # K not a multiple of 64
     assert plan(_capi.BF16, 8192, 4095, 4096) == (0, "general")      # N not a multiple of 4
     assert plan(_capi.BF16, 64, 64, 64, x=FAKE + 2) == (0, "general")  # rows not 16-byte aligned

@@ -42,6 +42,9 @@ CASES = [
     (1, 4, 64, "bf16", True, "mfma"),            # a single row
     (1100, 2300, 128, "f16", True, "mfma"),      # more than one 4 x 8 block of tiles
     (64, 768, 1024, "bf16", False, "mfma"),
+    (256, 256, 32, "f32", True, "mfma"),         # fp32 on the fp32 matrix cores: one tile, one k step
+    (300, 260, 160, "f32", True, "mfma"),
+    (1100, 520, 96, "f32", False, "mfma"),
     (2, 3, 5, "f32", True, "general"),
     (70, 90, 100, "f32", True, "general"),
     (129, 65, 200, "bf16", True, "general"),     # K not a multiple of 64
@@ -111,3 +114,7 @@ def test_full_size_projection_properties():
     assert float((y.float() - y0.float() - b.float()[None, :]).abs().max()) <= 3e-2   # two roundings apart
     y2 = linear(x * 2, w)   # doubling x is exact in bf16
     assert torch.equal(y2.float(), y0.float() * 2)
+    # the same projection in fp32 (full fp32 products): 1e-4 * sqrt(K) against fp64 on the sampled outputs
+    xf, wf, bf = x.float(), w.float(), b.float()
+    yf = linear(xf, wf, bf)
+    assert float((yf[rows, cols].double() - exact).abs().max()) <= 1e-4 * np.sqrt(K)

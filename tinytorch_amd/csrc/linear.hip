@@ -1,8 +1,8 @@
 // The linear layer y = x . w^T + bias on gfx950 (reference: op::matmul(input, weight, false, true, bias) behind
 // function::linear, src/Function/FuncNNLayer.h:14-19; device GEMM src/Operation/OpLinalgCuda.cuh:239-293).
 //
-// linear_mfma_kernel (fp16 / bf16): a workgroup of 8 wavefronts owns a 256 x 256 tile of the output and walks K in
-// steps of 64.  Both operands have K contiguous ("NT"), which is the layout v_mfma_f32_32x32x16 wants for both inputs:
+// linear_mfma_kernel (fp16 / bf16 on v_mfma_f32_32x32x16, fp32 on v_mfma_f32_32x32x2 with full fp32 products): a workgroup of 8 wavefronts owns a 256 x 256 tile of the output and walks K in
+// steps of 128 bytes (64 or 32 elements).  Both operands have K contiguous ("NT"), which is the layout v_mfma_f32_32x32x16 wants for both inputs:
 // a lane supplies 8 consecutive k of one row, so operand fragments are plain 16-byte LDS reads, no transposes.
 //   global -> LDS   global_load_lds_dwordx4, two stages of 64 KB (x tile 256 x 64, w tile 256 x 64); the 16-byte chunks
 //                   of a 128-byte LDS row are XOR-swizzled with half the row number so that the 32 rows a fragment read
@@ -33,8 +33,34 @@ struct LinArgs {
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 
-constexpr int BK = 64;
-constexpr int ROWB = BK * 2;  // bytes of an LDS row
+constexpr int ROWB = 128;  // bytes of an LDS row: 64 k of a 16-bit type, 32 k of fp32
+
+// What the kernel needs to know about the element type.  A fragment is the 16 bytes a lane reads per 32 x 32 block and
+// k-step: 8 consecutive k (16-bit: one v_mfma_f32_32x32x16) or 4 (fp32: four v_mfma_f32_32x32x2, MFMA e contracting the
+// lanes' e-th elements — lanes 0-31 hold k .. k+3, lanes 32-63 k+4 .. k+7, the same pairing for both operands).
+template <typename TR>
+struct Gemm {
+  typedef typename TR::elem elem;
+  typedef typename TR::vec8 frag;
+  typedef typename TR::vec4 out4;
+  static constexpr int KPC = 8;  // elements per 16-byte chunk
+  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) { return TR::mfma32(a, b, c); }
+  static __device__ __forceinline__ out4 cvt(f32x4 v) { return __builtin_convertvector(v, out4); }
+};
+struct F32 {};
+template <>
+struct Gemm<F32> {
+  typedef float elem;
+  typedef f32x4 frag;
+  typedef f32x4 out4;
+  static constexpr int KPC = 4;
+  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
+    return c;
+  }
+  static __device__ __forceinline__ out4 cvt(f32x4 v) { return v; }
+};
 
 // TM x TN: the workgroup's output tile, 256 x 256 (two stages of 64 KB) or 128 x 128 for problems with too few large
 // tiles to fill the chip.
@@ -44,9 +70,11 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
   constexpr int STAGE = (TM + TN) * ROWB;
   constexpr int XI = TM / 64, WI = TN / 64;  // load instructions per wavefront and tile
   constexpr int NI = TN / 128, MJ = TM / 64;  // 32 x 32 blocks of a wavefront's part: (TN/4 n) x (TM/2 m)
-  typedef typename TR::elem T;
-  typedef typename TR::vec8 vec8;
-  typedef typename TR::vec4 vec4;
+  typedef Gemm<TR> G;
+  typedef typename G::elem T;
+  typedef typename G::frag vec8;  // the 16-byte operand fragment
+  constexpr int BK = (ROWB / 16) * G::KPC;  // k per tile
+  constexpr int ESZ = 16 / G::KPC;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x;
@@ -76,14 +104,14 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
     const int row = (TM / 8) * wave + 8 * i + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     long long mr = m0 + row < a.M ? row : a.M - 1 - m0;
-    xoff[i] = (unsigned)((mr * a.ldx + 8 * chunk) * 2);
+    xoff[i] = (unsigned)((mr * a.ldx + G::KPC * chunk) * ESZ);
   }
 #pragma unroll
   for (int i = 0; i < WI; i++) {
     const int row = (TN / 8) * wave + 8 * i + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     long long nr = n0 + row < a.N ? row : a.N - 1 - n0;
-    woff[i] = (unsigned)((nr * a.ldw + 8 * chunk) * 2);
+    woff[i] = (unsigned)((nr * a.ldw + G::KPC * chunk) * ESZ);
   }
   const char* xbase = (const char*)((const T*)a.x + m0 * a.ldx);
   const char* wbase = (const char*)((const T*)a.w + n0 * a.ldw);
@@ -93,8 +121,8 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   auto dma_tile = [&](int t, int stage) __attribute__((always_inline)) {
-    const char* xs = xbase + (long long)t * BK * 2;
-    const char* ws = wbase + (long long)t * BK * 2;
+    const char* xs = xbase + (long long)t * ROWB;
+    const char* ws = wbase + (long long)t * ROWB;
     const unsigned dst = smem_addr + stage * STAGE;
 #pragma unroll
     for (int i = 0; i < XI; i++) dma_issue(xs, xoff[i], dst + ((TM / 8) * wave + 8 * i) * ROWB);
@@ -136,7 +164,7 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
 #pragma unroll
     for (int i = 0; i < NI; i++)
 #pragma unroll
-      for (int j = 0; j < MJ; j++) acc[i][j] = TR::mfma32(fw[buf][i], fx[buf][j], acc[i][j]);
+      for (int j = 0; j < MJ; j++) acc[i][j] = G::mma(fw[buf][i], fx[buf][j], acc[i][j]);
   };
 
   const int ntk = (int)(a.K / BK);
@@ -189,7 +217,7 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
           f32x4 v;
 #pragma unroll
           for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * rg + e];
-          *(vec4*)(orow + n) = __builtin_convertvector(v, vec4);
+          *(typename G::out4*)(orow + n) = G::cvt(v);
         }
       }
   }
@@ -259,9 +287,10 @@ int check(int dtype, const void* x, const void* w, const void* out, long long M,
   const size_t esz = dtype == TTSDPA_F32 ? 4 : 2;
   if (!aligned(x, esz) || !aligned(w, esz) || !aligned(out, esz)) return TTSDPA_ERR_STRIDE;
   if ((M + 63) / 64 > 65535 || (N + 63) / 64 > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
-  const bool mfma = dtype != TTSDPA_F32 && K > 0 && K % BK == 0 && N % 4 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldo % 4 == 0 &&
-                    aligned(x, 16) && aligned(w, 16) && aligned(out, 8) &&
-                    ldx < (1 << 22) && ldw < (1 << 22);  // 256 rows are addressed with 32-bit byte offsets
+  const long long kpc = 16 / (long long)esz;  // elements per 16 bytes
+  const bool mfma = K > 0 && K % (8 * kpc) == 0 && N % 4 == 0 && ldx % kpc == 0 && ldw % kpc == 0 && ldo % 4 == 0 &&
+                    aligned(x, 16) && aligned(w, 16) && aligned(out, 4 * esz) &&
+                    ldx < (1 << 21) && ldw < (1 << 21);  // 256 rows are addressed with 32-bit byte offsets
   *route = mfma ? TTLINEAR_ROUTE_MFMA : TTLINEAR_ROUTE_GENERAL;
   return TTSDPA_OK;
 }
@@ -320,7 +349,8 @@ int ttlinear_forward(int dtype, const void* x, const void* w, const void* bias, 
   if (bias && !aligned(bias, esz)) return TTSDPA_ERR_STRIDE;
   LinArgs a{x, w, bias, out, M, N, K, ldx, ldw, ldo};
   hipStream_t s = (hipStream_t)stream;
-  if (route == TTLINEAR_ROUTE_MFMA) return dtype == TTSDPA_F16 ? launch_mfma<F16>(a, s) : launch_mfma<BF16>(a, s);
+  if (route == TTLINEAR_ROUTE_MFMA)
+    return dtype == TTSDPA_F32 ? launch_mfma<F32>(a, s) : dtype == TTSDPA_F16 ? launch_mfma<F16>(a, s) : launch_mfma<BF16>(a, s);
   switch (dtype) {
     case TTSDPA_F32: return launch_general_linear<float>(a, s);
     case TTSDPA_F16: return launch_general_linear<_Float16>(a, s);
