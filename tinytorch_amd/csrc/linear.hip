@@ -64,12 +64,14 @@ struct Gemm<F32> {
 
 // TM x TN: the workgroup's output tile, 256 x 256 (two stages of 64 KB) or 128 x 128 for problems with too few large
 // tiles to fill the chip.
-template <typename TR, int TM, int TN>
-__global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
+// WN x WM wavefronts share the tile: a wavefront's part is (TN/WN n) x (TM/WM m).
+template <typename TR, int TM, int TN, int WN, int WM>
+__global__ __launch_bounds__(WN * WM * 64, 1) void linear_mfma_kernel(LinArgs a) {
+  constexpr int NW = WN * WM;
   constexpr int XTILE = TM * ROWB;
   constexpr int STAGE = (TM + TN) * ROWB;
-  constexpr int XI = TM / 64, WI = TN / 64;  // load instructions per wavefront and tile
-  constexpr int NI = TN / 128, MJ = TM / 64;  // 32 x 32 blocks of a wavefront's part: (TN/4 n) x (TM/2 m)
+  constexpr int XI = TM / NW / 8, WI = TN / NW / 8;  // load instructions per wavefront and tile
+  constexpr int NI = TN / WN / 32, MJ = TM / WM / 32;  // 32 x 32 blocks of a wavefront's part
   typedef Gemm<TR> G;
   typedef typename G::elem T;
   typedef typename G::frag vec8;  // the 16-byte operand fragment
@@ -98,51 +100,53 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
   // lane l fills (row l/8, chunk slot l%8) and therefore fetches chunk (l%8) ^ ((row / 2) % 8) — two rows share 256
   // bytes of LDS, so 16 consecutive rows of one logical chunk land in 16 different bank groups; rows past the end of the
   // matrix re-read its last row (their products land in outputs that are not stored)
-  unsigned xoff[XI], woff[WI];
-#pragma unroll
-  for (int i = 0; i < XI; i++) {
-    const int row = (TM / 8) * wave + 8 * i + (lane >> 3);
+  // The byte offset of a lane's chunk is recomputed per request (a handful of vector-ALU operations against the 2048+
+  // MFMA cycles of a tile) rather than held in registers for every row group.
+  const long long mlim = a.M - 1 - m0, nlim = a.N - 1 - n0;  // last valid row of the tiles
+  auto lane_off = [&](int row, long long lim, long long ld) __attribute__((always_inline)) {
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-    long long mr = m0 + row < a.M ? row : a.M - 1 - m0;
-    xoff[i] = (unsigned)((mr * a.ldx + G::KPC * chunk) * ESZ);
-  }
-#pragma unroll
-  for (int i = 0; i < WI; i++) {
-    const int row = (TN / 8) * wave + 8 * i + (lane >> 3);
-    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-    long long nr = n0 + row < a.N ? row : a.N - 1 - n0;
-    woff[i] = (unsigned)((nr * a.ldw + G::KPC * chunk) * ESZ);
-  }
+    const long long r = row < lim ? row : lim;
+    return (unsigned)((r * ld + G::KPC * chunk) * ESZ);
+  };
   const char* xbase = (const char*)((const T*)a.x + m0 * a.ldx);
   const char* wbase = (const char*)((const T*)a.w + n0 * a.ldw);
   const unsigned smem_addr = (unsigned)(unsigned long)(lds_void_t*)smem;
   // issued as asm so that the compiler does not treat it as an LDS store it must order every later LDS read behind
+  // (the lane's full address goes in a register pair: a scalar base operand is not always kept in scalar registers by
+  // the compiler once the tile requests are unrolled)
   auto dma_issue = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+    const char* p = sbase + voff;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(p), "s"(lds_addr) : "memory", "m0");
   };
   auto dma_tile = [&](int t, int stage) __attribute__((always_inline)) {
     const char* xs = xbase + (long long)t * ROWB;
     const char* ws = wbase + (long long)t * ROWB;
     const unsigned dst = smem_addr + stage * STAGE;
 #pragma unroll
-    for (int i = 0; i < XI; i++) dma_issue(xs, xoff[i], dst + ((TM / 8) * wave + 8 * i) * ROWB);
+    for (int i = 0; i < XI; i++) {
+      const int row = (TM / NW) * wave + 8 * i + (lane >> 3);
+      dma_issue(xs, lane_off(row, mlim, a.ldx), dst + ((TM / NW) * wave + 8 * i) * ROWB);
+    }
 #pragma unroll
-    for (int i = 0; i < WI; i++) dma_issue(ws, woff[i], dst + XTILE + ((TN / 8) * wave + 8 * i) * ROWB);
+    for (int i = 0; i < WI; i++) {
+      const int row = (TN / NW) * wave + 8 * i + (lane >> 3);
+      dma_issue(ws, lane_off(row, nlim, a.ldw), dst + XTILE + ((TN / NW) * wave + 8 * i) * ROWB);
+    }
   };
 
   // ---- this wavefront's part: n rows (TN/4)*wn .. of the w tile (A operand), m rows (TM/2)*wm .. of the x tile (B) ---------
-  const int wn = wave & 3, wm = wave >> 2;
+  const int wn = wave % WN, wm = wave / WN;
   // fragment (block, ks): row 32*block + lq, chunk 2*ks + lh at row*128 + 16 * (chunk ^ ((row/2) % 8)); (row/2) % 8 == (lq/2) % 8
   const unsigned frag = (unsigned)(lq * ROWB + 16 * (lh ^ ((lq >> 1) & 7)));
-  const unsigned wfrag = XTILE + ((TN / 4) * wn) * ROWB + frag;
-  const unsigned xfrag = ((TM / 2) * wm) * ROWB + frag;
+  const unsigned wfrag = XTILE + ((TN / WN) * wn) * ROWB + frag;
+  const unsigned xfrag = ((TM / WM) * wm) * ROWB + frag;
 
   f32x16 acc[NI][MJ];
 #pragma unroll
   for (int i = 0; i < NI; i++)
 #pragma unroll
     for (int r = 0; r < 16; r++) {
-      const long long n = n0 + (TN / 4) * wn + 32 * i + 8 * (r >> 2) + 4 * lh + (r & 3);
+      const long long n = n0 + (TN / WN) * wn + 32 * i + 8 * (r >> 2) + 4 * lh + (r & 3);
       const float b = (a.bias && n < a.N) ? (float)((const T*)a.bias)[n] : 0.f;
 #pragma unroll
       for (int j = 0; j < MJ; j++) acc[i][j][r] = b;
@@ -175,6 +179,7 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
       // tile 0's loads; tile 1's XI + WI may still be in flight
       if constexpr (XI + WI == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      static_assert(XI + WI == 8 || XI + WI == 4, "add the matching wait");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
@@ -205,14 +210,14 @@ __global__ __launch_bounds__(512, 2) void linear_mfma_kernel(LinArgs a) {
   // ---- store: register group rg of acc[i][j] is out[m = .. + 32j + lq][n = .. + 32i + 8rg + 4lh .. +3] ----------------------
 #pragma unroll
   for (int j = 0; j < MJ; j++) {
-    const long long m = m0 + (TM / 2) * wm + 32 * j + lq;
+    const long long m = m0 + (TM / WM) * wm + 32 * j + lq;
     if (m >= a.M) continue;
     T* orow = (T*)a.out + m * a.ldo;
 #pragma unroll
     for (int i = 0; i < NI; i++)
 #pragma unroll
       for (int rg = 0; rg < 4; rg++) {
-        const long long n = n0 + (TN / 4) * wn + 32 * i + 8 * rg + 4 * lh;
+        const long long n = n0 + (TN / WN) * wn + 32 * i + 8 * rg + 4 * lh;
         if (n < a.N) {  // N is a multiple of 4 on this route
           f32x4 v;
 #pragma unroll
@@ -295,18 +300,18 @@ int check(int dtype, const void* x, const void* w, const void* out, long long M,
   return TTSDPA_OK;
 }
 
-template <typename TR, int TM, int TN>
+template <typename TR, int TM, int TN, int WN, int WM>
 int launch_mfma_tile(const LinArgs& a, hipStream_t stream) {
   constexpr int lds = 2 * (TM + TN) * ROWB;
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)linear_mfma_kernel<TR, TM, TN>, lds, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)linear_mfma_kernel<TR, TM, TN, WN, WM>, lds, state, done);
   if (granted != hipSuccess) return (int)granted;
   const long long tiles_m = (a.M + TM - 1) / TM, tiles_n = (a.N + TN - 1) / TN;
   const long long nsuper = ((tiles_m + 3) / 4) * ((tiles_n + 7) / 8);
   const long long nwg = (nsuper + 7) / 8 * 8 * 32;
   if (nwg > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
-  hipLaunchKernelGGL((linear_mfma_kernel<TR, TM, TN>), dim3((unsigned)nwg), dim3(512), lds, stream, a);
+  hipLaunchKernelGGL((linear_mfma_kernel<TR, TM, TN, WN, WM>), dim3((unsigned)nwg), dim3(WN * WM * 64), lds, stream, a);
   return (int)hipGetLastError();
 }
 
@@ -314,7 +319,9 @@ template <typename TR>
 int launch_mfma(const LinArgs& a, hipStream_t stream) {
   // 256 x 256 tiles once they fill the 256 CUs; smaller problems get four times as many 128 x 128 tiles
   const long long big = ((a.M + 255) / 256) * ((a.N + 255) / 256);
-  return big >= 256 ? launch_mfma_tile<TR, 256, 256>(a, stream) : launch_mfma_tile<TR, 128, 128>(a, stream);
+  // (four wavefronts with 128 x 128 each — accumulators in AGPRs, half the LDS operand reads — measured 2-10 % slower
+  // than eight with 64 x 128: one wavefront per SIMD hides too little)
+  return big >= 256 ? launch_mfma_tile<TR, 256, 256, 4, 2>(a, stream) : launch_mfma_tile<TR, 128, 128, 4, 2>(a, stream);
 }
 
 template <typename T>
