@@ -93,11 +93,12 @@ def test_routes_depend_on_flags():
     p = params(*base)
     p.q = FAKE + 2
     assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL
-    # fp32: the MFMA kernel takes no attnMask and needs 16-byte aligned rows
+    # fp32: the MFMA kernel takes attnMask and per-batch key counts, and needs 16-byte aligned rows
     f32 = (_capi.F32, 2, 8, 2, 512, 512, 128)
     assert _capi.plan(params(*f32, causal=1))[1] == _capi.ROUTE_PREFILL
-    assert _capi.plan(params(*f32, mask_kind=_capi.MASK_ADD, mask=FAKE))[1] == _capi.ROUTE_GENERAL
-    assert _capi.plan(params(*f32, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(*f32, mask_kind=_capi.MASK_ADD, mask=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(*f32, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.F32, 2, 8, 2, 512, 512, 96, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
     p = params(*f32)
     p.v_stride[2] = 130
     assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL

@@ -548,3 +548,50 @@ def test_fp32_mfma_gqa_equals_repeated_kv_bitwise():
     rc2, b = call("prefill", dev[0], dev[1].repeat_interleave(G, 1), dev[2].repeat_interleave(G, 1), causal=True)
     assert rc == 0 and rc2 == 0
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("mshape,kind", [((2, 1, 1, 333), "bool"), ((200, 333), "bool"), ((2, 4, 200, 333), "float"),
+                                         ((4, 1, 333), "float"), ((333,), "bool")])
+@pytest.mark.parametrize("D", [64, 128])
+def test_fp32_mfma_masks(mshape, kind, D):
+    """attnMask on the fp32 MFMA kernel: every broadcastable shape, Bool and additive, against the oracle; rows whose
+    keys are all hidden give NaN on both sides."""
+    B, Hq, Hkv, L, S = 2, 4, 2, 200, 333
+    say("fp32 mfma mask", mshape, kind, D)
+    host, dev = make_inputs(6100 + D, B, Hq, Hkv, L, S, D, "f32")
+    rng = np.random.default_rng(len(mshape) * 10 + D)
+    if kind == "bool":
+        m = (rng.random(mshape) > 0.3)
+        m[..., 0] = True                     # at least one visible key per row
+        if len(mshape) >= 2 and mshape[-2] == L:
+            m[..., 5, :] = False              # except one row, hidden entirely
+        mh, md = m.astype(np.uint8), torch.from_numpy(m).cuda()
+    else:
+        mh = rng.standard_normal(mshape).astype(np.float32) * 2
+        md = torch.from_numpy(mh).cuda()
+    exp = oracle.sdpa_f32(*host, mask=mh)
+    assert route_of(*dev, mask=md) == "prefill"
+    rc, out = call("forward", *dev, mask=md)
+    assert rc == 0
+    y = to_host_f32(out)
+    assert np.array_equal(np.isnan(y), np.isnan(exp))
+    ok = ~np.isnan(exp)
+    assert np.abs(y[ok] - exp[ok]).max() <= TOL["f32"]
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_fp32_mfma_per_batch_key_counts(causal):
+    B, Hq, Hkv, L, S, D = 4, 4, 2, 150, 400, 128
+    host, dev = make_inputs(6200, B, Hq, Hkv, L, S, D, "f32")
+    lens = [400, 137, 0, 9999]
+    kv = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    assert route_of(*dev, causal=causal, kv_lens=kv) == "prefill"
+    rc, out = call("forward", *dev, causal=causal, kv_lens=kv)
+    assert rc == 0
+    for b, n in enumerate(lens):
+        n = min(n, S)
+        if n == 0:
+            assert torch.count_nonzero(out[b]) == 0
+            continue
+        exp = oracle.sdpa_f32(host[0][b:b + 1], host[1][b:b + 1, :, :n], host[2][b:b + 1, :, :n], causal=causal)
+        assert max_abs_err(out[b:b + 1], exp) <= TOL["f32"], b

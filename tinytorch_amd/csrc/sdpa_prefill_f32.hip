@@ -1,7 +1,7 @@
 // Flash-attention forward for fp32 tensors on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32, full fp32 products
 // and sums): fp32 is the reference's default dtype, and its fp32 path is what the 1e-4 parity bar is stated against.
 // Replaces the same device chain as the 16-bit kernels (reference src/Function/FuncNNLayer.h:237-265): the score
-// matrix never leaves registers.  head_dim 64 or 128, no attnMask (those calls take the vector-ALU kernel).
+// matrix never leaves registers.  head_dim 64 or 128; attnMask and per-batch key counts are applied in the kernel.
 //
 // A workgroup of 4 wavefronts owns 128 query rows of one (batch, query head), 32 rows per wavefront; keys/values come
 // in tiles of 32, staged global -> registers -> LDS, double-buffered.
@@ -36,7 +36,8 @@ struct F32Lds {
   static constexpr int BYTES = 2 * STAGE * 4;
 };
 
-template <int D, bool CAUSAL>
+// MASKED: an attnMask is applied (a variant of its own: the mask addressing costs registers the other variants keep).
+template <int D, bool CAUSAL, bool MASKED>
 __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
   typedef F32Lds<D> Lds;
   constexpr int K_PITCH = Lds::K_PITCH, V_PITCH = Lds::V_PITCH;
@@ -105,11 +106,24 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
   float mc = m_use * c;
   float l_run = 0.f;
 
-  int ntiles_kv = (a.S + BN - 1) / BN;
-  const int coff = CAUSAL ? causal_offset(a, a.S) : 0;  // query row i sees keys up to i + coff
+  int S = a.S;  // keys of this batch entry: all of them, or the filled prefix of a cache / the unpadded length
+  if (a.kv_len) {
+    int len = __builtin_amdgcn_readfirstlane(a.kv_len[b]);
+    S = len < 0 ? 0 : (len < S ? len : S);
+  }
+  if (S == 0) {  // no keys: zeros, the reference's empty contraction
+    const int qi = qw0 + lq;
+    if (qi < a.L) {
+      float* op = (float*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2];
+      for (int d = 4 * lh; d < D; d += 8) *(f32x4*)(op + d) = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+    return;
+  }
+  int ntiles_kv = (S + BN - 1) / BN;
+  const int coff = CAUSAL ? causal_offset(a, S) : 0;  // query row i sees keys up to i + coff
   if (CAUSAL) {
     int last = (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1) + coff;
-    int lastkv = last < a.S - 1 ? last : a.S - 1;
+    int lastkv = last < S - 1 ? last : S - 1;
     ntiles_kv = lastkv / BN + 1;
   }
 
@@ -126,7 +140,7 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
       int key = kv0 + lrow[i];
-      key = key < a.S ? key : a.S - 1;  // rows past the end re-read the last valid row (masked later)
+      key = key < S ? key : S - 1;  // rows past the end re-read the last valid row (masked later)
       kst[i] = *(const f32x4*)(kp + key * a.ks[2] + 4 * lcol[i]);
       vst[i] = *(const f32x4*)(vp + key * a.vs[2] + 4 * lcol[i]);
     }
@@ -177,13 +191,33 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
       for (int r = 0; r < 16; r++) s[r] = s0[r] + s1[r];
 
       // ---- mask the diagonal / ragged tile -----------------------------------------------------------------------------
-      if ((CAUSAL && kv0 + BN - 1 > qw0 + coff) || (kv0 + BN > a.S)) {
+      if ((CAUSAL && kv0 + BN - 1 > qw0 + coff) || (kv0 + BN > S)) {
         const int qi = qw0 + lq + coff;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-          bool hidden = key >= a.S || (CAUSAL && key > qi);
+          bool hidden = key >= S || (CAUSAL && key > qi);
           if (hidden) s[r] = -INFINITY;
+        }
+      }
+      // attnMask (reference src/Function/FuncNNLayer.h:249-260): Bool -> hidden keys get -inf; additive -> the bias joins
+      // the scaled score, i.e. bias / scale the raw score held here.  Element strides of 0 broadcast an axis.
+      if (MASKED) {
+        int qi = qw0 + lq;
+        qi = qi < a.L ? qi : a.L - 1;
+        const long long mrow = b * a.ms[0] + h * a.ms[1] + qi * a.ms[2];
+        const float inv_scale = 1.f / a.scale;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          if (key < S) {
+            const long long at = mrow + key * a.ms[3];
+            if (a.mask_kind == 1) {
+              if (((const uint8_t*)a.mask)[at] == 0) s[r] = -INFINITY;
+            } else {
+              s[r] += ((const float*)a.mask)[at] * inv_scale;
+            }
+          }
         }
       }
 
@@ -243,13 +277,13 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
   }
 }
 
-template <int D, bool CAUSAL>
+template <int D, bool CAUSAL, bool MASKED>
 int launch_f32_k(const KArgs& a, dim3 grid, hipStream_t stream) {
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)prefill_f32_kernel<D, CAUSAL>, F32Lds<D>::BYTES, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill_f32_kernel<D, CAUSAL, MASKED>, F32Lds<D>::BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
-  hipLaunchKernelGGL((prefill_f32_kernel<D, CAUSAL>), grid, dim3(256), F32Lds<D>::BYTES, stream, a);
+  hipLaunchKernelGGL((prefill_f32_kernel<D, CAUSAL, MASKED>), grid, dim3(256), F32Lds<D>::BYTES, stream, a);
   return (int)hipGetLastError();
 }
 
@@ -258,8 +292,11 @@ int launch_f32_k(const KArgs& a, dim3 grid, hipStream_t stream) {
 int launch_prefill_f32(const KArgs& a, hipStream_t stream) {
   long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM);
   dim3 grid((unsigned)nwg);
-  if (a.D == 128) return a.causal ? launch_f32_k<128, true>(a, grid, stream) : launch_f32_k<128, false>(a, grid, stream);
-  return a.causal ? launch_f32_k<64, true>(a, grid, stream) : launch_f32_k<64, false>(a, grid, stream);
+  if (a.mask_kind != 0)  // exclusive with causal (validated by the caller, as the reference asserts)
+    return a.D == 128 ? launch_f32_k<128, false, true>(a, grid, stream) : launch_f32_k<64, false, true>(a, grid, stream);
+  if (a.D == 128)
+    return a.causal ? launch_f32_k<128, true, false>(a, grid, stream) : launch_f32_k<128, false, false>(a, grid, stream);
+  return a.causal ? launch_f32_k<64, true, false>(a, grid, stream) : launch_f32_k<64, false, false>(a, grid, stream);
 }
 
 }  // namespace ttsdpa

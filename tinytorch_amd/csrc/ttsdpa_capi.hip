@@ -91,7 +91,7 @@ bool fast_layout_ok(const ttsdpa_params* p, bool masks_ok = false, bool pages_ok
 
 // fp32 tensors the fp32 MFMA kernel can read and write with 16-byte accesses.
 bool f32_prefill_ok(const ttsdpa_params* p) {
-  if (p->dtype != TTSDPA_F32 || p->mask_kind != TTSDPA_MASK_NONE || p->kv_len || p->block_table) return false;
+  if (p->dtype != TTSDPA_F32 || p->block_table) return false;
   if (p->D != 128 && p->D != 64) return false;
   if (!(p->scale > 0.f) || !isfinite(p->scale) || p->S < 1 || p->L < 1) return false;
   if (!dense_last_ok(p->q_stride, 4) || !dense_last_ok(p->k_stride, 4) || !dense_last_ok(p->v_stride, 4) ||
