@@ -82,10 +82,11 @@ def test_routes(args, route):
 def test_routes_depend_on_flags():
     base = (_capi.BF16, 2, 8, 2, 512, 512, 128)
     assert _capi.plan(params(*base, causal=1))[1] == _capi.ROUTE_PREFILL
-    # an attnMask is taken by the pipelined head_dim-128 kernel (L > 128); other masked shapes go to the general kernel
+    # an attnMask is taken by every MFMA prefill kernel; head sizes they do not cover go to the general kernel
     assert _capi.plan(params(*base, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_PREFILL
-    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 64, 512, 128, mask_kind=_capi.MASK_ADD, mask=FAKE))[1] == _capi.ROUTE_GENERAL
-    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 512, 512, 64, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 64, 512, 128, mask_kind=_capi.MASK_ADD, mask=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 512, 512, 64, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 512, 512, 80, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
     assert _capi.plan(params(*base, scale=-1.0))[1] == _capi.ROUTE_GENERAL
     p = params(*base)
     p.k_stride[2] = 132  # rows not 16-byte aligned
@@ -147,8 +148,9 @@ def test_kv_len_routes_and_append_validation():
     base = (_capi.BF16, 2, 32, 8, 4096, 4096, 128)
     assert _capi.plan(params(*base, causal=1))[1] == _capi.ROUTE_PREFILL
     assert _capi.plan(params(*base, causal=1, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
-    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 4096, 4096, 64, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
-    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 100, 4096, 128, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 4096, 4096, 64, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 100, 4096, 128, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 100, 4096, 80, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
     assert _capi.plan(params(_capi.BF16, 8, 32, 8, 1, 4096, 128, kv_len=FAKE))[1] == _capi.ROUTE_DECODE
     assert _capi.plan(params(_capi.BF16, 8, 32, 8, 1, 4096, 128, kv_len=FAKE + 2))[0] == _capi.ERR_STRIDE
     L = _capi.lib()

@@ -550,15 +550,21 @@ def test_fp32_mfma_gqa_equals_repeated_kv_bitwise():
     assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize("mshape,kind", [((2, 1, 1, 333), "bool"), ((200, 333), "bool"), ((2, 4, 200, 333), "float"),
-                                         ((4, 1, 333), "float"), ((333,), "bool")])
-@pytest.mark.parametrize("D", [64, 128])
-def test_fp32_mfma_masks(mshape, kind, D):
-    """attnMask on the fp32 MFMA kernel: every broadcastable shape, Bool and additive, against the oracle; rows whose
-    keys are all hidden give NaN on both sides."""
-    B, Hq, Hkv, L, S = 2, 4, 2, 200, 333
-    say("fp32 mfma mask", mshape, kind, D)
-    host, dev = make_inputs(6100 + D, B, Hq, Hkv, L, S, D, "f32")
+@pytest.mark.parametrize("mshape,kind", [((2, 1, 1, 336), "bool"), ((200, 336), "bool"), ((2, 4, 200, 336), "float"),
+                                         ((4, 1, 336), "float"), ((336,), "bool"), ((200, 333), "bool"),
+                                         ((2, 4, 200, 333), "float")])
+@pytest.mark.parametrize("D,dtype", [(64, "f32"), (128, "f32"), (64, "bf16"), (256, "f16"), (128, "bf16")])
+def test_masks_on_the_simple_mfma_kernels(mshape, kind, D, dtype):
+    """attnMask on the fp32 MFMA kernel and on the 4-wavefront 16-bit kernel (head_dim != 128, or few query rows):
+    every broadcastable shape, Bool and additive, against the oracle; rows whose keys are all hidden give NaN on both
+    sides.  These kernels read the mask four keys at a time; a key count that is not a multiple of 4 goes to the
+    vector-ALU kernel (the pipelined head_dim-128 kernel takes any mask)."""
+    S = mshape[-1]
+    B, Hq, Hkv, L = 2, 4, 2, (200 if not (D == 128 and dtype == "bf16") else 100)
+    if len(mshape) >= 2 and mshape[-2] == 200:
+        mshape = mshape[:-2] + (L, S)
+    say("mask on simple mfma kernels", mshape, kind, D, dtype)
+    host, dev = make_inputs(6100 + D, B, Hq, Hkv, L, S, D, dtype)
     rng = np.random.default_rng(len(mshape) * 10 + D)
     if kind == "bool":
         m = (rng.random(mshape) > 0.3)
@@ -567,16 +573,16 @@ def test_fp32_mfma_masks(mshape, kind, D):
             m[..., 5, :] = False              # except one row, hidden entirely
         mh, md = m.astype(np.uint8), torch.from_numpy(m).cuda()
     else:
-        mh = rng.standard_normal(mshape).astype(np.float32) * 2
-        md = torch.from_numpy(mh).cuda()
+        mv, mb = oracle.round_to(rng.standard_normal(mshape).astype(np.float32) * 2, dtype)
+        mh, md = mv, to_device(mv, mb, dtype)
     exp = oracle.sdpa_f32(*host, mask=mh)
-    assert route_of(*dev, mask=md) == "prefill"
+    assert route_of(*dev, mask=md) == ("prefill" if S % 4 == 0 else "general")
     rc, out = call("forward", *dev, mask=md)
     assert rc == 0
     y = to_host_f32(out)
     assert np.array_equal(np.isnan(y), np.isnan(exp))
     ok = ~np.isnan(exp)
-    assert np.abs(y[ok] - exp[ok]).max() <= TOL["f32"]
+    assert np.abs(y[ok] - exp[ok]).max() <= TOL[dtype]
 
 
 @pytest.mark.parametrize("causal", [False, True])

@@ -24,6 +24,7 @@ struct KArgs {
   float scale;
   long long qs[3], ks[3], vs[3], os[3];  // element strides: batch, head, sequence
   long long ms[4];                       // mask element strides: batch, head, query row, key (0 = broadcast)
+  int mask_vec4;  // keys are contiguous in the mask and groups of 4 keys starting at a multiple of 4 are naturally aligned
 };
 
 // Offset of the causal diagonal in key coordinates for a batch entry with S keys.
@@ -102,6 +103,49 @@ __device__ __forceinline__ float load_as_float(const _Float16* p) { return (floa
 __device__ __forceinline__ void store_from_float(float* p, float x) { *p = x; }
 __device__ __forceinline__ void store_from_float(__bf16* p, float x) { *p = (__bf16)x; }
 __device__ __forceinline__ void store_from_float(_Float16* p, float x) { *p = (_Float16)x; }
+
+// attnMask applied to the 32 x 32 score block of an MFMA accumulator (reference src/Function/FuncNNLayer.h:249-260):
+// a lane holds one query row (mask row offset `mrow`, in elements) and, in register group rg, the four consecutive
+// keys kv0 + 8*rg + 4*lh .. +3.  Bool: hidden keys get -inf; additive: the bias joins the scaled score, i.e.
+// bias * inv_scale the raw score held here.  Element strides of 0 broadcast an axis.  Keys at or beyond S are left
+// alone (masked by the caller).  With a.mask_vec4 a group of four keys is one load.  VEC_ONLY: the caller guarantees
+// a.mask_vec4 and S % 4 == 0, and the element-wise path (and its registers) is left out.
+template <typename T, bool VEC_ONLY>
+__device__ __forceinline__ void apply_attn_mask(const KArgs& a, f32x16& s, long long mrow, int kv0, int lh, int S,
+                                                float inv_scale) {
+#pragma unroll
+  for (int rg = 0; rg < 4; rg++) {
+    const int key0 = kv0 + 8 * rg + 4 * lh;
+    if (VEC_ONLY && key0 >= S) continue;
+    if (VEC_ONLY || (a.mask_vec4 && key0 + 3 < S)) {
+      const long long at = mrow + key0;
+      if (a.mask_kind == 1) {
+        const uint32_t w = *(const uint32_t*)((const uint8_t*)a.mask + at);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (((w >> (8 * e)) & 0xffu) == 0) s[4 * rg + e] = -INFINITY;
+      } else {
+        typedef T vec4t __attribute__((ext_vector_type(4)));
+        const vec4t w = *(const vec4t*)((const T*)a.mask + at);
+#pragma unroll
+        for (int e = 0; e < 4; e++) s[4 * rg + e] += (float)w[e] * inv_scale;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int key = key0 + e;
+        if (key < S) {
+          const long long at = mrow + key * a.ms[3];
+          if (a.mask_kind == 1) {
+            if (((const uint8_t*)a.mask)[at] == 0) s[4 * rg + e] = -INFINITY;
+          } else {
+            s[4 * rg + e] += (float)((const T*)a.mask)[at] * inv_scale;
+          }
+        }
+      }
+    }
+  }
+}
 
 // Host-side launchers (one per kernel family); each returns a hipError_t as int.
 int launch_general(const KArgs& a, int dtype, hipStream_t stream);

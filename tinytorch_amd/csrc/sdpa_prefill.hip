@@ -59,7 +59,8 @@ __device__ __forceinline__ vec8 v_operand(const void* lane_base, int byte_off_lo
   return __builtin_bit_cast(vec8, r);
 }
 
-template <typename TR, int D, bool CAUSAL>
+// MASKED: an attnMask is applied (a variant of its own: the mask addressing costs registers the other variants keep).
+template <typename TR, int D, bool CAUSAL, bool MASKED>
 __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
@@ -126,11 +127,27 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
   float mc = m_use * c;
   float l_run = 0.f;     // this lane's share of the running row sum
 
-  int ntiles_kv = (a.S + BN - 1) / BN;
-  const int coff = CAUSAL ? causal_offset(a, a.S) : 0;  // query row i sees keys up to i + coff
+  int S = a.S;  // keys of this batch entry: all of them, or the filled prefix of a cache / the unpadded length
+  if (a.kv_len) {
+    int len = __builtin_amdgcn_readfirstlane(a.kv_len[b]);
+    S = len < 0 ? 0 : (len < S ? len : S);
+  }
+  if (S == 0) {  // no keys: zeros, the reference's empty contraction
+    const int qi = qw0 + lq;
+    if (qi < a.L) {
+      T* op = (T*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2];
+      typename TR::vec4 zero;
+#pragma unroll
+      for (int i = 0; i < 4; i++) zero[i] = (T)0.f;
+      for (int d = 4 * lh; d < D; d += 8) *(typename TR::vec4*)(op + d) = zero;
+    }
+    return;
+  }
+  int ntiles_kv = (S + BN - 1) / BN;
+  const int coff = CAUSAL ? causal_offset(a, S) : 0;  // query row i sees keys up to i + coff
   if (CAUSAL) {
     int last = (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1) + coff;  // last key of the workgroup's last query row
-    int lastkv = last < a.S - 1 ? last : a.S - 1;
+    int lastkv = last < S - 1 ? last : S - 1;
     ntiles_kv = lastkv / BN + 1;
   }
 
@@ -150,7 +167,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
   auto load_tile = [&](int kv0) {
     const char* kt = (const char*)(kp + kv0 * a.ks[2]);
     const char* vt = (const char*)(vp + kv0 * a.vs[2]);
-    if (kv0 + BN <= a.S) {
+    if (kv0 + BN <= S) {
 #pragma unroll
       for (int i = 0; i < NLD; i++) {
         kst[i] = *(const u32x4*)(kt + koff[i]);
@@ -160,7 +177,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
 #pragma unroll
       for (int i = 0; i < NLD; i++) {
         int key = kv0 + lrow[i];
-        key = key < a.S ? key : a.S - 1;
+        key = key < S ? key : S - 1;
         kst[i] = *(const u32x4*)(kp + key * a.ks[2] + 8 * lcol[i]);
         vst[i] = *(const u32x4*)(vp + key * a.vs[2] + 8 * lcol[i]);
       }
@@ -212,7 +229,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
       }
 
       // ---- mask the diagonal / ragged tile -----------------------------------------------------------------------
-      const bool need_mask = (CAUSAL && kv0 + BN - 1 > qw0 + coff) || (kv0 + BN > a.S);
+      const bool need_mask = (CAUSAL && kv0 + BN - 1 > qw0 + coff) || (kv0 + BN > S);
       if (need_mask) {
         const int qi = qw0 + lq + coff;
 #pragma unroll
@@ -220,9 +237,16 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
 #pragma unroll
           for (int r = 0; r < 16; r++) {
             int key = kv0 + 32 * blk + 8 * (r >> 2) + 4 * lh + (r & 3);
-            bool hidden = key >= a.S || (CAUSAL && key > qi);
+            bool hidden = key >= S || (CAUSAL && key > qi);
             if (hidden) sacc[blk][r] = -INFINITY;
           }
+      }
+      if (MASKED) {
+        int qi = qw0 + lq;
+        qi = qi < a.L ? qi : a.L - 1;
+        const long long mrow = b * a.ms[0] + h * a.ms[1] + qi * a.ms[2];
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) apply_attn_mask<T, true>(a, sacc[blk], mrow, kv0 + 32 * blk, lh, S, 1.f / a.scale);
       }
 
       // ---- online softmax with a lazily raised maximum ---------------------------------------------------------------
@@ -297,13 +321,13 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
   }
 }
 
-template <typename TR, int D, bool CAUSAL>
+template <typename TR, int D, bool CAUSAL, bool MASKED>
 int launch_prefill_k(const KArgs& a, dim3 grid, hipStream_t stream) {
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)prefill_kernel<TR, D, CAUSAL>, PrefillLds<D>::BYTES, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill_kernel<TR, D, CAUSAL, MASKED>, PrefillLds<D>::BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
-  hipLaunchKernelGGL((prefill_kernel<TR, D, CAUSAL>), grid, dim3(256), PrefillLds<D>::BYTES, stream, a);
+  hipLaunchKernelGGL((prefill_kernel<TR, D, CAUSAL, MASKED>), grid, dim3(256), PrefillLds<D>::BYTES, stream, a);
   return (int)hipGetLastError();
 }
 
@@ -311,7 +335,8 @@ template <typename TR, int D>
 int launch_prefill_t(const KArgs& a, hipStream_t stream) {
   long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM);
   dim3 grid((unsigned)nwg);
-  return a.causal ? launch_prefill_k<TR, D, true>(a, grid, stream) : launch_prefill_k<TR, D, false>(a, grid, stream);
+  if (a.mask_kind != 0) return launch_prefill_k<TR, D, false, true>(a, grid, stream);  // exclusive with causal (validated)
+  return a.causal ? launch_prefill_k<TR, D, true, false>(a, grid, stream) : launch_prefill_k<TR, D, false, false>(a, grid, stream);
 }
 
 }  // namespace

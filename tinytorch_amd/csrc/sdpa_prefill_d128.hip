@@ -306,25 +306,10 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     }
   };
 
-  // attnMask (reference src/Function/FuncNNLayer.h:249-260): Bool -> hidden keys get -inf; additive -> the bias is
-  // added to the scaled score, i.e. bias / scale to the raw score held here.  Element strides of 0 broadcast an axis.
   auto user_mask_half = [&](f32x16& s, int kv0) __attribute__((always_inline)) {
     int qi = qw0 + lq;
     qi = qi < a.L ? qi : a.L - 1;
-    const long long mrow = b * a.ms[0] + h * a.ms[1] + qi * a.ms[2];
-    const float inv_scale = 1.f / a.scale;
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-      if (key < S) {
-        const long long at = mrow + key * a.ms[3];
-        if (a.mask_kind == 1) {
-          if (((const uint8_t*)a.mask)[at] == 0) s[r] = -INFINITY;
-        } else {
-          s[r] += (float)((const T*)a.mask)[at] * inv_scale;
-        }
-      }
-    }
+    apply_attn_mask<T, false>(a, s, b * a.ms[0] + h * a.ms[1] + qi * a.ms[2], kv0, lh, S, 1.f / a.scale);
   };
 
   auto row_max = [&](const f32x16& s) __attribute__((always_inline)) {

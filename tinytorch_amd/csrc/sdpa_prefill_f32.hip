@@ -200,25 +200,10 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
           if (hidden) s[r] = -INFINITY;
         }
       }
-      // attnMask (reference src/Function/FuncNNLayer.h:249-260): Bool -> hidden keys get -inf; additive -> the bias joins
-      // the scaled score, i.e. bias / scale the raw score held here.  Element strides of 0 broadcast an axis.
       if (MASKED) {
         int qi = qw0 + lq;
         qi = qi < a.L ? qi : a.L - 1;
-        const long long mrow = b * a.ms[0] + h * a.ms[1] + qi * a.ms[2];
-        const float inv_scale = 1.f / a.scale;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-          if (key < S) {
-            const long long at = mrow + key * a.ms[3];
-            if (a.mask_kind == 1) {
-              if (((const uint8_t*)a.mask)[at] == 0) s[r] = -INFINITY;
-            } else {
-              s[r] += ((const float*)a.mask)[at] * inv_scale;
-            }
-          }
-        }
+        apply_attn_mask<float, true>(a, s, b * a.ms[0] + h * a.ms[1] + qi * a.ms[2], kv0, lh, S, 1.f / a.scale);
       }
 
       // ---- online softmax with a lazily raised maximum -----------------------------------------------------------------

@@ -25,6 +25,14 @@ int effective_causal(const ttsdpa_params* p) {
   return TTSDPA_CAUSAL_BOTTOM_RIGHT;
 }
 
+// Groups of four consecutive keys of the mask (starting at multiples of 4) can be read with one aligned load.
+bool mask_vec4_ok(const ttsdpa_params* p) {
+  if (p->mask_kind != TTSDPA_MASK_BOOL && p->mask_kind != TTSDPA_MASK_ADD) return false;
+  const size_t mesz = p->mask_kind == TTSDPA_MASK_BOOL ? 1 : (p->dtype == TTSDPA_F32 ? 4 : 2);
+  return p->mask_stride[3] == 1 && p->mask_stride[0] % 4 == 0 && p->mask_stride[1] % 4 == 0 && p->mask_stride[2] % 4 == 0 &&
+         ptr_aligned(p->mask, 4 * mesz);
+}
+
 // Validation shared by every entry point; fills the kernel argument block.
 int validate(const ttsdpa_params* p, KArgs* a) {
   if (!p) return TTSDPA_ERR_NULL;
@@ -55,6 +63,7 @@ int validate(const ttsdpa_params* p, KArgs* a) {
     a->ms[i] = p->mask_kind != TTSDPA_MASK_NONE ? p->mask_stride[i] : 0;
   }
   if (p->mask_kind == TTSDPA_MASK_ADD && !ptr_aligned(p->mask, esz)) return TTSDPA_ERR_STRIDE;
+  a->mask_vec4 = mask_vec4_ok(p) ? 1 : 0;
   if (p->kv_len && !ptr_aligned(p->kv_len, 4)) return TTSDPA_ERR_STRIDE;
   a->kv_len = p->kv_len;
   a->block_table = p->block_table, a->page_shift = 0, a->bt_stride = p->block_table_stride;
@@ -89,9 +98,14 @@ bool fast_layout_ok(const ttsdpa_params* p, bool masks_ok = false, bool pages_ok
   return ptr_aligned(p->q, 16) && ptr_aligned(p->k, 16) && ptr_aligned(p->v, 16) && ptr_aligned(p->out, 16);
 }
 
+// The 4-wavefront and fp32 kernels read an attnMask four keys at a time: aligned groups, whole groups only.
+bool simple_mask_ok(const ttsdpa_params* p) {
+  return p->mask_kind == TTSDPA_MASK_NONE || (mask_vec4_ok(p) && p->S % 4 == 0 && !p->kv_len);
+}
+
 // fp32 tensors the fp32 MFMA kernel can read and write with 16-byte accesses.
 bool f32_prefill_ok(const ttsdpa_params* p) {
-  if (p->dtype != TTSDPA_F32 || p->block_table) return false;
+  if (p->dtype != TTSDPA_F32 || p->block_table || !simple_mask_ok(p)) return false;
   if (p->D != 128 && p->D != 64) return false;
   if (!(p->scale > 0.f) || !isfinite(p->scale) || p->S < 1 || p->L < 1) return false;
   if (!dense_last_ok(p->q_stride, 4) || !dense_last_ok(p->k_stride, 4) || !dense_last_ok(p->v_stride, 4) ||
@@ -100,13 +114,15 @@ bool f32_prefill_ok(const ttsdpa_params* p) {
   return ptr_aligned(p->q, 16) && ptr_aligned(p->k, 16) && ptr_aligned(p->v, 16) && ptr_aligned(p->out, 16);
 }
 
+bool pipelined_ok(const ttsdpa_params* p) {
+  return p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
+}
+
 bool prefill_ok(const ttsdpa_params* p) {
   if (f32_prefill_ok(p)) return true;
-  // an attnMask or per-batch key counts are taken by the pipelined head_dim-128 kernel only
-  const bool pipelined = p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
-  if (p->kv_len && !pipelined) return false;
+  // the pipelined head_dim-128 kernel takes any attnMask; the 4-wavefront kernel those it can read four keys at a time
   const bool mfma_head_dim = p->D == 32 || p->D == 64 || p->D == 96 || p->D == 128 || p->D == 256;
-  return fast_layout_ok(p, pipelined) && mfma_head_dim && p->S >= 1 && p->L >= 1;
+  return fast_layout_ok(p, true) && mfma_head_dim && p->S >= 1 && p->L >= 1 && (pipelined_ok(p) || simple_mask_ok(p));
 }
 
 bool decode_ok(const ttsdpa_params* p) {
@@ -205,8 +221,7 @@ int ttsdpa_prefill(const ttsdpa_params* p, void* stream) {
   if (p->dtype == TTSDPA_F32) return launch_prefill_f32(a, (hipStream_t)stream);
   // head_dim 128 with enough rows to fill 256-row workgroups takes the software-pipelined kernel (its tile loads
   // address 64 rows with 32-bit byte offsets)
-  if (a.D == 128 && a.L > 128 && a.ks[2] < (1 << 24) && a.vs[2] < (1 << 24))
-    return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
+  if (pipelined_ok(p)) return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
   return launch_prefill(a, p->dtype, (hipStream_t)stream);
 }
 
