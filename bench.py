@@ -4,9 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3] [--no-secondary] [--no-cpu]
 
 A step is one call of the hot path (ttsdpa_forward through the C ABI) over one batch of synthetic input already
-resident in HBM.  The headline workload is BASELINE.json's configs[2] (bf16 causal GQA prefill, B2 32q/8kv S4096
-D128: the shape the prefill target is quoted on); the decode workload configs[3] (bf16, B64 32q/8kv KV 8192) is
-measured in the same run and reported under "secondary", and config 3's shape in fp32 (the reference's default dtype,
+resident in HBM.  The headline workload is "config3" (bf16 causal GQA prefill, B2 32q/8kv S4096 D128: the shape the
+prefill throughput target is quoted on); the decode workload "config4" (bf16, B64 32q/8kv KV 8192) is measured in the
+same run and reported under "secondary", config 3's shape in fp32 (the reference's default dtype,
 on the fp32 MFMA kernel, against the 157.3 TFLOP/s fp32 peak) under "fp32", and the row-wise neighbour ops (rmsNorm,
 fusedAddRmsNorm, siluMul, softmax; HBM-bound) under "fused_ops" and the linear layer (QKV projection of the same
 token batch; MFMA-bound) under "linear".  One JSON line is printed.
