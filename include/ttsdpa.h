@@ -133,7 +133,9 @@ void ttsdpa_params_init(ttsdpa_params* p, int dtype, int B, int Hq, int Hkv, int
  * needs no GPU.  Plays the role of the reference's shape checks before a device op (src/Operation/OpLinalg.cpp:62-89). */
 int ttsdpa_plan(const ttsdpa_params* p, int* route);
 
-/* Bytes of device scratch ttsdpa_forward / ttsdpa_decode need for *p (0 for routes that need none).
+/* Bytes of device scratch ttsdpa_forward / ttsdpa_decode use for *p (0 for calls that need none): the split-KV
+ * partials of the decode route, and of short-L calls on the prefill route whose keys are divided among workgroups.
+ * The decode route refuses to run with less (TTSDPA_ERR_WORKSPACE); the prefill route then runs unsplit.
  * The reference's precedent for op-owned device scratch is src/Operation/OpNNLayerCuda.cuh:415. */
 size_t ttsdpa_workspace_bytes(const ttsdpa_params* p);
 

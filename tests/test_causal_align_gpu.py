@@ -100,3 +100,58 @@ def test_chunked_prefill_equals_one_pass():
         err = (part.float() - full[:, :, c * C:end].float()).abs().max().item()
         assert err <= TOL["bf16"], (c, err)
     torch.cuda.synchronize()
+
+
+# ---- many query rows per KV head against a long cache: packed heads, split keys ----------------------------------------
+
+MULTIROW_CASES = [
+    # B, Hq, Hkv, L, S, D, dtype, causal (bottom-right)
+    (2, 32, 8, 8, 4096, 128, "bf16", True),      # 32 rows per KV head: packed into one row tile, keys split
+    (2, 32, 8, 8, 4096, 128, "f16", False),
+    (1, 8, 2, 20, 1000, 64, "bf16", True),       # head_dim 64, ragged key count
+    (1, 28, 4, 5, 3000, 128, "bf16", True),      # 7 heads per KV head: 35 rows
+    (1, 64, 8, 40, 2100, 128, "f16", True),      # 320 packed rows: three row tiles per KV head
+    (1, 4, 4, 17, 8192, 128, "bf16", True),      # one head per KV head: nothing to pack, keys split
+    (16, 16, 8, 12, 700, 128, "bf16", False),    # enough (batch, head) pairs: packed, not split
+]
+
+
+@pytest.mark.parametrize("case", MULTIROW_CASES, ids=lambda c: "B%dH%dk%dL%dS%dD%d-%s-c%d" % c)
+def test_packed_heads_and_split_keys(case):
+    """Short-L calls beyond the decode kernel's 16 rows: the G heads of a KV head share a row tile of the 4-wavefront
+    kernel and the keys may be divided among workgroups (partials merged by the decode path's merge kernel).  Both are
+    internal to the prefill route: the result is the oracle's, with and without scratch."""
+    B, Hq, Hkv, L, S, D, dtype, causal = case
+    say("multi-row", case)
+    host, dev = make_inputs(7700 + L + S, B, Hq, Hkv, L, S, D, dtype)
+    exp = oracle.sdpa_f32(*host, mask=br_mask(L, S)) if causal else oracle.sdpa_f32(*host)
+    kw = dict(causal=causal, align="bottom-right")
+    assert route_of(*dev, **kw) == "prefill"
+    rc, out = call("forward", *dev, **kw)    # with the scratch ttsdpa_workspace_bytes asks for
+    assert rc == 0
+    assert max_abs_err(out, exp) <= TOL[dtype]
+    rc, out2 = call("prefill", *dev, **kw)   # no scratch: no split
+    assert rc == 0 and max_abs_err(out2, exp) <= TOL[dtype]
+    # per-batch key counts on the same path
+    lens = [S - 37 * b for b in range(B)]
+    kv = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    rc, out3 = call("forward", *dev, kv_lens=kv, **kw)
+    assert rc == 0
+    for b in (0, B - 1):
+        n = lens[b]
+        e = oracle.sdpa_f32(host[0][b:b + 1], host[1][b:b + 1, :, :n], host[2][b:b + 1, :, :n],
+                            mask=br_mask(L, n) if causal else None)
+        assert max_abs_err(out3[b:b + 1], e) <= TOL[dtype], b
+
+
+def test_split_keys_need_scratch_only_when_asked():
+    import ctypes
+    from tinytorch_amd import _capi, build_params
+    host, dev = make_inputs(1, 1, 32, 8, 8, 8192, 128, "bf16")
+    out = torch.empty_like(dev[0])
+    p = build_params(*dev, out, True, causalAlign="bottom-right")
+    need = _capi.lib().ttsdpa_workspace_bytes(ctypes.byref(p))
+    assert need > 0 and need % 4 == 0           # one (batch) x 8 KV heads: the keys are split
+    big = make_inputs(2, 64, 32, 8, 8, 1024, 128, "bf16")[1]
+    p2 = build_params(*big, torch.empty_like(big[0]), True, causalAlign="bottom-right")
+    assert _capi.lib().ttsdpa_workspace_bytes(ctypes.byref(p2)) == 0   # 512 pairs fill the chip unsplit

@@ -24,12 +24,20 @@ struct KArgs {
   float scale;
   long long qs[3], ks[3], vs[3], os[3];  // element strides: batch, head, sequence
   long long ms[4];                       // mask element strides: batch, head, query row, key (0 = broadcast)
+  // Packed query heads (4-wavefront prefill kernel only): the G query heads of a KV head are presented as one head of
+  // G * pack_L rows (dense q / out make that a plain reshape); row x is query position x % pack_L.  0 = not packed.
+  int pack_L;
+  // Split keys (4-wavefront prefill kernel, one query head per KV head after packing): workgroup (.., split) covers keys
+  // split * kv_chunk .. + kv_chunk - 1 and writes a (acc[D], max, sum) record per row to ws instead of the output;
+  // the decode path's merge kernel combines them.  kv_splits <= 1: no split.
+  int kv_splits, kv_chunk;
+  float* ws;
   int mask_vec4;  // keys are contiguous in the mask and groups of 4 keys starting at a multiple of 4 are naturally aligned
 };
 
 // Offset of the causal diagonal in key coordinates for a batch entry with S keys.
 __device__ __forceinline__ int causal_offset(const KArgs& a, int S) {
-  const int d = S - a.L;
+  const int d = S - (a.pack_L ? a.pack_L : a.L);
   return (a.causal_br && d > 0) ? d : 0;
 }
 
@@ -153,6 +161,8 @@ int launch_prefill(const KArgs& a, int dtype, hipStream_t stream);       // 128-
 int launch_prefill_d128(const KArgs& a, int dtype, hipStream_t stream);  // 256-row workgroups, pipelined; head_dim 128
 int launch_prefill_f32(const KArgs& a, hipStream_t stream);              // fp32 tensors on the fp32 matrix cores; head_dim 64 or 128
 int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream);
+// combines per-split records [pair][split][row][D + 2] (pair = batch * Hkv + kv head, row = l * G + g) into a.out
+int launch_merge(const KArgs& a, int dtype, int splits, const float* ws, hipStream_t stream);
 int launch_zero(const KArgs& a, int dtype, hipStream_t stream);
 struct KvAppendArgs {
   void* kc;

@@ -84,9 +84,11 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
   const int inner = a.G * ntile;           // workgroups that share one (batch, kv head)
   const int npair = a.B * a.Hkv;
   int pair, in;
+  const int nsplit = a.kv_splits > 1 ? a.kv_splits : 1;
+  const int split = blockIdx.x % nsplit;    // key range of this workgroup (the only one unless the keys are split)
   {
-    int n = blockIdx.x;
-    if ((npair & 7) == 0) {                // workgroup n runs on XCD n % 8: keep a pair on one XCD
+    int n = blockIdx.x / nsplit;
+    if ((npair & 7) == 0 && nsplit == 1) {  // workgroup n runs on XCD n % 8: keep a pair on one XCD
       int xcd = n & 7, slot = n >> 3;
       pair = (slot / inner) * 8 + xcd;
       in = slot % inner;
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
     int len = __builtin_amdgcn_readfirstlane(a.kv_len[b]);
     S = len < 0 ? 0 : (len < S ? len : S);
   }
-  if (S == 0) {  // no keys: zeros, the reference's empty contraction
+  if (S == 0 && nsplit == 1) {  // no keys: zeros, the reference's empty contraction
     const int qi = qw0 + lq;
     if (qi < a.L) {
       T* op = (T*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2];
@@ -144,11 +146,21 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
     return;
   }
   int ntiles_kv = (S + BN - 1) / BN;
-  const int coff = CAUSAL ? causal_offset(a, S) : 0;  // query row i sees keys up to i + coff
+  const int coff = CAUSAL ? causal_offset(a, S) : 0;  // query position i sees keys up to i + coff
+  // Query position of a row under the causal mask: the row itself, or with packed heads row % pack_L — then positions
+  // are not monotone in the row, and the tile-level tests below use the range of all positions.
+  const int pos_lo = a.pack_L ? 0 : qw0, pos_hi = a.pack_L ? a.pack_L - 1 : qw0 + 31;
   if (CAUSAL) {
-    int last = (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1) + coff;  // last key of the workgroup's last query row
+    int last = (a.pack_L ? a.pack_L - 1 : (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1)) + coff;  // last key any row of the workgroup sees
     int lastkv = last < S - 1 ? last : S - 1;
-    ntiles_kv = lastkv / BN + 1;
+    ntiles_kv = S > 0 ? lastkv / BN + 1 : 0;
+  }
+  // tiles jt0 .. jt1-1 are this workgroup's: all of them, or those of its split (kv_chunk is a multiple of the tile)
+  int jt0 = 0, jt1 = ntiles_kv;
+  if (nsplit > 1) {
+    jt0 = split * (a.kv_chunk / BN);
+    const int end = jt0 + a.kv_chunk / BN;
+    jt1 = end < jt1 ? end : jt1;
   }
 
   // ---- global -> register -> LDS staging of one K/V tile --------------------------------------------------------
@@ -197,20 +209,22 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
   const int k_lane = lq * K_PITCH + 8 * lh;                                              // elements
   const int v_lane = (4 * lh + ((lane & 15) >> 2)) * V_PITCH + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);  // elements
 
-  load_tile(0);
-  store_tile(0);
-  if (ntiles_kv > 1) load_tile(BN);
+  if (jt0 < jt1) {
+    load_tile(jt0 * BN);
+    store_tile(0);
+    if (jt0 + 1 < jt1) load_tile((jt0 + 1) * BN);
+  }
   __syncthreads();
 
-  for (int jt = 0; jt < ntiles_kv; jt++) {
+  for (int jt = jt0; jt < jt1; jt++) {
     const int kv0 = jt * BN;
-    const int cur = jt & 1;
-    if (jt + 1 < ntiles_kv) {
+    const int cur = (jt - jt0) & 1;
+    if (jt + 1 < jt1) {
       store_tile(cur ^ 1);  // stage cur^1 was last read before the barrier that ended the previous iteration
-      if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BN);
+      if (jt + 2 < jt1) load_tile(kv0 + 2 * BN);
     }
 
-    if (!CAUSAL || kv0 <= qw0 + 31 + coff) {  // else: the whole tile is above this wavefront's diagonal
+    if (!CAUSAL || kv0 <= pos_hi + coff) {  // else: the whole tile is above this wavefront's diagonal
       const T* Ks = smem + cur * Lds::STAGE;
       const T* Vs = Ks + BN * K_PITCH;
 
@@ -229,9 +243,9 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
       }
 
       // ---- mask the diagonal / ragged tile -----------------------------------------------------------------------
-      const bool need_mask = (CAUSAL && kv0 + BN - 1 > qw0 + coff) || (kv0 + BN > S);
+      const bool need_mask = (CAUSAL && kv0 + BN - 1 > pos_lo + coff) || (kv0 + BN > S);
       if (need_mask) {
-        const int qi = qw0 + lq + coff;
+        const int qi = (a.pack_L ? (qw0 + lq) % a.pack_L : qw0 + lq) + coff;
 #pragma unroll
         for (int blk = 0; blk < 2; blk++)
 #pragma unroll
@@ -304,8 +318,23 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
 
   // ---- normalise and store ----------------------------------------------------------------------------------------------
   float l_tot = l_run + __shfl_xor(l_run, 32);
-  const float inv = 1.f / l_tot;
   const int qi = qw0 + lq;
+  if (nsplit > 1) {  // a partial result: unnormalised accumulator, the maximum it is relative to, the sum
+    if (qi < a.L) {
+      float* rec = a.ws + ((long long)(pair * nsplit + split) * a.L + qi) * (D + 2);  // 8-byte aligned
+#pragma unroll
+      for (int db = 0; db < DBLK; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          float* dst = rec + 32 * db + 8 * rg + 4 * lh;
+          *(float2*)dst = make_float2(oacc[db][4 * rg], oacc[db][4 * rg + 1]);
+          *(float2*)(dst + 2) = make_float2(oacc[db][4 * rg + 2], oacc[db][4 * rg + 3]);
+        }
+      if (lh == 0) rec[D] = m_use, rec[D + 1] = l_tot;
+    }
+    return;
+  }
+  const float inv = 1.f / l_tot;
   if (qi < a.L) {
     T* op = (T*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2];
 #pragma unroll
@@ -333,7 +362,7 @@ int launch_prefill_k(const KArgs& a, dim3 grid, hipStream_t stream) {
 
 template <typename TR, int D>
 int launch_prefill_t(const KArgs& a, hipStream_t stream) {
-  long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM);
+  long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM) * (a.kv_splits > 1 ? a.kv_splits : 1);
   dim3 grid((unsigned)nwg);
   if (a.mask_kind != 0) return launch_prefill_k<TR, D, false, true>(a, grid, stream);  // exclusive with causal (validated)
   return a.causal ? launch_prefill_k<TR, D, true, false>(a, grid, stream) : launch_prefill_k<TR, D, false, false>(a, grid, stream);

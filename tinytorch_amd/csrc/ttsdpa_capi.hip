@@ -64,6 +64,7 @@ int validate(const ttsdpa_params* p, KArgs* a) {
   }
   if (p->mask_kind == TTSDPA_MASK_ADD && !ptr_aligned(p->mask, esz)) return TTSDPA_ERR_STRIDE;
   a->mask_vec4 = mask_vec4_ok(p) ? 1 : 0;
+  a->pack_L = 0, a->kv_splits = 1, a->kv_chunk = 0, a->ws = nullptr;
   if (p->kv_len && !ptr_aligned(p->kv_len, 4)) return TTSDPA_ERR_STRIDE;
   a->kv_len = p->kv_len;
   a->block_table = p->block_table, a->page_shift = 0, a->bt_stride = p->block_table_stride;
@@ -117,6 +118,51 @@ bool f32_prefill_ok(const ttsdpa_params* p) {
 bool pipelined_ok(const ttsdpa_params* p) {
   return p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
 }
+
+// Few query rows per head against many keys on the 4-wavefront kernel: the G heads of a KV head share one row tile
+// (dense q / out make [B,Hq,L,D] a [B,Hkv,G*L,D] tensor), so K/V are streamed once per KV head instead of once per
+// query head and the tile is not mostly padding.
+bool pack_heads_ok(const ttsdpa_params* p) {
+  const int G = p->Hq / p->Hkv;
+  if (p->dtype == TTSDPA_F32 || pipelined_ok(p) || G < 2 || p->mask_kind != TTSDPA_MASK_NONE || p->L > 64 || p->S < 256)
+    return false;
+  return p->q_stride[1] == (int64_t)p->L * p->q_stride[2] && p->o_stride[1] == (int64_t)p->L * p->o_stride[2];
+}
+
+void pack_heads(KArgs* a) {
+  a->pack_L = a->L;
+  a->L = a->L * a->G, a->Hq = a->Hkv;
+  a->qs[1] *= a->G, a->os[1] *= a->G;
+  a->G = 1;
+}
+
+// Key splits of a short-L call on the 4-wavefront kernel (one query head per KV head, possibly after packing): when
+// batch x heads x row tiles leave most of the 256 CUs idle, the keys are divided among several workgroups whose
+// partial results the decode path's merge kernel combines.  Needs head_dim 64 or 128 (the merge kernel's) and scratch.
+struct SplitPlan {
+  int splits, chunk;
+  size_t ws_bytes;
+};
+SplitPlan plan_prefill_splits(const ttsdpa_params* p, const KArgs& a /* after packing */) {
+  SplitPlan s{1, 0, 0};
+  if (a.G != 1 || (a.D != 64 && a.D != 128) || p->dtype == TTSDPA_F32 || p->mask_kind != TTSDPA_MASK_NONE ||
+      pipelined_ok(p))
+    return s;
+  const long long wgs = (long long)a.B * a.Hq * ((a.L + 127) / 128);
+  long long want = (2 * 256 + wgs - 1) / wgs;  // aim for two workgroups per CU
+  const long long most = a.S / 512;            // at least 8 key tiles per split
+  if (want > most) want = most;
+  if (want > 64) want = 64;                    // the merge kernel's limit
+  if (want < 2) return s;
+  int chunk = (int)((a.S + want - 1) / want);
+  chunk = (chunk + 63) / 64 * 64;
+  s.splits = (a.S + chunk - 1) / chunk;
+  s.chunk = chunk;
+  if (s.splits < 2) return SplitPlan{1, 0, 0};
+  s.ws_bytes = (size_t)a.B * a.Hq * s.splits * a.L * (a.D + 2) * sizeof(float);
+  return s;
+}
+
 
 bool prefill_ok(const ttsdpa_params* p) {
   if (f32_prefill_ok(p)) return true;
@@ -197,8 +243,13 @@ int ttsdpa_plan(const ttsdpa_params* p, int* route) {
 size_t ttsdpa_workspace_bytes(const ttsdpa_params* p) {
   KArgs a;
   if (validate(p, &a) != TTSDPA_OK) return 0;
-  if (p->B == 0 || p->L == 0 || p->S == 0 || !decode_ok(p)) return 0;
-  return plan_decode(a).ws_bytes;
+  switch (pick_route(p)) {
+    case TTSDPA_ROUTE_DECODE: return plan_decode(a).ws_bytes;
+    case TTSDPA_ROUTE_PREFILL:
+      if (pack_heads_ok(p)) pack_heads(&a);
+      return plan_prefill_splits(p, a).ws_bytes;
+    default: return 0;
+  }
 }
 
 int ttsdpa_general(const ttsdpa_params* p, void* stream) {
@@ -211,7 +262,8 @@ int ttsdpa_general(const ttsdpa_params* p, void* stream) {
   return launch_general(a, p->dtype, (hipStream_t)stream);
 }
 
-int ttsdpa_prefill(const ttsdpa_params* p, void* stream) {
+// ttsdpa_prefill with optional scratch: with it, a short-L call may divide its keys among workgroups.
+static int prefill_impl(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream) {
   KArgs a;
   int rc = validate(p, &a);
   if (rc != TTSDPA_OK) return rc;
@@ -222,8 +274,20 @@ int ttsdpa_prefill(const ttsdpa_params* p, void* stream) {
   // head_dim 128 with enough rows to fill 256-row workgroups takes the software-pipelined kernel (its tile loads
   // address 64 rows with 32-bit byte offsets)
   if (pipelined_ok(p)) return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
+  if (pack_heads_ok(p)) pack_heads(&a);
+  a.kv_splits = 1, a.kv_chunk = 0, a.ws = nullptr;
+  const SplitPlan sp = plan_prefill_splits(p, a);
+  if (sp.splits > 1 && workspace && workspace_bytes >= sp.ws_bytes && ptr_aligned(workspace, 16) && p->S > 0) {
+    a.kv_splits = sp.splits, a.kv_chunk = sp.chunk, a.ws = (float*)workspace;
+    if ((rc = check_grid((long long)a.B * a.Hq * ((a.L + 127) / 128) * sp.splits)) != TTSDPA_OK) return rc;
+    rc = launch_prefill(a, p->dtype, (hipStream_t)stream);
+    if (rc != 0) return rc;
+    return launch_merge(a, p->dtype, sp.splits, a.ws, (hipStream_t)stream);
+  }
   return launch_prefill(a, p->dtype, (hipStream_t)stream);
 }
+
+int ttsdpa_prefill(const ttsdpa_params* p, void* stream) { return prefill_impl(p, nullptr, 0, stream); }
 
 int ttsdpa_decode(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream) {
   KArgs a;
@@ -246,7 +310,7 @@ int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_byt
     case TTSDPA_ROUTE_NONE: return TTSDPA_OK;
     case TTSDPA_ROUTE_ZERO: return launch_zero(a, p->dtype, (hipStream_t)stream);
     case TTSDPA_ROUTE_DECODE: return ttsdpa_decode(p, workspace, workspace_bytes, stream);
-    case TTSDPA_ROUTE_PREFILL: return ttsdpa_prefill(p, stream);
+    case TTSDPA_ROUTE_PREFILL: return prefill_impl(p, workspace, workspace_bytes, stream);
     default: return ttsdpa_general(p, stream);
   }
 }
