@@ -104,11 +104,15 @@ def test_routes_depend_on_flags():
     p.v_stride[2] = 130
     assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL
     # bottom-right aligned causal: a few new rows against a long cache stream it; one new row hides nothing
-    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 4, 1024, 128, causal=2))[1] == _capi.ROUTE_DECODE
+    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 2, 1024, 128, causal=2))[1] == _capi.ROUTE_DECODE   # 8 rows per KV head
+    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 4, 1024, 128, causal=2))[1] == _capi.ROUTE_PREFILL  # 16: packed heads on the MFMA kernel
+    strided = params(_capi.BF16, 4, 8, 2, 4, 1024, 128, causal=2)
+    strided.q_stride[1] = 4 * 128 + 128   # heads not dense: cannot be packed, the streaming kernel takes its 16 rows
+    assert _capi.plan(strided)[1] == _capi.ROUTE_DECODE
     assert _capi.plan(params(_capi.BF16, 4, 8, 2, 1, 1024, 128, causal=2))[1] == _capi.ROUTE_DECODE
     assert _capi.plan(params(_capi.BF16, 4, 8, 2, 512, 1024, 128, causal=2))[1] == _capi.ROUTE_PREFILL
     assert _capi.plan(params(_capi.F32, 4, 8, 2, 512, 1024, 128, causal=2))[1] == _capi.ROUTE_PREFILL
-    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 4, 1024, 128, causal=2, kv_len=FAKE))[1] == _capi.ROUTE_DECODE
+    assert _capi.plan(params(_capi.BF16, 4, 8, 2, 2, 1024, 128, causal=2, kv_len=FAKE))[1] == _capi.ROUTE_DECODE
     # decode with causal set is the top-left triangle (only key 0 visible): not the streaming kernel's case
     assert _capi.plan(params(_capi.BF16, 4, 8, 2, 1, 1024, 128, causal=1))[1] == _capi.ROUTE_PREFILL
 

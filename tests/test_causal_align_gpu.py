@@ -36,10 +36,13 @@ CASES = [
     (2, 2, 2, 77, 99, 64, "f32", "prefill"),
     (1, 2, 2, 70, 131, 96, "f32", "general"),       # vector-ALU kernel
     (1, 2, 1, 40, 90, 80, "bf16", "general"),
-    (2, 8, 2, 4, 2048, 128, "bf16", "decode"),      # 16 rows per KV head: 4 new tokens
+    (2, 8, 2, 4, 2048, 128, "bf16", "prefill"),     # 16 rows per KV head: 4 new tokens, packed heads on the MFMA kernel
+    (2, 8, 2, 2, 2048, 128, "bf16", "decode"),      # 8 rows per KV head: the streaming kernel
     (1, 4, 4, 3, 1000, 128, "f16", "decode"),       # 3 rows per KV head
-    (2, 8, 4, 5, 700, 64, "bf16", "decode"),        # head_dim 64, 10 rows per KV head
-    (1, 28, 4, 2, 5000, 128, "bf16", "decode"),     # 7 heads per KV head, split cache
+    (2, 8, 4, 5, 700, 64, "bf16", "prefill"),       # head_dim 64, 10 rows per KV head
+    (2, 8, 4, 3, 700, 64, "bf16", "decode"),        # head_dim 64, 6 rows per KV head
+    (1, 28, 4, 2, 5000, 128, "bf16", "prefill"),    # 7 heads per KV head, 14 rows: packed, keys split
+    (1, 28, 4, 1, 5000, 128, "bf16", "decode"),     # 7 rows per KV head, split cache
     (1, 4, 2, 1, 512, 128, "bf16", "decode"),       # one new token sees every key
     (1, 4, 2, 300, 200, 128, "bf16", "prefill"),    # fewer keys than queries: offset 0, the top-left mask
 ]
@@ -113,6 +116,9 @@ MULTIROW_CASES = [
     (1, 64, 8, 40, 2100, 128, "f16", True),      # 320 packed rows: three row tiles per KV head
     (1, 4, 4, 17, 8192, 128, "bf16", True),      # one head per KV head: nothing to pack, keys split
     (16, 16, 8, 12, 700, 128, "bf16", False),    # enough (batch, head) pairs: packed, not split
+    (2, 16, 4, 1, 3000, 128, "f32", False),      # fp32 decode step: packed heads and split keys on the fp32 MFMA kernel
+    (1, 8, 2, 6, 2500, 64, "f32", True),
+    (1, 4, 4, 3, 4100, 128, "f32", True),        # fp32, one head per KV head: keys split
 ]
 
 

@@ -478,7 +478,8 @@ def test_per_batch_key_counts_on_the_mfma_route(causal, dtype):
 def test_decode_head_dim_64(case):
     B, Hq, Hkv, L, S, dtype = case
     host, dev = make_inputs(99 + S, B, Hq, Hkv, L, S, 64, dtype)
-    assert route_of(*dev) == "decode"
+    # up to 8 rows per KV head stream through the decode kernel; 9-16 take the packed-heads MFMA path when S >= 256
+    assert route_of(*dev) == ("decode" if L * (Hq // Hkv) <= 8 or S < 256 else "prefill")
     exp = oracle.sdpa_f32(*host)
     rc, out = call("forward", *dev)
     assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]

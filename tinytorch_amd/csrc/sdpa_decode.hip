@@ -373,7 +373,10 @@ DecodePlan plan_decode(const KArgs& a) {
 
 int launch_merge(const KArgs& a, int dtype, int splits, const float* ws, hipStream_t stream) {
   const dim3 grid((unsigned)((long long)a.B * a.Hkv * a.L * a.G));
-  if (a.D == 64) {
+  if (dtype == 0) {
+    if (a.D == 64) hipLaunchKernelGGL((merge_kernel<float, 64>), grid, dim3(64), 0, stream, a, splits, ws);
+    else hipLaunchKernelGGL((merge_kernel<float, 128>), grid, dim3(128), 0, stream, a, splits, ws);
+  } else if (a.D == 64) {
     if (dtype == 1) hipLaunchKernelGGL((merge_kernel<_Float16, 64>), grid, dim3(64), 0, stream, a, splits, ws);
     else hipLaunchKernelGGL((merge_kernel<__bf16, 64>), grid, dim3(64), 0, stream, a, splits, ws);
   } else {

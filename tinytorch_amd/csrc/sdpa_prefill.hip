@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
       if (jt + 2 < jt1) load_tile(kv0 + 2 * BN);
     }
 
-    if (!CAUSAL || kv0 <= pos_hi + coff) {  // else: the whole tile is above this wavefront's diagonal
+    if (qw0 < a.L && (!CAUSAL || kv0 <= pos_hi + coff)) {  // else: no rows here, or the whole tile is above the diagonal
       const T* Ks = smem + cur * Lds::STAGE;
       const T* Vs = Ks + BN * K_PITCH;
 

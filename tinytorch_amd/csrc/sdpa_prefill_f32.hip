@@ -59,9 +59,11 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
   const int inner = a.G * ntile;
   const int npair = a.B * a.Hkv;
   int pair, in;
+  const int nsplit = a.kv_splits > 1 ? a.kv_splits : 1;
+  const int split = blockIdx.x % nsplit;  // key range of this workgroup (the only one unless the keys are split)
   {
-    int n = blockIdx.x;
-    if ((npair & 7) == 0) {
+    int n = blockIdx.x / nsplit;
+    if ((npair & 7) == 0 && nsplit == 1) {
       int xcd = n & 7, slot = n >> 3;
       pair = (slot / inner) * 8 + xcd;
       in = slot % inner;
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
     int len = __builtin_amdgcn_readfirstlane(a.kv_len[b]);
     S = len < 0 ? 0 : (len < S ? len : S);
   }
-  if (S == 0) {  // no keys: zeros, the reference's empty contraction
+  if (S == 0 && nsplit == 1) {  // no keys: zeros, the reference's empty contraction
     const int qi = qw0 + lq;
     if (qi < a.L) {
       float* op = (float*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2];
@@ -120,12 +122,23 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
     return;
   }
   int ntiles_kv = (S + BN - 1) / BN;
-  const int coff = CAUSAL ? causal_offset(a, S) : 0;  // query row i sees keys up to i + coff
+  const int coff = CAUSAL ? causal_offset(a, S) : 0;  // query position i sees keys up to i + coff
+  // Query position of a row under the causal mask: the row itself, or with packed heads row % pack_L — then positions
+  // are not monotone in the row, and the tile-level tests below use the range of all positions.
+  const int pos_lo = a.pack_L ? 0 : qw0, pos_hi = a.pack_L ? a.pack_L - 1 : qw0 + 31;
   if (CAUSAL) {
-    int last = (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1) + coff;
+    int last = (a.pack_L ? a.pack_L - 1 : (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1)) + coff;
     int lastkv = last < S - 1 ? last : S - 1;
-    ntiles_kv = lastkv / BN + 1;
+    ntiles_kv = S > 0 ? lastkv / BN + 1 : 0;
   }
+  // tiles jt0 .. jt1-1 are this workgroup's: all of them, or those of its split (kv_chunk is a multiple of the tile)
+  int jt0 = 0, jt1 = ntiles_kv;
+  if (nsplit > 1) {
+    jt0 = split * (a.kv_chunk / BN);
+    const int end = jt0 + a.kv_chunk / BN;
+    jt1 = end < jt1 ? end : jt1;
+  }
+  const bool wave_live = qw0 < a.L;  // a wavefront without query rows only helps to stage the tiles
 
   // ---- global -> register -> LDS staging: thread t moves 16-byte chunks t, t+256, ... of a tile ----------------------
   f32x4 kst[NLD], vst[NLD];
@@ -159,20 +172,22 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
   const int k_lane = lq * K_PITCH + lh * (D / 2);  // floats
   const int v_lane = 4 * lh * V_PITCH + lq;        // floats; + (8*(t/4) + t%4) * V_PITCH + 32*db
 
-  load_tile(0);
-  store_tile(0);
-  if (ntiles_kv > 1) load_tile(BN);
+  if (jt0 < jt1) {
+    load_tile(jt0 * BN);
+    store_tile(0);
+    if (jt0 + 1 < jt1) load_tile((jt0 + 1) * BN);
+  }
   __syncthreads();
 
-  for (int jt = 0; jt < ntiles_kv; jt++) {
+  for (int jt = jt0; jt < jt1; jt++) {
     const int kv0 = jt * BN;
-    const int cur = jt & 1;
-    if (jt + 1 < ntiles_kv) {
+    const int cur = (jt - jt0) & 1;
+    if (jt + 1 < jt1) {
       store_tile(cur ^ 1);  // stage cur^1 was last read before the barrier that ended the previous iteration
-      if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BN);
+      if (jt + 2 < jt1) load_tile(kv0 + 2 * BN);
     }
 
-    if (!CAUSAL || kv0 <= qw0 + 31 + coff) {  // else: the whole tile is above this wavefront's diagonal
+    if (wave_live && (!CAUSAL || kv0 <= pos_hi + coff)) {  // else: the whole tile is above this wavefront's diagonal
       const float* Ks = smem + cur * Lds::STAGE;
       const float* Vs = Ks + BN * K_PITCH;
 
@@ -191,8 +206,8 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
       for (int r = 0; r < 16; r++) s[r] = s0[r] + s1[r];
 
       // ---- mask the diagonal / ragged tile -----------------------------------------------------------------------------
-      if ((CAUSAL && kv0 + BN - 1 > qw0 + coff) || (kv0 + BN > S)) {
-        const int qi = qw0 + lq + coff;
+      if ((CAUSAL && kv0 + BN - 1 > pos_lo + coff) || (kv0 + BN > S)) {
+        const int qi = (a.pack_L ? (qw0 + lq) % a.pack_L : qw0 + lq) + coff;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
@@ -246,8 +261,23 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
 
   // ---- normalise and store ----------------------------------------------------------------------------------------------
   float l_tot = l_run + __shfl_xor(l_run, 32);
-  const float inv = 1.f / l_tot;
   const int qi = qw0 + lq;
+  if (nsplit > 1) {  // a partial result: unnormalised accumulator, the maximum it is relative to, the sum
+    if (qi < a.L) {
+      float* rec = a.ws + ((long long)(pair * nsplit + split) * a.L + qi) * (D + 2);  // 8-byte aligned
+#pragma unroll
+      for (int db = 0; db < DBLK; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          float* dst = rec + 32 * db + 8 * rg + 4 * lh;
+          *(float2*)dst = make_float2(oacc[db][4 * rg], oacc[db][4 * rg + 1]);
+          *(float2*)(dst + 2) = make_float2(oacc[db][4 * rg + 2], oacc[db][4 * rg + 3]);
+        }
+      if (lh == 0) rec[D] = m_use, rec[D + 1] = l_tot;
+    }
+    return;
+  }
+  const float inv = 1.f / l_tot;
   if (qi < a.L) {
     float* op = (float*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2];
 #pragma unroll
@@ -275,7 +305,7 @@ int launch_f32_k(const KArgs& a, dim3 grid, hipStream_t stream) {
 }  // namespace
 
 int launch_prefill_f32(const KArgs& a, hipStream_t stream) {
-  long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM);
+  long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM) * (a.kv_splits > 1 ? a.kv_splits : 1);
   dim3 grid((unsigned)nwg);
   if (a.mask_kind != 0)  // exclusive with causal (validated by the caller, as the reference asserts)
     return a.D == 128 ? launch_f32_k<128, false, true>(a, grid, stream) : launch_f32_k<64, false, true>(a, grid, stream);

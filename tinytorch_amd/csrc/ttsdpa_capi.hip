@@ -124,8 +124,8 @@ bool pipelined_ok(const ttsdpa_params* p) {
 // query head and the tile is not mostly padding.
 bool pack_heads_ok(const ttsdpa_params* p) {
   const int G = p->Hq / p->Hkv;
-  if (p->dtype == TTSDPA_F32 || pipelined_ok(p) || G < 2 || p->mask_kind != TTSDPA_MASK_NONE || p->L > 64 || p->S < 256)
-    return false;
+  if (pipelined_ok(p) || G < 2 || p->mask_kind != TTSDPA_MASK_NONE || p->L > 64 || p->S < 256) return false;
+  if (p->dtype == TTSDPA_F32 && !f32_prefill_ok(p)) return false;
   return p->q_stride[1] == (int64_t)p->L * p->q_stride[2] && p->o_stride[1] == (int64_t)p->L * p->o_stride[2];
 }
 
@@ -145,9 +145,7 @@ struct SplitPlan {
 };
 SplitPlan plan_prefill_splits(const ttsdpa_params* p, const KArgs& a /* after packing */) {
   SplitPlan s{1, 0, 0};
-  if (a.G != 1 || (a.D != 64 && a.D != 128) || p->dtype == TTSDPA_F32 || p->mask_kind != TTSDPA_MASK_NONE ||
-      pipelined_ok(p))
-    return s;
+  if (a.G != 1 || (a.D != 64 && a.D != 128) || p->mask_kind != TTSDPA_MASK_NONE || pipelined_ok(p)) return s;
   const long long wgs = (long long)a.B * a.Hq * ((a.L + 127) / 128);
   long long want = (2 * 256 + wgs - 1) / wgs;  // aim for two workgroups per CU
   const long long most = a.S / 512;            // at least 8 key tiles per split
@@ -184,7 +182,13 @@ int pick_route(const ttsdpa_params* p) {
   if (p->B == 0 || p->L == 0) return TTSDPA_ROUTE_NONE;
   if (p->S == 0) return TTSDPA_ROUTE_ZERO;
   // Few query rows against many keys: streaming the cache once for the whole head group beats a 128-row tile.
-  if (decode_ok(p) && p->S >= 256) return TTSDPA_ROUTE_DECODE;
+  if (decode_ok(p) && p->S >= 256) {
+    // 9-16 rows per KV head: the streaming kernel does P.V on the vector ALUs and measures 5.5 TB/s there; the
+    // 4-wavefront MFMA kernel with packed heads and split keys 5.85 TB/s, when the call allows it
+    const long long rows = (long long)p->L * (p->Hq / p->Hkv);
+    if (rows > 8 && prefill_ok(p) && !pipelined_ok(p) && (p->Hq == p->Hkv || pack_heads_ok(p))) return TTSDPA_ROUTE_PREFILL;
+    return TTSDPA_ROUTE_DECODE;
+  }
   if (prefill_ok(p) && p->L >= 16) return TTSDPA_ROUTE_PREFILL;
   if (decode_ok(p)) return TTSDPA_ROUTE_DECODE;
   if (prefill_ok(p)) return TTSDPA_ROUTE_PREFILL;
@@ -243,13 +247,15 @@ int ttsdpa_plan(const ttsdpa_params* p, int* route) {
 size_t ttsdpa_workspace_bytes(const ttsdpa_params* p) {
   KArgs a;
   if (validate(p, &a) != TTSDPA_OK) return 0;
-  switch (pick_route(p)) {
-    case TTSDPA_ROUTE_DECODE: return plan_decode(a).ws_bytes;
-    case TTSDPA_ROUTE_PREFILL:
-      if (pack_heads_ok(p)) pack_heads(&a);
-      return plan_prefill_splits(p, a).ws_bytes;
-    default: return 0;
+  if (p->B == 0 || p->L == 0 || p->S == 0) return 0;
+  // enough for ttsdpa_forward's route and for an explicit ttsdpa_decode of the same call
+  size_t need = decode_ok(p) ? plan_decode(a).ws_bytes : 0;
+  if (pick_route(p) == TTSDPA_ROUTE_PREFILL) {
+    if (pack_heads_ok(p)) pack_heads(&a);
+    const size_t split = plan_prefill_splits(p, a).ws_bytes;
+    need = split > need ? split : need;
   }
+  return need;
 }
 
 int ttsdpa_general(const ttsdpa_params* p, void* stream) {
@@ -270,21 +276,23 @@ static int prefill_impl(const ttsdpa_params* p, void* workspace, size_t workspac
   if (p->B == 0 || p->L == 0) return TTSDPA_OK;
   if (!prefill_ok(p)) return TTSDPA_ERR_UNSUPPORTED;
   if ((rc = check_grid((long long)a.B * a.Hq * ((a.L + 127) / 128))) != TTSDPA_OK) return rc;
-  if (p->dtype == TTSDPA_F32) return launch_prefill_f32(a, (hipStream_t)stream);
   // head_dim 128 with enough rows to fill 256-row workgroups takes the software-pipelined kernel (its tile loads
   // address 64 rows with 32-bit byte offsets)
-  if (pipelined_ok(p)) return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
+  if (p->dtype != TTSDPA_F32 && pipelined_ok(p)) return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
+  auto launch = [&](const KArgs& k) {
+    return p->dtype == TTSDPA_F32 ? launch_prefill_f32(k, (hipStream_t)stream) : launch_prefill(k, p->dtype, (hipStream_t)stream);
+  };
   if (pack_heads_ok(p)) pack_heads(&a);
   a.kv_splits = 1, a.kv_chunk = 0, a.ws = nullptr;
   const SplitPlan sp = plan_prefill_splits(p, a);
   if (sp.splits > 1 && workspace && workspace_bytes >= sp.ws_bytes && ptr_aligned(workspace, 16) && p->S > 0) {
     a.kv_splits = sp.splits, a.kv_chunk = sp.chunk, a.ws = (float*)workspace;
     if ((rc = check_grid((long long)a.B * a.Hq * ((a.L + 127) / 128) * sp.splits)) != TTSDPA_OK) return rc;
-    rc = launch_prefill(a, p->dtype, (hipStream_t)stream);
+    rc = launch(a);
     if (rc != 0) return rc;
     return launch_merge(a, p->dtype, sp.splits, a.ws, (hipStream_t)stream);
   }
-  return launch_prefill(a, p->dtype, (hipStream_t)stream);
+  return launch(a);
 }
 
 int ttsdpa_prefill(const ttsdpa_params* p, void* stream) { return prefill_impl(p, nullptr, 0, stream); }
