@@ -115,7 +115,7 @@ typedef struct ttsdpa_params {
    * j % page_size of page block_table[b * block_table_stride + j / page_size] (int32, device memory).  S is the
    * logical capacity: the table holds at least ceil(S / page_size) entries per batch entry, of which those below
    * ceil(kv_len[b] / page_size) are read.  page_size must be a power of two; the decode kernel takes pages of 32 rows
-   * or more, anything else paged goes to the general kernel. */
+   * or more and the MFMA prefill kernels pages of 64 rows or more, smaller pages go to the general kernel. */
   const int32_t* block_table;
   int32_t page_size;
   int32_t block_table_stride;

@@ -237,14 +237,20 @@ def test_fused_ops_argument_checks_without_a_gpu():
 
 
 def test_paged_cache_routes_and_validation():
-    """block_table: decode kernel for pages of 32 rows or more, general kernel otherwise; page sizes are powers of two."""
+    """block_table: decode kernel for pages of 32 rows or more, MFMA prefill kernels for 64 or more, general kernel
+    otherwise; page sizes are powers of two."""
     dec = (_capi.BF16, 4, 32, 8, 1, 4096, 128)
     paged = dict(block_table=FAKE, page_size=64, block_table_stride=64)
     assert _capi.plan(params(*dec, **paged))[1] == _capi.ROUTE_DECODE
     assert _capi.plan(params(*dec, **paged, kv_len=FAKE))[1] == _capi.ROUTE_DECODE
     assert _capi.plan(params(*dec, block_table=FAKE, page_size=16, block_table_stride=256))[1] == _capi.ROUTE_GENERAL
-    assert _capi.plan(params(_capi.BF16, 4, 32, 8, 512, 4096, 128, causal=2, **paged))[1] == _capi.ROUTE_GENERAL  # prefill kernels read contiguous K/V
-    assert _capi.plan(params(_capi.F32, 4, 32, 8, 1, 4096, 128, **paged))[1] == _capi.ROUTE_GENERAL
+    # the MFMA prefill kernels stage 64-key tiles: pages of 64 rows or more
+    assert _capi.plan(params(_capi.BF16, 4, 32, 8, 512, 4096, 128, causal=2, **paged))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.F32, 4, 32, 8, 1, 4096, 128, **paged))[1] == _capi.ROUTE_PREFILL
+    small = dict(block_table=FAKE, page_size=32, block_table_stride=128)
+    assert _capi.plan(params(_capi.BF16, 4, 32, 8, 512, 4096, 128, causal=2, **small))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.F32, 4, 32, 8, 1, 4096, 128, **small))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(*dec, **small))[1] == _capi.ROUTE_DECODE
     assert _capi.plan(params(*dec, block_table=FAKE, page_size=48, block_table_stride=128))[0] == _capi.ERR_SHAPE
     assert _capi.plan(params(*dec, block_table=FAKE, page_size=0, block_table_stride=128))[0] == _capi.ERR_SHAPE
     assert _capi.plan(params(*dec, block_table=FAKE + 2, page_size=64, block_table_stride=64))[0] == _capi.ERR_STRIDE

@@ -42,10 +42,19 @@ CASES = [
     (4, 8, 2, 1, 2048, 128, "bf16", 64, "decode"),
     (2, 32, 8, 1, 8192, 128, "bf16", 256, "decode"),     # split cache + merge
     (3, 8, 4, 1, 1000, 64, "f16", 32, "decode"),         # ragged last page, head_dim 64
-    (2, 8, 2, 4, 3000, 128, "bf16", 128, "decode"),      # 16 rows per KV head
+    (2, 8, 2, 2, 3000, 128, "bf16", 128, "decode"),      # 8 rows per KV head
+    (2, 8, 2, 4, 3000, 128, "bf16", 128, "prefill"),     # 16 rows per KV head: packed heads on the MFMA kernel
+    (2, 8, 2, 4, 3000, 128, "bf16", 32, "decode"),       # ... or the streaming kernel when the pages are too small for it
     (2, 4, 2, 1, 300, 128, "bf16", 16, "general"),       # pages smaller than a key block
     (2, 4, 2, 40, 200, 96, "f32", 8, "general"),
-    (1, 4, 4, 70, 500, 128, "f16", 64, "general"),       # many query rows: the prefill kernels need contiguous K/V
+    (1, 4, 4, 70, 500, 128, "f16", 64, "prefill"),       # many query rows: the 4-wavefront MFMA kernel, ragged last tile
+    (1, 4, 4, 70, 500, 128, "f16", 32, "general"),       # ... whose 64-key tiles need pages of 64 rows or more
+    (2, 8, 2, 300, 1500, 128, "bf16", 128, "prefill"),   # the pipelined head_dim-128 kernel over pages
+    (2, 8, 4, 200, 777, 64, "bf16", 64, "prefill"),      # head_dim 64, ragged last page
+    (2, 4, 2, 130, 600, 96, "f16", 256, "prefill"),      # head_dim 96
+    (2, 8, 2, 150, 900, 128, "f32", 64, "prefill"),      # the fp32 MFMA kernel
+    (2, 8, 4, 1, 2000, 64, "f32", 128, "prefill"),       # fp32 decode: packed heads + split keys over pages
+    (2, 32, 8, 8, 4096, 128, "bf16", 256, "prefill"),    # 32 rows per KV head: packed heads + split keys over pages
 ]
 
 
@@ -121,3 +130,29 @@ def test_paged_equals_contiguous_bitwise_at_full_size():
     ref = sdpAttention(q, k, v)
     out = sdpAttention(q, kp, vp, blockTable=perm)
     assert torch.equal(ref, out)
+
+
+def test_paged_chunked_prefill_equals_contiguous_bitwise():
+    """Config 3's shape as four chunks of 1024 tokens: each chunk's K/V rows are appended into pages of 128 rows, then
+    its queries attend bottom-right causally to the cache so far.  The pipelined kernel over pages gives the bits it
+    gives over the contiguous prefix (same tiles, same order; only the tile addresses differ)."""
+    B, Hq, Hkv, S, D, C, page = 2, 32, 8, 4096, 128, 1024, 128
+    gen = torch.Generator(device="cuda").manual_seed(12)
+    q = torch.randn(B, Hq, S, D, device="cuda", generator=gen).bfloat16()
+    k = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).bfloat16()
+    v = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).bfloat16()
+    n = S // page
+    table = torch.randperm(B * n + 5, device="cuda", generator=gen)[:B * n].int().view(B, n).contiguous()
+    kp = torch.full((B * n + 5, Hkv, page, D), float("nan"), dtype=torch.bfloat16, device="cuda")
+    vp = torch.full_like(kp, float("nan"))
+    for c in range(S // C):
+        say("paged chunk", c)
+        end = (c + 1) * C
+        kvCacheAppend(kp, vp, k[:, :, c * C:end], v[:, :, c * C:end], c * C, blockTable=table)
+        lens = torch.full((B,), end, dtype=torch.int32, device="cuda")
+        qc = q[:, :, c * C:end]
+        o = torch.empty_like(qc)
+        assert route_of(qc, kp, vp, kv_lens=lens, block_table=table, out=o, causal=True, align="bottom-right") == "prefill"
+        paged = sdpAttention(qc, kp, vp, isCausal=True, causalAlign="bottom-right", kvLens=lens, blockTable=table)
+        flat = sdpAttention(qc, k[:, :, :end], v[:, :, :end], isCausal=True, causalAlign="bottom-right")
+        assert torch.equal(paged, flat), c

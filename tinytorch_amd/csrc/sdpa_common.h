@@ -41,6 +41,15 @@ __device__ __forceinline__ int causal_offset(const KArgs& a, int S) {
   return (a.causal_br && d > 0) ? d : 0;
 }
 
+// Element offset of key tile kv0 (a multiple of the tile length, which divides the page size) from the K or V pointer
+// of a (batch, kv head): `table` is the batch entry's row of the block table, or nullptr for a contiguous cache.  For
+// paged caches the (batch, kv head) pointer carries the head offset only: pstride is the pool's page stride.
+__device__ __forceinline__ long long kv_tile_offset(const KArgs& a, const int* table, int kv0, long long rstride, long long pstride) {
+  if (!table) return (long long)kv0 * rstride;
+  const int page = __builtin_amdgcn_readfirstlane(table[kv0 >> a.page_shift]);
+  return (long long)page * pstride + (long long)(kv0 & ((1 << a.page_shift) - 1)) * rstride;
+}
+
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));

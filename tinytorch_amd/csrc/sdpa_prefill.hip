@@ -105,8 +105,9 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
   const int qw0 = q0 + wave * 32;
 
   const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
-  const T* kp = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
-  const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
+  const int* table = a.block_table ? a.block_table + (long long)b * a.bt_stride : nullptr;  // paged cache
+  const T* kp = (const T*)a.k + (table ? 0 : b * a.ks[0]) + hk * a.ks[1];
+  const T* vp = (const T*)a.v + (table ? 0 : b * a.vs[0]) + hk * a.vs[1];
 
   // ---- Q rows of this wavefront, kept in registers as MFMA B operands -----------------------------------------
   vec8 qreg[KSTEPS];
@@ -177,8 +178,10 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
     voff[i] = (unsigned)(lrow[i] * a.vs[2] + 8 * lcol[i]) * 2u;
   }
   auto load_tile = [&](int kv0) {
-    const char* kt = (const char*)(kp + kv0 * a.ks[2]);
-    const char* vt = (const char*)(vp + kv0 * a.vs[2]);
+    const T* ktile = kp + kv_tile_offset(a, table, kv0, a.ks[2], a.ks[0]);
+    const T* vtile = vp + kv_tile_offset(a, table, kv0, a.vs[2], a.vs[0]);
+    const char* kt = (const char*)ktile;
+    const char* vt = (const char*)vtile;
     if (kv0 + BN <= S) {
 #pragma unroll
       for (int i = 0; i < NLD; i++) {
@@ -188,10 +191,10 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
     } else {  // ragged last tile: rows past the end re-read the last valid row (masked later)
 #pragma unroll
       for (int i = 0; i < NLD; i++) {
-        int key = kv0 + lrow[i];
-        key = key < S ? key : S - 1;
-        kst[i] = *(const u32x4*)(kp + key * a.ks[2] + 8 * lcol[i]);
-        vst[i] = *(const u32x4*)(vp + key * a.vs[2] + 8 * lcol[i]);
+        int row = lrow[i];
+        row = kv0 + row < S ? row : S - 1 - kv0;
+        kst[i] = *(const u32x4*)(ktile + row * a.ks[2] + 8 * lcol[i]);
+        vst[i] = *(const u32x4*)(vtile + row * a.vs[2] + 8 * lcol[i]);
       }
     }
   };

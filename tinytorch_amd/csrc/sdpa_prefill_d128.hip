@@ -108,8 +108,9 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   const int h = hk * a.G + g;
 
   const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
-  const T* kp = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
-  const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
+  const int* table = a.block_table ? a.block_table + (long long)b * a.bt_stride : nullptr;  // paged cache
+  const T* kp = (const T*)a.k + (table ? 0 : b * a.ks[0]) + hk * a.ks[1];
+  const T* vp = (const T*)a.v + (table ? 0 : b * a.vs[0]) + hk * a.vs[1];
   int S = a.S;  // keys of this batch entry: all of them, or the filled prefix of a cache / the unpadded length
   if (a.kv_len) {
     int len = __builtin_amdgcn_readfirstlane(a.kv_len[b]);
@@ -191,9 +192,10 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   const unsigned smem_addr = (unsigned)(unsigned long)(lds_void*)smem;
-  auto dma_tile = [&](const T* base, long long rstride, const unsigned (&off)[2], int kv0, unsigned stage_addr) __attribute__((always_inline)) {
+  auto dma_tile = [&](const T* base, long long rstride, long long pstride, const unsigned (&off)[2], int kv0, unsigned stage_addr) __attribute__((always_inline)) {
+    const T* tile = base + kv_tile_offset(a, table, kv0, rstride, pstride);
     if (kv0 + BN <= S) {
-      const char* src = (const char*)(base + kv0 * rstride);
+      const char* src = (const char*)tile;
 #pragma unroll
       for (int i = 0; i < 2; i++) dma_issue(src, off[i], stage_addr + (8 * wave + 4 * i) * ROW_BYTES);
     } else {  // ragged last tile: rows past the end re-read the last valid row (their scores are masked)
@@ -204,12 +206,12 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
         int chunk = (lane & 15) ^ swz(row);
         int rowc = row < S - kv0 ? row : S - 1 - kv0;
         unsigned voff = ((unsigned)rowc * (unsigned)rstride + 8u * chunk) * 2u;
-        dma_issue((const char*)(base + kv0 * rstride), voff, stage_addr + (8 * wave + 4 * i) * ROW_BYTES);
+        dma_issue((const char*)tile, voff, stage_addr + (8 * wave + 4 * i) * ROW_BYTES);
       }
     }
   };
-  auto dma_k = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(kp, a.ks[2], ld_koff, tile * BN, smem_addr + stage * STAGE_BYTES); };
-  auto dma_v = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(vp, a.vs[2], ld_voff, tile * BN, smem_addr + (KSTAGES + stage) * STAGE_BYTES); };
+  auto dma_k = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(kp, a.ks[2], a.ks[0], ld_koff, tile * BN, smem_addr + stage * STAGE_BYTES); };
+  auto dma_v = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(vp, a.vs[2], a.vs[0], ld_voff, tile * BN, smem_addr + (KSTAGES + stage) * STAGE_BYTES); };
   // Wait until at most `keep` of this wavefront's global->LDS loads are still in flight (they complete in issue
   // order), then meet the other wavefronts: what was issued before the newest `keep` loads is visible to all.
   auto dma_wait_and_sync = [&](int keep) __attribute__((always_inline)) {

@@ -80,8 +80,9 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
   const int qw0 = q0 + wave * 32;
 
   const float* qp = (const float*)a.q + b * a.qs[0] + h * a.qs[1];
-  const float* kp = (const float*)a.k + b * a.ks[0] + hk * a.ks[1];
-  const float* vp = (const float*)a.v + b * a.vs[0] + hk * a.vs[1];
+  const int* table = a.block_table ? a.block_table + (long long)b * a.bt_stride : nullptr;  // paged cache
+  const float* kp = (const float*)a.k + (table ? 0 : b * a.ks[0]) + hk * a.ks[1];
+  const float* vp = (const float*)a.v + (table ? 0 : b * a.vs[0]) + hk * a.vs[1];
 
   // ---- Q: this lane's half of its query row, the B operands of the S^T MFMAs ---------------------------------------
   float qreg[KSTEPS];
@@ -150,12 +151,14 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
     lcol[i] = cidx % (D / 4);
   }
   auto load_tile = [&](int kv0) {
+    const float* ktile = kp + kv_tile_offset(a, table, kv0, a.ks[2], a.ks[0]);
+    const float* vtile = vp + kv_tile_offset(a, table, kv0, a.vs[2], a.vs[0]);
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
-      int key = kv0 + lrow[i];
-      key = key < S ? key : S - 1;  // rows past the end re-read the last valid row (masked later)
-      kst[i] = *(const f32x4*)(kp + key * a.ks[2] + 4 * lcol[i]);
-      vst[i] = *(const f32x4*)(vp + key * a.vs[2] + 4 * lcol[i]);
+      int row = lrow[i];
+      row = kv0 + row < S ? row : S - 1 - kv0;  // rows past the end re-read the last valid row (masked later)
+      kst[i] = *(const f32x4*)(ktile + row * a.ks[2] + 4 * lcol[i]);
+      vst[i] = *(const f32x4*)(vtile + row * a.vs[2] + 4 * lcol[i]);
     }
   };
   auto store_tile = [&](int stage) {

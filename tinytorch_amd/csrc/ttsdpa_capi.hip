@@ -87,6 +87,9 @@ int validate(const ttsdpa_params* p, KArgs* a) {
   return TTSDPA_OK;
 }
 
+// The MFMA prefill kernels stage key tiles of up to 64 rows: over a paged cache a tile must lie in one page.
+constexpr int kPrefillMinPage = 64;
+
 // 16-bit tensors the MFMA kernels can read with 16-byte loads and write with 8-byte stores.
 bool fast_layout_ok(const ttsdpa_params* p, bool masks_ok = false, bool pages_ok = false) {
   if (p->block_table && !pages_ok) return false;
@@ -106,7 +109,7 @@ bool simple_mask_ok(const ttsdpa_params* p) {
 
 // fp32 tensors the fp32 MFMA kernel can read and write with 16-byte accesses.
 bool f32_prefill_ok(const ttsdpa_params* p) {
-  if (p->dtype != TTSDPA_F32 || p->block_table || !simple_mask_ok(p)) return false;
+  if (p->dtype != TTSDPA_F32 || (p->block_table && p->page_size < kPrefillMinPage) || !simple_mask_ok(p)) return false;
   if (p->D != 128 && p->D != 64) return false;
   if (!(p->scale > 0.f) || !isfinite(p->scale) || p->S < 1 || p->L < 1) return false;
   if (!dense_last_ok(p->q_stride, 4) || !dense_last_ok(p->k_stride, 4) || !dense_last_ok(p->v_stride, 4) ||
@@ -166,7 +169,8 @@ bool prefill_ok(const ttsdpa_params* p) {
   if (f32_prefill_ok(p)) return true;
   // the pipelined head_dim-128 kernel takes any attnMask; the 4-wavefront kernel those it can read four keys at a time
   const bool mfma_head_dim = p->D == 32 || p->D == 64 || p->D == 96 || p->D == 128 || p->D == 256;
-  return fast_layout_ok(p, true) && mfma_head_dim && p->S >= 1 && p->L >= 1 && (pipelined_ok(p) || simple_mask_ok(p));
+  if (p->block_table && p->page_size < kPrefillMinPage) return false;
+  return fast_layout_ok(p, true, true) && mfma_head_dim && p->S >= 1 && p->L >= 1 && (pipelined_ok(p) || simple_mask_ok(p));
 }
 
 bool decode_ok(const ttsdpa_params* p) {
