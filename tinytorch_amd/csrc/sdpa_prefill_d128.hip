@@ -70,7 +70,9 @@ typedef __attribute__((address_space(1))) const void gbl_void;
 
 __device__ __forceinline__ int swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
-template <typename TR, bool CAUSAL>
+// PAGED: K/V are page pools addressed through a block table (a variant of its own: the table look-ups cost the
+// contiguous path 1-3 % when they are a run-time branch).
+template <typename TR, bool CAUSAL, bool PAGED>
 __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
@@ -108,9 +110,9 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   const int h = hk * a.G + g;
 
   const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
-  const int* table = a.block_table ? a.block_table + (long long)b * a.bt_stride : nullptr;  // paged cache
-  const T* kp = (const T*)a.k + (table ? 0 : b * a.ks[0]) + hk * a.ks[1];
-  const T* vp = (const T*)a.v + (table ? 0 : b * a.vs[0]) + hk * a.vs[1];
+  const int* table = PAGED ? a.block_table + (long long)b * a.bt_stride : nullptr;
+  const T* kp = (const T*)a.k + (PAGED ? 0 : b * a.ks[0]) + hk * a.ks[1];
+  const T* vp = (const T*)a.v + (PAGED ? 0 : b * a.vs[0]) + hk * a.vs[1];
   int S = a.S;  // keys of this batch entry: all of them, or the filled prefix of a cache / the unpadded length
   if (a.kv_len) {
     int len = __builtin_amdgcn_readfirstlane(a.kv_len[b]);
@@ -192,8 +194,21 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   const unsigned smem_addr = (unsigned)(unsigned long)(lds_void*)smem;
-  auto dma_tile = [&](const T* base, long long rstride, long long pstride, const unsigned (&off)[2], int kv0, unsigned stage_addr) __attribute__((always_inline)) {
-    const T* tile = base + kv_tile_offset(a, table, kv0, rstride, pstride);
+  // Paged cache: the table entry of a tile is fetched while the previous tile of the same stream (K or V) is issued,
+  // so that the address of a tile does not wait for a scalar load: {entry index, page} of the prefetched entry.
+  int kpage[2] = {-1, 0}, vpage[2] = {-1, 0};
+  auto dma_tile = [&](const T* base, long long rstride, long long pstride, int (&pc)[2], const unsigned (&off)[2], int kv0, unsigned stage_addr) __attribute__((always_inline)) {
+    long long toff = (long long)kv0 * rstride;
+    if (PAGED) {
+      const int want = kv0 >> a.page_shift;
+      int page = pc[1];
+      if (pc[0] != want) page = __builtin_amdgcn_readfirstlane(table[want]);
+      toff = (long long)page * pstride + (long long)(kv0 & ((1 << a.page_shift) - 1)) * rstride;
+      const int nxt = (kv0 + BN) >> a.page_shift;
+      pc[0] = want, pc[1] = page;
+      if (nxt != want && kv0 + BN < S) pc[0] = nxt, pc[1] = __builtin_amdgcn_readfirstlane(table[nxt]);
+    }
+    const T* tile = base + toff;
     if (kv0 + BN <= S) {
       const char* src = (const char*)tile;
 #pragma unroll
@@ -210,8 +225,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       }
     }
   };
-  auto dma_k = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(kp, a.ks[2], a.ks[0], ld_koff, tile * BN, smem_addr + stage * STAGE_BYTES); };
-  auto dma_v = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(vp, a.vs[2], a.vs[0], ld_voff, tile * BN, smem_addr + (KSTAGES + stage) * STAGE_BYTES); };
+  auto dma_k = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(kp, a.ks[2], a.ks[0], kpage, ld_koff, tile * BN, smem_addr + stage * STAGE_BYTES); };
+  auto dma_v = [&](int tile, int stage) __attribute__((always_inline)) { dma_tile(vp, a.vs[2], a.vs[0], vpage, ld_voff, tile * BN, smem_addr + (KSTAGES + stage) * STAGE_BYTES); };
   // Wait until at most `keep` of this wavefront's global->LDS loads are still in flight (they complete in issue
   // order), then meet the other wavefronts: what was issued before the newest `keep` loads is visible to all.
   auto dma_wait_and_sync = [&](int keep) __attribute__((always_inline)) {
@@ -543,14 +558,19 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }  // part
 }
 
-template <typename TR, bool CAUSAL>
-int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
+template <typename TR, bool CAUSAL, bool PAGED>
+int launch_v(const KArgs& a, dim3 grid, hipStream_t stream) {
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)prefill128_kernel<TR, CAUSAL>, LDS_BYTES, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill128_kernel<TR, CAUSAL, PAGED>, LDS_BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
-  hipLaunchKernelGGL((prefill128_kernel<TR, CAUSAL>), grid, dim3(NW * 64), LDS_BYTES, stream, a);
+  hipLaunchKernelGGL((prefill128_kernel<TR, CAUSAL, PAGED>), grid, dim3(NW * 64), LDS_BYTES, stream, a);
   return (int)hipGetLastError();
+}
+
+template <typename TR, bool CAUSAL>
+int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
+  return a.block_table ? launch_v<TR, CAUSAL, true>(a, grid, stream) : launch_v<TR, CAUSAL, false>(a, grid, stream);
 }
 
 }  // namespace
