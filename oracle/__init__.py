@@ -53,6 +53,9 @@ def lib():
         L.oracle_sdpa_rows_f32.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p] + [_i64] * 6 + [
             ctypes.c_int, ctypes.c_float, _c_i64p, _i64, ctypes.c_int]
         L.oracle_sdpa_rows_f32.restype = ctypes.c_int
+        L.oracle_sdpa_backward_f32.argtypes = [_c_f32p] * 7 + [_i64] * 6 + [
+            ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_int]
+        L.oracle_sdpa_backward_f32.restype = ctypes.c_int
         L.oracle_rms_norm.argtypes = [_c_f32p, _c_f32p, _c_f32p, _i64, _i64, ctypes.c_float, ctypes.c_int]
         L.oracle_rms_norm.restype = None
         L.oracle_fused_add_rms_norm.argtypes = [_c_f32p, _c_f32p, _c_f32p, _i64, _i64, ctypes.c_float, ctypes.c_int]
@@ -194,6 +197,40 @@ def sdpa_rows_f32(q, k, v, rows, causal=False, scale=None, nthreads=None):
     if rc != 0:
         raise RuntimeError("oracle_sdpa_rows_f32 failed: %d" % rc)
     return out
+
+
+def sdpa_backward_f32(q, k, v, dout, causal=False, scale=None, mask=None, nthreads=None):
+    """Gradients (dq, dk, dv) of sum(sdpa(q, k, v) * dout): the chain rule through the restated forward, accumulated in
+    double.  Same shapes and mask conventions as sdpa_f32."""
+    q, k, v, dout = _f32(q), _f32(k), _f32(v), _f32(dout)
+    B, Hq, Hkv, L, S, D = _dims(q, k, v)
+    assert dout.shape == q.shape
+    sc = np.float32(1.0) / np.sqrt(np.float32(D)) if scale is None else np.float32(scale)
+    if mask is not None and tuple(mask.shape) != (L, S):
+        full = np.broadcast_to(mask, (B, Hq, L, S))   # every (batch, head) slice sees its own [L,S] slice
+        G = Hq // Hkv
+        dq = np.empty(q.shape, dtype=np.float32)
+        dk = np.zeros(k.shape, dtype=np.float64)
+        dv = np.zeros(v.shape, dtype=np.float64)
+        for b in range(B):
+            for h in range(Hq):
+                hk = h // G
+                a, bk, bv = sdpa_backward_f32(q[b:b + 1, h:h + 1], k[b:b + 1, hk:hk + 1], v[b:b + 1, hk:hk + 1],
+                                              dout[b:b + 1, h:h + 1], scale=sc, mask=np.ascontiguousarray(full[b, h]),
+                                              nthreads=nthreads)
+                dq[b, h] = a[0, 0]
+                dk[b, hk] += bk[0, 0]
+                dv[b, hk] += bv[0, 0]
+        return dq, dk.astype(np.float32), dv.astype(np.float32)
+    kind, keep, mp = _mask_args(mask, L, S)
+    dq = np.empty(q.shape, dtype=np.float32)
+    dk = np.zeros(k.shape, dtype=np.float32)
+    dv = np.zeros(v.shape, dtype=np.float32)
+    rc = lib().oracle_sdpa_backward_f32(_p(q), _p(k), _p(v), _p(dout), _p(dq), _p(dk), _p(dv), B, Hq, Hkv, L, S, D,
+                                        int(bool(causal)), float(sc), kind, mp, nthreads or default_threads())
+    if rc != 0:
+        raise RuntimeError("oracle_sdpa_backward_f32 failed: %d" % rc)
+    return dq, dk, dv
 
 
 def ref_sdpa_f32(q, k, v, causal=False, scale=None, mask=None):

@@ -375,3 +375,102 @@ int oracle_sdpa_rows_f32(const float* q, const float* k, const float* v, float* 
   size_t scratch = sizeof(float) * (size_t)(S > 0 ? S : 1);
   return run_pool(row_task, &c, nrows, scratch, nthreads);
 }
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Gradients of the attention path.  The reference has none (FuncSDPAttention::backward and FuncMatmul::backward are
+ * NOT_IMPLEMENTED, reference src/Function/FuncNNLayer.h:267, src/Function/FuncLinalg.h:20): this is the chain rule
+ * through the forward above, accumulated in double.  The softmax step is the reference's own
+ * (src/Operation/OpNNLayerCpu.h:79-109: dx_j = y_j * (dy_j - sum_t y_t dy_t)); the matmul steps are dA = dC B^T,
+ * dB = A^T dC.  One task per (batch, kv head): dK and dV sum over the query heads of the group in head order.
+ * ---------------------------------------------------------------------------------------------------------------- */
+
+typedef struct {
+  const float *q, *k, *v, *dout;
+  float *dq, *dk, *dv;
+  int64_t B, Hq, Hkv, L, S, D;
+  int causal;
+  float scale;
+  int mask_kind;
+  const void* mask;
+} sdpa_bwd_ctx;
+
+/* scratch: p [S] double, dp [S] double, dk [S*D] double, dv [S*D] double */
+static void bwd_task(void* vctx, int64_t task, void* scratch) {
+  sdpa_bwd_ctx* c = (sdpa_bwd_ctx*)vctx;
+  const int64_t b = task / c->Hkv, hk = task % c->Hkv;
+  const int64_t G = c->Hq / c->Hkv, L = c->L, S = c->S, D = c->D;
+  const float* k = c->k + (b * c->Hkv + hk) * S * D;
+  const float* v = c->v + (b * c->Hkv + hk) * S * D;
+  double* p = (double*)scratch;
+  double* dp = p + S;
+  double* dka = dp + S;
+  double* dva = dka + S * D;
+  for (int64_t i = 0; i < S * D; i++) dka[i] = 0.0, dva[i] = 0.0;
+  for (int64_t g = 0; g < G; g++) {
+    const int64_t h = hk * G + g;
+    const float* q = c->q + (b * c->Hq + h) * L * D;
+    const float* go = c->dout + (b * c->Hq + h) * L * D;
+    float* dq = c->dq + (b * c->Hq + h) * L * D;
+    for (int64_t i = 0; i < L; i++) {
+      /* scores of row i with the forward's bias, softmax in double */
+      double mx = -INFINITY;
+      for (int64_t j = 0; j < S; j++) {
+        double s = 0.0;
+        for (int64_t d = 0; d < D; d++) s += (double)q[i * D + d] * (double)k[j * D + d];
+        s *= (double)c->scale;
+        if (c->causal && j > i) s = -INFINITY;
+        if (c->mask_kind == ORACLE_MASK_BOOL && !((const uint8_t*)c->mask)[i * S + j]) s = -INFINITY;
+        if (c->mask_kind == ORACLE_MASK_FLOAT) s += (double)((const float*)c->mask)[i * S + j];
+        p[j] = s;
+        if (s > mx) mx = s;
+      }
+      double sum = 0.0;
+      for (int64_t j = 0; j < S; j++) {
+        p[j] = exp(p[j] - mx);
+        sum += p[j];
+      }
+      for (int64_t j = 0; j < S; j++) p[j] /= sum;
+      /* out = P V:  dV += P^T dOut,  dP = dOut V^T */
+      double dot = 0.0;
+      for (int64_t j = 0; j < S; j++) {
+        double t = 0.0;
+        for (int64_t d = 0; d < D; d++) {
+          t += (double)go[i * D + d] * (double)v[j * D + d];
+          dva[j * D + d] += p[j] * (double)go[i * D + d];
+        }
+        dp[j] = t;
+        dot += p[j] * t;
+      }
+      /* softmax: dS_j = P_j (dP_j - sum_t P_t dP_t); scores = scale * Q K^T: dQ = scale dS K, dK += scale dS^T Q */
+      double acc[1024]; /* dQ row i; D <= 1024 is checked by the entry point */
+      for (int64_t d = 0; d < D; d++) acc[d] = 0.0;
+      for (int64_t j = 0; j < S; j++) {
+        const double ds = p[j] * (dp[j] - dot) * (double)c->scale;
+        if (ds == 0.0) continue;
+        for (int64_t d = 0; d < D; d++) {
+          acc[d] += ds * (double)k[j * D + d];
+          dka[j * D + d] += ds * (double)q[i * D + d];
+        }
+      }
+      for (int64_t d = 0; d < D; d++) dq[i * D + d] = (float)acc[d];
+    }
+  }
+  float* dk = c->dk + (b * c->Hkv + hk) * S * D;
+  float* dv = c->dv + (b * c->Hkv + hk) * S * D;
+  for (int64_t i = 0; i < S * D; i++) dk[i] = (float)dka[i], dv[i] = (float)dva[i];
+}
+
+int oracle_sdpa_backward_f32(const float* q, const float* k, const float* v, const float* dout, float* dq, float* dk,
+                             float* dv, int64_t B, int64_t Hq, int64_t Hkv, int64_t L, int64_t S, int64_t D,
+                             int causal, float scale, int mask_kind, const void* mask, int nthreads) {
+  if (bad_dims(B, Hq, Hkv, L, S, D) || D > 1024) return -1;
+  if (mask_kind != ORACLE_MASK_NONE && !mask) return -1;
+  if (B == 0) return 0;
+  sdpa_bwd_ctx c;
+  memset(&c, 0, sizeof(c));
+  c.q = q, c.k = k, c.v = v, c.dout = dout, c.dq = dq, c.dk = dk, c.dv = dv;
+  c.B = B, c.Hq = Hq, c.Hkv = Hkv, c.L = L, c.S = S, c.D = D;
+  c.causal = causal, c.scale = scale, c.mask_kind = mask_kind, c.mask = mask;
+  size_t scratch = sizeof(double) * (size_t)(2 * S + 2 * S * D + 1);
+  return run_pool(bwd_task, &c, B * Hkv, scratch, nthreads);
+}

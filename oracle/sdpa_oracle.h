@@ -8,6 +8,10 @@
  *   oracle_sdpa_f32            pinned: reference KATs (test/test_function.cpp:393-419), bit-exact against the compiled
  *                              reference (oracle/_ref) and against fixtures written from it, fp64 closed form,
  *                              invariants (causal row 0 == v[0], rows of P sum to 1, uniform-K running mean).
+ *   oracle_sdpa_backward_f32   the reference has no attention (or matmul) backward to compare with: pinned by central
+ *                              differences of an independent float64 forward, by closed forms (one key; zero
+ *                              queries) and by invariants (columns of dK sum to 0, GQA == repeated K/V summed over
+ *                              the group) in tests/test_oracle_backward.py.
  *   oracle_round_bf16 / _f16   pinned: bit-exact against the reference's own casts over a sweep that includes
  *                              ties, subnormals, overflow, inf and NaN; and against numpy float16 casts.
  *   oracle_randn               not a reference function (the harness's own PRNG); pinned by moments and by a
@@ -55,6 +59,14 @@ int oracle_sdpa_f32(const float* q, const float* k, const float* v, float* out, 
 int oracle_sdpa_rows_f32(const float* q, const float* k, const float* v, float* out, int64_t B, int64_t Hq,
                          int64_t Hkv, int64_t L, int64_t S, int64_t D, int causal, float scale, const int64_t* rows,
                          int64_t nrows, int nthreads);
+
+/* Gradients of oracle_sdpa_f32's output with respect to q, k, v for an upstream gradient dout [B,Hq,L,D]: the chain
+ * rule through scores = scale * Q K^T + bias, P = softmax(scores), out = P V, accumulated in double and rounded to
+ * fp32 once.  dq [B,Hq,L,D]; dk, dv [B,Hkv,S,D] sum over the query heads that share a kv head.  Same causal / mask
+ * arguments as the forward; D <= 1024.  S == 0 gives dq = 0 and writes nothing to dk / dv. */
+int oracle_sdpa_backward_f32(const float* q, const float* k, const float* v, const float* dout, float* dq, float* dk,
+                             float* dv, int64_t B, int64_t Hq, int64_t Hkv, int64_t L, int64_t S, int64_t D,
+                             int causal, float scale, int mask_kind, const void* mask, int nthreads);
 
 /* Row-wise neighbour ops (fused_oracle.c): rmsNorm, fusedAddRmsNorm (in place), siluMul, softmax / logSoftmax over
  * [outer, dim, inner].  dtype: 0 fp32, 1 fp16, 2 bf16 = the element type the reference would store in. */
