@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TTSDPA_ABI_VERSION 5
+#define TTSDPA_ABI_VERSION 6
 
 /* Element types; numbering is the reference's DType enum (reference src/Tensor/DType.h:20-28). */
 enum ttsdpa_dtype { TTSDPA_F32 = 0, TTSDPA_F16 = 1, TTSDPA_BF16 = 2 };
@@ -152,6 +152,44 @@ int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_byt
 int ttsdpa_prefill(const ttsdpa_params* p, void* stream);
 int ttsdpa_decode(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream);
 int ttsdpa_general(const ttsdpa_params* p, void* stream);
+
+/*
+ * Backward of the attention call.  The reference declares it and stops there: FuncSDPAttention::backward is
+ * NOT_IMPLEMENTED() (reference src/Function/FuncNNLayer.h:267), as is FuncMatmul::backward (src/Function/FuncLinalg.h:20),
+ * so a model that attends cannot be trained with it.  This entry point is what that backward would call: for the
+ * forward call `fwd` (same tensors, mask, causal mode and scale; fwd.out is the forward's result and is READ here) and
+ * the upstream gradient dout [B,Hq,L,D] it writes dq [B,Hq,L,D], dk and dv [B,Hkv,S,D] — the chain rule through
+ * matmul -> scale -> bias -> softmax -> matmul (src/Function/FuncNNLayer.h:237-265), with the reference's own softmax
+ * backward step (src/Operation/OpNNLayerCpu.h:79-109).  dk / dv sum over the query heads of a KV head; rows of dk / dv
+ * at or beyond kv_len[b] are written as zeros.  Gradients have the element type of the inputs; strides are in elements
+ * {batch, head, sequence}, head_dim stride 1.  Paged caches (fwd.block_table) are not differentiated:
+ * TTSDPA_ERR_UNSUPPORTED.  A query row whose keys are all hidden gets dq = 0 and adds nothing to dk / dv.
+ * Scratch: ttsdpa_backward_workspace_bytes() bytes of device memory (per-row softmax statistics, and fp32 partial
+ * gradients where a kernel needs them); TTSDPA_ERR_WORKSPACE with less.  No allocation, no synchronisation; results
+ * do not depend on timing (no atomics).
+ */
+typedef struct ttsdpa_backward_params {
+  uint32_t struct_size; /* sizeof(ttsdpa_backward_params) */
+  uint32_t reserved;    /* 0 */
+  ttsdpa_params fwd;
+  const void* dout;
+  void* dq;
+  void* dk;
+  void* dv;
+  int64_t dout_stride[3];
+  int64_t dq_stride[3];
+  int64_t dk_stride[3];
+  int64_t dv_stride[3];
+} ttsdpa_backward_params;
+
+/* Fill *p for dense tensors (ttsdpa_params_init for fwd, dense gradient strides); pointers NULL. */
+void ttsdpa_backward_params_init(ttsdpa_backward_params* p, int dtype, int B, int Hq, int Hkv, int L, int S, int D);
+/* Validate and report the kernels ttsdpa_backward would use: TTSDPA_ROUTE_PREFILL = the MFMA backward kernels
+ * (fp16/bf16, head_dim 64 or 128, no attnMask, no kv_len), TTSDPA_ROUTE_GENERAL = the vector-ALU kernels,
+ * TTSDPA_ROUTE_NONE = nothing to compute.  Needs no GPU. */
+int ttsdpa_backward_plan(const ttsdpa_backward_params* p, int* route);
+size_t ttsdpa_backward_workspace_bytes(const ttsdpa_backward_params* p);
+int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * KV-cache append.  The reference has no KV cache: a caller that generates token by token grows K and V with

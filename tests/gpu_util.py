@@ -74,3 +74,36 @@ def max_abs_err(out_dev, expect):
     assert y.shape == expect.shape
     assert np.isfinite(y).all(), "non-finite values in the GPU result"
     return float(np.abs(y.astype(np.float64) - expect.astype(np.float64)).max())
+
+
+def backward_call(q, k, v, out, dout, causal=False, mask=None, scale=None, kv_lens=None, align="top-left", grads=None,
+                  ws_bytes=None):
+    """ttsdpa_backward through the C ABI -> (status, (dq, dk, dv))."""
+    from tinytorch_amd.function import build_backward_params
+    if grads is None:
+        grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+    bp = build_backward_params(q, k, v, out, dout, grads[0], grads[1], grads[2], causal, mask, scale, kv_lens, align)
+    L = _capi.lib()
+    nbytes = L.ttsdpa_backward_workspace_bytes(ctypes.byref(bp)) if ws_bytes is None else ws_bytes
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+    rc = L.ttsdpa_backward(ctypes.byref(bp), ws.data_ptr() if nbytes else None, nbytes, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return rc, grads
+
+
+def backward_route_of(q, k, v, out, dout, causal=False, mask=None, scale=None, kv_lens=None, align="top-left"):
+    from tinytorch_amd.function import build_backward_params
+    g = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+    bp = build_backward_params(q, k, v, out, dout, g[0], g[1], g[2], causal, mask, scale, kv_lens, align)
+    r = ctypes.c_int(-1)
+    assert _capi.lib().ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0
+    return _capi.ROUTE_NAMES[r.value]
+
+
+def grad_err(got_dev, expect):
+    """Max abs error of a gradient, in units of max(1, largest expected magnitude): the forward's bar applied to a
+    tensor whose entries are sums over many rows and exceed 1."""
+    y = to_host_f32(got_dev)
+    assert y.shape == expect.shape
+    assert np.isfinite(y).all(), "non-finite values in the GPU gradient"
+    return float(np.abs(y.astype(np.float64) - expect.astype(np.float64)).max() / max(1.0, float(np.abs(expect).max())))

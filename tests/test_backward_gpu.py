@@ -1,0 +1,165 @@
+"""Attention backward through the C ABI (ttsdpa_backward) against the oracle's gradients on the same seeded inputs.
+
+The reference has no attention backward (reference src/Function/FuncNNLayer.h:267 is NOT_IMPLEMENTED), so the oracle's
+gradients are pinned by differences, closed forms and invariants (tests/test_oracle_backward.py) rather than against
+reference vectors.  Bars: the forward's (fp32 1e-4, fp16/bf16 2e-2), in units of max(1, largest expected magnitude) —
+gradient entries are sums over many rows.  `out` handed to the backward is what the GPU forward produced."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import (TOL, TORCH_DTYPE, backward_call, backward_route_of, call, grad_err, make_inputs, to_device,
+                      to_host_f32)
+from tinytorch_amd import sdpAttention, sdpAttentionBackward
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def upstream(seed, shape, dtype):
+    vals, bits = oracle.round_to(oracle.randn(seed, 7, shape), dtype)
+    return vals, to_device(vals, bits, dtype)
+
+
+def check(case_name, host, dev, dtype, causal=False, mask_h=None, mask_d=None, scale=None, kv_lens=None, align="top-left",
+          oracle_mask=None, route=None):
+    say("backward", case_name)
+    q, k, v = dev
+    go_h, go = upstream(hash(case_name) % 1000, q.shape, dtype)
+    rc, out = call("forward", q, k, v, causal=causal, mask=mask_d, scale=scale, kv_lens=kv_lens, align=align)
+    assert rc == 0
+    if route is not None:
+        assert backward_route_of(q, k, v, out, go, causal, mask_d, scale, kv_lens, align) == route
+    rc, (dq, dk, dv) = backward_call(q, k, v, out, go, causal, mask_d, scale, kv_lens, align)
+    assert rc == 0
+    om = oracle_mask if oracle_mask is not None else mask_h
+    ocausal = causal and oracle_mask is None
+    eq, ek, ev = oracle.sdpa_backward_f32(host[0], host[1], host[2], go_h, causal=ocausal, scale=scale, mask=om)
+    for name, got, exp in (("dq", dq, eq), ("dk", dk, ek), ("dv", dv, ev)):
+        err = grad_err(got, exp)
+        assert err <= TOL[dtype], (name, err)
+
+
+GENERAL_CASES = [
+    # B, Hq, Hkv, L, S, D, dtype, causal
+    (1, 1, 1, 3, 5, 8, "f32", False),
+    (2, 4, 4, 33, 33, 64, "f32", True),
+    (2, 8, 2, 70, 130, 40, "f32", False),      # grouped heads, head_dim not a multiple of 64
+    (1, 4, 2, 65, 20, 96, "f32", True),        # L > S, top-left causal: rows past S see every key
+    (1, 2, 1, 17, 200, 256, "f32", False),     # the largest head_dim
+    (2, 4, 2, 50, 77, 64, "bf16", True),
+    (2, 4, 2, 50, 77, 128, "f16", False),
+    (1, 6, 3, 129, 64, 32, "bf16", False),
+]
+
+
+@pytest.mark.parametrize("case", GENERAL_CASES, ids=lambda c: "B%dH%dk%dL%dS%dD%d-%s-c%d" % c)
+def test_backward_against_oracle(case):
+    B, Hq, Hkv, L, S, D, dtype, causal = case
+    host, dev = make_inputs(4000 + L + S + D, B, Hq, Hkv, L, S, D, dtype)
+    check("plain-%s" % (case,), host, dev, dtype, causal=causal)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("kind", ["bool", "add", "keypad", "perhead"])
+def test_backward_with_masks(dtype, kind):
+    B, Hq, Hkv, L, S, D = 2, 4, 2, 19, 45, 64
+    host, dev = make_inputs(4100, B, Hq, Hkv, L, S, D, dtype)
+    rng = np.random.default_rng(3)
+    if kind == "bool":
+        m = rng.random((L, S)) < 0.7
+        m[:, 0] = True
+    elif kind == "add":
+        m = oracle.round_to(rng.standard_normal((L, S)).astype(np.float32), dtype)[0]
+    elif kind == "keypad":
+        m = np.arange(S)[None, None, None, :] < np.array([S, 30])[:, None, None, None]   # [B,1,1,S]
+    else:
+        m = rng.random((Hq, L, S)) < 0.7                                                    # [Hq,L,S]
+        m[..., 0] = True
+    md = torch.from_numpy(np.ascontiguousarray(m)).cuda()
+    if md.dtype != torch.bool:
+        md = md.to(TORCH_DTYPE[dtype])
+    check("mask-%s-%s" % (kind, dtype), host, dev, dtype, mask_h=m, mask_d=md, route="general")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_backward_bottom_right_causal_and_key_counts(dtype):
+    """Bottom-right alignment with per-batch key counts: the oracle sees it as a Bool mask per batch entry; rows of
+    dk / dv at or beyond the count are zero."""
+    B, Hq, Hkv, L, S, D = 3, 4, 2, 12, 90, 64
+    host, dev = make_inputs(4200, B, Hq, Hkv, L, S, D, dtype)
+    lens = [90, 40, 13]
+    kv = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    m = np.zeros((B, 1, L, S), dtype=bool)
+    for b in range(B):
+        m[b, 0] = np.arange(S)[None, :] <= np.arange(L)[:, None] + lens[b] - L
+        m[b, 0, :, lens[b]:] = False
+    check("br-%s" % dtype, host, dev, dtype, causal=True, kv_lens=kv, align="bottom-right", oracle_mask=m)
+    q, k, v = dev
+    go = upstream(1, q.shape, dtype)[1]
+    out = sdpAttention(q, k, v, isCausal=True, causalAlign="bottom-right", kvLens=kv)
+    _, dk, dv = sdpAttentionBackward(go, q, k, v, out, isCausal=True, causalAlign="bottom-right", kvLens=kv)
+    for b in range(B):
+        assert torch.all(dk[b, :, lens[b]:] == 0) and torch.all(dv[b, :, lens[b]:] == 0)
+
+
+def test_backward_strided_views_and_scale():
+    """q/k/v as slices of one packed projection output, gradients into slices of one packed buffer."""
+    B, H, N, D = 2, 4, 40, 64
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    qkv = torch.randn(B, N, 3, H, D, device="cuda", generator=gen)
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))      # [B,H,N,D] views, row stride 3*H*D
+    go = torch.randn(B, H, N, D, device="cuda", generator=gen)
+    out = sdpAttention(q, k, v, isCausal=True, scale=0.2)
+    dqkv = torch.full_like(qkv, float("nan"))
+    grads = tuple(dqkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    rc, _ = backward_call(q, k, v, out, go, causal=True, scale=0.2, grads=grads)
+    assert rc == 0 and torch.isfinite(dqkv).all()
+    eq, ek, ev = oracle.sdpa_backward_f32(to_host_f32(q), to_host_f32(k), to_host_f32(v), to_host_f32(go), causal=True, scale=0.2)
+    for got, exp in zip(grads, (eq, ek, ev)):
+        assert grad_err(got, exp) <= TOL["f32"]
+
+
+def test_backward_validation_and_empty_shapes():
+    from tinytorch_amd import _capi
+    q = torch.randn(1, 2, 4, 64, device="cuda")
+    k = torch.randn(1, 2, 6, 64, device="cuda")
+    v = torch.randn(1, 2, 6, 64, device="cuda")
+    out = sdpAttention(q, k, v)
+    go = torch.randn_like(q)
+    rc, _ = backward_call(q, k, v, out, go, ws_bytes=8)      # scratch too small
+    assert rc == _capi.ERR_WORKSPACE
+    with pytest.raises(ValueError):
+        sdpAttentionBackward(go[:, :1], q, k, v, out)
+    with pytest.raises(TypeError):
+        sdpAttentionBackward(go.half(), q, k, v, out)
+    # no keys: dq = 0, nothing else to write; no queries: dk = dv = 0
+    k0, v0 = k[:, :, :0], v[:, :, :0]
+    dq, dk, dv = sdpAttentionBackward(go, q, k0, v0, sdpAttention(q, k0, v0))
+    assert torch.all(dq == 0) and dk.numel() == 0
+    q0 = q[:, :, :0]
+    dq, dk, dv = sdpAttentionBackward(q0, q0, k, v, sdpAttention(q0, k, v))
+    assert dq.numel() == 0 and torch.all(dk == 0) and torch.all(dv == 0)
+
+
+def test_backward_matches_torch_autograd():
+    """A second, independent check: torch's autograd through plain fp32 matmul / softmax / matmul on the same device."""
+    B, Hq, Hkv, L, S, D = 2, 6, 2, 37, 53, 64
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    q = torch.randn(B, Hq, L, D, device="cuda", generator=gen, requires_grad=True)
+    k = torch.randn(B, Hkv, S, D, device="cuda", generator=gen, requires_grad=True)
+    v = torch.randn(B, Hkv, S, D, device="cuda", generator=gen, requires_grad=True)
+    go = torch.randn(B, Hq, L, D, device="cuda", generator=gen)
+    G = Hq // Hkv
+    s = (q @ k.repeat_interleave(G, 1).transpose(-1, -2)) / D ** 0.5
+    s = s.masked_fill(~torch.ones(L, S, dtype=torch.bool, device="cuda").tril(), float("-inf"))
+    ref = torch.softmax(s, -1) @ v.repeat_interleave(G, 1)
+    ref.backward(go)
+    out = sdpAttention(q.detach(), k.detach(), v.detach(), isCausal=True)
+    dq, dk, dv = sdpAttentionBackward(go, q.detach(), k.detach(), v.detach(), out, isCausal=True)
+    for got, exp in ((dq, q.grad), (dk, k.grad), (dv, v.grad)):
+        assert (got - exp).abs().max().item() <= 1e-4 * max(1.0, exp.abs().max().item())

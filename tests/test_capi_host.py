@@ -289,3 +289,40 @@ def test_linear_routes_and_validation():
     assert plan(_capi.BF16, 64, 64, 64, x=None)[0] == _capi.ERR_NULL
     assert L.ttlinear_forward(_capi.BF16, None, None, None, None, 0, 64, 64, 64, 64, 64, None) == 0
     assert L.ttlinear_forward(_capi.BF16, FAKE, FAKE, None, None, 8, 64, 64, 64, 64, 64, None) == _capi.ERR_NULL
+
+
+def test_backward_params_layout_routes_and_validation():
+    """struct ttsdpa_backward_params as the header lays it out; plan and validation of ttsdpa_backward without a GPU."""
+    L = _capi.lib()
+    bp = _capi.BackwardParams()
+    L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.BF16, 2, 8, 2, 64, 96, 128)
+    assert bp.struct_size == ctypes.sizeof(_capi.BackwardParams) == 8 + ctypes.sizeof(_capi.Params) + 4 * 8 + 4 * 24
+    assert bp.fwd.struct_size == ctypes.sizeof(_capi.Params) and bp.fwd.L == 64 and bp.fwd.S == 96
+    assert list(bp.dq_stride) == list(bp.fwd.q_stride) == [8 * 64 * 128, 64 * 128, 128]
+    assert list(bp.dk_stride) == list(bp.dv_stride) == list(bp.fwd.k_stride) == [2 * 96 * 128, 96 * 128, 128]
+    r = ctypes.c_int(-1)
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == _capi.ERR_NULL      # no tensors yet
+    bp.fwd.q = bp.fwd.k = bp.fwd.v = bp.fwd.out = FAKE
+    bp.dout = bp.dq = bp.dk = bp.dv = FAKE
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value in (_capi.ROUTE_GENERAL, _capi.ROUTE_PREFILL)
+    assert L.ttsdpa_backward_workspace_bytes(ctypes.byref(bp)) >= 2 * 8 * 64 * 2 * 4
+    assert L.ttsdpa_backward(ctypes.byref(bp), None, 0, None) == _capi.ERR_WORKSPACE
+    bp.dk = None
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == _capi.ERR_NULL
+    bp.dk = FAKE + 1
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == _capi.ERR_STRIDE
+    bp.dk = FAKE
+    bp.dv_stride[2] = 64
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == _capi.ERR_STRIDE
+    bp.dv_stride[2] = 128
+    bp.fwd.block_table, bp.fwd.page_size, bp.fwd.block_table_stride = FAKE, 64, 64
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == _capi.ERR_UNSUPPORTED
+    bp.fwd.block_table = None
+    bp.struct_size -= 8
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == _capi.ERR_ABI
+    # fp32 and masks: the vector-ALU kernels
+    L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.F32, 1, 4, 4, 32, 32, 64)
+    bp.fwd.q = bp.fwd.k = bp.fwd.v = bp.fwd.out = bp.dout = bp.dq = bp.dk = bp.dv = FAKE
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_GENERAL
+    L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.F32, 0, 4, 4, 32, 32, 64)
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_NONE

@@ -9,7 +9,7 @@ from . import _capi
 _capi.lib()  # fail loudly when the extension is missing
 
 from .function import (sdpAttention, kvCacheAppend, build_params, rmsNorm, fusedAddRmsNorm, siluMul, softmax,  # noqa: E402
-                       logSoftmax, linear)
+                       logSoftmax, linear, sdpAttentionBackward, build_backward_params)
 
 __all__ = ["sdpAttention", "kvCacheAppend", "build_params", "rmsNorm", "fusedAddRmsNorm", "siluMul", "softmax",
-           "logSoftmax", "linear"]
+           "logSoftmax", "linear", "sdpAttentionBackward", "build_backward_params"]

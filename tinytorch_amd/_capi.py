@@ -21,6 +21,7 @@ EXPORTS = [
     "ttsdpa_abi_version", "ttsdpa_status_string", "ttsdpa_params_init", "ttsdpa_plan", "ttsdpa_workspace_bytes",
     "ttsdpa_forward", "ttsdpa_prefill", "ttsdpa_decode", "ttsdpa_general",
     "ttsdpa_kv_append_params_init", "ttsdpa_kv_append", "ttsdpa_probe",
+    "ttsdpa_backward_params_init", "ttsdpa_backward_plan", "ttsdpa_backward_workspace_bytes", "ttsdpa_backward",
     # include/ttfused.h
     "ttfused_rms_norm", "ttfused_add_rms_norm", "ttfused_silu_mul", "ttfused_softmax",
     # include/ttlinear.h
@@ -53,6 +54,23 @@ class Params(ctypes.Structure):
         ("block_table", ctypes.c_void_p),
         ("page_size", ctypes.c_int32),
         ("block_table_stride", ctypes.c_int32),
+    ]
+
+
+class BackwardParams(ctypes.Structure):
+    """struct ttsdpa_backward_params"""
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32),
+        ("fwd", Params),
+        ("dout", ctypes.c_void_p),
+        ("dq", ctypes.c_void_p),
+        ("dk", ctypes.c_void_p),
+        ("dv", ctypes.c_void_p),
+        ("dout_stride", ctypes.c_int64 * 3),
+        ("dq_stride", ctypes.c_int64 * 3),
+        ("dk_stride", ctypes.c_int64 * 3),
+        ("dv_stride", ctypes.c_int64 * 3),
     ]
 
 
@@ -115,6 +133,15 @@ def lib():
         L.ttsdpa_kv_append_params_init.restype = None
         L.ttsdpa_kv_append.argtypes = [ctypes.POINTER(KvAppendParams), ctypes.c_void_p]
         L.ttsdpa_kv_append.restype = ctypes.c_int
+        BP = ctypes.POINTER(BackwardParams)
+        L.ttsdpa_backward_params_init.argtypes = [BP] + [ctypes.c_int] * 7
+        L.ttsdpa_backward_params_init.restype = None
+        L.ttsdpa_backward_plan.argtypes = [BP, ctypes.POINTER(ctypes.c_int)]
+        L.ttsdpa_backward_plan.restype = ctypes.c_int
+        L.ttsdpa_backward_workspace_bytes.argtypes = [BP]
+        L.ttsdpa_backward_workspace_bytes.restype = ctypes.c_size_t
+        L.ttsdpa_backward.argtypes = [BP, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        L.ttsdpa_backward.restype = ctypes.c_int
         L.ttsdpa_probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
                                    ctypes.POINTER(ctypes.c_double)]
         L.ttsdpa_probe.restype = ctypes.c_int
@@ -131,7 +158,7 @@ def lib():
         L.ttlinear_forward.restype = ctypes.c_int
         L.ttlinear_plan.argtypes = [ctypes.c_int, vp, vp, vp, vp] + [i64] * 6 + [ctypes.POINTER(ctypes.c_int)]
         L.ttlinear_plan.restype = ctypes.c_int
-        if L.ttsdpa_abi_version() != 5:
+        if L.ttsdpa_abi_version() != 6:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L
     return _lib

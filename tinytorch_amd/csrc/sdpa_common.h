@@ -164,6 +164,20 @@ __device__ __forceinline__ void apply_attn_mask(const KArgs& a, f32x16& s, long 
   }
 }
 
+// Backward call: the forward's arguments (f.out holds the forward's result, an input here) plus the upstream gradient
+// and the three gradients to write.  stats is scratch [B,Hq,L,2] floats: per query row the natural-log sum of
+// exponentials of its scaled, biased scores, and delta = dout . out.
+struct BwdArgs {
+  KArgs f;
+  const void* dout;
+  void* dq;
+  void* dk;
+  void* dv;
+  long long dos[3], dqs[3], dks[3], dvs[3];  // element strides: batch, head, sequence
+  float* stats;
+};
+int launch_backward_general(const BwdArgs& a, int dtype, hipStream_t stream);
+
 // Host-side launchers (one per kernel family); each returns a hipError_t as int.
 int launch_general(const KArgs& a, int dtype, hipStream_t stream);
 int launch_prefill(const KArgs& a, int dtype, hipStream_t stream);       // 128-row workgroups; head_dim 64 or 128

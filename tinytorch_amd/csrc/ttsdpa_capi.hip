@@ -199,6 +199,39 @@ int pick_route(const ttsdpa_params* p) {
   return TTSDPA_ROUTE_GENERAL;
 }
 
+// ---- backward ---------------------------------------------------------------------------------------------------------
+int validate_backward(const ttsdpa_backward_params* p, BwdArgs* a) {
+  if (!p) return TTSDPA_ERR_NULL;
+  if (p->struct_size != sizeof(ttsdpa_backward_params)) return TTSDPA_ERR_ABI;
+  int rc = validate(&p->fwd, &a->f);
+  if (rc != TTSDPA_OK) return rc;
+  const ttsdpa_params* f = &p->fwd;
+  if (f->block_table) return TTSDPA_ERR_UNSUPPORTED;
+  const size_t esz = f->dtype == TTSDPA_F32 ? 4 : 2;
+  if (f->B > 0 && f->L > 0 && (!p->dout || !p->dq)) return TTSDPA_ERR_NULL;
+  if (f->B > 0 && f->S > 0 && (!p->dk || !p->dv || !f->k || !f->v)) return TTSDPA_ERR_NULL;
+  if (!ptr_aligned(p->dout, esz) || !ptr_aligned(p->dq, esz) || !ptr_aligned(p->dk, esz) || !ptr_aligned(p->dv, esz))
+    return TTSDPA_ERR_STRIDE;
+  for (int i = 0; i < 3; i++) {
+    if (p->dout_stride[i] < 0 || p->dq_stride[i] < 0 || p->dk_stride[i] < 0 || p->dv_stride[i] < 0) return TTSDPA_ERR_STRIDE;
+    a->dos[i] = p->dout_stride[i], a->dqs[i] = p->dq_stride[i], a->dks[i] = p->dk_stride[i], a->dvs[i] = p->dv_stride[i];
+  }
+  if ((p->dout_stride[2] < f->D || p->dq_stride[2] < f->D) && f->L > 1) return TTSDPA_ERR_STRIDE;
+  if ((p->dk_stride[2] < f->D || p->dv_stride[2] < f->D) && f->S > 1) return TTSDPA_ERR_STRIDE;
+  a->dout = p->dout, a->dq = p->dq, a->dk = p->dk, a->dv = p->dv, a->stats = nullptr;
+  return TTSDPA_OK;
+}
+
+int pick_backward_route(const ttsdpa_backward_params* p) {
+  const ttsdpa_params* f = &p->fwd;
+  if (f->B == 0 || (f->L == 0 && f->S == 0)) return TTSDPA_ROUTE_NONE;
+  return TTSDPA_ROUTE_GENERAL;
+}
+
+size_t backward_stats_bytes(const ttsdpa_backward_params* p) {
+  return (size_t)p->fwd.B * p->fwd.Hq * p->fwd.L * 2 * sizeof(float);
+}
+
 int check_grid(long long nwg) { return nwg > 0x7fffffffLL ? TTSDPA_ERR_SHAPE : TTSDPA_OK; }
 
 }  // namespace
@@ -325,6 +358,42 @@ int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_byt
     case TTSDPA_ROUTE_PREFILL: return prefill_impl(p, workspace, workspace_bytes, stream);
     default: return ttsdpa_general(p, stream);
   }
+}
+
+void ttsdpa_backward_params_init(ttsdpa_backward_params* p, int dtype, int B, int Hq, int Hkv, int L, int S, int D) {
+  memset(p, 0, sizeof(*p));
+  p->struct_size = sizeof(*p);
+  ttsdpa_params_init(&p->fwd, dtype, B, Hq, Hkv, L, S, D);
+  for (int i = 0; i < 3; i++) {
+    p->dout_stride[i] = p->dq_stride[i] = p->fwd.q_stride[i];
+    p->dk_stride[i] = p->dv_stride[i] = p->fwd.k_stride[i];
+  }
+}
+
+int ttsdpa_backward_plan(const ttsdpa_backward_params* p, int* route) {
+  BwdArgs a;
+  int rc = validate_backward(p, &a);
+  if (rc != TTSDPA_OK) return rc;
+  if (route) *route = pick_backward_route(p);
+  return TTSDPA_OK;
+}
+
+size_t ttsdpa_backward_workspace_bytes(const ttsdpa_backward_params* p) {
+  BwdArgs a;
+  if (validate_backward(p, &a) != TTSDPA_OK) return 0;
+  return backward_stats_bytes(p);
+}
+
+int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t workspace_bytes, void* stream) {
+  BwdArgs a;
+  int rc = validate_backward(p, &a);
+  if (rc != TTSDPA_OK) return rc;
+  const int route = pick_backward_route(p);
+  if (route == TTSDPA_ROUTE_NONE) return TTSDPA_OK;
+  const size_t need = backward_stats_bytes(p);
+  if (need > 0 && (!workspace || workspace_bytes < need || !ptr_aligned(workspace, 16))) return TTSDPA_ERR_WORKSPACE;
+  a.stats = (float*)workspace;
+  return launch_backward_general(a, p->fwd.dtype, (hipStream_t)stream);
 }
 
 void ttsdpa_kv_append_params_init(ttsdpa_kv_append_params* p, int dtype, int B, int Hkv, int Smax, int Lnew, int D) {

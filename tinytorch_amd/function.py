@@ -136,6 +136,57 @@ def sdpAttention(query, key, value, isCausal=False, attnMask=None, dropoutP=0.0,
     return out
 
 
+def build_backward_params(query, key, value, out, gradOut, gradQuery, gradKey, gradValue, isCausal=False, attnMask=None,
+                          scale=None, kvLens=None, causalAlign="top-left"):
+    """Fill a ttsdpa_backward_params: the forward call of build_params plus the four gradient tensors."""
+    bp = _capi.BackwardParams()
+    bp.struct_size = ctypes.sizeof(_capi.BackwardParams)
+    bp.fwd = build_params(query, key, value, out, isCausal, attnMask, scale, kvLens, causalAlign)
+    bp.dout, bp.dq, bp.dk, bp.dv = gradOut.data_ptr(), gradQuery.data_ptr(), gradKey.data_ptr(), gradValue.data_ptr()
+    for name, t in (("dout_stride", gradOut), ("dq_stride", gradQuery), ("dk_stride", gradKey), ("dv_stride", gradValue)):
+        st = _strides3(t)
+        for i in range(3):
+            getattr(bp, name)[i] = st[i]
+    return bp
+
+
+def sdpAttentionBackward(gradOut, query, key, value, out, isCausal=False, attnMask=None, scale=None, kvLens=None,
+                         causalAlign="top-left"):
+    """(gradQuery, gradKey, gradValue) of sdpAttention(query, key, value, ...) for the upstream gradient gradOut.
+
+    What FuncSDPAttention::backward would compute; the reference leaves it NOT_IMPLEMENTED (reference
+    src/Function/FuncNNLayer.h:267).  `out` is the forward's result for the same arguments.  gradKey / gradValue have
+    the shape of key / value: with grouped heads they sum over the query heads of a KV head; rows at or beyond
+    kvLens[b] are zero.
+    """
+    if any(t.dim() != 4 for t in (gradOut, query, key, value, out)):
+        raise ValueError("sdpAttentionBackward: expected 4-D tensors [B, H, N, D]")
+    if not query.is_cuda:
+        raise RuntimeError("tinytorch_amd.sdpAttentionBackward runs on the GPU only; got a %s tensor" % query.device)
+    if any(t.device != query.device for t in (gradOut, key, value, out)):
+        raise RuntimeError("sdpAttentionBackward: all tensors must live on the same device")
+    if gradOut.shape != query.shape or out.shape != query.shape:
+        raise ValueError("sdpAttentionBackward: gradOut %s and out %s must have the shape of query %s"
+                         % (tuple(gradOut.shape), tuple(out.shape), tuple(query.shape)))
+    if gradOut.dtype != query.dtype or out.dtype != query.dtype:
+        raise TypeError("sdpAttentionBackward: gradOut and out must have the dtype of query")
+    fix = lambda t: t if (t.stride(-1) == 1 or t.size(-1) == 1) else t.contiguous()
+    gradOut, query, key, value, out = fix(gradOut), fix(query), fix(key), fix(value), fix(out)
+    gq, gk, gv = torch.empty_like(query), torch.empty_like(key), torch.empty_like(value)
+    if gq.stride(-1) != 1 or gk.stride(-1) != 1 or gv.stride(-1) != 1:
+        gq, gk, gv = (torch.empty(t.shape, dtype=t.dtype, device=t.device) for t in (query, key, value))
+    bp = build_backward_params(query, key, value, out, gradOut, gq, gk, gv, isCausal, attnMask, scale, kvLens, causalAlign)
+    L = _capi.lib()
+    with torch.cuda.device(query.device):
+        nbytes = L.ttsdpa_backward_workspace_bytes(ctypes.byref(bp))
+        ws = _workspace(query.device, nbytes) if nbytes else None
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = L.ttsdpa_backward(ctypes.byref(bp), ws.data_ptr() if ws is not None else None, nbytes, stream)
+    if rc != 0:
+        raise RuntimeError("ttsdpa_backward failed: %d (%s)" % (rc, _capi.status_string(rc)))
+    return gq, gk, gv
+
+
 def kvCacheAppend(kCache, vCache, kNew, vNew, positions, blockTable=None):
     """Write kNew/vNew [B,Hkv,Lnew,D] into the caches [B,Hkv,Smax,D] at rows positions[b] .. positions[b]+Lnew-1.
 
