@@ -64,6 +64,58 @@ def test_backward_against_oracle(case):
     check("plain-%s" % (case,), host, dev, dtype, causal=causal)
 
 
+MFMA_CASES = [
+    # B, Hq, Hkv, L, S, D, dtype, causal ("br" = bottom-right aligned)
+    (2, 8, 2, 256, 256, 128, "bf16", True),
+    (1, 4, 4, 200, 333, 64, "f16", False),        # ragged last tiles on both sides
+    (2, 6, 2, 130, 70, 128, "f16", True),         # L > S, top-left: rows past S see every key
+    (1, 8, 8, 64, 500, 128, "bf16", "br"),        # a chunk of 64 queries at the end of 500 keys
+    (2, 4, 1, 96, 96, 64, "bf16", True),          # four heads per KV head, head_dim 64
+    (1, 2, 2, 1, 129, 128, "bf16", False),        # one query row
+    (1, 2, 1, 300, 17, 64, "f16", "br"),          # more queries than keys, bottom-right: offset 0
+    (3, 4, 2, 33, 257, 128, "f16", False),
+]
+
+
+@pytest.mark.parametrize("case", MFMA_CASES, ids=lambda c: "B%dH%dk%dL%dS%dD%d-%s-%s" % c)
+def test_backward_mfma_against_oracle(case):
+    B, Hq, Hkv, L, S, D, dtype, causal = case
+    host, dev = make_inputs(4300 + L + S + D, B, Hq, Hkv, L, S, D, dtype)
+    if causal == "br":
+        m = np.arange(S)[None, :] <= np.arange(L)[:, None] + max(0, S - L)
+        check("mfma-%s" % (case,), host, dev, dtype, causal=True, align="bottom-right", oracle_mask=m, route="prefill")
+    else:
+        check("mfma-%s" % (case,), host, dev, dtype, causal=causal, route="prefill")
+
+
+def test_backward_mfma_properties_at_size():
+    """Config 3's shape (B2 32q/8kv 4096 x 4096 x 128 bf16, causal), where the oracle would take minutes: the gradients are
+    linear in dout (doubling it doubles them exactly: every product has one factor from dout), the columns of dk sum to ~0
+    (softmax ignores a shift common to all keys), and a sample of dq / dk / dv rows agrees with the vector-ALU kernels run
+    on fp32 copies of the same tensors."""
+    B, Hq, Hkv, N, D = 2, 32, 8, 4096, 128
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    q = torch.randn(B, Hq, N, D, device="cuda", generator=gen).bfloat16()
+    k = torch.randn(B, Hkv, N, D, device="cuda", generator=gen).bfloat16()
+    v = torch.randn(B, Hkv, N, D, device="cuda", generator=gen).bfloat16()
+    go = torch.randn(B, Hq, N, D, device="cuda", generator=gen).bfloat16()
+    out = sdpAttention(q, k, v, isCausal=True)
+    assert backward_route_of(q, k, v, out, go, True) == "prefill"
+    dq, dk, dv = sdpAttentionBackward(go, q, k, v, out, isCausal=True)
+    dq2, dk2, dv2 = sdpAttentionBackward(go * 2, q, k, v, out, isCausal=True)
+    assert torch.equal(dq2, dq * 2) and torch.equal(dk2, dk * 2) and torch.equal(dv2, dv * 2)
+    colsum = dk.float().sum(dim=2).abs().max().item()
+    assert colsum <= 2e-2 * N ** 0.5 * max(1.0, dk.float().abs().max().item()), colsum
+    # one batch entry, one KV head (its four query heads) on the fp32 kernels
+    sl = lambda t, h0, h1: t[1:2, h0:h1].float().contiguous()
+    qf, kf, vf, gf = sl(q, 8, 12), sl(k, 2, 3), sl(v, 2, 3), sl(go, 8, 12)
+    of = sdpAttention(qf, kf, vf, isCausal=True)
+    rq, rk, rv = sdpAttentionBackward(gf, qf, kf, vf, of, isCausal=True)
+    for got, ref in ((dq[1:2, 8:12], rq), (dk[1:2, 2:3], rk), (dv[1:2, 2:3], rv)):
+        err = (got.float() - ref).abs().max().item() / max(1.0, ref.abs().max().item())
+        assert err <= TOL["bf16"], err
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("kind", ["bool", "add", "keypad", "perhead"])
 def test_backward_with_masks(dtype, kind):

@@ -1,0 +1,496 @@
+// Attention backward for fp16 / bf16 on gfx950 matrix cores, head_dim 64 or 128, optional causal mask (either
+// alignment), grouped heads.  The reference has no attention backward (reference src/Function/FuncNNLayer.h:267 is
+// NOT_IMPLEMENTED); this is the chain rule through its forward chain matmul -> scale -> bias -> softmax -> matmul
+// (src/Function/FuncNNLayer.h:237-265, softmax step as src/Operation/OpNNLayerCpu.h:79-109) without ever storing an
+// [L,S] matrix:
+//   P_ij = exp(scale * q_i.k_j - lse_i)    dP_ij = dout_i.v_j    delta_i = dout_i.out_i    dS_ij = P_ij (dP_ij - delta_i)
+//   dq_i = scale * sum_j dS_ij k_j         dk_j = scale * sum_i dS_ij q_i                  dv_j = sum_i P_ij dout_i
+//
+// Two kernels, no atomics (fixed summation order, reproducible results):
+//   1. backward_dq_mfma_kernel — a workgroup owns 128 query rows of one (batch, query head), a wavefront 32 of them,
+//      and streams the keys in tiles of 64 exactly like the forward kernel: S^T = K.Q^T, an online softmax with a lazily
+//      raised maximum (so lse_i needs no pass of its own), dP^T = V.dout^T, dS^T, dq^T += K^T.dS^T.  At the end
+//      dq = scale/l * accumulator, and (lse_i, delta_i) go to scratch for the second kernel.
+//   2. backward_dkv_mfma_kernel — a workgroup owns 128 keys of one (batch, kv head), a wavefront 32 of them, and
+//      streams the query rows of every head of the group in tiles of 32: S = Q.K^T, P from lse, dP = dout.V^T, dS,
+//      dv^T += dout^T.P, dk^T += Q^T.dS.
+// Both compute 32 x 32 score blocks with v_mfma_f32_32x32x16 whose accumulator layout (lane = column, registers = rows)
+// is the B operand of the following product, so P and dS go from registers to the matrix cores without touching LDS;
+// the streamed tiles are staged in LDS twice where both a row-major operand and a transposed one
+// (ds_read_b64_tr_b16) are read from them, each copy with the row pitch that makes its reads conflict-free.
+// Seven matrix products in all, against five in the textbook count (the scores are computed in both kernels).
+
+#include "sdpa_common.h"
+
+namespace ttsdpa {
+
+namespace {
+
+constexpr int BM = 128;  // rows of the owning side per workgroup (queries in kernel 1, keys in kernel 2)
+constexpr int BN = 64;   // keys per streamed tile, kernel 1
+constexpr int BQ = 32;   // query rows per streamed tile, kernel 2
+constexpr float kLazyExp = 8.f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+
+template <int D>
+struct BwdLds {
+  static constexpr int RP = D + 8;    // row pitch (elements) of a tile read as a row-major operand (ds_read_b128)
+  static constexpr int TP = D + 32;   // row pitch of a tile read as a transposed operand (ds_read_b64_tr_b16)
+  static constexpr int DQ_STAGE = BN * (2 * RP + TP);       // K row-major, V row-major, K for transposed reads
+  static constexpr int DQ_BYTES = 2 * DQ_STAGE * 2;
+  static constexpr int KV_STAGE = BQ * (2 * RP + 2 * TP);   // Q and dout, each in both layouts
+  static constexpr int KV_STATS = 2 * BQ;                   // floats per stage: (lse, delta) per query row
+  static constexpr int KV_BYTES = 2 * KV_STAGE * 2 + 2 * KV_STATS * 4;
+};
+
+// One MFMA A operand of X^T from a row-major tile X with pitch TP: lane l (column d = d0 + l%32, half h = l/32)
+// receives the 8 rows base + {4h + 0..3, 8 + 4h + 0..3} — the order in which a 32x32 accumulator's registers 8t..8t+7
+// hold rows, so the other operand can be taken straight from such registers.
+template <typename vec8>
+__device__ __forceinline__ vec8 transposed_operand(const void* lane_base, int byte_off_lo, int byte_off_hi) {
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)((const char*)lane_base + byte_off_lo));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)((const char*)lane_base + byte_off_hi));
+  s16x8 r = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(vec8, r);
+}
+
+template <typename vec8>
+__device__ __forceinline__ vec8 regs_to_operand(const f32x16& acc, int t) {
+  f32x8 x;
+#pragma unroll
+  for (int i = 0; i < 8; i++) x[i] = acc[8 * t + i];
+  return __builtin_convertvector(x, vec8);
+}
+
+// ---- kernel 1: dq, lse, delta ----------------------------------------------------------------------------------------
+template <typename TR, int D, bool CAUSAL>
+__global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel(BwdArgs a) {
+  typedef typename TR::elem T;
+  typedef typename TR::vec8 vec8;
+  typedef BwdLds<D> Lds;
+  constexpr int RP = Lds::RP, TP = Lds::TP;
+  constexpr int KSTEPS = D / 16, DBLK = D / 32;
+  constexpr int NLD = (BN * D / 8) / 256;
+  const KArgs& f = a.f;
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  T* smem = (T*)smem_raw;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, lh = lane >> 5;
+
+  const int ntile = (f.L + BM - 1) / BM;
+  int n = blockIdx.x;
+  const int in = n % ntile;
+  n /= ntile;
+  const int h = n % f.Hq, b = n / f.Hq;
+  const int hk = h / f.G;
+  const int rt = CAUSAL ? ntile - 1 - in : in;  // longest rows first
+  const int q0 = rt * BM, qw0 = q0 + wave * 32;
+  const bool wave_live = qw0 < f.L;
+
+  const T* kp = (const T*)f.k + b * f.ks[0] + hk * f.ks[1];
+  const T* vp = (const T*)f.v + b * f.vs[0] + hk * f.vs[1];
+
+  // ---- this lane's query row: q and dout as B operands, delta = dout . out ------------------------------------------------
+  vec8 qreg[KSTEPS], greg[KSTEPS];
+  float delta;
+  {
+    int row = qw0 + lq;
+    row = row < f.L ? row : f.L - 1;
+    const T* qr = (const T*)f.q + b * f.qs[0] + h * f.qs[1] + row * f.qs[2] + 8 * lh;
+    const T* gr = (const T*)a.dout + b * a.dos[0] + h * a.dos[1] + row * a.dos[2] + 8 * lh;
+    const T* orow = (const T*)f.out + b * f.os[0] + h * f.os[1] + row * f.os[2] + 8 * lh;
+    float part = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      qreg[ks] = *(const vec8*)(qr + 16 * ks);
+      greg[ks] = *(const vec8*)(gr + 16 * ks);
+      const vec8 o = *(const vec8*)(orow + 16 * ks);
+#pragma unroll
+      for (int i = 0; i < 8; i++) part = fmaf((float)o[i], (float)greg[ks][i], part);
+    }
+    delta = part + __shfl_xor(part, 32);
+  }
+
+  f32x16 dqacc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dqacc[i][r] = 0.f;
+  const float c = f.scale * kLog2e;
+  const float lazy = kLazyExp / c;
+  float m_use = -1e30f, mc = m_use * c, l_run = 0.f;
+
+  const int S = f.S;
+  const int coff = CAUSAL ? causal_offset(f, S) : 0;
+  int ntiles_kv = (S + BN - 1) / BN;
+  if (CAUSAL) {
+    const int last = (q0 + BM - 1 < f.L - 1 ? q0 + BM - 1 : f.L - 1) + coff;  // last key any row of the workgroup sees
+    const int lastkv = last < S - 1 ? last : S - 1;
+    ntiles_kv = lastkv / BN + 1;
+  }
+
+  // ---- global -> register -> LDS staging of one K/V tile (thread t moves 16-byte chunks t, t+256, ...) ----------------------
+  u32x4 kst[NLD], vst[NLD];
+  int lrow[NLD], lcol[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; i++) {
+    const int cidx = tid + 256 * i;
+    lrow[i] = cidx / (D / 8);
+    lcol[i] = cidx % (D / 8);
+  }
+  auto load_tile = [&](int kv0) {
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+      int key = kv0 + lrow[i];
+      key = key < S ? key : S - 1;  // rows past the end re-read the last valid row (hidden below)
+      kst[i] = *(const u32x4*)(kp + key * f.ks[2] + 8 * lcol[i]);
+      vst[i] = *(const u32x4*)(vp + key * f.vs[2] + 8 * lcol[i]);
+    }
+  };
+  auto store_tile = [&](int stage) {
+    T* Kr = smem + stage * Lds::DQ_STAGE;
+    T* Vr = Kr + BN * RP;
+    T* Kt = Vr + BN * RP;
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+      *(u32x4*)(Kr + lrow[i] * RP + 8 * lcol[i]) = kst[i];
+      *(u32x4*)(Kt + lrow[i] * TP + 8 * lcol[i]) = kst[i];
+      *(u32x4*)(Vr + lrow[i] * RP + 8 * lcol[i]) = vst[i];
+    }
+  };
+  const int r_lane = lq * RP + 8 * lh;
+  const int t_lane = (4 * lh + ((lane & 15) >> 2)) * TP + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  if (ntiles_kv > 0) {
+    load_tile(0);
+    store_tile(0);
+    if (1 < ntiles_kv) load_tile(BN);
+  }
+  __syncthreads();
+
+  for (int jt = 0; jt < ntiles_kv; jt++) {
+    const int kv0 = jt * BN;
+    const int cur = jt & 1;
+    if (jt + 1 < ntiles_kv) {
+      store_tile(cur ^ 1);
+      if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BN);
+    }
+    if (wave_live && (!CAUSAL || kv0 <= qw0 + 31 + coff)) {
+      const T* Kr = smem + cur * Lds::DQ_STAGE;
+      const T* Vr = Kr + BN * RP;
+      const T* Kt = Vr + BN * RP;
+
+      f32x16 sacc[2];
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[blk][r] = 0.f;
+        const T* krow = Kr + r_lane + 32 * blk * RP;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) sacc[blk] = TR::mfma32(*(const vec8*)(krow + 16 * ks), qreg[ks], sacc[blk]);
+      }
+      if ((CAUSAL && kv0 + BN - 1 > qw0 + coff) || kv0 + BN > S) {
+        const int qi = qw0 + lq + coff;
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int key = kv0 + 32 * blk + 8 * (r >> 2) + 4 * lh + (r & 3);
+            if (key >= S || (CAUSAL && key > qi)) sacc[blk][r] = -INFINITY;
+          }
+      }
+      float mloc = sacc[0][0];
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, sacc[blk][r]);
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+      if (__builtin_amdgcn_ballot_w64(mloc > m_use + lazy) != 0) {
+        const float m_new = fmaxf(m_use, mloc);
+        const float alpha = fast_exp2((m_use - m_new) * c);
+        m_use = m_new;
+        mc = m_new * c;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DBLK; i++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) dqacc[i][r] *= alpha;
+      }
+      // dP^T = V . dout^T
+      f32x16 dpacc[2];
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) dpacc[blk][r] = 0.f;
+        const T* vrow = Vr + r_lane + 32 * blk * RP;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) dpacc[blk] = TR::mfma32(*(const vec8*)(vrow + 16 * ks), greg[ks], dpacc[blk]);
+      }
+      float psum = 0.f;
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float p = fast_exp2(fmaf(sacc[blk][r], c, -mc));  // relative to m_use; normalised at the end
+          psum += p;
+          sacc[blk][r] = p * (dpacc[blk][r] - delta);
+        }
+      l_run += psum;
+      vec8 dsb[4];
+#pragma unroll
+      for (int t = 0; t < 4; t++) dsb[t] = regs_to_operand<vec8>(sacc[t >> 1], t & 1);
+      // dq^T += K^T . dS^T
+      const T* kl = Kt + t_lane;
+#pragma unroll
+      for (int db = 0; db < DBLK; db++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          const vec8 ka = transposed_operand<vec8>(kl, ((16 * t) * TP + 32 * db) * 2, ((16 * t + 8) * TP + 32 * db) * 2);
+          dqacc[db] = TR::mfma32(ka, dsb[t], dqacc[db]);
+        }
+    }
+    __syncthreads();
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const int qi = qw0 + lq;
+  if (qi < f.L) {
+    const long long row_id = ((long long)b * f.Hq + h) * f.L + qi;
+    if (lh == 0) *(float2*)(a.stats + 2 * row_id) = make_float2(m_use * f.scale + __logf(l_tot), delta);
+    const float w = f.scale / l_tot;
+    T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
+#pragma unroll
+    for (int db = 0; db < DBLK; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        f32x4 x;
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = dqacc[db][4 * rg + i] * w;
+        *(typename TR::vec4*)(dqp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
+      }
+  }
+}
+
+// ---- kernel 2: dk, dv ---------------------------------------------------------------------------------------------------
+template <typename TR, int D, bool CAUSAL>
+__global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kernel(BwdArgs a) {
+  typedef typename TR::elem T;
+  typedef typename TR::vec8 vec8;
+  typedef BwdLds<D> Lds;
+  constexpr int RP = Lds::RP, TP = Lds::TP;
+  constexpr int KSTEPS = D / 16, DBLK = D / 32;
+  constexpr int NLD = (BQ * D / 8) / 256;
+  const KArgs& f = a.f;
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  T* smem = (T*)smem_raw;
+  float* sstats = (float*)(smem_raw + 2 * Lds::KV_STAGE * 2);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, lh = lane >> 5;
+
+  const int nkb = (f.S + BM - 1) / BM;
+  int n = blockIdx.x;
+  const int kb = n % nkb;
+  n /= nkb;
+  const int hk = n % f.Hkv, b = n / f.Hkv;
+  const int k0 = kb * BM, kw0 = k0 + wave * 32;
+  const int S = f.S;
+  const bool wave_live = kw0 < S;
+  const int coff = CAUSAL ? causal_offset(f, S) : 0;
+
+  // ---- this lane's key: k and v rows as B operands -------------------------------------------------------------------------
+  vec8 kreg[KSTEPS], vreg[KSTEPS];
+  {
+    int row = kw0 + lq;
+    row = row < S ? row : S - 1;
+    const T* kr = (const T*)f.k + b * f.ks[0] + hk * f.ks[1] + row * f.ks[2] + 8 * lh;
+    const T* vr = (const T*)f.v + b * f.vs[0] + hk * f.vs[1] + row * f.vs[2] + 8 * lh;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      kreg[ks] = *(const vec8*)(kr + 16 * ks);
+      vreg[ks] = *(const vec8*)(vr + 16 * ks);
+    }
+  }
+  f32x16 dkacc[DBLK], dvacc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dkacc[i][r] = 0.f, dvacc[i][r] = 0.f;
+  const float c = f.scale * kLog2e;
+
+  // query tiles it0 .. ntq-1 of each of the G heads see keys of this workgroup
+  const int ntq = (f.L + BQ - 1) / BQ;
+  int it0 = 0;
+  if (CAUSAL) it0 = (k0 - coff > 0 ? k0 - coff : 0) / BQ;
+  const int nt = ntq > it0 ? ntq - it0 : 0;
+  const int total = f.G * nt;
+
+  u32x4 qst[NLD], gst[NLD];
+  float2 sst = make_float2(0.f, 0.f);
+  int lrow[NLD], lcol[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; i++) {
+    const int cidx = tid + 256 * i;
+    lrow[i] = cidx / (D / 8);
+    lcol[i] = cidx % (D / 8);
+  }
+  auto load_tile = [&](int idx) {
+    const int h = hk * f.G + idx / nt;
+    const int i0 = (it0 + idx % nt) * BQ;
+    const T* qp = (const T*)f.q + b * f.qs[0] + h * f.qs[1];
+    const T* gp = (const T*)a.dout + b * a.dos[0] + h * a.dos[1];
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+      int row = i0 + lrow[i];
+      row = row < f.L ? row : f.L - 1;  // rows past the end re-read the last valid row (their weight is forced to 0)
+      qst[i] = *(const u32x4*)(qp + row * f.qs[2] + 8 * lcol[i]);
+      gst[i] = *(const u32x4*)(gp + row * a.dos[2] + 8 * lcol[i]);
+    }
+    if (tid < BQ) {
+      const int row = i0 + tid;
+      sst = row < f.L ? *(const float2*)(a.stats + 2 * (((long long)b * f.Hq + h) * f.L + row)) : make_float2(1e30f, 0.f);
+    }
+  };
+  auto store_tile = [&](int stage) {
+    T* Qr = smem + stage * Lds::KV_STAGE;
+    T* Gr = Qr + BQ * RP;
+    T* Qt = Gr + BQ * RP;
+    T* Gt = Qt + BQ * TP;
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+      *(u32x4*)(Qr + lrow[i] * RP + 8 * lcol[i]) = qst[i];
+      *(u32x4*)(Qt + lrow[i] * TP + 8 * lcol[i]) = qst[i];
+      *(u32x4*)(Gr + lrow[i] * RP + 8 * lcol[i]) = gst[i];
+      *(u32x4*)(Gt + lrow[i] * TP + 8 * lcol[i]) = gst[i];
+    }
+    if (tid < BQ) *(float2*)(sstats + stage * Lds::KV_STATS + 2 * tid) = sst;
+  };
+  const int r_lane = lq * RP + 8 * lh;
+  const int t_lane = (4 * lh + ((lane & 15) >> 2)) * TP + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  if (total > 0) {
+    load_tile(0);
+    store_tile(0);
+    if (1 < total) load_tile(1);
+  }
+  __syncthreads();
+
+  for (int idx = 0; idx < total; idx++) {
+    const int cur = idx & 1;
+    if (idx + 1 < total) {
+      store_tile(cur ^ 1);
+      if (idx + 2 < total) load_tile(idx + 2);
+    }
+    const int i0 = (it0 + idx % nt) * BQ;
+    if (wave_live && (!CAUSAL || kw0 <= i0 + BQ - 1 + coff)) {
+      const T* Qr = smem + cur * Lds::KV_STAGE;
+      const T* Gr = Qr + BQ * RP;
+      const T* Qt = Gr + BQ * RP;
+      const T* Gt = Qt + BQ * TP;
+      const float* st = sstats + cur * Lds::KV_STATS;
+
+      f32x16 sacc, dpacc;
+#pragma unroll
+      for (int r = 0; r < 16; r++) sacc[r] = 0.f, dpacc[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) sacc = TR::mfma32(*(const vec8*)(Qr + r_lane + 16 * ks), kreg[ks], sacc);
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) dpacc = TR::mfma32(*(const vec8*)(Gr + r_lane + 16 * ks), vreg[ks], dpacc);
+
+      const int key = kw0 + lq;
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        const f32x4 s0 = *(const f32x4*)(st + 2 * (8 * rg + 4 * lh));      // (lse, delta) of rows 8rg+4lh+0, +1
+        const f32x4 s1 = *(const f32x4*)(st + 2 * (8 * rg + 4 * lh) + 4);  // ... +2, +3
+        const float lse[4] = {s0[0], s0[2], s1[0], s1[2]};
+        const float dl[4] = {s0[1], s0[3], s1[1], s1[3]};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int r = 4 * rg + e;
+          const int qrow = i0 + 8 * rg + 4 * lh + e;
+          const bool hidden = key >= S || (CAUSAL && key > qrow + coff);
+          float p = fast_exp2(fmaf(sacc[r], c, -lse[e] * kLog2e));
+          p = hidden ? 0.f : p;
+          sacc[r] = p;
+          dpacc[r] = p * (dpacc[r] - dl[e]);
+        }
+      }
+      vec8 pb[2], dsb[2];
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        pb[t] = regs_to_operand<vec8>(sacc, t);
+        dsb[t] = regs_to_operand<vec8>(dpacc, t);
+      }
+      const T* gl = Gt + t_lane;
+      const T* ql = Qt + t_lane;
+#pragma unroll
+      for (int db = 0; db < DBLK; db++)
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const int lo = ((16 * t) * TP + 32 * db) * 2, hi = ((16 * t + 8) * TP + 32 * db) * 2;
+          dvacc[db] = TR::mfma32(transposed_operand<vec8>(gl, lo, hi), pb[t], dvacc[db]);
+          dkacc[db] = TR::mfma32(transposed_operand<vec8>(ql, lo, hi), dsb[t], dkacc[db]);
+        }
+    }
+    __syncthreads();
+  }
+
+  const int key = kw0 + lq;
+  if (key < S) {
+    T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
+    T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
+#pragma unroll
+    for (int db = 0; db < DBLK; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        f32x4 x, y;
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = dkacc[db][4 * rg + i] * f.scale, y[i] = dvacc[db][4 * rg + i];
+        *(typename TR::vec4*)(dkp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
+        *(typename TR::vec4*)(dvp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(y, typename TR::vec4);
+      }
+  }
+}
+
+template <typename TR, int D, bool CAUSAL>
+int launch_k(const BwdArgs& a, hipStream_t stream) {
+  typedef BwdLds<D> Lds;
+  static hipError_t state1[kMaxDevices], state2[kMaxDevices];
+  static bool done1[kMaxDevices], done2[kMaxDevices];
+  hipError_t e = grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL>, Lds::DQ_BYTES, state1, done1);
+  if (e != hipSuccess) return (int)e;
+  e = grant_dynamic_lds((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL>, Lds::KV_BYTES, state2, done2);
+  if (e != hipSuccess) return (int)e;
+  const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
+  const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM);
+  hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g1), dim3(256), Lds::DQ_BYTES, stream, a);
+  e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
+  return (int)hipGetLastError();
+}
+
+template <typename TR>
+int launch_t(const BwdArgs& a, hipStream_t stream) {
+  if (a.f.D == 64) return a.f.causal ? launch_k<TR, 64, true>(a, stream) : launch_k<TR, 64, false>(a, stream);
+  return a.f.causal ? launch_k<TR, 128, true>(a, stream) : launch_k<TR, 128, false>(a, stream);
+}
+
+}  // namespace
+
+int launch_backward_mfma(const BwdArgs& a, int dtype, hipStream_t stream) {
+  return dtype == 1 ? launch_t<F16>(a, stream) : launch_t<BF16>(a, stream);
+}
+
+}  // namespace ttsdpa

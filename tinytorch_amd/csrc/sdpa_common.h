@@ -177,6 +177,7 @@ struct BwdArgs {
   float* stats;
 };
 int launch_backward_general(const BwdArgs& a, int dtype, hipStream_t stream);
+int launch_backward_mfma(const BwdArgs& a, int dtype, hipStream_t stream);  // fp16/bf16, head_dim 64 or 128, no attnMask / kv_len
 
 // Host-side launchers (one per kernel family); each returns a hipError_t as int.
 int launch_general(const KArgs& a, int dtype, hipStream_t stream);

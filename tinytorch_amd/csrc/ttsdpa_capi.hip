@@ -222,10 +222,21 @@ int validate_backward(const ttsdpa_backward_params* p, BwdArgs* a) {
   return TTSDPA_OK;
 }
 
+// The MFMA backward kernels: 16-bit tensors they can read and write with 16-byte / 8-byte accesses, head_dim 64 or
+// 128, no attnMask, no per-batch key counts.
+bool backward_mfma_ok(const ttsdpa_backward_params* p) {
+  const ttsdpa_params* f = &p->fwd;
+  if (!fast_layout_ok(f) || f->kv_len || (f->D != 64 && f->D != 128) || f->L < 1 || f->S < 1) return false;
+  if (!dense_last_ok(p->dout_stride, 8) || !dense_last_ok(p->dq_stride, 8) || !dense_last_ok(p->dk_stride, 8) ||
+      !dense_last_ok(p->dv_stride, 8))
+    return false;
+  return ptr_aligned(p->dout, 16) && ptr_aligned(p->dq, 16) && ptr_aligned(p->dk, 16) && ptr_aligned(p->dv, 16);
+}
+
 int pick_backward_route(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
   if (f->B == 0 || (f->L == 0 && f->S == 0)) return TTSDPA_ROUTE_NONE;
-  return TTSDPA_ROUTE_GENERAL;
+  return backward_mfma_ok(p) ? TTSDPA_ROUTE_PREFILL : TTSDPA_ROUTE_GENERAL;
 }
 
 size_t backward_stats_bytes(const ttsdpa_backward_params* p) {
@@ -393,6 +404,11 @@ int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t wor
   const size_t need = backward_stats_bytes(p);
   if (need > 0 && (!workspace || workspace_bytes < need || !ptr_aligned(workspace, 16))) return TTSDPA_ERR_WORKSPACE;
   a.stats = (float*)workspace;
+  if (route == TTSDPA_ROUTE_PREFILL) {
+    const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + 127) / 128), g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + 127) / 128);
+    if (check_grid(g1) != TTSDPA_OK || check_grid(g2) != TTSDPA_OK) return TTSDPA_ERR_SHAPE;
+    return launch_backward_mfma(a, p->fwd.dtype, (hipStream_t)stream);
+  }
   return launch_backward_general(a, p->fwd.dtype, (hipStream_t)stream);
 }
 
