@@ -58,6 +58,22 @@ __device__ __forceinline__ vec8 transposed_operand(const void* lane_base, int by
   return __builtin_bit_cast(vec8, r);
 }
 
+// Workgroup n -> (pair, block) for npair (batch, head) pairs of nblk blocks each, block 0 the longest under a causal
+// mask.  Workgroups are handed to the 8 XCDs round-robin (n % 8) and start in order: every XCD gets whole pairs (a
+// contiguous range, so the heads of a group share its L2) and takes their blocks longest first across all its pairs,
+// which keeps the XCDs evenly loaded and the short blocks for the end.  Without a multiple of 8 pairs: longest first
+// over all pairs.
+__device__ __forceinline__ void map_workgroup(int n, int npair, int nblk, int* pair, int* blk) {
+  if ((npair & 7) == 0) {
+    const int xcd = n & 7, slot = n >> 3, ppx = npair >> 3;
+    *blk = slot / ppx;
+    *pair = xcd * ppx + slot % ppx;
+  } else {
+    *blk = n / npair;
+    *pair = n % npair;
+  }
+}
+
 template <typename vec8>
 __device__ __forceinline__ vec8 regs_to_operand(const f32x16& acc, int t) {
   f32x8 x;
@@ -86,10 +102,9 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
   const int lq = lane & 31, lh = lane >> 5;
 
   const int ntile = (f.L + BM - 1) / BM;
-  int n = blockIdx.x;
-  const int in = n % ntile;
-  n /= ntile;
-  const int h = n % f.Hq, b = n / f.Hq;
+  int pair, in;
+  map_workgroup(blockIdx.x, f.B * f.Hq, ntile, &pair, &in);
+  const int h = pair % f.Hq, b = pair / f.Hq;
   const int hk = h / f.G;
   const int rt = CAUSAL ? ntile - 1 - in : in;  // longest rows first
   const int q0 = rt * BM, qw0 = q0 + wave * 32;
@@ -300,10 +315,9 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   const int lq = lane & 31, lh = lane >> 5;
 
   const int nkb = (f.S + BM - 1) / BM;
-  int n = blockIdx.x;
-  const int kb = n % nkb;
-  n /= nkb;
-  const int hk = n % f.Hkv, b = n / f.Hkv;
+  int pair, kb;  // the first key block is seen by every query row: the longest
+  map_workgroup(blockIdx.x, f.B * f.Hkv, nkb, &pair, &kb);
+  const int hk = pair % f.Hkv, b = pair / f.Hkv;
   const int k0 = kb * BM, kw0 = k0 + wave * 32;
   const int S = f.S;
   const bool wave_live = kw0 < S;
