@@ -9,12 +9,14 @@ prefill throughput target is quoted on); the decode workload "config4" (bf16, B6
 same run and reported under "secondary", config 3's shape in fp32 (the reference's default dtype,
 on the fp32 MFMA kernel, against the 157.3 TFLOP/s fp32 peak) under "fp32", and the row-wise neighbour ops (rmsNorm,
 fusedAddRmsNorm, siluMul, softmax; HBM-bound) under "fused_ops" and the linear layer (QKV projection of the same
-token batch; MFMA-bound) under "linear".  One JSON line is printed.
+token batch; MFMA-bound) under "linear", and the attention backward (dq, dk, dv at config 3's shape; MFMA-bound) under
+"backward".  One JSON line is printed.
 
 Algorithmic work per launch (what "achieved" divides by the measured launch time):
   prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)
   prefill, full:    4 * B * Hq * L * S * D flop
   decode:           2 * B*Hkv*S*D*2 bytes (K and V once) + 2 * B*Hq*D*2 bytes (q in, out)
+  backward, causal: 2.5 x the causal prefill's flop (five matrix products; the kernels execute seven)
 """
 import argparse
 import ctypes
@@ -323,6 +325,68 @@ def run_linear(steps, warmup, cpu=True):
     return res
 
 
+def run_backward(steps, warmup, cpu=True):
+    """Attention backward (ttsdpa_backward) at config 3's shape, bf16, causal: dq, dk, dv per launch pair.  Flop count:
+    the textbook five matrix products (2.5 x the forward's), halved by the causal mask; the two kernels execute seven."""
+    import ctypes
+    import numpy as np
+    import torch
+    from tinytorch_amd import _capi, build_backward_params, sdpAttention
+
+    B, Hq, Hkv, L, S, D = 2, 32, 8, 4096, 4096, 128
+    lib = _capi.lib()
+    stream = torch.cuda.current_stream()
+    gen = torch.Generator(device="cuda").manual_seed(0x5EED)
+    q = torch.randn(B, Hq, L, D, device="cuda", generator=gen).bfloat16()
+    k = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).bfloat16()
+    v = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).bfloat16()
+    go = torch.randn(B, Hq, L, D, device="cuda", generator=gen).bfloat16()
+    out = sdpAttention(q, k, v, isCausal=True)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    bp = build_backward_params(q, k, v, out, go, dq, dk, dv, True)
+    nbytes = lib.ttsdpa_backward_workspace_bytes(ctypes.byref(bp))
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+    route = ctypes.c_int(-1)
+    lib.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(route))
+
+    def step():
+        rc = lib.ttsdpa_backward(ctypes.byref(bp), ws.data_ptr(), nbytes, stream.cuda_stream)
+        if rc != 0:
+            raise RuntimeError("ttsdpa_backward: %s" % _capi.status_string(rc))
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    flops = 2.5 * 4.0 * B * Hq * L * S * D * 0.5
+    tf = flops / (ms * 1e-3) / 1e12
+    res = {"workload": "attention backward bf16 B%d %dq/%dkv L=S=%d D%d causal" % (B, Hq, Hkv, L, D), "dtype": "bf16",
+           "route": _capi.ROUTE_NAMES[route.value], "ms_per_step": round(ms, 5), "value": round(tf, 1), "unit": "TFLOP/s",
+           "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                        "frac": round(tf / PEAK_TFLOPS["bf16"], 4), "traffic": measured_traffic("backward"),
+                        "algorithmic_flops": flops, "kernels": "backward_dq_mfma_kernel + backward_dkv_mfma_kernel per step"}}
+    if cpu:
+        import oracle
+        # the causal top-left corner is a problem of its own for dq: rows below n see keys below n only
+        n = 2048
+        qh, kh, vh, gh = (t[:1, :h, :n].float().cpu().numpy() for t, h in ((q, Hq // Hkv), (k, 1), (v, 1), (go, Hq // Hkv)))
+        t0 = time.perf_counter()
+        rq, _, _ = oracle.sdpa_backward_f32(qh, kh, vh, gh, causal=True, nthreads=1)
+        spent = time.perf_counter() - t0
+        got = dq[:1, :Hq // Hkv, :n].float().cpu().numpy()
+        res["cpu_baseline"] = {"value": float("%.4g" % (2.5 * 4.0 * (Hq // Hkv) * n * n * D * 0.5 / spent / 1e12)), "unit": "TFLOP/s",
+                               "cores": 1, "kind": "port",
+                               "sample": "the first %d queries x %d keys of one KV head (its %d query heads), %.1f s, one thread, double accumulation"
+                               % (n, n, Hq // Hkv, spent),
+                               "max_abs_err_gpu_vs_cpu_dq": float("%.3g" % float(np.abs(rq - got).max()))}
+    return res
+
+
 def run_cpu_baseline(name, tensors, budget_s=20.0):
     """The reference CPU path (compiled reference if oracle/_ref is present, else this repository's C restatement)
     on one host core, over as many (batch, head) slices of the same inputs as fit the time budget."""
@@ -377,6 +441,7 @@ def main():
     ap.add_argument("--fused-only", default=None, choices=sorted(FUSED_WORKLOADS),
                     help="measure one row-wise op only and print its line (for profiling)")
     ap.add_argument("--linear-only", action="store_true", help="measure the linear layer only and print its line (for profiling)")
+    ap.add_argument("--backward-only", action="store_true", help="measure the attention backward only and print its line (for profiling)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one device-to-device copy of 1 GiB (a kernel of known traffic that calibrates "
                          "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc)")
@@ -399,6 +464,9 @@ def main():
         return
     if args.linear_only:
         print(json.dumps(run_linear(args.steps, args.warmup, cpu=not args.no_cpu)), flush=True)
+        return
+    if args.backward_only:
+        print(json.dumps(run_backward(args.steps, args.warmup, cpu=not args.no_cpu)), flush=True)
         return
     main_res, tensors = run_gpu(args.workload, args.steps, args.warmup)
     ceilings = None if args.no_probes else run_probes()
@@ -430,6 +498,8 @@ def main():
                              for n in ("rms_norm", "fused_add_rms_norm", "silu_mul", "softmax")]
         torch.cuda.empty_cache()
         line["linear"] = run_linear(max(1, min(args.steps, 100)), min(args.warmup, 50), cpu=not args.no_cpu)
+        torch.cuda.empty_cache()
+        line["backward"] = run_backward(max(1, min(args.steps, 50)), min(args.warmup, 20), cpu=not args.no_cpu)
     print(json.dumps(line), flush=True)
 
 

@@ -290,6 +290,80 @@ static void test_kv_cache() {
   }
 }
 
+// Plain double-precision gradients of sum(attention(q,k,v) * go) for one head (causal top-left), for the check below.
+static void cpuAttentionBackward(const std::vector<float>& q, const std::vector<float>& k, const std::vector<float>& v,
+                                 const std::vector<float>& go, int L, int S, int D, float scale, bool causal,
+                                 std::vector<double>& dq, std::vector<double>& dk, std::vector<double>& dv) {
+  dq.assign(static_cast<size_t>(L) * D, 0.0), dk.assign(static_cast<size_t>(S) * D, 0.0), dv.assign(static_cast<size_t>(S) * D, 0.0);
+  std::vector<double> p(S), dp(S);
+  for (int i = 0; i < L; i++) {
+    double mx = -1e300, sum = 0.0, dot = 0.0;
+    for (int j = 0; j < S; j++) {
+      double s = 0.0;
+      for (int d = 0; d < D; d++) s += static_cast<double>(q[i * D + d]) * k[j * D + d];
+      p[j] = (causal && j > i) ? -1e300 : s * scale;
+      mx = std::max(mx, p[j]);
+    }
+    for (int j = 0; j < S; j++) sum += (p[j] = std::exp(p[j] - mx));
+    for (int j = 0; j < S; j++) {
+      p[j] /= sum;
+      dp[j] = 0.0;
+      for (int d = 0; d < D; d++) dp[j] += static_cast<double>(go[i * D + d]) * v[j * D + d];
+      dot += p[j] * dp[j];
+    }
+    for (int j = 0; j < S; j++) {
+      const double ds = p[j] * (dp[j] - dot) * scale;
+      for (int d = 0; d < D; d++) {
+        dq[i * D + d] += ds * k[j * D + d];
+        dk[j * D + d] += ds * q[i * D + d];
+        dv[j * D + d] += p[j] * go[i * D + d];
+      }
+    }
+  }
+}
+
+static void test_backward() {
+  std::printf("FuncSDPAttention::backward (the reference stops at NOT_IMPLEMENTED)\n");
+  const Options gpu = options::device(DeviceType::GPU);
+  const int L = 9, S = 9, D = 16;
+  std::vector<float> q = pseudoRandom(static_cast<size_t>(L) * D, 71), k = pseudoRandom(static_cast<size_t>(S) * D, 72),
+                     v = pseudoRandom(static_cast<size_t>(S) * D, 73), go = pseudoRandom(static_cast<size_t>(L) * D, 74);
+  Tensor tq(q, {1, 1, L, D}, gpu), tk(k, {1, 1, S, D}, gpu), tv(v, {1, 1, S, D}, gpu), tgo(go, {1, 1, L, D}, gpu);
+  tq.setRequiresGrad(true);
+  tv.setRequiresGrad(true);
+  Tensor y = function::sdpAttention(tq, tk, tv, true);
+  EXPECT_TRUE(y.gradFn() != nullptr && !tq.grad().defined());
+  y.gradFn()->backward(tgo);
+  EXPECT_TRUE(tq.grad().defined() && tv.grad().defined() && !tk.grad().defined());  // k does not require grad
+  std::vector<double> dq, dk, dv;
+  cpuAttentionBackward(q, k, v, go, L, S, D, 1.f / std::sqrt(static_cast<float>(D)), true, dq, dk, dv);
+  std::vector<float> gq = tq.grad().toList<float>(), gv = tv.grad().toList<float>();
+  bool ok = gq.size() == dq.size() && gv.size() == dv.size();
+  for (size_t i = 0; ok && i < dq.size(); i++) ok = std::fabs(gq[i] - dq[i]) < 1e-4;
+  for (size_t i = 0; ok && i < dv.size(); i++) ok = std::fabs(gv[i] - dv[i]) < 1e-4;
+  EXPECT_TRUE(ok);
+  // the op itself, bf16 with grouped heads: dk / dv have the shape of key / value
+  const Options bf = options::device(DeviceType::GPU).dtype(DType::BFloat16);
+  Tensor bq = Tensor::ones({2, 4, 64, 128}, bf), bk = Tensor::ones({2, 2, 64, 128}, bf), bv = Tensor::ones({2, 2, 64, 128}, bf);
+  Tensor bo = op::sdpAttention(bq, bk, bv, false, Tensor{}, 0.f, 0.1f);
+  auto grads = op::sdpAttentionBackward(bq, bq, bk, bv, bo, false, Tensor{}, 0.1f);
+  EXPECT_TRUE(grads.size() == 3 && grads[0].shape() == bq.shape() && grads[1].shape() == bk.shape() && grads[2].shape() == bv.shape());
+  if (grads.size() == 3) {
+    // equal keys: P is uniform, dP is constant per row, so dS = 0: dq = dk = 0, dv = (2 heads * 64 rows / 64 keys) * 1 = 2
+    bool z = true;
+    for (float f : grads[0].toList<float>()) z = z && std::fabs(f) < 1e-3f;
+    for (float f : grads[1].toList<float>()) z = z && std::fabs(f) < 1e-3f;
+    for (float f : grads[2].toList<float>()) z = z && std::fabs(f - 2.f) < 2e-2f;
+    EXPECT_TRUE(z);
+  }
+  // a second gradient for the same tensor needs an accumulate this layer does not have: loud failure
+  AssertHandler old = setAssertHandler(countingAssertHandler);
+  const int before = g_asserts;
+  y.gradFn()->backward(tgo);
+  EXPECT_TRUE(g_asserts > before);
+  setAssertHandler(old);
+}
+
 static void test_grad_bookkeeping_and_errors() {
   std::printf("Function::apply bookkeeping, dispatcher failure, allocator reuse\n");
   const Options gpu = options::device(DeviceType::GPU).dtype(DType::BFloat16);
@@ -309,11 +383,8 @@ static void test_grad_bookkeeping_and_errors() {
   for (float f : ones) allOne = allOne && std::fabs(f - 1.f) < 1e-2f;
   EXPECT_TRUE(allOne);
 
-  // backward is not implemented (as in the reference): it must fail through ASSERT
   AssertHandler old = setAssertHandler(countingAssertHandler);
   int before = g_asserts;
-  y.gradFn()->backward(y);
-  EXPECT_TRUE(g_asserts == before + 1);
   // a CPU tensor has no implementation behind op::sdpAttention: loud failure, undefined result
   Tensor cq = Tensor::ones({1, 1, 4, 64}, options::device(DeviceType::CPU));
   before = g_asserts;
@@ -441,6 +512,7 @@ int main() {
   test_broadcast_masks();
   test_kv_cache();
   test_row_wise_ops();
+  test_backward();
   test_grad_bookkeeping_and_errors();
   std::printf(g_failures == 0 ? "ALL PASSED\n" : "%d FAILURES\n", g_failures);
   return g_failures == 0 ? 0 : 1;

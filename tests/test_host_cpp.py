@@ -35,7 +35,7 @@ def test_cpp_sources_keep_the_reference_interface():
     assert "class FuncSDPAttention : public Function<FuncSDPAttention>" in func
     assert "inline Tensor sdpAttention(const Tensor& query, const Tensor& key, const Tensor& value, bool isCausal = false," in func
     assert "const Tensor& attnMask = {}, float dropoutP = 0.f," in func and "std::optional<float> scale = std::nullopt" in func
-    assert "NOT_IMPLEMENTED();" in func
+    assert "static void backward(AutogradContext* ctx, const Tensor& grad)" in func and "op::sdpAttentionBackward(" in func
     disp = open(os.path.join(ROOT, "tinytorch_amd", "host", "Dispatch.h")).read()
     assert "#define DEFINE_OP(NAME, FN_TYPE)" in disp and "#define REGISTER_OP_IMPL(NAME, DEVICE, DTYPE, FUNC)" in disp
     op = open(os.path.join(ROOT, "tinytorch_amd", "host", "OpAttention.cpp")).read()

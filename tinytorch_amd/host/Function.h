@@ -37,6 +37,9 @@ struct AutogradContext {
   std::vector<Tensor> savedInputs;
   std::vector<Tensor> savedForBackward;
   void saveForBackward(const Tensor& t) { savedForBackward.push_back(t); }
+  // non-tensor arguments a backward needs (the reference keeps such values in an IValue list, src/Tensor/IValue.h)
+  bool isCausal = false;
+  float scale = 1.f;
 };
 
 struct FunctionBase {

@@ -17,17 +17,18 @@ int dtypeCode(DType t) {
   }
 }
 
-// GPU entry of op::sdpAttention for every floating dtype: one enqueue on the thread's current stream, output and
-// scratch from the caching allocator, no host synchronisation.
-Tensor sdpAttentionGpuImpl(const Tensor& query, const Tensor& key, const Tensor& value, bool isCausal,
-                           const Tensor& attnMask, float dropoutP, float scale) {
+// Checks the arguments of an attention call and fills *p for dense tensors (pointers of q, k, v and the mask; p->out
+// is left to the caller).  false after a failed precondition.
+bool fillAttentionParams(ttsdpa_params* pp, const Tensor& query, const Tensor& key, const Tensor& value, bool isCausal,
+                         const Tensor& attnMask, float dropoutP, float scale) {
+  ttsdpa_params& p = *pp;
   ASSERT(query.defined() && key.defined() && value.defined());
   ASSERT(query.dim() == key.dim() && key.dim() == value.dim() && (query.dim() == 4 || query.dim() == 3));
   ASSERT(key.dtype() == query.dtype() && value.dtype() == query.dtype());
   ASSERT(key.device() == query.device() && value.device() == query.device());
   ASSERT(dropoutP == 0.f);  // the fused path has no dropout (the reference's composite passes p through inverted)
   ASSERT(!(isCausal && attnMask.defined()));  // reference src/Function/FuncNNLayer.h:242
-  if (query.dim() != key.dim() || dropoutP != 0.f || (isCausal && attnMask.defined())) return {};
+  if (query.dim() != key.dim() || dropoutP != 0.f || (isCausal && attnMask.defined())) return false;
 
   const int nd = static_cast<int>(query.dim());
   const int B = nd == 4 ? static_cast<int>(query.size(0)) : 1;
@@ -36,12 +37,10 @@ Tensor sdpAttentionGpuImpl(const Tensor& query, const Tensor& key, const Tensor&
   const int D = static_cast<int>(query.size(-1));
   ASSERT(key.shape() == value.shape() && key.size(-1) == D && Hkv >= 1 && Hq % Hkv == 0);
   ASSERT(nd == 3 || key.size(0) == B);
-  if (key.shape() != value.shape() || key.size(-1) != D || Hkv < 1 || Hq % Hkv != 0) return {};
+  if (key.shape() != value.shape() || key.size(-1) != D || Hkv < 1 || Hq % Hkv != 0) return false;
 
-  ttsdpa_params p;
   ttsdpa_params_init(&p, dtypeCode(query.dtype()), B, Hq, Hkv, L, S, D);
-  Tensor out = Tensor::empty(query.shape(), query.options().noGrad());
-  p.q = query.rawPtr(), p.k = key.rawPtr(), p.v = value.rawPtr(), p.out = out.rawPtr();
+  p.q = query.rawPtr(), p.k = key.rawPtr(), p.v = value.rawPtr();
   p.scale = scale;
   p.causal = isCausal ? TTSDPA_CAUSAL_TOP_LEFT : TTSDPA_CAUSAL_NONE;  // the reference's alignment
   if (attnMask.defined()) {
@@ -51,21 +50,31 @@ Tensor sdpAttentionGpuImpl(const Tensor& query, const Tensor& key, const Tensor&
     // (src/Function/FuncNNLayer.h:249-260): right-align the mask's axes, size-1 and missing axes get stride 0.
     const int md = static_cast<int>(attnMask.dim());
     ASSERT(md >= 1 && md <= 4);
-    if (md < 1 || md > 4) return {};
+    if (md < 1 || md > 4) return false;
     const int64_t target[4] = {B, Hq, L, S};
     int64_t dense = 1;
     for (int i = 3; i >= 0; i--) {
       const int mi = i - (4 - md);
       const int64_t n = mi >= 0 ? attnMask.size(mi) : 1;
       ASSERT(n == target[i] || n == 1);
-      if (n != target[i] && n != 1) return {};
+      if (n != target[i] && n != 1) return false;
       p.mask_stride[i] = n == 1 ? 0 : dense;
       dense *= n;
     }
     p.mask_kind = attnMask.dtype() == DType::Bool ? TTSDPA_MASK_BOOL : TTSDPA_MASK_ADD;
     p.mask = attnMask.rawPtr();
   }
+  return true;
+}
 
+// GPU entry of op::sdpAttention for every floating dtype: one enqueue on the thread's current stream, output and
+// scratch from the caching allocator, no host synchronisation.
+Tensor sdpAttentionGpuImpl(const Tensor& query, const Tensor& key, const Tensor& value, bool isCausal,
+                           const Tensor& attnMask, float dropoutP, float scale) {
+  ttsdpa_params p;
+  if (!fillAttentionParams(&p, query, key, value, isCausal, attnMask, dropoutP, scale)) return {};
+  Tensor out = Tensor::empty(query.shape(), query.options().noGrad());
+  p.out = out.rawPtr();
   const DeviceIndex dev = query.device().index;
   HIP_CHECK(hipSetDevice(dev));
   const size_t wsBytes = ttsdpa_workspace_bytes(&p);
@@ -78,6 +87,43 @@ Tensor sdpAttentionGpuImpl(const Tensor& query, const Tensor& key, const Tensor&
     return {};
   }
   return out;
+}
+
+// GPU entry of op::sdpAttentionBackward: {dq, dk, dv} for the forward call with the same arguments, whose result is
+// `out`.  One enqueue of two kernels on the thread's current stream; gradients and scratch from the caching allocator.
+std::vector<Tensor> sdpAttentionBackwardGpuImpl(const Tensor& gradOut, const Tensor& query, const Tensor& key,
+                                                const Tensor& value, const Tensor& out, bool isCausal,
+                                                const Tensor& attnMask, float scale) {
+  ttsdpa_backward_params bp;
+  ASSERT(gradOut.defined() && out.defined());
+  if (!gradOut.defined() || !out.defined()) return {};
+  if (!fillAttentionParams(&bp.fwd, query, key, value, isCausal, attnMask, 0.f, scale)) return {};
+  ASSERT(gradOut.shape() == query.shape() && out.shape() == query.shape());
+  ASSERT(gradOut.dtype() == query.dtype() && out.dtype() == query.dtype());
+  ASSERT(gradOut.device() == query.device() && out.device() == query.device());
+  if (gradOut.shape() != query.shape() || out.shape() != query.shape() || gradOut.dtype() != query.dtype() ||
+      out.dtype() != query.dtype())
+    return {};
+  const ttsdpa_params fwd = bp.fwd;
+  ttsdpa_backward_params_init(&bp, fwd.dtype, fwd.B, fwd.Hq, fwd.Hkv, fwd.L, fwd.S, fwd.D);
+  bp.fwd = fwd;
+  bp.fwd.out = out.rawPtr();
+  Tensor dq = Tensor::empty(query.shape(), query.options().noGrad());
+  Tensor dk = Tensor::empty(key.shape(), key.options().noGrad());
+  Tensor dv = Tensor::empty(value.shape(), value.options().noGrad());
+  bp.dout = gradOut.rawPtr(), bp.dq = dq.rawPtr(), bp.dk = dk.rawPtr(), bp.dv = dv.rawPtr();
+  const DeviceIndex dev = query.device().index;
+  HIP_CHECK(hipSetDevice(dev));
+  const size_t wsBytes = ttsdpa_backward_workspace_bytes(&bp);
+  std::shared_ptr<Storage> ws;
+  if (wsBytes) ws = std::make_shared<Storage>(wsBytes, query.device());
+  const int rc = ttsdpa_backward(&bp, ws ? ws->data() : nullptr, wsBytes, getCurrentStream(dev));
+  if (rc != TTSDPA_OK) {
+    LOGE("ttsdpa_backward failed: %d (%s)", rc, ttsdpa_status_string(rc));
+    ASSERT(rc == TTSDPA_OK);
+    return {};
+  }
+  return {dq, dk, dv};
 }
 
 // Fills the block-table fields of a parameter struct; false after a failed precondition.
@@ -176,6 +222,9 @@ void registerAttentionGpu() {
   REGISTER_OP_IMPL(sdpAttention, GPU, Float32, &sdpAttentionGpuImpl);
   REGISTER_OP_IMPL(sdpAttention, GPU, Float16, &sdpAttentionGpuImpl);
   REGISTER_OP_IMPL(sdpAttention, GPU, BFloat16, &sdpAttentionGpuImpl);
+  REGISTER_OP_IMPL(sdpAttentionBackward, GPU, Float32, &sdpAttentionBackwardGpuImpl);
+  REGISTER_OP_IMPL(sdpAttentionBackward, GPU, Float16, &sdpAttentionBackwardGpuImpl);
+  REGISTER_OP_IMPL(sdpAttentionBackward, GPU, BFloat16, &sdpAttentionBackwardGpuImpl);
   REGISTER_OP_IMPL(kvCacheAppend, GPU, Float32, &kvCacheAppendGpuImpl);
   REGISTER_OP_IMPL(kvCacheAppend, GPU, Float16, &kvCacheAppendGpuImpl);
   REGISTER_OP_IMPL(kvCacheAppend, GPU, BFloat16, &kvCacheAppendGpuImpl);

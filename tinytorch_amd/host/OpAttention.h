@@ -19,6 +19,15 @@ using SdpAttentionOpFn = Tensor (*)(const Tensor& query, const Tensor& key, cons
 
 DEFINE_OP(sdpAttention, SdpAttentionOpFn)
 
+// Gradients {dQuery, dKey, dValue} of op::sdpAttention(query, key, value, isCausal, attnMask, 0, scale) for the upstream
+// gradient gradOut; `out` is that call's result.  dKey / dValue have the shapes of key / value (grouped heads are
+// summed).  The reference stops at NOT_IMPLEMENTED here (src/Function/FuncNNLayer.h:267).  Empty vector after a failed
+// ASSERT.
+using SdpAttentionBackwardOpFn = std::vector<Tensor> (*)(const Tensor& gradOut, const Tensor& query, const Tensor& key,
+                                                         const Tensor& value, const Tensor& out, bool isCausal,
+                                                         const Tensor& attnMask, float scale);
+DEFINE_OP(sdpAttentionBackward, SdpAttentionBackwardOpFn)
+
 // KV cache (no counterpart in the reference, whose callers would grow K/V with op::concat on the sequence axis,
 // src/Operation/OpTransform.cpp:306-357, copying the whole history per generated token).
 // kvCacheAppend writes kNew/vNew [B,Hkv,Lnew,D] into the preallocated caches [B,Hkv,Smax,D] in place, at rows

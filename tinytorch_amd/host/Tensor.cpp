@@ -271,6 +271,7 @@ struct Tensor::Impl {
   Options options;
   std::shared_ptr<Storage> storage;
   std::shared_ptr<FunctionBase> gradFn;
+  Tensor grad;
 };
 
 Tensor::Tensor(const std::vector<int64_t>& shape, Options options) {
@@ -303,6 +304,29 @@ bool Tensor::requiresGrad() const { return impl_ && impl_->options.requiresGrad_
 void Tensor::setRequiresGrad(bool r) { impl_->options.requiresGrad_ = r; }
 std::shared_ptr<FunctionBase> Tensor::gradFn() const { return impl_ ? impl_->gradFn : nullptr; }
 void Tensor::setGradFn(std::shared_ptr<FunctionBase> fn) { impl_->gradFn = std::move(fn); }
+const Tensor& Tensor::grad() const {
+  static const Tensor none;
+  return impl_ ? impl_->grad : none;
+}
+void Tensor::addGrad(Tensor&& g) {
+  ASSERT(impl_ && requiresGrad());
+  ASSERT(!impl_->grad.defined());  // accumulation needs an elementwise add, which this layer does not carry
+  if (impl_ && !impl_->grad.defined()) impl_->grad = std::move(g);
+}
+Tensor Tensor::detach() const {
+  Tensor t;
+  if (impl_) {
+    t.impl_ = std::make_shared<Impl>();
+    t.impl_->shape = impl_->shape;
+    t.impl_->numel = impl_->numel;
+    t.impl_->options = impl_->options.noGrad();
+    t.impl_->storage = impl_->storage;
+  }
+  return t;
+}
+void Tensor::zeroGrad() {
+  if (impl_) impl_->grad = Tensor();
+}
 void* Tensor::rawPtr() const { return impl_->storage->data(); }
 
 void Tensor::reshape_(const std::vector<int64_t>& shape) {

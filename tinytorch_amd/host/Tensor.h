@@ -107,6 +107,11 @@ class Tensor {
   void setRequiresGrad(bool r);
   std::shared_ptr<FunctionBase> gradFn() const;
   void setGradFn(std::shared_ptr<FunctionBase> fn);
+  // Gradient slot of a tensor that requires grad (reference src/Tensor/Tensor.h grad()/addGrad()).  This layer has no
+  // elementwise add: the first gradient is stored, a second one for the same tensor fails loudly.
+  const Tensor& grad() const;
+  void addGrad(Tensor&& g);
+  void zeroGrad();
 
   void* rawPtr() const;
   template <typename T>
@@ -116,6 +121,7 @@ class Tensor {
   Tensor to(Device device) const;
   Tensor to(DType dtype) const;  // Float32 <-> Float16 / BFloat16, round to nearest even; done on the host
   Tensor clone() const;
+  Tensor detach() const;  // the same storage without the autograd links (reference Tensor::detach)
   void fill_(float value);
 
   // Values as T on the host (Float32 / Float16 / BFloat16 / Bool / Int tensors are converted element-wise).
