@@ -30,7 +30,6 @@ constexpr int BM = 128;  // rows of the owning side per workgroup (queries in ke
 constexpr int BN = 64;   // keys per streamed tile, kernel 1
 constexpr int BQ = 32;   // query rows per streamed tile, kernel 2
 constexpr float kLazyExp = 8.f;
-constexpr float kLn2 = 0.6931471805599453f;
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -72,6 +71,15 @@ __device__ __forceinline__ void map_workgroup(int n, int npair, int nblk, int* p
     *blk = n / npair;
     *pair = n % npair;
   }
+}
+
+// head_dim 128 needs more than 256 registers per lane: one wavefront per SIMD, the gradient accumulators in the
+// accumulation registers.  Pinning them there at the end of every iteration keeps the loop-carried values in that
+// register class, so the matrix instructions accumulate in place instead of being fed through copies (128 moves each
+// way per tile otherwise).
+template <bool PIN>
+__device__ __forceinline__ void pin_accumulator(f32x16& acc) {
+  if constexpr (PIN) asm volatile("" : "+a"(acc));
 }
 
 template <typename vec8>
@@ -272,6 +280,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
           dqacc[db] = TR::mfma32(ka, dsb[t], dqacc[db]);
         }
     }
+#pragma unroll
+    for (int db = 0; db < DBLK; db++) pin_accumulator<(D > 64)>(dqacc[db]);
     __syncthreads();
   }
 
@@ -279,7 +289,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
   const int qi = qw0 + lq;
   if (qi < f.L) {
     const long long row_id = ((long long)b * f.Hq + h) * f.L + qi;
-    if (lh == 0) *(float2*)(a.stats + 2 * row_id) = make_float2(m_use * f.scale + __logf(l_tot), delta);
+    // log2 of the row's sum of exponentials, the unit the second kernel's exp2 wants
+    if (lh == 0) *(float2*)(a.stats + 2 * row_id) = make_float2(m_use * c + __log2f(l_tot), delta);
     const float w = f.scale / l_tot;
     T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
 #pragma unroll
@@ -423,21 +434,27 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
       for (int ks = 0; ks < KSTEPS; ks++) dpacc = TR::mfma32(*(const vec8*)(Gr + r_lane + 16 * ks), vreg[ks], dpacc);
 
       const int key = kw0 + lq;
+      // only tiles on the diagonal, and the last key block, hide anything (rows past L carry lse = 1e30: weight 0)
+      const bool need_mask = (CAUSAL && kw0 + 31 > i0 + coff) || kw0 + 32 > S;
 #pragma unroll
       for (int rg = 0; rg < 4; rg++) {
-        const f32x4 s0 = *(const f32x4*)(st + 2 * (8 * rg + 4 * lh));      // (lse, delta) of rows 8rg+4lh+0, +1
+        const f32x4 s0 = *(const f32x4*)(st + 2 * (8 * rg + 4 * lh));      // (lse2, delta) of rows 8rg+4lh+0, +1
         const f32x4 s1 = *(const f32x4*)(st + 2 * (8 * rg + 4 * lh) + 4);  // ... +2, +3
-        const float lse[4] = {s0[0], s0[2], s1[0], s1[2]};
+        const float lse2[4] = {s0[0], s0[2], s1[0], s1[2]};
         const float dl[4] = {s0[1], s0[3], s1[1], s1[3]};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 4 * rg + e;
-          const int qrow = i0 + 8 * rg + 4 * lh + e;
-          const bool hidden = key >= S || (CAUSAL && key > qrow + coff);
-          float p = fast_exp2(fmaf(sacc[r], c, -lse[e] * kLog2e));
-          p = hidden ? 0.f : p;
+          const float p = fast_exp2(fmaf(sacc[r], c, -lse2[e]));
           sacc[r] = p;
           dpacc[r] = p * (dpacc[r] - dl[e]);
+        }
+      }
+      if (need_mask) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int qrow = i0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          if (key >= S || (CAUSAL && key > qrow + coff)) sacc[r] = 0.f, dpacc[r] = 0.f;
         }
       }
       vec8 pb[2], dsb[2];
@@ -457,6 +474,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
           dkacc[db] = TR::mfma32(transposed_operand<vec8>(ql, lo, hi), dsb[t], dkacc[db]);
         }
     }
+#pragma unroll
+    for (int db = 0; db < DBLK; db++) pin_accumulator<(D > 64)>(dkacc[db]), pin_accumulator<(D > 64)>(dvacc[db]);
     __syncthreads();
   }
 

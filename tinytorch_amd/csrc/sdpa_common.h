@@ -165,8 +165,9 @@ __device__ __forceinline__ void apply_attn_mask(const KArgs& a, f32x16& s, long 
 }
 
 // Backward call: the forward's arguments (f.out holds the forward's result, an input here) plus the upstream gradient
-// and the three gradients to write.  stats is scratch [B,Hq,L,2] floats: per query row the natural-log sum of
-// exponentials of its scaled, biased scores, and delta = dout . out.
+// and the three gradients to write.  stats is scratch [B,Hq,L,2] floats: per query row the log of the sum of
+// exponentials of its scaled, biased scores (natural log in the vector-ALU kernels, log2 in the MFMA kernels: the two
+// kernels of a call are always of one family), and delta = dout . out.
 struct BwdArgs {
   KArgs f;
   const void* dout;
