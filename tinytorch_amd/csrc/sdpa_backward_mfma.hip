@@ -27,7 +27,6 @@ namespace ttsdpa {
 namespace {
 
 constexpr int BM = 128;  // rows of the owning side per workgroup (queries in kernel 1, keys in kernel 2)
-constexpr int BN = 64;   // keys per streamed tile, kernel 1
 constexpr int BQ = 32;   // query rows per streamed tile, kernel 2
 constexpr float kLazyExp = 8.f;
 
@@ -38,11 +37,17 @@ template <int D>
 struct BwdLds {
   static constexpr int RP = D + 8;    // row pitch (elements) of a tile read as a row-major operand (ds_read_b128)
   static constexpr int TP = D + 32;   // row pitch of a tile read as a transposed operand (ds_read_b64_tr_b16)
-  static constexpr int DQ_STAGE = BN * (2 * RP + TP);       // K row-major, V row-major, K for transposed reads
-  static constexpr int DQ_BYTES = 2 * DQ_STAGE * 2;
   static constexpr int KV_STAGE = BQ * (2 * RP + 2 * TP);   // Q and dout, each in both layouts
   static constexpr int KV_STATS = 2 * BQ;                   // floats per stage: (lse, delta) per query row
   static constexpr int KV_BYTES = 2 * KV_STAGE * 2 + 2 * KV_STATS * 4;
+};
+
+// Key tile of the dq kernel: keys per tile, elements per LDS stage (K row-major, V row-major, K for transposed reads).
+template <int D>
+struct DqTile {
+  static constexpr int BN = D > 64 ? 32 : 64;
+  static constexpr int STAGE = BN * (2 * BwdLds<D>::RP + BwdLds<D>::TP);
+  static constexpr int BYTES = 2 * STAGE * 2;
 };
 
 // One MFMA A operand of X^T from a row-major tile X with pitch TP: lane l (column d = d0 + l%32, half h = l/32)
@@ -91,12 +96,16 @@ __device__ __forceinline__ vec8 regs_to_operand(const f32x16& acc, int t) {
 }
 
 // ---- kernel 1: dq, lse, delta ----------------------------------------------------------------------------------------
+// BN: keys per streamed tile.  64 for head_dim 64; 32 for head_dim 128, which keeps a wavefront under 256 registers:
+// two wavefronts per SIMD (one's vector work overlaps the other's matrix work), accumulators in ordinary registers.
 template <typename TR, int D, bool CAUSAL>
-__global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel(BwdArgs a) {
+__global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
+  constexpr int BN = DqTile<D>::BN;
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
   typedef BwdLds<D> Lds;
   constexpr int RP = Lds::RP, TP = Lds::TP;
+  constexpr int NBLK = BN / 32;            // 32-key blocks per tile
   constexpr int KSTEPS = D / 16, DBLK = D / 32;
   constexpr int NLD = (BN * D / 8) / 256;
   const KArgs& f = a.f;
@@ -179,7 +188,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
     }
   };
   auto store_tile = [&](int stage) {
-    T* Kr = smem + stage * Lds::DQ_STAGE;
+    T* Kr = smem + stage * DqTile<D>::STAGE;
     T* Vr = Kr + BN * RP;
     T* Kt = Vr + BN * RP;
 #pragma unroll
@@ -207,13 +216,13 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
       if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BN);
     }
     if (wave_live && (!CAUSAL || kv0 <= qw0 + 31 + coff)) {
-      const T* Kr = smem + cur * Lds::DQ_STAGE;
+      const T* Kr = smem + cur * DqTile<D>::STAGE;
       const T* Vr = Kr + BN * RP;
       const T* Kt = Vr + BN * RP;
 
-      f32x16 sacc[2];
+      f32x16 sacc[NBLK];
 #pragma unroll
-      for (int blk = 0; blk < 2; blk++) {
+      for (int blk = 0; blk < NBLK; blk++) {
 #pragma unroll
         for (int r = 0; r < 16; r++) sacc[blk][r] = 0.f;
         const T* krow = Kr + r_lane + 32 * blk * RP;
@@ -223,7 +232,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
       if ((CAUSAL && kv0 + BN - 1 > qw0 + coff) || kv0 + BN > S) {
         const int qi = qw0 + lq + coff;
 #pragma unroll
-        for (int blk = 0; blk < 2; blk++)
+        for (int blk = 0; blk < NBLK; blk++)
 #pragma unroll
           for (int r = 0; r < 16; r++) {
             const int key = kv0 + 32 * blk + 8 * (r >> 2) + 4 * lh + (r & 3);
@@ -232,7 +241,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
       }
       float mloc = sacc[0][0];
 #pragma unroll
-      for (int blk = 0; blk < 2; blk++)
+      for (int blk = 0; blk < NBLK; blk++)
 #pragma unroll
         for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, sacc[blk][r]);
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
@@ -248,9 +257,9 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
           for (int r = 0; r < 16; r++) dqacc[i][r] *= alpha;
       }
       // dP^T = V . dout^T
-      f32x16 dpacc[2];
+      f32x16 dpacc[NBLK];
 #pragma unroll
-      for (int blk = 0; blk < 2; blk++) {
+      for (int blk = 0; blk < NBLK; blk++) {
 #pragma unroll
         for (int r = 0; r < 16; r++) dpacc[blk][r] = 0.f;
         const T* vrow = Vr + r_lane + 32 * blk * RP;
@@ -259,7 +268,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
       }
       float psum = 0.f;
 #pragma unroll
-      for (int blk = 0; blk < 2; blk++)
+      for (int blk = 0; blk < NBLK; blk++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const float p = fast_exp2(fmaf(sacc[blk][r], c, -mc));  // relative to m_use; normalised at the end
@@ -267,21 +276,19 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_mfma_kernel
           sacc[blk][r] = p * (dpacc[blk][r] - delta);
         }
       l_run += psum;
-      vec8 dsb[4];
+      vec8 dsb[2 * NBLK];
 #pragma unroll
-      for (int t = 0; t < 4; t++) dsb[t] = regs_to_operand<vec8>(sacc[t >> 1], t & 1);
+      for (int t = 0; t < 2 * NBLK; t++) dsb[t] = regs_to_operand<vec8>(sacc[t >> 1], t & 1);
       // dq^T += K^T . dS^T
       const T* kl = Kt + t_lane;
 #pragma unroll
       for (int db = 0; db < DBLK; db++)
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
+        for (int t = 0; t < 2 * NBLK; t++) {
           const vec8 ka = transposed_operand<vec8>(kl, ((16 * t) * TP + 32 * db) * 2, ((16 * t + 8) * TP + 32 * db) * 2);
           dqacc[db] = TR::mfma32(ka, dsb[t], dqacc[db]);
         }
     }
-#pragma unroll
-    for (int db = 0; db < DBLK; db++) pin_accumulator<(D > 64)>(dqacc[db]);
     __syncthreads();
   }
 
@@ -501,13 +508,13 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   typedef BwdLds<D> Lds;
   static hipError_t state1[kMaxDevices], state2[kMaxDevices];
   static bool done1[kMaxDevices], done2[kMaxDevices];
-  hipError_t e = grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL>, Lds::DQ_BYTES, state1, done1);
+  hipError_t e = grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL>, DqTile<D>::BYTES, state1, done1);
   if (e != hipSuccess) return (int)e;
   e = grant_dynamic_lds((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL>, Lds::KV_BYTES, state2, done2);
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM);
-  hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g1), dim3(256), Lds::DQ_BYTES, stream, a);
+  hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g1), dim3(256), DqTile<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
