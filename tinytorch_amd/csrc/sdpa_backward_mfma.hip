@@ -503,6 +503,218 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   }
 }
 
+// ---- kernel 2 for head_dim 128: the same products with the tiles brought in by direct global->LDS loads ----------------
+// With register-staged tiles the kernel above needs ~330 registers per lane at head_dim 128: one wavefront per SIMD,
+// whose vector work nothing overlaps.  Here the Q / dout tiles (and this wavefront's V rows, once) go from global memory
+// straight into LDS (global_load_lds_dwordx4: 64 lanes x 16 bytes = four 256-byte rows per instruction, unpadded), which
+// frees the staging registers and the V fragments: under 256 registers, two workgroups per CU.  Rows are 16 chunks of
+// 16 bytes; chunk c of row r sits in slot c ^ f(r), f(r) = 4*(r%4) + (r/4)%4, which makes both the row-major operand
+// reads (ds_read_b128) and the transposed ones (ds_read_b64_tr_b16) conflict-free on one copy of a tile.
+namespace dkv128 {
+constexpr int D = 128;
+constexpr int ROW_BYTES = D * 2;
+constexpr int TILE_BYTES = BQ * ROW_BYTES;              // one 32-row tile of Q or dout
+constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * BQ * 4;  // Q, dout, (lse2, delta) per row
+constexpr int V_BYTES = BM * ROW_BYTES;                 // the workgroup's V rows
+constexpr int LDS_BYTES = V_BYTES + 2 * STAGE_BYTES;
+__device__ __forceinline__ int swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+}  // namespace dkv128
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+template <typename TR, bool CAUSAL>
+__global__ __launch_bounds__(256, 2) void backward_dkv128_kernel(BwdArgs a) {
+  using namespace dkv128;
+  typedef typename TR::elem T;
+  typedef typename TR::vec8 vec8;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  constexpr int KSTEPS = D / 16, DBLK = D / 32;
+  const KArgs& f = a.f;
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const unsigned smem_addr = (unsigned)(unsigned long)(lds_void*)smem;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, lh = lane >> 5;
+
+  const int nkb = (f.S + BM - 1) / BM;
+  int pair, kb;
+  map_workgroup(blockIdx.x, f.B * f.Hkv, nkb, &pair, &kb);
+  const int hk = pair % f.Hkv, b = pair / f.Hkv;
+  const int k0 = kb * BM, kw0 = k0 + wave * 32;
+  const int S = f.S;
+  const int coff = CAUSAL ? causal_offset(f, S) : 0;
+
+  // Issued as asm so that the compiler does not see stores to LDS (it would make every LDS read wait for all loads).
+  auto dma16 = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+  };
+  auto dma4 = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+  };
+  const int drow = lane >> 4, dslot = lane & 15;  // this lane's row and slot inside a 4-row group of a load
+
+  // ---- this wavefront's V rows into LDS (read only by itself), its K rows into registers -------------------------------
+  {
+    const char* vb = (const char*)((const T*)f.v + b * f.vs[0] + hk * f.vs[1] + (long long)k0 * f.vs[2]);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int row = 32 * wave + 4 * i + drow;
+      const int rowc = k0 + row < S ? row : S - 1 - k0;  // rows past the end re-read the last key (never stored)
+      const unsigned voff = ((unsigned)rowc * (unsigned)f.vs[2] + 8u * (unsigned)(dslot ^ swz(row))) * 2u;
+      dma16(vb, voff, smem_addr + (32 * wave + 4 * i) * ROW_BYTES);
+    }
+  }
+  vec8 kreg[KSTEPS];
+  {
+    int row = kw0 + lq;
+    row = row < S ? row : S - 1;
+    const T* kr = (const T*)f.k + b * f.ks[0] + hk * f.ks[1] + row * f.ks[2] + 8 * lh;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) kreg[ks] = *(const vec8*)(kr + 16 * ks);
+  }
+  f32x16 dkacc[DBLK], dvacc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dkacc[i][r] = 0.f, dvacc[i][r] = 0.f;
+  const float c = f.scale * kLog2e;
+
+  const int ntq = (f.L + BQ - 1) / BQ;
+  int it0 = 0;
+  if (CAUSAL) it0 = (k0 - coff > 0 ? k0 - coff : 0) / BQ;
+  const int nt = ntq > it0 ? ntq - it0 : 0;
+  const int total = f.G * nt;
+
+  // wavefront w brings rows 8w .. 8w+7 of the Q tile and of the dout tile (two loads each); wavefront 0 the statistics
+  auto dma_tile = [&](int idx, int stage) __attribute__((always_inline)) {
+    const int h = hk * f.G + idx / nt;
+    const int i0 = (it0 + idx % nt) * BQ;
+    const char* qb = (const char*)((const T*)f.q + b * f.qs[0] + h * f.qs[1] + (long long)i0 * f.qs[2]);
+    const char* gb = (const char*)((const T*)a.dout + b * a.dos[0] + h * a.dos[1] + (long long)i0 * a.dos[2]);
+    const unsigned at = smem_addr + V_BYTES + stage * STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const int row = 8 * wave + 4 * i + drow;
+      const int rowc = i0 + row < f.L ? row : f.L - 1 - i0;  // rows past the end re-read the last row (weight forced to 0)
+      const unsigned chunk = (unsigned)(dslot ^ swz(row));
+      dma16(qb, ((unsigned)rowc * (unsigned)f.qs[2] + 8u * chunk) * 2u, at + (8 * wave + 4 * i) * ROW_BYTES);
+      dma16(gb, ((unsigned)rowc * (unsigned)a.dos[2] + 8u * chunk) * 2u, at + TILE_BYTES + (8 * wave + 4 * i) * ROW_BYTES);
+    }
+    if (wave == 0) {  // 32 rows x (lse2, delta): 64 floats, one per lane
+      const char* sb = (const char*)(a.stats + 2 * (((long long)b * f.Hq + h) * f.L + i0));
+      const int row = lane >> 1;
+      const int rowc = i0 + row < f.L ? row : f.L - 1 - i0;
+      dma4(sb, (unsigned)(2 * rowc + (lane & 1)) * 4u, at + 2 * TILE_BYTES);
+    }
+  };
+
+  // ---- LDS operand addresses (bytes inside a tile), loop-invariant ----------------------------------------------------
+  // row-major operand, k-step ks: row lq, chunk 2ks + lh  ->  lq*256 + 16*((2ks + lh) ^ f(lq)) = r_base ^ (32*ks)
+  const unsigned r_base = (unsigned)(lq * ROW_BYTES + 16 * (lh ^ swz(lq)));
+  // transposed operand (db, ld) of k-step t: this lane points at row 16t + 8ld + 4lh + s/4, elements
+  // 32db + 16*dhalf + 4*(s%4) .. +3 (s = lane%16, dhalf = (lane/16)%2) and receives X[16t + 8ld + 4lh + 0..3][32db + lq]
+  unsigned t_base[2];
+  {
+    const int s = lane & 15, dhalf = (lane >> 4) & 1;
+#pragma unroll
+    for (int ld = 0; ld < 2; ld++) {
+      const int row = 8 * ld + 4 * lh + (s >> 2);  // f(row) does not depend on t
+      const int c0 = 2 * dhalf + ((s & 3) >> 1);
+      t_base[ld] = (unsigned)(row * ROW_BYTES + 16 * (c0 ^ swz(row)) + 8 * (s & 1));  // ^ (64*db) selects the 32-column block
+    }
+  }
+  const char* vown = smem + 32 * wave * ROW_BYTES;
+
+  if (total > 0) dma_tile(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  const int key = kw0 + lq;
+  for (int idx = 0; idx < total; idx++) {
+    const int cur = idx & 1;
+    if (idx + 1 < total) dma_tile(idx + 1, cur ^ 1);  // that stage was last read before the barrier that ended idx-1
+    const int i0 = (it0 + idx % nt) * BQ;
+    {
+      const char* qt = smem + V_BYTES + cur * STAGE_BYTES;
+      const char* gt = qt + TILE_BYTES;
+      const float* st = (const float*)(qt + 2 * TILE_BYTES);
+
+      f32x16 sacc, dpacc;
+#pragma unroll
+      for (int r = 0; r < 16; r++) sacc[r] = 0.f, dpacc[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) sacc = TR::mfma32(*(const vec8*)(qt + (r_base ^ (unsigned)(32 * ks))), kreg[ks], sacc);
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++)
+        dpacc = TR::mfma32(*(const vec8*)(gt + (r_base ^ (unsigned)(32 * ks))), *(const vec8*)(vown + (r_base ^ (unsigned)(32 * ks))), dpacc);
+
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        const f32x4 s0 = *(const f32x4*)(st + 2 * (8 * rg + 4 * lh));      // (lse2, delta) of rows 8rg+4lh+0, +1
+        const f32x4 s1 = *(const f32x4*)(st + 2 * (8 * rg + 4 * lh) + 4);  // ... +2, +3
+        const float lse2[4] = {s0[0], s0[2], s1[0], s1[2]};
+        const float dl[4] = {s0[1], s0[3], s1[1], s1[3]};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int r = 4 * rg + e;
+          const float p = fast_exp2(fmaf(sacc[r], c, -lse2[e]));
+          sacc[r] = p;
+          dpacc[r] = p * (dpacc[r] - dl[e]);
+        }
+      }
+      // only tiles on or above the diagonal, the last key block and the last query tile hide anything; a wavefront whose
+      // keys no row of the tile sees runs the tile with every weight 0
+      if ((CAUSAL && kw0 + 31 > i0 + coff) || kw0 + 32 > S || i0 + BQ > f.L) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int qrow = i0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          if (key >= S || qrow >= f.L || (CAUSAL && key > qrow + coff)) sacc[r] = 0.f, dpacc[r] = 0.f;
+        }
+      }
+      vec8 pb[2], dsb[2];
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        pb[t] = regs_to_operand<vec8>(sacc, t);
+        dsb[t] = regs_to_operand<vec8>(dpacc, t);
+      }
+#pragma unroll
+      for (int db = 0; db < DBLK; db++)
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const unsigned lo = (t_base[0] ^ (unsigned)(64 * db)) + 16 * t * ROW_BYTES, hi = (t_base[1] ^ (unsigned)(64 * db)) + 16 * t * ROW_BYTES;
+          const s16x4 glo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(gt + lo));
+          const s16x4 ghi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(gt + hi));
+          const s16x4 qlo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(qt + lo));
+          const s16x4 qhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(qt + hi));
+          dvacc[db] = TR::mfma32(__builtin_bit_cast(vec8, __builtin_shufflevector(glo, ghi, 0, 1, 2, 3, 4, 5, 6, 7)), pb[t], dvacc[db]);
+          dkacc[db] = TR::mfma32(__builtin_bit_cast(vec8, __builtin_shufflevector(qlo, qhi, 0, 1, 2, 3, 4, 5, 6, 7)), dsb[t], dkacc[db]);
+        }
+    }
+    // the next tile has landed (this wavefront's part; the barrier covers the others') and nobody reads this one any more
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  if (key < S) {
+    T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
+    T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
+#pragma unroll
+    for (int db = 0; db < DBLK; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        f32x4 x, y;
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = dkacc[db][4 * rg + i] * f.scale, y[i] = dvacc[db][4 * rg + i];
+        *(typename TR::vec4*)(dkp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
+        *(typename TR::vec4*)(dvp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(y, typename TR::vec4);
+      }
+  }
+}
+
 template <typename TR, int D, bool CAUSAL>
 int launch_k(const BwdArgs& a, hipStream_t stream) {
   typedef BwdLds<D> Lds;
@@ -510,14 +722,22 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   static bool done1[kMaxDevices], done2[kMaxDevices];
   hipError_t e = grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL>, DqTile<D>::BYTES, state1, done1);
   if (e != hipSuccess) return (int)e;
-  e = grant_dynamic_lds((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL>, Lds::KV_BYTES, state2, done2);
+  if (D == 128) {
+    e = grant_dynamic_lds((const void*)backward_dkv128_kernel<TR, CAUSAL>, dkv128::LDS_BYTES, state2, done2);
+  } else {
+    e = grant_dynamic_lds((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL>, Lds::KV_BYTES, state2, done2);
+  }
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM);
   hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g1), dim3(256), DqTile<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
-  hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
+  if (D == 128) {
+    hipLaunchKernelGGL((backward_dkv128_kernel<TR, CAUSAL>), dim3((unsigned)g2), dim3(256), dkv128::LDS_BYTES, stream, a);
+  } else {
+    hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
+  }
   return (int)hipGetLastError();
 }
 
