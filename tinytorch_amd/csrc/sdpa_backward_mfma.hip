@@ -8,16 +8,17 @@
 //
 // Two kernels, no atomics (fixed summation order, reproducible results):
 //   1. backward_dq_mfma_kernel — a workgroup owns 128 query rows of one (batch, query head), a wavefront 32 of them,
-//      and streams the keys in tiles of 64 exactly like the forward kernel: S^T = K.Q^T, an online softmax with a lazily
+//      and streams the keys in tiles of 64 (32 at head_dim 128) like the forward kernel: S^T = K.Q^T, an online softmax with a lazily
 //      raised maximum (so lse_i needs no pass of its own), dP^T = V.dout^T, dS^T, dq^T += K^T.dS^T.  At the end
 //      dq = scale/l * accumulator, and (lse_i, delta_i) go to scratch for the second kernel.
-//   2. backward_dkv_mfma_kernel — a workgroup owns 128 keys of one (batch, kv head), a wavefront 32 of them, and
-//      streams the query rows of every head of the group in tiles of 32: S = Q.K^T, P from lse, dP = dout.V^T, dS,
-//      dv^T += dout^T.P, dk^T += Q^T.dS.
+//   2. backward_dkv_mfma_kernel (head_dim 64) / backward_dkv128_kernel (head_dim 128) — a workgroup owns 128 keys of
+//      one (batch, kv head), a wavefront 32 of them, and streams the query rows of every head of the group in tiles
+//      of 32: S = Q.K^T, P from lse, dP = dout.V^T, dS, dv^T += dout^T.P, dk^T += Q^T.dS.
 // Both compute 32 x 32 score blocks with v_mfma_f32_32x32x16 whose accumulator layout (lane = column, registers = rows)
 // is the B operand of the following product, so P and dS go from registers to the matrix cores without touching LDS;
-// the streamed tiles are staged in LDS twice where both a row-major operand and a transposed one
-// (ds_read_b64_tr_b16) are read from them, each copy with the row pitch that makes its reads conflict-free.
+// the register-staged tiles are kept in LDS twice where both a row-major operand and a transposed one
+// (ds_read_b64_tr_b16) are read from them, each copy with the row pitch that makes its reads conflict-free; the
+// head_dim-128 dk/dv kernel keeps one swizzled copy instead (see there).
 // Seven matrix products in all, against five in the textbook count (the scores are computed in both kernels).
 
 #include "sdpa_common.h"
@@ -361,7 +362,10 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
     for (int r = 0; r < 16; r++) dkacc[i][r] = 0.f, dvacc[i][r] = 0.f;
   const float c = f.scale * kLog2e;
 
-  // query tiles it0 .. ntq-1 of each of the G heads see keys of this workgroup
+  // Query tiles it0 .. ntq-1 of each of the G heads see keys of this workgroup.  They are taken from the last tile down,
+  // the heads of a tile one after the other: every key block of a (batch, kv head) then starts at the same tile and walks
+  // in step with the others (a block further down the causal triangle just stops earlier), so the tile one workgroup
+  // fetches from HBM is in the XCD's L2 for the others.
   const int ntq = (f.L + BQ - 1) / BQ;
   int it0 = 0;
   if (CAUSAL) it0 = (k0 - coff > 0 ? k0 - coff : 0) / BQ;
@@ -378,8 +382,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
     lcol[i] = cidx % (D / 8);
   }
   auto load_tile = [&](int idx) {
-    const int h = hk * f.G + idx / nt;
-    const int i0 = (it0 + idx % nt) * BQ;
+    const int h = hk * f.G + idx % f.G;
+    const int i0 = (ntq - 1 - idx / f.G) * BQ;
     const T* qp = (const T*)f.q + b * f.qs[0] + h * f.qs[1];
     const T* gp = (const T*)a.dout + b * a.dos[0] + h * a.dos[1];
 #pragma unroll
@@ -424,7 +428,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
       store_tile(cur ^ 1);
       if (idx + 2 < total) load_tile(idx + 2);
     }
-    const int i0 = (it0 + idx % nt) * BQ;
+    const int i0 = (ntq - 1 - idx / f.G) * BQ;
     if (wave_live && (!CAUSAL || kw0 <= i0 + BQ - 1 + coff)) {
       const T* Qr = smem + cur * Lds::KV_STAGE;
       const T* Gr = Qr + BQ * RP;
@@ -590,8 +594,8 @@ __global__ __launch_bounds__(256, 2) void backward_dkv128_kernel(BwdArgs a) {
 
   // wavefront w brings rows 8w .. 8w+7 of the Q tile and of the dout tile (two loads each); wavefront 0 the statistics
   auto dma_tile = [&](int idx, int stage) __attribute__((always_inline)) {
-    const int h = hk * f.G + idx / nt;
-    const int i0 = (it0 + idx % nt) * BQ;
+    const int h = hk * f.G + idx % f.G;
+    const int i0 = (ntq - 1 - idx / f.G) * BQ;
     const char* qb = (const char*)((const T*)f.q + b * f.qs[0] + h * f.qs[1] + (long long)i0 * f.qs[2]);
     const char* gb = (const char*)((const T*)a.dout + b * a.dos[0] + h * a.dos[1] + (long long)i0 * a.dos[2]);
     const unsigned at = smem_addr + V_BYTES + stage * STAGE_BYTES;
@@ -637,7 +641,7 @@ __global__ __launch_bounds__(256, 2) void backward_dkv128_kernel(BwdArgs a) {
   for (int idx = 0; idx < total; idx++) {
     const int cur = idx & 1;
     if (idx + 1 < total) dma_tile(idx + 1, cur ^ 1);  // that stage was last read before the barrier that ended idx-1
-    const int i0 = (it0 + idx % nt) * BQ;
+    const int i0 = (ntq - 1 - idx / f.G) * BQ;
     {
       const char* qt = smem + V_BYTES + cur * STAGE_BYTES;
       const char* gt = qt + TILE_BYTES;
