@@ -509,25 +509,32 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
 
 // ---- kernel 2 for head_dim 128: the same products with the tiles brought in by direct global->LDS loads ----------------
 // With register-staged tiles the kernel above needs ~330 registers per lane at head_dim 128: one wavefront per SIMD,
-// whose vector work nothing overlaps.  Here the Q / dout tiles (and this wavefront's V rows, once) go from global memory
+// whose vector work nothing overlaps.  Here the Q / dout tiles (and the workgroup's V rows, once) go from global memory
 // straight into LDS (global_load_lds_dwordx4: 64 lanes x 16 bytes = four 256-byte rows per instruction, unpadded), which
-// frees the staging registers and the V fragments: under 256 registers, two workgroups per CU.  Rows are 16 chunks of
+// frees the staging registers and the V fragments: under 256 registers, two wavefronts per SIMD.  Rows are 16 chunks of
 // 16 bytes; chunk c of row r sits in slot c ^ f(r), f(r) = 4*(r%4) + (r/4)%4, which makes both the row-major operand
 // reads (ds_read_b128) and the transposed ones (ds_read_b64_tr_b16) conflict-free on one copy of a tile.
+//
+// Eight wavefronts in two groups of four: both groups own the same 128 keys and take alternate tiles of the query
+// stream, each with its own three-stage ring of tiles, and group 1's partial dk / dv are added to group 0's through
+// LDS at the end.  Under a causal mask the first key block of a KV head sees every query row of every head of the
+// group — the longest workgroup of the launch; two groups halve that critical path.
 namespace dkv128 {
 constexpr int D = 128;
 constexpr int ROW_BYTES = D * 2;
-constexpr int TILE_BYTES = BQ * ROW_BYTES;              // one 32-row tile of Q or dout
+constexpr int TILE_BYTES = BQ * ROW_BYTES;                // one 32-row tile of Q or dout
 constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * BQ * 4;  // Q, dout, (lse2, delta) per row
-constexpr int V_BYTES = BM * ROW_BYTES;                 // the workgroup's V rows
-constexpr int LDS_BYTES = V_BYTES + 2 * STAGE_BYTES;
+constexpr int NSTAGE = 3;
+constexpr int V_BYTES = BM * ROW_BYTES;                   // the workgroup's V rows
+constexpr int LDS_BYTES = V_BYTES + 2 * NSTAGE * STAGE_BYTES;
+static_assert(LDS_BYTES >= 2 * 128 * 64 * 4, "the reduction of one gradient needs 64 KiB");
 __device__ __forceinline__ int swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 }  // namespace dkv128
 
 typedef __attribute__((address_space(3))) void lds_void;
 
 template <typename TR, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void backward_dkv128_kernel(BwdArgs a) {
+__global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
   using namespace dkv128;
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
@@ -541,13 +548,14 @@ __global__ __launch_bounds__(256, 2) void backward_dkv128_kernel(BwdArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave >> 2, gw = wave & 3;  // group, wavefront inside the group
   const int lq = lane & 31, lh = lane >> 5;
 
   const int nkb = (f.S + BM - 1) / BM;
   int pair, kb;
   map_workgroup(blockIdx.x, f.B * f.Hkv, nkb, &pair, &kb);
   const int hk = pair % f.Hkv, b = pair / f.Hkv;
-  const int k0 = kb * BM, kw0 = k0 + wave * 32;
+  const int k0 = kb * BM, kw0 = k0 + gw * 32;
   const int S = f.S;
   const int coff = CAUSAL ? causal_offset(f, S) : 0;
 
@@ -560,15 +568,15 @@ __global__ __launch_bounds__(256, 2) void backward_dkv128_kernel(BwdArgs a) {
   };
   const int drow = lane >> 4, dslot = lane & 15;  // this lane's row and slot inside a 4-row group of a load
 
-  // ---- this wavefront's V rows into LDS (read only by itself), its K rows into registers -------------------------------
+  // ---- the workgroup's V rows into LDS (wavefront w brings rows 16w .. 16w+15), this wavefront's K rows into registers ----
   {
     const char* vb = (const char*)((const T*)f.v + b * f.vs[0] + hk * f.vs[1] + (long long)k0 * f.vs[2]);
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int row = 32 * wave + 4 * i + drow;
+    for (int i = 0; i < 4; i++) {
+      const int row = 16 * wave + 4 * i + drow;
       const int rowc = k0 + row < S ? row : S - 1 - k0;  // rows past the end re-read the last key (never stored)
       const unsigned voff = ((unsigned)rowc * (unsigned)f.vs[2] + 8u * (unsigned)(dslot ^ swz(row))) * 2u;
-      dma16(vb, voff, smem_addr + (32 * wave + 4 * i) * ROW_BYTES);
+      dma16(vb, voff, smem_addr + (16 * wave + 4 * i) * ROW_BYTES);
     }
   }
   vec8 kreg[KSTEPS];
@@ -586,28 +594,35 @@ __global__ __launch_bounds__(256, 2) void backward_dkv128_kernel(BwdArgs a) {
     for (int r = 0; r < 16; r++) dkacc[i][r] = 0.f, dvacc[i][r] = 0.f;
   const float c = f.scale * kLog2e;
 
+  // Query tiles it0 .. ntq-1 of each of the G heads see keys of this workgroup.  They are taken from the last tile down,
+  // the heads of a tile one after the other: every key block of a (batch, kv head) then starts at the same tile and walks
+  // in step with the others (a block further down the causal triangle just stops earlier), so the tile one workgroup
+  // fetches from HBM is in the XCD's L2 for the others.  Entry idx of that list belongs to group idx % 2.
   const int ntq = (f.L + BQ - 1) / BQ;
   int it0 = 0;
   if (CAUSAL) it0 = (k0 - coff > 0 ? k0 - coff : 0) / BQ;
   const int nt = ntq > it0 ? ntq - it0 : 0;
   const int total = f.G * nt;
+  const int niter = (total + 1) / 2;  // iterations of either group (the second may have one entry less)
 
-  // wavefront w brings rows 8w .. 8w+7 of the Q tile and of the dout tile (two loads each); wavefront 0 the statistics
+  // wavefront gw of a group brings rows 8gw .. 8gw+7 of the Q tile and of the dout tile (two loads each) into the
+  // group's ring; its first wavefront the statistics as well
+  const unsigned ring_addr = smem_addr + V_BYTES + grp * NSTAGE * STAGE_BYTES;
   auto dma_tile = [&](int idx, int stage) __attribute__((always_inline)) {
     const int h = hk * f.G + idx % f.G;
     const int i0 = (ntq - 1 - idx / f.G) * BQ;
     const char* qb = (const char*)((const T*)f.q + b * f.qs[0] + h * f.qs[1] + (long long)i0 * f.qs[2]);
     const char* gb = (const char*)((const T*)a.dout + b * a.dos[0] + h * a.dos[1] + (long long)i0 * a.dos[2]);
-    const unsigned at = smem_addr + V_BYTES + stage * STAGE_BYTES;
+    const unsigned at = ring_addr + stage * STAGE_BYTES;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-      const int row = 8 * wave + 4 * i + drow;
+      const int row = 8 * gw + 4 * i + drow;
       const int rowc = i0 + row < f.L ? row : f.L - 1 - i0;  // rows past the end re-read the last row (weight forced to 0)
       const unsigned chunk = (unsigned)(dslot ^ swz(row));
-      dma16(qb, ((unsigned)rowc * (unsigned)f.qs[2] + 8u * chunk) * 2u, at + (8 * wave + 4 * i) * ROW_BYTES);
-      dma16(gb, ((unsigned)rowc * (unsigned)a.dos[2] + 8u * chunk) * 2u, at + TILE_BYTES + (8 * wave + 4 * i) * ROW_BYTES);
+      dma16(qb, ((unsigned)rowc * (unsigned)f.qs[2] + 8u * chunk) * 2u, at + (8 * gw + 4 * i) * ROW_BYTES);
+      dma16(gb, ((unsigned)rowc * (unsigned)a.dos[2] + 8u * chunk) * 2u, at + TILE_BYTES + (8 * gw + 4 * i) * ROW_BYTES);
     }
-    if (wave == 0) {  // 32 rows x (lse2, delta): 64 floats, one per lane
+    if (gw == 0) {  // 32 rows x (lse2, delta): 64 floats, one per lane
       const char* sb = (const char*)(a.stats + 2 * (((long long)b * f.Hq + h) * f.L + i0));
       const int row = lane >> 1;
       const int rowc = i0 + row < f.L ? row : f.L - 1 - i0;
@@ -630,20 +645,26 @@ __global__ __launch_bounds__(256, 2) void backward_dkv128_kernel(BwdArgs a) {
       t_base[ld] = (unsigned)(row * ROW_BYTES + 16 * (c0 ^ swz(row)) + 8 * (s & 1));  // ^ (64*db) selects the 32-column block
     }
   }
-  const char* vown = smem + 32 * wave * ROW_BYTES;
+  const char* vown = smem + 32 * gw * ROW_BYTES;
+  const char* ring = smem + V_BYTES + grp * NSTAGE * STAGE_BYTES;
 
-  if (total > 0) dma_tile(0, 0);
+  // entries grp, grp + 2 of the list on their way, everything landed before the first use
+  if (grp < total) dma_tile(grp, 0);
+  if (grp + 2 < total) dma_tile(grp + 2, 1);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 
   const int key = kw0 + lq;
-  for (int idx = 0; idx < total; idx++) {
-    const int cur = idx & 1;
-    if (idx + 1 < total) dma_tile(idx + 1, cur ^ 1);  // that stage was last read before the barrier that ended idx-1
-    const int i0 = (ntq - 1 - idx / f.G) * BQ;
-    {
-      const char* qt = smem + V_BYTES + cur * STAGE_BYTES;
+  int cur = 0;  // j % 3
+  for (int j = 0; j < niter; j++) {
+    const int idx = 2 * j + grp;
+    const int nxt2 = cur == 0 ? 2 : cur - 1;  // (j + 2) % 3: last read in iteration j-1, which a barrier ended
+    const bool more = idx + 4 < total;
+    if (more) dma_tile(idx + 4, nxt2);
+    if (idx < total) {
+      const int i0 = (ntq - 1 - idx / f.G) * BQ;
+      const char* qt = ring + cur * STAGE_BYTES;
       const char* gt = qt + TILE_BYTES;
       const float* st = (const float*)(qt + 2 * TILE_BYTES);
 
@@ -698,12 +719,44 @@ __global__ __launch_bounds__(256, 2) void backward_dkv128_kernel(BwdArgs a) {
           dkacc[db] = TR::mfma32(__builtin_bit_cast(vec8, __builtin_shufflevector(qlo, qhi, 0, 1, 2, 3, 4, 5, 6, 7)), dsb[t], dkacc[db]);
         }
     }
-    // the next tile has landed (this wavefront's part; the barrier covers the others') and nobody reads this one any more
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // Entry idx + 2 must have landed before the next iteration; the loads of entry idx + 4, issued above, may stay in
+    // flight (four per wavefront, five for the one that also brings the statistics; they complete in issue order).
+    if (more) {
+      if (gw == 0) {
+        asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      }
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    cur = cur == 2 ? 0 : cur + 1;
+  }
+
+  // ---- group 1's partial gradients join group 0's, one gradient (64 KiB of fp32) at a time ------------------------------
+  float* red = (float*)smem;
+  const int slot = gw * 64 + lane;
+#pragma unroll
+  for (int which = 0; which < 2; which++) {
+    f32x16* acc = which == 0 ? dkacc : dvacc;
+    if (grp == 1) {
+#pragma unroll
+      for (int db = 0; db < DBLK; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) red[(db * 16 + r) * 256 + slot] = acc[db][r];
+    }
+    __syncthreads();
+    if (grp == 0) {
+#pragma unroll
+      for (int db = 0; db < DBLK; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[db][r] += red[(db * 16 + r) * 256 + slot];
+    }
     __syncthreads();
   }
 
-  if (key < S) {
+  if (grp == 0 && key < S) {
     T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
     T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
 #pragma unroll
@@ -738,7 +791,7 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   if (D == 128) {
-    hipLaunchKernelGGL((backward_dkv128_kernel<TR, CAUSAL>), dim3((unsigned)g2), dim3(256), dkv128::LDS_BYTES, stream, a);
+    hipLaunchKernelGGL((backward_dkv128_kernel<TR, CAUSAL>), dim3((unsigned)g2), dim3(512), dkv128::LDS_BYTES, stream, a);
   } else {
     hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
   }
