@@ -159,6 +159,36 @@ def test_backward_bottom_right_causal_and_key_counts(dtype):
         assert torch.all(dk[b, :, lens[b]:] == 0) and torch.all(dv[b, :, lens[b]:] == 0)
 
 
+@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_backward_mfma_per_batch_key_counts(dtype, D, causal):
+    """kv_len on the MFMA pair: each batch entry against the oracle on its own key prefix (bottom-right causal when
+    asked); an empty entry gets dq = 0; dk / dv beyond a count are zeros."""
+    B, Hq, Hkv, L, S = 3, 8, 2, 70, 300
+    host, dev = make_inputs(4400 + D, B, Hq, Hkv, L, S, D, dtype)
+    lens = [300, 129, 0]
+    kv = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    q, k, v = dev
+    go_h, go = upstream(5, q.shape, dtype)
+    say("backward kv_len", dtype, D, causal)
+    out = sdpAttention(q, k, v, isCausal=causal, causalAlign="bottom-right", kvLens=kv)
+    assert backward_route_of(q, k, v, out, go, causal, None, None, kv, "bottom-right") == "prefill"
+    rc, (dq, dk, dv) = backward_call(q, k, v, out, go, causal=causal, kv_lens=kv, align="bottom-right")
+    assert rc == 0
+    for b in range(B):
+        n = lens[b]
+        if n == 0:
+            assert torch.all(dq[b] == 0) and torch.all(dk[b] == 0) and torch.all(dv[b] == 0)
+            continue
+        m = (np.arange(n)[None, :] <= np.arange(L)[:, None] + max(0, n - L)) if causal else None
+        eq, ek, ev = oracle.sdpa_backward_f32(host[0][b:b + 1], host[1][b:b + 1, :, :n], host[2][b:b + 1, :, :n],
+                                              go_h[b:b + 1], mask=m)
+        assert grad_err(dq[b:b + 1], eq) <= TOL[dtype], b
+        assert grad_err(dk[b:b + 1, :, :n], ek) <= TOL[dtype], b
+        assert grad_err(dv[b:b + 1, :, :n], ev) <= TOL[dtype], b
+        assert torch.all(dk[b, :, n:] == 0) and torch.all(dv[b, :, n:] == 0)
+
+
 def test_backward_strided_views_and_scale():
     """q/k/v as slices of one packed projection output, gradients into slices of one packed buffer."""
     B, H, N, D = 2, 4, 40, 64

@@ -88,6 +88,32 @@ __device__ __forceinline__ void pin_accumulator(f32x16& acc) {
   if constexpr (PIN) asm volatile("" : "+a"(acc));
 }
 
+// Keys of batch entry b: all S of them, or the filled prefix of a cache / the unpadded length (kv_len).
+__device__ __forceinline__ int keys_of_batch(const KArgs& f, int b) {
+  int S = f.S;
+  if (f.kv_len) {
+    const int len = __builtin_amdgcn_readfirstlane(f.kv_len[b]);
+    S = len < 0 ? 0 : (len < S ? len : S);
+  }
+  return S;
+}
+
+// dk and dv rows of a key no query row attends to (at or beyond the batch entry's key count): zeros.
+template <typename TR, int D>
+__device__ __forceinline__ void zero_key_rows(const BwdArgs& a, int b, int hk, int key, int lh) {
+  typedef typename TR::elem T;
+  if (key >= a.f.S) return;
+  T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
+  T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
+  typename TR::vec4 zero;
+#pragma unroll
+  for (int i = 0; i < 4; i++) zero[i] = (T)0.f;
+  for (int d = 4 * lh; d < D; d += 8) {
+    *(typename TR::vec4*)(dkp + d) = zero;
+    *(typename TR::vec4*)(dvp + d) = zero;
+  }
+}
+
 template <typename vec8>
 __device__ __forceinline__ vec8 regs_to_operand(const f32x16& acc, int t) {
   f32x8 x;
@@ -161,7 +187,18 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
   const float lazy = kLazyExp / c;
   float m_use = -1e30f, mc = m_use * c, l_run = 0.f;
 
-  const int S = f.S;
+  const int S = keys_of_batch(f, b);
+  if (S == 0) {  // no keys (an empty cache entry): the output did not depend on q
+    const int qi = qw0 + lq;
+    if (qi < f.L) {
+      T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
+      typename TR::vec4 zero;
+#pragma unroll
+      for (int i = 0; i < 4; i++) zero[i] = (T)0.f;
+      for (int d = 4 * lh; d < D; d += 8) *(typename TR::vec4*)(dqp + d) = zero;
+    }
+    return;
+  }
   const int coff = CAUSAL ? causal_offset(f, S) : 0;
   int ntiles_kv = (S + BN - 1) / BN;
   if (CAUSAL) {
@@ -338,7 +375,11 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   map_workgroup(blockIdx.x, f.B * f.Hkv, nkb, &pair, &kb);
   const int hk = pair % f.Hkv, b = pair / f.Hkv;
   const int k0 = kb * BM, kw0 = k0 + wave * 32;
-  const int S = f.S;
+  const int S = keys_of_batch(f, b);  // rows of dk / dv from here to f.S are written as zeros
+  if (k0 >= S) {
+    zero_key_rows<TR, D>(a, b, hk, kw0 + lq, lh);
+    return;
+  }
   const bool wave_live = kw0 < S;
   const int coff = CAUSAL ? causal_offset(f, S) : 0;
 
@@ -491,7 +532,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   }
 
   const int key = kw0 + lq;
-  if (key < S) {
+  if (key < f.S) {
     T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
     T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
 #pragma unroll
@@ -556,7 +597,11 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
   map_workgroup(blockIdx.x, f.B * f.Hkv, nkb, &pair, &kb);
   const int hk = pair % f.Hkv, b = pair / f.Hkv;
   const int k0 = kb * BM, kw0 = k0 + gw * 32;
-  const int S = f.S;
+  const int S = keys_of_batch(f, b);  // rows of dk / dv from here to f.S are written as zeros
+  if (k0 >= S) {
+    if (grp == 0) zero_key_rows<TR, D>(a, b, hk, kw0 + lq, lh);
+    return;
+  }
   const int coff = CAUSAL ? causal_offset(f, S) : 0;
 
   // Issued as asm so that the compiler does not see stores to LDS (it would make every LDS read wait for all loads).
@@ -756,7 +801,7 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
     __syncthreads();
   }
 
-  if (grp == 0 && key < S) {
+  if (grp == 0 && key < f.S) {
     T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
     T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
 #pragma unroll
