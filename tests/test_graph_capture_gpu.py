@@ -78,3 +78,46 @@ def test_decode_step_in_a_graph(B, Hq, Hkv, Smax):
         assert torch.equal(eager, out_buf)
     for b in range(B):
         assert torch.equal(kc[b, :, :cur[b]], kd[b, :, :cur[b]])
+
+
+def test_forward_and_backward_in_a_graph():
+    """A training-style step (attention forward, then its backward) recorded once and replayed on new inputs: both
+    calls only enqueue kernels and use caller-provided scratch, so every replay reproduces the eager bits."""
+    import ctypes
+    from tinytorch_amd import _capi, build_backward_params, build_params
+    B, Hq, Hkv, N, D = 2, 8, 2, 384, 128
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    mk = lambda *shape: torch.randn(*shape, device="cuda", generator=gen).bfloat16()
+    q, k, v, go = mk(B, Hq, N, D), mk(B, Hkv, N, D), mk(B, Hkv, N, D), mk(B, Hq, N, D)
+    out, dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    L = _capi.lib()
+    fp = build_params(q, k, v, out, True)
+    bp = build_backward_params(q, k, v, out, go, dq, dk, dv, True)
+    nbytes = L.ttsdpa_backward_workspace_bytes(ctypes.byref(bp))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+
+    def step():
+        st = torch.cuda.current_stream().cuda_stream
+        assert L.ttsdpa_forward(ctypes.byref(fp), None, 0, st) == 0
+        assert L.ttsdpa_backward(ctypes.byref(bp), ws.data_ptr(), nbytes, st) == 0
+
+    step()   # eager once: one-time set-up of the kernels happens outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    for t in range(3):
+        for buf in (q, k, v, go):
+            buf.copy_(mk(*buf.shape))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [x.clone() for x in (out, dq, dk, dv)]
+        for x in (out, dq, dk, dv):
+            x.zero_()
+        step()   # the same step eagerly
+        torch.cuda.synchronize()
+        for a, b in zip(got, (out, dq, dk, dv)):
+            assert torch.equal(a, b), t
