@@ -40,6 +40,19 @@ int ttlinear_forward(int dtype, const void* x, const void* w, const void* bias, 
 int ttlinear_plan(int dtype, const void* x, const void* w, const void* bias, const void* out, int64_t M, int64_t N,
                   int64_t K, int64_t ldx, int64_t ldw, int64_t ldo, int* route);
 
+/* out[m, n] = bias[n] + sum_k A(m, k) * B(k, n) with the reference's transpose flags — op::matmul(a, b, transA, transB,
+ * bias) for 2-D operands (reference src/Operation/OpLinalgCpu.h:119-150: a is [M, K], or [K, M] with transA; b is [K, N], or
+ * [N, K] with transB).  (false, true) is ttlinear_forward; FuncLinear::backward (reference
+ * src/Function/FuncNNLayer.h:20-33) uses the other two that matter: (false, false) for the input gradient
+ * dy[M, N] . w[N, K], and (true, false) for the weight gradient dy^T . x.  lda / ldb / ldo are row strides in elements.
+ * workspace: ttlinear_matmul_workspace_bytes() bytes of device scratch, 256-byte aligned — the MFMA route first makes
+ * dense row-major copies of the operands that are stored contraction-major; with less (or NULL), or for shapes the MFMA
+ * kernel does not take, the vector-ALU kernel reads the operands in place.  Same return codes as ttlinear_forward. */
+size_t ttlinear_matmul_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b);
+int ttlinear_matmul(int dtype, const void* a, const void* b, const void* bias, void* out, int64_t M, int64_t N, int64_t K,
+                    int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldo, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

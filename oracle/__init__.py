@@ -66,6 +66,8 @@ def lib():
         L.oracle_softmax.restype = None
         L.oracle_linear.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int]
         L.oracle_linear.restype = None
+        L.oracle_matmul.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        L.oracle_matmul.restype = None
         _lib = L
     return _lib
 
@@ -96,6 +98,8 @@ def ref():
         R.tt_ref_softmax.restype = ctypes.c_int
         R.tt_ref_linear.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64]
         R.tt_ref_linear.restype = ctypes.c_int
+        R.tt_ref_matmul.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int]
+        R.tt_ref_matmul.restype = ctypes.c_int
         _ref = R
     return _ref
 
@@ -357,6 +361,34 @@ def linear(x, w, bias=None, dtype="f32"):
     N = w.shape[0]
     out = np.empty((M, N), dtype=np.float32)
     lib().oracle_linear(_p(x), _p(w), _p(b) if b is not None else None, _p(out), M, N, K, _dt(dtype))
+    return out
+
+
+def _matmul_dims(a, b, transA, transB):
+    K, M = a.shape if transA else a.shape[::-1]
+    Kb, N = b.shape[::-1] if transB else b.shape
+    assert K == Kb
+    return M, N, K
+
+
+def matmul(a, b, transA=False, transB=False, bias=None, dtype="f32"):
+    """op(a) . op(b) + bias in the reference's loop order: a [M,K] ([K,M] with transA), b [K,N] ([N,K] with transB)."""
+    a, b = _f32(a), _f32(b)
+    bs = _f32(bias) if bias is not None else None
+    M, N, K = _matmul_dims(a, b, transA, transB)
+    out = np.empty((M, N), dtype=np.float32)
+    lib().oracle_matmul(_p(a), _p(b), _p(bs) if bs is not None else None, _p(out), M, N, K, int(transA), int(transB), _dt(dtype))
+    return out
+
+
+def ref_matmul(a, b, transA=False, transB=False, bias=None):
+    """op::matmul of the compiled reference (fp32, CPU)."""
+    a, b = _f32(a), _f32(b)
+    bs = _f32(bias) if bias is not None else None
+    M, N, K = _matmul_dims(a, b, transA, transB)
+    out = np.empty((M, N), dtype=np.float32)
+    rc = ref().tt_ref_matmul(_p(a), _p(b), _p(bs) if bs is not None else None, _p(out), M, N, K, int(transA), int(transB))
+    assert rc == 0
     return out
 
 

@@ -17,6 +17,8 @@
  *                              (op::siluMul) bit-exact in fp32
  *   oracle_linear              reference KAT test/test_function.cpp:234-241; oracle/_ref (function::linear) bit-exact
  *                              in fp32; fp64 closed form
+ *   oracle_matmul              oracle/_ref (op::matmul with every transpose flag pair, with and without bias) bit-exact in
+ *                              fp32; fp64 closed form; (false, true) == oracle_linear
  *   oracle_softmax             reference KATs test/test_function.cpp:147-176; oracle/_ref (function::softmax /
  *                              logSoftmax, every axis) bit-exact in fp32; rows sum to 1
  */
@@ -113,6 +115,21 @@ void oracle_softmax(const float* x, float* out, int64_t outer, int64_t dim, int6
  * c[i][j] += a[i][p] * b[j][p] in i, p, j order, all in fp32; `dtype` rounds the result once (16-bit tensors: fp32
  * accumulation as in the device GEMM).  Pinned by the reference KAT test/test_function.cpp:234-241, bit-exact against
  * oracle/_ref (function::linear) in fp32, and the fp64 closed form. */
+/* reference src/Operation/OpLinalgCpu.h:119-150 (gemmCpuImpl, the in-tree loop): C = bias rows or zeros, then for i, p, j:
+ * c[i][j] += A(i,p) * B(p,j) with A(i,p) = transA ? a[p*m + i] : a[i*k + p], B(p,j) = transB ? b[j*k + p] : b[p*n + j]. */
+void oracle_matmul(const float* a, const float* b, const float* bias, float* out, int64_t M, int64_t N, int64_t K,
+                   int trans_a, int trans_b, int dtype) {
+  for (int64_t i = 0; i < M; i++)
+    for (int64_t j = 0; j < N; j++) out[i * N + j] = bias ? bias[j] : 0.f;
+  for (int64_t i = 0; i < M; i++)
+    for (int64_t p = 0; p < K; p++) {
+      const float av = trans_a ? a[p * M + i] : a[i * K + p];
+      for (int64_t j = 0; j < N; j++) out[i * N + j] += av * (trans_b ? b[j * K + p] : b[p * N + j]);
+    }
+  if (dtype != 0)
+    for (int64_t e = 0; e < M * N; e++) out[e] = round_t(out[e], dtype);
+}
+
 void oracle_linear(const float* x, const float* w, const float* bias, float* out, int64_t M, int64_t N, int64_t K,
                    int dtype) {
   for (int64_t i = 0; i < M; i++)

@@ -177,4 +177,19 @@ int tt_ref_linear(const float* x, const float* w, const float* bias, float* out,
   return 0;
 }
 
+int tt_ref_matmul(const float* a, const float* b, const float* bias, float* out, int64_t M, int64_t N, int64_t K,
+                  int transA, int transB) {
+  ensureCpu();
+  NoGradGuard guard;
+  Tensor tb;
+  if (bias) tb = fromF32(bias, {N});
+  Tensor ta = transA ? fromF32(a, {K, M}) : fromF32(a, {M, K});
+  Tensor tw = transB ? fromF32(b, {N, K}) : fromF32(b, {K, N});
+  Tensor y = op::matmul(ta, tw, transA != 0, transB != 0, tb);
+  auto r = y.toList<float>();
+  if (static_cast<int64_t>(r.size()) != M * N) return -2;
+  std::memcpy(out, r.data(), sizeof(float) * r.size());
+  return 0;
+}
+
 }  // extern "C"

@@ -118,3 +118,64 @@ def test_full_size_projection_properties():
     xf, wf, bf = x.float(), w.float(), b.float()
     yf = linear(xf, wf, bf)
     assert float((yf[rows, cols].double() - exact).abs().max()) <= 1e-4 * np.sqrt(K)
+
+
+MATMUL_CASES = [
+    # M, N, K, transA, transB, dtype, bias
+    (512, 384, 256, False, False, "bf16", False),   # input gradient of a linear layer: dy [M, N'] . w [N', K']
+    (384, 256, 512, True, False, "bf16", False),    # weight gradient: dy^T . x
+    (300, 260, 192, False, False, "f16", True),
+    (260, 192, 320, True, False, "f16", False),
+    (256, 128, 64, True, True, "bf16", True),
+    (300, 260, 160, False, False, "f32", True),     # fp32 on the fp32 matrix cores after the copies
+    (260, 96, 320, True, False, "f32", False),
+    (70, 90, 100, False, False, "f32", True),       # shapes the MFMA kernel does not take: read in place
+    (33, 47, 65, True, False, "bf16", True),
+    (5, 3, 2, True, True, "f32", False),
+    (64, 64, 64, False, True, "bf16", True),        # the linear layer's own form
+]
+
+
+@pytest.mark.parametrize("case", MATMUL_CASES, ids=lambda c: "M%dN%dK%d-tA%d-tB%d-%s-b%d" % c)
+def test_matmul_transpose_flags_against_oracle(case):
+    from tinytorch_amd import matmul
+    M, N, K, ta, tb, dtype, has_bias = case
+    say("matmul", case)
+    ah, ad = inputs(700 + M + K, 0, (K, M) if ta else (M, K), dtype)
+    bh, bd = inputs(700 + M + K, 1, (N, K) if tb else (K, N), dtype)
+    ch, cd = inputs(700 + M + K, 2, (N,), dtype) if has_bias else (None, None)
+    exp = oracle.matmul(ah, bh, ta, tb, ch, dtype)
+    y = to_host_f32(matmul(ad, bd, ta, tb, cd))
+    assert y.shape == exp.shape and np.isfinite(y).all()
+    scale = max(1.0, np.sqrt(K))
+    tol = 1e-4 * scale if dtype == "f32" else 2e-2 * scale
+    err = float(np.abs(y.astype(np.float64) - exp).max())
+    say("   max-abs-err", err, "tol", tol)
+    assert err <= tol
+    # without scratch the operands are read in place on the vector ALUs: the same result to the same bar
+    L = _capi.lib()
+    out = torch.empty(M, N, dtype=ad.dtype, device="cuda")
+    code = {"f32": _capi.F32, "f16": _capi.F16, "bf16": _capi.BF16}[dtype]
+    rc = L.ttlinear_matmul(code, ad.data_ptr(), bd.data_ptr(), cd.data_ptr() if cd is not None else None, out.data_ptr(),
+                           M, N, K, int(ta), int(tb), ad.stride(0), bd.stride(0), N, None, 0, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0
+    assert float(np.abs(to_host_f32(out).astype(np.float64) - exp).max()) <= tol
+
+
+def test_linear_backward_against_torch_autograd():
+    """FuncLinear::backward (reference src/Function/FuncNNLayer.h:20-33) at a projection's shape: grad . w, grad^T . x and
+    the column sums of grad, against torch's fp32 autograd on the same bf16 values."""
+    from tinytorch_amd import linearBackward
+    M, N, K = 2048, 1536, 1024
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(M, K, device="cuda", generator=gen).bfloat16()
+    w = (torch.randn(N, K, device="cuda", generator=gen) * K ** -0.5).bfloat16()
+    g = torch.randn(M, N, device="cuda", generator=gen).bfloat16()
+    xf, wf = x.float().requires_grad_(), w.float().requires_grad_()
+    bf = torch.zeros(N, device="cuda", requires_grad=True)
+    torch.nn.functional.linear(xf, wf, bf).backward(g.float())
+    gi, gw, gb = linearBackward(g, x, w)
+    for got, exp, k in ((gi, xf.grad, N), (gw, wf.grad, M), (gb, bf.grad, M)):
+        err = (got.float() - exp).abs().max().item()
+        assert err <= 2e-2 * max(1.0, k ** 0.5), err

@@ -131,3 +131,34 @@ def test_linear_known_answer_reference_and_closed_form(oracle_mod):
     wb, _ = o.round_to(w, "bf16")
     y16 = o.linear(xb, wb, None, "bf16")
     assert np.array_equal(y16, o.round_to(o.linear(xb, wb), "bf16")[0])
+
+
+def test_matmul_transpose_flags_reference_and_closed_form(oracle_mod):
+    """oracle_matmul with every transpose flag pair: bit-exact against the compiled reference's op::matmul (with and without
+    bias), the fp64 closed form, (False, True) == oracle_linear, and a wrong flag must change the answer."""
+    o = oracle_mod
+    r = rng(31)
+    for M, N, K in ((1, 1, 1), (5, 7, 3), (16, 16, 16), (33, 65, 129)):
+        for ta in (False, True):
+            for tb in (False, True):
+                a = r.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+                b = r.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+                bias = r.standard_normal(N).astype(np.float32)
+                y = o.matmul(a, b, ta, tb, bias)
+                A = a.T if ta else a
+                Bm = b.T if tb else b
+                ref64 = A.astype(np.float64) @ Bm.astype(np.float64) + bias
+                assert np.abs(y - ref64).max() < 1e-4 * max(1.0, np.sqrt(K)), (M, N, K, ta, tb)
+                assert np.abs(o.matmul(a, b, ta, tb) - (ref64 - bias)).max() < 1e-4 * max(1.0, np.sqrt(K))
+                if o.have_ref():
+                    assert np.array_equal(y, o.ref_matmul(a, b, ta, tb, bias)), (M, N, K, ta, tb)
+                    assert np.array_equal(o.matmul(a, b, ta, tb), o.ref_matmul(a, b, ta, tb))
+                if not ta and tb:
+                    assert np.array_equal(y, o.linear(a, b, bias))
+                if M == N == K and K > 1:   # square: the flags are not interchangeable
+                    assert np.abs(y - o.matmul(a, b, not ta, tb, bias)).max() > 0.1
+                    assert np.abs(y - o.matmul(a, b, ta, not tb, bias)).max() > 0.1
+    a16, _ = o.round_to(r.standard_normal((8, 12)).astype(np.float32), "bf16")
+    b16, _ = o.round_to(r.standard_normal((8, 20)).astype(np.float32), "bf16")
+    y16 = o.matmul(a16, b16, True, False, None, "bf16")
+    assert np.array_equal(y16, o.round_to(o.matmul(a16, b16, True, False), "bf16")[0])

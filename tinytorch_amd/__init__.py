@@ -9,7 +9,8 @@ from . import _capi
 _capi.lib()  # fail loudly when the extension is missing
 
 from .function import (sdpAttention, kvCacheAppend, build_params, rmsNorm, fusedAddRmsNorm, siluMul, softmax,  # noqa: E402
-                       logSoftmax, linear, sdpAttentionBackward, build_backward_params)
+                       logSoftmax, linear, sdpAttentionBackward, build_backward_params, matmul, linearBackward)
 
 __all__ = ["sdpAttention", "kvCacheAppend", "build_params", "rmsNorm", "fusedAddRmsNorm", "siluMul", "softmax",
-           "logSoftmax", "linear", "sdpAttentionBackward", "build_backward_params"]
+           "logSoftmax", "linear", "sdpAttentionBackward", "build_backward_params", "matmul",
+           "linearBackward"]

@@ -25,7 +25,7 @@ EXPORTS = [
     # include/ttfused.h
     "ttfused_rms_norm", "ttfused_add_rms_norm", "ttfused_silu_mul", "ttfused_softmax",
     # include/ttlinear.h
-    "ttlinear_forward", "ttlinear_plan",
+    "ttlinear_forward", "ttlinear_plan", "ttlinear_matmul", "ttlinear_matmul_workspace_bytes",
 ]
 LINEAR_ROUTE_NAMES = {0: "none", 1: "mfma", 2: "general"}
 
@@ -158,6 +158,11 @@ def lib():
         L.ttlinear_forward.restype = ctypes.c_int
         L.ttlinear_plan.argtypes = [ctypes.c_int, vp, vp, vp, vp] + [i64] * 6 + [ctypes.POINTER(ctypes.c_int)]
         L.ttlinear_plan.restype = ctypes.c_int
+        L.ttlinear_matmul_workspace_bytes.argtypes = [ctypes.c_int, i64, i64, i64, ctypes.c_int, ctypes.c_int]
+        L.ttlinear_matmul_workspace_bytes.restype = ctypes.c_size_t
+        L.ttlinear_matmul.argtypes = [ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, ctypes.c_int, ctypes.c_int, i64, i64, i64,
+                                      vp, ctypes.c_size_t, vp]
+        L.ttlinear_matmul.restype = ctypes.c_int
         if L.ttsdpa_abi_version() != 6:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L

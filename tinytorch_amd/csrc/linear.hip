@@ -29,6 +29,8 @@ struct LinArgs {
   const void* bias;
   void* out;
   long long M, N, K, ldx, ldw, ldo;
+  // general kernel only: x is stored [K, M] (x(m,k) = x[k*ldx + m]) / w is stored [K, N] (w(n,k) = w[k*ldw + n])
+  int xt = 0, wt = 0;
 };
 
 typedef __attribute__((address_space(3))) void lds_void_t;
@@ -252,8 +254,10 @@ __global__ __launch_bounds__(256) void linear_general_kernel(LinArgs a) {
       const int e = tid + 256 * i;
       const int row = e >> 4, kk = e & 15;
       const bool kin = k0 + kk < a.K;
-      Xs[kk][row] = (kin && m0 + row < a.M) ? load_as_float(x + (m0 + row) * a.ldx + k0 + kk) : 0.f;
-      Ws[kk][row] = (kin && n0 + row < a.N) ? load_as_float(w + (n0 + row) * a.ldw + k0 + kk) : 0.f;
+      const long long xat = a.xt ? (k0 + kk) * a.ldx + m0 + row : (m0 + row) * a.ldx + k0 + kk;
+      const long long wat = a.wt ? (k0 + kk) * a.ldw + n0 + row : (n0 + row) * a.ldw + k0 + kk;
+      Xs[kk][row] = (kin && m0 + row < a.M) ? load_as_float(x + xat) : 0.f;
+      Ws[kk][row] = (kin && n0 + row < a.N) ? load_as_float(w + wat) : 0.f;
     }
     __syncthreads();
 #pragma unroll
@@ -277,6 +281,33 @@ __global__ __launch_bounds__(256) void linear_general_kernel(LinArgs a) {
       if (n < a.N) store_from_float((T*)a.out + m * a.ldo + n, acc[i][j]);
     }
   }
+}
+
+// dst[c, r] = src[r, c] for src [R, C] with row stride ld; dst dense [C, R].  64 x 64 tiles through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* src, T* dst, long long R, long long C, long long ld) {
+  __shared__ T tile[64][64 + 2];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const long long r0 = (long long)blockIdx.y * 64, c0 = (long long)blockIdx.x * 64;
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    const long long r = r0 + ty + 4 * i, c = c0 + tx;
+    if (r < R && c < C) tile[ty + 4 * i][tx] = src[r * ld + c];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    const long long c = c0 + ty + 4 * i, r = r0 + tx;
+    if (r < R && c < C) dst[c * R + r] = tile[tx][ty + 4 * i];
+  }
+}
+
+template <typename T>
+int launch_transpose(const void* src, void* dst, long long R, long long C, long long ld, hipStream_t stream) {
+  if ((R + 63) / 64 > 65535 || (C + 63) / 64 > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
+  dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64));
+  hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, stream, (const T*)src, (T*)dst, R, C, ld);
+  return (int)hipGetLastError();
 }
 
 bool aligned(const void* p, size_t n) { return ((uintptr_t)p % n) == 0; }
@@ -362,6 +393,67 @@ int ttlinear_forward(int dtype, const void* x, const void* w, const void* bias, 
     case TTSDPA_F32: return launch_general_linear<float>(a, s);
     case TTSDPA_F16: return launch_general_linear<_Float16>(a, s);
     default: return launch_general_linear<__bf16>(a, s);
+  }
+}
+
+// Bytes of the dense transposed copies the MFMA route of ttlinear_matmul makes: a as [M, K] when it is stored [K, M],
+// b as [N, K] when it is stored [K, N]; each rounded up to 256 bytes.
+static size_t matmul_copy_bytes(int dtype, int64_t rows, int64_t K) {
+  const size_t esz = dtype == TTSDPA_F32 ? 4 : 2;
+  return ((size_t)rows * (size_t)K * esz + 255) / 256 * 256;
+}
+
+size_t ttlinear_matmul_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  return (trans_a ? matmul_copy_bytes(dtype, M, K) : 0) + (!trans_b ? matmul_copy_bytes(dtype, N, K) : 0);
+}
+
+int ttlinear_matmul(int dtype, const void* a, const void* b, const void* bias, void* out, int64_t M, int64_t N, int64_t K,
+                    int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldo, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  if (!trans_a && trans_b) return ttlinear_forward(dtype, a, b, bias, out, M, N, K, lda, ldb, ldo, stream);
+  if (dtype != TTSDPA_F32 && dtype != TTSDPA_F16 && dtype != TTSDPA_BF16) return TTSDPA_ERR_DTYPE;
+  if (M < 0 || N < 0 || K < 0) return TTSDPA_ERR_SHAPE;
+  if (M == 0 || N == 0) return TTSDPA_OK;
+  if (!out || (K > 0 && (!a || !b))) return TTSDPA_ERR_NULL;
+  if (lda < (trans_a ? M : K) || ldb < (trans_b ? K : N) || ldo < N) return TTSDPA_ERR_STRIDE;
+  const size_t esz = dtype == TTSDPA_F32 ? 4 : 2;
+  if (!aligned(a, esz) || !aligned(b, esz) || !aligned(out, esz) || (bias && !aligned(bias, esz))) return TTSDPA_ERR_STRIDE;
+  if ((M + 63) / 64 > 65535 || (N + 63) / 64 > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+
+  // MFMA route: dense row-major copies of the operands that are stored contraction-major, then the x . w^T kernel
+  const size_t need = ttlinear_matmul_workspace_bytes(dtype, M, N, K, trans_a, trans_b);
+  if (K > 0 && workspace && workspace_bytes >= need && aligned(workspace, 256)) {
+    const void* x = a;
+    const void* w = b;
+    long long ldx = lda, ldw = ldb;
+    char* ws = (char*)workspace;
+    int route = TTLINEAR_ROUTE_NONE;
+    const void* xprobe = trans_a ? (const void*)ws : a;
+    const void* wprobe = !trans_b ? (const void*)(ws + (trans_a ? matmul_copy_bytes(dtype, M, K) : 0)) : b;
+    if (check(dtype, xprobe, wprobe, out, M, N, K, trans_a ? K : lda, !trans_b ? K : ldb, ldo, &route) == TTSDPA_OK &&
+        route == TTLINEAR_ROUTE_MFMA) {
+      int rc = 0;
+      if (trans_a) {  // a is [K, M]
+        rc = dtype == TTSDPA_F32 ? launch_transpose<float>(a, ws, K, M, lda, s) : launch_transpose<uint16_t>(a, ws, K, M, lda, s);
+        if (rc != 0) return rc;
+        x = ws, ldx = K;
+        ws += matmul_copy_bytes(dtype, M, K);
+      }
+      if (!trans_b) {  // b is [K, N]
+        rc = dtype == TTSDPA_F32 ? launch_transpose<float>(b, ws, K, N, ldb, s) : launch_transpose<uint16_t>(b, ws, K, N, ldb, s);
+        if (rc != 0) return rc;
+        w = ws, ldw = K;
+      }
+      return ttlinear_forward(dtype, x, w, bias, out, M, N, K, ldx, ldw, ldo, stream);
+    }
+  }
+  LinArgs g{a, b, bias, out, M, N, K, lda, ldb, ldo, trans_a ? 1 : 0, trans_b ? 0 : 1};
+  switch (dtype) {
+    case TTSDPA_F32: return launch_general_linear<float>(g, s);
+    case TTSDPA_F16: return launch_general_linear<_Float16>(g, s);
+    default: return launch_general_linear<__bf16>(g, s);
   }
 }
 

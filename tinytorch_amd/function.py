@@ -358,3 +358,47 @@ def linear(input, weight, bias=None):
             b.data_ptr() if b is not None else None, out.data_ptr(), M, N, K,
             x.stride(0) if M > 1 else max(K, 1), w.stride(0) if N > 1 else max(K, 1), N)
     return out.reshape(input.shape[:-1] + (N,))
+
+
+def matmul(a, b, transA=False, transB=False, bias=None):
+    """op(a) . op(b) + bias for 2-D tensors with the reference's transpose flags (op::matmul, reference
+    src/Operation/OpLinalg.cpp:244-276): a is [M, K], or [K, M] with transA; b is [K, N], or [N, K] with transB.
+    (False, True) is the linear layer; (False, False) and (True, False) are what FuncLinear::backward calls for the
+    input and the weight gradient (reference src/Function/FuncNNLayer.h:20-33)."""
+    _check_rowwise("matmul", a, b, bias)
+    if a.dim() != 2 or b.dim() != 2:
+        raise ValueError("matmul: expected 2-D tensors")
+    K, M = a.shape if transA else (a.shape[1], a.shape[0])
+    Kb, N = (b.shape[1], b.shape[0]) if transB else b.shape
+    if K != Kb:
+        raise ValueError("matmul: inner sizes differ: %s (transA=%s), %s (transB=%s)" % (tuple(a.shape), transA, tuple(b.shape), transB))
+    if bias is not None and tuple(bias.shape) != (N,):
+        raise ValueError("matmul: bias must have shape [%d]" % N)
+    a = a if (a.stride(-1) == 1 or a.shape[-1] == 1) else a.contiguous()
+    b = b if (b.stride(-1) == 1 or b.shape[-1] == 1) else b.contiguous()
+    bs = bias.contiguous() if bias is not None else None
+    out = torch.empty(M, N, dtype=a.dtype, device=a.device)
+    L = _capi.lib()
+    nbytes = L.ttlinear_matmul_workspace_bytes(_DTYPES[a.dtype], M, N, K, int(transA), int(transB))
+    ws = _workspace(a.device, nbytes) if nbytes else None
+    lda = a.stride(0) if a.shape[0] > 1 else max(a.shape[1], 1)
+    ldb = b.stride(0) if b.shape[0] > 1 else max(b.shape[1], 1)
+    with torch.cuda.device(a.device):
+        rc = L.ttlinear_matmul(_DTYPES[a.dtype], a.data_ptr(), b.data_ptr(), bs.data_ptr() if bs is not None else None,
+                               out.data_ptr(), M, N, K, int(transA), int(transB), lda, ldb, N,
+                               ws.data_ptr() if ws is not None else None, nbytes, torch.cuda.current_stream().cuda_stream)
+    if rc != 0:
+        raise RuntimeError("ttlinear_matmul failed: %d (%s)" % (rc, _capi.status_string(rc)))
+    return out
+
+
+def linearBackward(gradOut, input, weight, needBias=True):
+    """(gradInput, gradWeight, gradBias) of linear(input, weight, bias) — FuncLinear::backward (reference
+    src/Function/FuncNNLayer.h:20-33): grad . weight, grad^T . input, and the column sums of grad."""
+    N, K = weight.shape
+    g = gradOut.reshape(-1, N)
+    x = input.reshape(-1, K)
+    gi = matmul(g, weight, False, False).reshape(input.shape)
+    gw = matmul(g, x, True, False)
+    gb = g.float().sum(dim=0).to(g.dtype) if needBias else None   # the reference's op::sumOnDim(grad, 0)
+    return gi, gw, gb
