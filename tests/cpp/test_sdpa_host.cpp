@@ -362,6 +362,36 @@ static void test_backward() {
   y.gradFn()->backward(tgo);
   EXPECT_TRUE(g_asserts > before);
   setAssertHandler(old);
+
+  // FuncLinear::backward (reference src/Function/FuncNNLayer.h:20-33): grad . w, grad^T . x, column sums of grad
+  {
+    const int M = 6, N = 5, K = 7;
+    std::vector<float> x = pseudoRandom(static_cast<size_t>(M) * K, 81), w = pseudoRandom(static_cast<size_t>(N) * K, 82),
+                       bb = pseudoRandom(N, 83), g = pseudoRandom(static_cast<size_t>(M) * N, 84);
+    Tensor tx(x, {M, K}, gpu), tw(w, {N, K}, gpu), tb(bb, {N}, gpu), tg(g, {M, N}, gpu);
+    tx.setRequiresGrad(true), tw.setRequiresGrad(true), tb.setRequiresGrad(true);
+    Tensor out = function::linear(tx, tw, tb);
+    out.gradFn()->backward(tg);
+    std::vector<float> gx = tx.grad().toList<float>(), gw = tw.grad().toList<float>(), gb = tb.grad().toList<float>();
+    bool good = gx.size() == x.size() && gw.size() == w.size() && gb.size() == bb.size();
+    for (int m = 0; good && m < M; m++)
+      for (int k = 0; k < K; k++) {
+        double s = 0;
+        for (int n = 0; n < N; n++) s += static_cast<double>(g[m * N + n]) * w[n * K + k];
+        good = good && std::fabs(gx[m * K + k] - s) < 1e-4;
+      }
+    for (int n = 0; good && n < N; n++) {
+      double sb = 0;
+      for (int m = 0; m < M; m++) sb += g[m * N + n];
+      good = good && std::fabs(gb[n] - sb) < 1e-4;
+      for (int k = 0; k < K; k++) {
+        double s = 0;
+        for (int m = 0; m < M; m++) s += static_cast<double>(g[m * N + n]) * x[m * K + k];
+        good = good && std::fabs(gw[n * K + k] - s) < 1e-4;
+      }
+    }
+    EXPECT_TRUE(good);
+  }
 }
 
 static void test_grad_bookkeeping_and_errors() {

@@ -50,8 +50,9 @@ class FuncSoftmaxT : public Function<FuncSoftmaxT<LOG>> {
   }
 };
 
-// function::linear (reference src/Function/FuncNNLayer.h:14-36, 270-272): forward is the reference's single op call;
-// the backward (three more matmul forms) is not part of this inference path.
+// function::linear (reference src/Function/FuncNNLayer.h:14-36, 270-272): forward is the reference's single op call,
+// backward its three: grad . weight, grad^T . input and the column sums of grad (here: ones[1, M] . grad, this layer
+// having no reduction op).
 class FuncLinear : public Function<FuncLinear> {
  public:
   static Tensor forward(AutogradContext* ctx, const Tensor& input, const Tensor& weight, const Tensor& bias) {
@@ -59,8 +60,22 @@ class FuncLinear : public Function<FuncLinear> {
     return op::matmul(input, weight, false, true, bias);
   }
   static void backward(AutogradContext* ctx, const Tensor& grad) {
-    (void)ctx, (void)grad;
-    NOT_IMPLEMENTED();
+    ASSERT(ctx && ctx->savedInputs.size() >= 2);
+    if (!ctx || ctx->savedInputs.size() < 2) return;
+    Tensor& input = ctx->savedInputs[0];
+    Tensor& weight = ctx->savedInputs[1];
+    if (input.requiresGrad()) input.addGrad(op::matmul(grad, weight, false, false, Tensor{}));
+    const int64_t N = weight.size(0), K = weight.size(1);
+    Tensor g2 = grad.detach(), x2 = input.detach();  // [M, N] and [M, K] views of the same storage
+    g2.reshape_({-1, N});
+    x2.reshape_({-1, K});
+    if (weight.requiresGrad()) weight.addGrad(op::matmul(g2, x2, true, false, Tensor{}));
+    if (ctx->savedInputs.size() > 2 && ctx->savedInputs[2].requiresGrad()) {
+      Tensor ones = Tensor::ones({1, g2.size(0)}, g2.options().noGrad());
+      Tensor gb = op::matmul(ones, g2, false, false, Tensor{});
+      gb.reshape_({N});
+      ctx->savedInputs[2].addGrad(std::move(gb));
+    }
   }
 };
 

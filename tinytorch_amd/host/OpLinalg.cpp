@@ -8,9 +8,53 @@ namespace tinytorch::op {
 
 namespace {
 
+// The other transpose flag pairs of op::matmul for 2-D operands (reference src/Operation/OpLinalgCpu.h:119-150): a is
+// [M, K], or [K, M] with transA; b is [K, N], or [N, K] with transB.  The first operand may carry leading batch axes when
+// it is not transposed (they are part of M).
+Tensor matmulFlagsGpuImpl(const Tensor& a, const Tensor& b, bool transA, bool transB, const Tensor& bias) {
+  ASSERT(a.dim() >= 2 && b.dim() == 2 && (!transA || a.dim() == 2));
+  ASSERT(b.dtype() == a.dtype() && b.device() == a.device());
+  if (a.dim() < 2 || b.dim() != 2 || (transA && a.dim() != 2) || b.dtype() != a.dtype()) return {};
+  const int64_t K = transA ? a.size(0) : a.size(-1);
+  const int64_t N = transB ? b.size(0) : b.size(1);
+  ASSERT((transB ? b.size(1) : b.size(0)) == K);
+  if ((transB ? b.size(1) : b.size(0)) != K) return {};
+  if (bias.defined()) {
+    ASSERT(bias.dim() == 1 && bias.size(0) == N && bias.dtype() == a.dtype());
+    if (bias.dim() != 1 || bias.size(0) != N || bias.dtype() != a.dtype()) return {};
+  }
+  std::vector<int64_t> shape;
+  int64_t M = 1;
+  if (transA) {
+    M = a.size(1);
+    shape = {M, N};
+  } else {
+    shape = a.shape();
+    shape.back() = N;
+    for (size_t i = 0; i + 1 < shape.size(); i++) M *= shape[i];
+  }
+  Tensor out = Tensor::empty(shape, a.options().noGrad());
+  const int dtype = a.dtype() == DType::Float32 ? TTSDPA_F32 : a.dtype() == DType::Float16 ? TTSDPA_F16 : TTSDPA_BF16;
+  const DeviceIndex dev = a.device().index;
+  HIP_CHECK(hipSetDevice(dev));
+  const size_t wsBytes = ttlinear_matmul_workspace_bytes(dtype, M, N, K, transA, transB);
+  std::shared_ptr<Storage> ws;  // back to the allocator's cache on scope exit; the stream orders its reuse
+  if (wsBytes) ws = std::make_shared<Storage>(wsBytes, a.device());
+  const int rc = ttlinear_matmul(dtype, a.rawPtr(), b.rawPtr(), bias.defined() ? bias.rawPtr() : nullptr, out.rawPtr(), M, N, K,
+                                 transA, transB, transA ? M : K, transB ? K : N, N, ws ? ws->data() : nullptr, wsBytes,
+                                 getCurrentStream(dev));
+  if (rc != TTSDPA_OK) {
+    LOGE("ttlinear_matmul failed: %d (%s)", rc, ttsdpa_status_string(rc));
+    ASSERT(rc == TTSDPA_OK);
+    return {};
+  }
+  return out;
+}
+
 Tensor matmulGpuImpl(const Tensor& a, const Tensor& b, bool transA, bool transB, const Tensor& bias) {
   ASSERT(a.defined() && b.defined());
-  ASSERT(!transA && transB);  // the linear layer's call; the reference's other flag combinations are not built here
+  if (!a.defined() || !b.defined()) return {};
+  if (transA || !transB) return matmulFlagsGpuImpl(a, b, transA, transB, bias);
   ASSERT(a.dim() >= 1 && b.dim() == 2 && a.size(-1) == b.size(1));
   ASSERT(b.dtype() == a.dtype() && b.device() == a.device());
   if (!a.defined() || !b.defined() || transA || !transB || a.dim() < 1 || b.dim() != 2 || a.size(-1) != b.size(1) ||

@@ -8,7 +8,9 @@
 
 namespace tinytorch::op {
 
-// a [..., K], b [N, K] with transA == false, transB == true; bias undefined or [N].  Returns [..., N].
+// a [..., K], b [N, K] with transA == false, transB == true (the linear layer); bias undefined or [N].  Returns [..., N].
+// The other flag pairs take 2-D operands: a [M, K] ([K, M] with transA; leading batch axes allowed without it), b [K, N]
+// ([N, K] with transB).
 using MatmulOpFn = Tensor (*)(const Tensor& a, const Tensor& b, bool transA, bool transB, const Tensor& bias);
 
 DEFINE_OP(matmul, MatmulOpFn)
