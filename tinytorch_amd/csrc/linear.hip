@@ -283,22 +283,47 @@ __global__ __launch_bounds__(256) void linear_general_kernel(LinArgs a) {
   }
 }
 
-// dst[c, r] = src[r, c] for src [R, C] with row stride ld; dst dense [C, R].  64 x 64 tiles through LDS.
-template <typename T>
+// dst[c, r] = src[r, c] for src [R, C] with row stride ld; dst dense [C, R].  64 x 64 tiles through LDS, 16 bytes per
+// global access where the row lengths allow it (VECOK: ld and R multiples of 16 bytes, both pointers 16-byte aligned).
+template <typename T, bool VECOK>
 __global__ __launch_bounds__(256) void transpose_kernel(const T* src, T* dst, long long R, long long C, long long ld) {
-  __shared__ T tile[64][64 + 2];
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int PITCH = 64 + VEC;  // rows stay 16-byte aligned
+  typedef T vecT __attribute__((ext_vector_type(VEC)));
+  __shared__ __attribute__((aligned(16))) T tile[64][PITCH];
   const long long r0 = (long long)blockIdx.y * 64, c0 = (long long)blockIdx.x * 64;
+  constexpr int CPR = 64 / VEC;  // 16-byte chunks per tile row
 #pragma unroll
-  for (int i = 0; i < 16; i++) {
-    const long long r = r0 + ty + 4 * i, c = c0 + tx;
-    if (r < R && c < C) tile[ty + 4 * i][tx] = src[r * ld + c];
+  for (int i = 0; i < 64 * CPR / 256; i++) {
+    const int chunk = threadIdx.x + 256 * i;
+    const int row = chunk / CPR, cc = (chunk % CPR) * VEC;
+    const long long r = r0 + row, c = c0 + cc;
+    if (r >= R) continue;
+    if (VECOK && c + VEC <= C) {
+      *(vecT*)&tile[row][cc] = *(const vecT*)(src + r * ld + c);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; e++)
+        if (c + e < C) tile[row][cc + e] = src[r * ld + c + e];
+    }
   }
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 16; i++) {
-    const long long c = c0 + ty + 4 * i, r = r0 + tx;
-    if (r < R && c < C) dst[c * R + r] = tile[tx][ty + 4 * i];
+  for (int i = 0; i < 64 * CPR / 256; i++) {
+    const int chunk = threadIdx.x + 256 * i;
+    const int orow = chunk / CPR, oc = (chunk % CPR) * VEC;  // output row = source column; first of VEC source rows
+    const long long c = c0 + orow, r = r0 + oc;
+    if (c >= C) continue;
+    if (VECOK && r + VEC <= R) {
+      vecT v;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) v[e] = tile[oc + e][orow];
+      *(vecT*)(dst + c * R + r) = v;
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; e++)
+        if (r + e < R) dst[c * R + r + e] = tile[oc + e][orow];
+    }
   }
 }
 
@@ -306,7 +331,13 @@ template <typename T>
 int launch_transpose(const void* src, void* dst, long long R, long long C, long long ld, hipStream_t stream) {
   if ((R + 63) / 64 > 65535 || (C + 63) / 64 > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
   dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64));
-  hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, stream, (const T*)src, (T*)dst, R, C, ld);
+  constexpr long long VEC = 16 / sizeof(T);
+  const bool vecok = ld % VEC == 0 && R % VEC == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)dst % 16) == 0;
+  if (vecok) {
+    hipLaunchKernelGGL((transpose_kernel<T, true>), grid, dim3(256), 0, stream, (const T*)src, (T*)dst, R, C, ld);
+  } else {
+    hipLaunchKernelGGL((transpose_kernel<T, false>), grid, dim3(256), 0, stream, (const T*)src, (T*)dst, R, C, ld);
+  }
   return (int)hipGetLastError();
 }
 
