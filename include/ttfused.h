@@ -47,6 +47,15 @@ int ttfused_silu_mul(int dtype, const void* x, void* out, int64_t rows, int64_t 
 int ttfused_softmax(int dtype, const void* x, void* out, int64_t outer, int64_t dim, int64_t inner, int log_form,
                     void* stream);
 
+/* Backward of softmax / logSoftmax over the same [outer, dim, inner] view (reference op::softmaxBackward /
+ * op::logSoftmaxBackward, src/Operation/OpNNLayerCpu.h:79-109, 123-150; called by FuncSoftmax / FuncLogSoftmax::backward,
+ * src/Function/FuncActivation.h:53-61, 76-84): from the upstream gradient `grad` and the forward's `output`,
+ *   softmax:    out_j = output_j * (grad_j - sum_t output_t * grad_t)
+ *   logSoftmax: out_j = grad_j - exp(output_j) * sum_t grad_t
+ * with the sums in fp32 and one rounding of the result.  out may alias grad. */
+int ttfused_softmax_backward(int dtype, const void* grad, const void* output, void* out, int64_t outer, int64_t dim,
+                             int64_t inner, int log_form, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -64,6 +64,8 @@ def lib():
         L.oracle_silu_mul.restype = None
         L.oracle_softmax.argtypes = [_c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int]
         L.oracle_softmax.restype = None
+        L.oracle_softmax_backward.argtypes = [_c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int]
+        L.oracle_softmax_backward.restype = None
         L.oracle_linear.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int]
         L.oracle_linear.restype = None
         L.oracle_matmul.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int, ctypes.c_int]
@@ -96,6 +98,8 @@ def ref():
         R.tt_ref_silu_mul.restype = ctypes.c_int
         R.tt_ref_softmax.argtypes = [_c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int]
         R.tt_ref_softmax.restype = ctypes.c_int
+        R.tt_ref_softmax_backward.argtypes = [_c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int]
+        R.tt_ref_softmax_backward.restype = ctypes.c_int
         R.tt_ref_linear.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64]
         R.tt_ref_linear.restype = ctypes.c_int
         R.tt_ref_matmul.argtypes = [_c_f32p, _c_f32p, _c_f32p, _c_f32p, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int]
@@ -314,6 +318,25 @@ def softmax(x, dim=-1, log=False, dtype="f32"):
     out = np.empty_like(x)
     outer, n, inner = _softmax_dims(x.shape, dim)
     lib().oracle_softmax(_p(x), _p(out), outer, n, inner, int(log), _dt(dtype))
+    return out
+
+
+def softmax_backward(grad, output, dim=-1, log=False, dtype="f32"):
+    """Gradient of softmax / logSoftmax along `dim` from the upstream gradient and the forward's output."""
+    g, y = _f32(grad), _f32(output)
+    assert g.shape == y.shape
+    out = np.empty_like(g)
+    outer, n, inner = _softmax_dims(g.shape, dim)
+    lib().oracle_softmax_backward(_p(g), _p(y), _p(out), outer, n, inner, int(log), _dt(dtype))
+    return out
+
+
+def ref_softmax_backward(grad, output, dim=-1, log=False):
+    g, y = _f32(grad), _f32(output)
+    out = np.empty_like(g)
+    outer, n, inner = _softmax_dims(g.shape, dim)
+    rc = ref().tt_ref_softmax_backward(_p(g), _p(y), _p(out), outer, n, inner, int(log))
+    assert rc == 0
     return out
 
 

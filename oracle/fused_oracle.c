@@ -17,6 +17,8 @@
  *                              (op::siluMul) bit-exact in fp32
  *   oracle_linear              reference KAT test/test_function.cpp:234-241; oracle/_ref (function::linear) bit-exact
  *                              in fp32; fp64 closed form
+ *   oracle_softmax_backward    oracle/_ref (op::softmaxBackward / op::logSoftmaxBackward, every axis) bit-exact in fp32;
+ *                              central differences of the fp64 forward; rows of the softmax gradient sum to 0
  *   oracle_matmul              oracle/_ref (op::matmul with every transpose flag pair, with and without bias) bit-exact in
  *                              fp32; fp64 closed form; (false, true) == oracle_linear
  *   oracle_softmax             reference KATs test/test_function.cpp:147-176; oracle/_ref (function::softmax /
@@ -115,6 +117,23 @@ void oracle_softmax(const float* x, float* out, int64_t outer, int64_t dim, int6
  * c[i][j] += a[i][p] * b[j][p] in i, p, j order, all in fp32; `dtype` rounds the result once (16-bit tensors: fp32
  * accumulation as in the device GEMM).  Pinned by the reference KAT test/test_function.cpp:234-241, bit-exact against
  * oracle/_ref (function::linear) in fp32, and the fp64 closed form. */
+/* reference src/Operation/OpNNLayerCpu.h:79-109 (softmax) and 123-150 (logSoftmax): sequential fp32 sum over the axis,
+ * then out = y * (g - sum)  /  out = g - expf(y) * sum.  16-bit: float arithmetic on the rounded inputs, one rounding. */
+void oracle_softmax_backward(const float* g, const float* y, float* out, int64_t outer, int64_t dim, int64_t inner,
+                             int log_form, int dtype) {
+  for (int64_t o = 0; o < outer; o++)
+    for (int64_t i = 0; i < inner; i++) {
+      const int64_t base = o * dim * inner + i;
+      float sum = 0.f;
+      for (int64_t d = 0; d < dim; d++) sum += log_form ? g[base + d * inner] : y[base + d * inner] * g[base + d * inner];
+      for (int64_t d = 0; d < dim; d++) {
+        const int64_t at = base + d * inner;
+        const float v = log_form ? g[at] - expf(y[at]) * sum : y[at] * (g[at] - sum);
+        out[at] = round_t(v, dtype);
+      }
+    }
+}
+
 /* reference src/Operation/OpLinalgCpu.h:119-150 (gemmCpuImpl, the in-tree loop): C = bias rows or zeros, then for i, p, j:
  * c[i][j] += A(i,p) * B(p,j) with A(i,p) = transA ? a[p*m + i] : a[i*k + p], B(p,j) = transB ? b[j*k + p] : b[p*n + j]. */
 void oracle_matmul(const float* a, const float* b, const float* bias, float* out, int64_t M, int64_t N, int64_t K,

@@ -164,6 +164,19 @@ int tt_ref_softmax(const float* x, float* out, int64_t outer, int64_t dim, int64
   return 0;
 }
 
+// op::softmaxBackward / op::logSoftmaxBackward (reference src/Operation/OpNNLayer.h:46-51) over axis 1 of [outer, dim, inner].
+int tt_ref_softmax_backward(const float* g, const float* y, float* out, int64_t outer, int64_t dim, int64_t inner,
+                            int log_form) {
+  ensureCpu();
+  NoGradGuard guard;
+  Tensor tg = fromF32(g, {outer, dim, inner}), ty = fromF32(y, {outer, dim, inner});
+  Tensor r = log_form ? op::logSoftmaxBackward(tg, ty, 1) : op::softmaxBackward(tg, ty, 1);
+  auto v = r.toList<float>();
+  if (static_cast<int64_t>(v.size()) != outer * dim * inner) return -2;
+  std::memcpy(out, v.data(), sizeof(float) * v.size());
+  return 0;
+}
+
 // function::linear (reference src/Function/FuncNNLayer.h:270-272): x [M,K], w [N,K], bias [N] or NULL -> out [M,N].
 int tt_ref_linear(const float* x, const float* w, const float* bias, float* out, int64_t M, int64_t N, int64_t K) {
   ensureCpu();

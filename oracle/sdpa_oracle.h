@@ -78,6 +78,9 @@ void oracle_softmax(const float* x, float* out, int64_t outer, int64_t dim, int6
 /* out[M,N] = bias[N] (or 0) + x[M,K] . w[N,K]^T, the reference's gemm loop order. */
 void oracle_linear(const float* x, const float* w, const float* bias, float* out, int64_t M, int64_t N, int64_t K,
                    int dtype);
+/* softmax / logSoftmax backward over [outer, dim, inner] from the upstream gradient g and the forward's output y. */
+void oracle_softmax_backward(const float* g, const float* y, float* out, int64_t outer, int64_t dim, int64_t inner,
+                             int log_form, int dtype);
 /* out[M,N] = bias[N] (or 0) + op(a) . op(b): a is [M,K], or [K,M] with trans_a; b is [K,N], or [N,K] with trans_b. */
 void oracle_matmul(const float* a, const float* b, const float* bias, float* out, int64_t M, int64_t N, int64_t K,
                    int trans_a, int trans_b, int dtype);

@@ -363,6 +363,29 @@ static void test_backward() {
   EXPECT_TRUE(g_asserts > before);
   setAssertHandler(old);
 
+  // FuncSoftmax / FuncLogSoftmax::backward (reference src/Function/FuncActivation.h:53-61, 76-84) against the formulas
+  {
+    std::vector<float> x = pseudoRandom(3 * 5, 91), g = pseudoRandom(3 * 5, 92);
+    for (int logForm = 0; logForm < 2; logForm++) {
+      Tensor tx(x, {3, 5}, gpu), tg(g, {3, 5}, gpu);
+      tx.setRequiresGrad(true);
+      Tensor out = logForm ? function::logSoftmax(tx, -1) : function::softmax(tx, -1);
+      std::vector<float> yv = out.toList<float>();
+      out.gradFn()->backward(tg);
+      std::vector<float> dx = tx.grad().toList<float>();
+      bool good = dx.size() == x.size();
+      for (int r = 0; good && r < 3; r++) {
+        double s = 0;
+        for (int j = 0; j < 5; j++) s += logForm ? g[r * 5 + j] : static_cast<double>(yv[r * 5 + j]) * g[r * 5 + j];
+        for (int j = 0; j < 5; j++) {
+          const double e = logForm ? g[r * 5 + j] - std::exp(static_cast<double>(yv[r * 5 + j])) * s : yv[r * 5 + j] * (g[r * 5 + j] - s);
+          good = good && std::fabs(dx[r * 5 + j] - e) < 1e-5;
+        }
+      }
+      EXPECT_TRUE(good);
+    }
+  }
+
   // FuncLinear::backward (reference src/Function/FuncNNLayer.h:20-33): grad . w, grad^T . x, column sums of grad
   {
     const int M = 6, N = 5, K = 7;

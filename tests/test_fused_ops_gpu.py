@@ -92,6 +92,29 @@ def test_softmax_and_log_softmax(shape, dim, dtype):
     assert (np.abs(yl - el) <= tol).all()
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("shape,dim", [((4,), 0), ((3, 7), -1), ((3, 7), 0), ((64, 1000), 1), ((5, 32000), -1),
+                                       ((4, 9, 6), 1), ((2, 3, 300, 64), 2), ((8, 4096), 1), ((6, 128, 33), 1)])
+def test_softmax_backward(shape, dim, dtype):
+    """op::softmaxBackward / op::logSoftmaxBackward (reference src/Operation/OpNNLayerCpu.h:79-150) from the same rounded
+    gradient and forward output the oracle sees.  The sums run over up to 32000 terms in another order than the oracle's
+    left-to-right loop: the bar is the forward's, widened by the size of the terms that cancel in (g - sum)."""
+    from tinytorch_amd import logSoftmaxBackward, softmaxBackward
+    say("softmax backward", shape, dim, dtype)
+    xh, _ = inputs(450 + sum(shape), 0, shape, dtype, 2.0)
+    gh, gd = inputs(450 + sum(shape), 1, shape, dtype)
+    for log, fn in ((False, softmaxBackward), (True, logSoftmaxBackward)):
+        yh, yb = oracle.round_to(oracle.softmax(xh, dim, log), dtype)
+        yd = to_device(yh, yb, dtype)
+        exp = oracle.softmax_backward(gh, yh, dim, log, dtype)
+        got = to_host_f32(fn(gd, yd, dim))
+        assert got.shape == exp.shape and np.isfinite(got).all()
+        n = shape[dim]
+        scale = np.abs(gh).max() * (np.sqrt(n) if log else 1.0)   # |sum| the result is a difference against
+        tol = (1e-4 if dtype == "f32" else 1.01 * ULP[dtype] * np.abs(exp)) + 1e-5 * max(1.0, scale)
+        assert (np.abs(got.astype(np.float64) - exp) <= tol).all(), (log, float(np.abs(got - exp).max()))
+
+
 def test_reference_known_answers_on_the_gpu():
     """reference test/test_function.cpp:147-152, 385-391 through the HIP kernels."""
     x = torch.tensor([[1.4176, 0.1874, 0.8367], [-0.1203, 2.5638, -1.2554]], device="cuda")

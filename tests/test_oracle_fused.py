@@ -162,3 +162,42 @@ def test_matmul_transpose_flags_reference_and_closed_form(oracle_mod):
     b16, _ = o.round_to(r.standard_normal((8, 20)).astype(np.float32), "bf16")
     y16 = o.matmul(a16, b16, True, False, None, "bf16")
     assert np.array_equal(y16, o.round_to(o.matmul(a16, b16, True, False), "bf16")[0])
+
+
+def test_softmax_backward_reference_and_differences(oracle_mod):
+    """oracle_softmax_backward: bit-exact against the compiled reference's op::softmaxBackward / op::logSoftmaxBackward on
+    every axis; central differences of a float64 forward; the softmax gradient sums to 0 along the axis."""
+    o = oracle_mod
+    r = rng(41)
+    for shape, dim in (((5, 7), 1), ((4, 6, 3), 1), ((3, 4, 5), 0), ((2, 3, 4, 5), 2), ((6, 33), -1)):
+        x = r.standard_normal(shape).astype(np.float32)
+        g = r.standard_normal(shape).astype(np.float32)
+        for log in (False, True):
+            y = o.softmax(x, dim, log)
+            d = o.softmax_backward(g, y, dim, log)
+            if o.have_ref():
+                assert np.array_equal(d, o.ref_softmax_backward(g, y, dim, log)), (shape, dim, log)
+            # d/dx of sum(f(x) * g) by central differences in float64
+            def f(z):
+                z = z - z.max(axis=dim, keepdims=True)
+                e = np.exp(z)
+                s = e.sum(axis=dim, keepdims=True)
+                return z - np.log(s) if log else e / s
+            x64 = x.astype(np.float64)
+            num = np.zeros_like(x64)
+            flat = x64.reshape(-1)
+            for i in range(flat.size):
+                old = flat[i]
+                flat[i] = old + 1e-5
+                up = (f(x64) * g).sum()
+                flat[i] = old - 1e-5
+                dn = (f(x64) * g).sum()
+                flat[i] = old
+                num.reshape(-1)[i] = (up - dn) / 2e-5
+            assert np.abs(num - d).max() < 2e-5 * max(1.0, np.abs(num).max()), (shape, dim, log)
+            if not log:
+                assert np.abs(d.sum(axis=dim)).max() < 1e-5
+    g16, _ = o.round_to(g, "bf16")
+    y16, _ = o.round_to(o.softmax(x, -1), "bf16")
+    d16 = o.softmax_backward(g16, y16, -1, False, "bf16")
+    assert np.array_equal(d16, o.round_to(o.softmax_backward(g16, y16, -1), "bf16")[0])

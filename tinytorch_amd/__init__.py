@@ -9,8 +9,9 @@ from . import _capi
 _capi.lib()  # fail loudly when the extension is missing
 
 from .function import (sdpAttention, kvCacheAppend, build_params, rmsNorm, fusedAddRmsNorm, siluMul, softmax,  # noqa: E402
-                       logSoftmax, linear, sdpAttentionBackward, build_backward_params, matmul, linearBackward)
+                       logSoftmax, linear, sdpAttentionBackward, build_backward_params, matmul, linearBackward, softmaxBackward,
+                       logSoftmaxBackward)
 
 __all__ = ["sdpAttention", "kvCacheAppend", "build_params", "rmsNorm", "fusedAddRmsNorm", "siluMul", "softmax",
            "logSoftmax", "linear", "sdpAttentionBackward", "build_backward_params", "matmul",
-           "linearBackward"]
+           "linearBackward", "softmaxBackward", "logSoftmaxBackward"]

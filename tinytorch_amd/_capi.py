@@ -23,7 +23,7 @@ EXPORTS = [
     "ttsdpa_kv_append_params_init", "ttsdpa_kv_append", "ttsdpa_probe",
     "ttsdpa_backward_params_init", "ttsdpa_backward_plan", "ttsdpa_backward_workspace_bytes", "ttsdpa_backward",
     # include/ttfused.h
-    "ttfused_rms_norm", "ttfused_add_rms_norm", "ttfused_silu_mul", "ttfused_softmax",
+    "ttfused_rms_norm", "ttfused_add_rms_norm", "ttfused_silu_mul", "ttfused_softmax", "ttfused_softmax_backward",
     # include/ttlinear.h
     "ttlinear_forward", "ttlinear_plan", "ttlinear_matmul", "ttlinear_matmul_workspace_bytes",
 ]
@@ -154,6 +154,8 @@ def lib():
         L.ttfused_silu_mul.restype = ctypes.c_int
         L.ttfused_softmax.argtypes = [ctypes.c_int, vp, vp, i64, i64, i64, ctypes.c_int, vp]
         L.ttfused_softmax.restype = ctypes.c_int
+        L.ttfused_softmax_backward.argtypes = [ctypes.c_int, vp, vp, vp, i64, i64, i64, ctypes.c_int, vp]
+        L.ttfused_softmax_backward.restype = ctypes.c_int
         L.ttlinear_forward.argtypes = [ctypes.c_int, vp, vp, vp, vp] + [i64] * 6 + [vp]
         L.ttlinear_forward.restype = ctypes.c_int
         L.ttlinear_plan.argtypes = [ctypes.c_int, vp, vp, vp, vp] + [i64] * 6 + [ctypes.POINTER(ctypes.c_int)]

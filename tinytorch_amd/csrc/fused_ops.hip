@@ -384,6 +384,121 @@ int launch_softmax_rows(const void* x, void* out, long long rows, int dim, hipSt
   return (int)hipGetLastError();
 }
 
+// ---- softmax / logSoftmax backward (reference src/Operation/OpNNLayerCpu.h:79-109, 123-150) -----------------------------
+// softmax:    dx_j = y_j * (g_j - sum_t y_t g_t)        logSoftmax: dx_j = g_j - exp(y_j) * sum_t g_t
+// over [outer, dim, inner]; inner == 1 is the last axis.  One workgroup lane group walks a row twice: the sum, then the
+// result (the second read of a row comes from L2).  Lanes run along the contiguous axis in both layouts.
+template <typename T, int VEC, int LPR, bool LOG>
+__global__ __launch_bounds__(256) void softmax_backward_rows_kernel(const T* g, const T* y, T* out, long long rows, int dim) {
+  typedef typename Pack<T, VEC>::type V;
+  __shared__ float lds[4];
+  constexpr int RPB = 256 / LPR;
+  const int lr = threadIdx.x % LPR;
+  const long long row = (long long)blockIdx.x * RPB + threadIdx.x / LPR;
+  const bool live = row < rows;
+  const int nvec = dim / VEC;
+  const T* gr = g + row * dim;
+  const T* yr = y + row * dim;
+  float part = 0.f;
+  if (live) {
+    for (int i = lr; i < nvec; i += LPR) {
+      const V a = load_plain<T, VEC>(gr + (long long)i * VEC);
+      if (LOG) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) part += (float)a[e];
+      } else {
+        const V b = load_plain<T, VEC>(yr + (long long)i * VEC);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) part = fmaf((float)a[e], (float)b[e], part);
+      }
+    }
+  }
+  const float sum = row_reduce<LPR, SumOp>(part, lds, 0);
+  if (!live) return;
+  for (int i = lr; i < nvec; i += LPR) {
+    const V a = load_plain<T, VEC>(gr + (long long)i * VEC);
+    const V b = load_stream<T, VEC>(yr + (long long)i * VEC);
+    V o;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) o[e] = (T)(LOG ? (float)a[e] - __expf((float)b[e]) * sum : (float)b[e] * ((float)a[e] - sum));
+    store_pack<T, VEC>(out + row * dim + (long long)i * VEC, o);
+  }
+}
+
+template <typename T, int VEC, bool LOG>
+__global__ __launch_bounds__(256) void softmax_backward_strided_kernel(const T* g, const T* y, T* out, long long outer, int dim,
+                                                                       long long inner) {
+  typedef typename Pack<T, VEC>::type V;
+  const long long ivec = inner / VEC;
+  const long long cg = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (cg >= outer * ivec) return;
+  const long long base = (cg / ivec) * dim * inner + (cg % ivec) * VEC;
+  float sum[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; e++) sum[e] = 0.f;
+  for (int d = 0; d < dim; d++) {
+    const V a = load_plain<T, VEC>(g + base + d * inner);
+    if (LOG) {
+#pragma unroll
+      for (int e = 0; e < VEC; e++) sum[e] += (float)a[e];
+    } else {
+      const V b = load_plain<T, VEC>(y + base + d * inner);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) sum[e] = fmaf((float)a[e], (float)b[e], sum[e]);
+    }
+  }
+  for (int d = 0; d < dim; d++) {
+    const V a = load_plain<T, VEC>(g + base + d * inner);
+    const V b = load_plain<T, VEC>(y + base + d * inner);
+    V o;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) o[e] = (T)(LOG ? (float)a[e] - __expf((float)b[e]) * sum[e] : (float)b[e] * ((float)a[e] - sum[e]));
+    store_pack<T, VEC>(out + base + d * inner, o);
+  }
+}
+
+template <typename T>
+int softmax_backward_dispatch(const void* g, const void* y, void* out, long long outer, int dim, long long inner, bool log_form,
+                              hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  if (inner == 1) {
+    const bool vec = dim % VEC == 0 && aligned16(g) && aligned16(y) && aligned16(out);
+    const int lpr = pick_lpr(vec ? dim / VEC : dim);
+    const long long rpb = 256 / lpr;
+    const unsigned grid = (unsigned)((outer + rpb - 1) / rpb);
+#define TT_SMB(V_, LPR_, LOG_) \
+  hipLaunchKernelGGL((softmax_backward_rows_kernel<T, V_, LPR_, LOG_>), dim3(grid), dim3(256), 0, s, (const T*)g, (const T*)y, (T*)out, outer, dim)
+#define TT_SMB_L(V_, LOG_)                  \
+  switch (lpr) {                            \
+    case 8: TT_SMB(V_, 8, LOG_); break;     \
+    case 16: TT_SMB(V_, 16, LOG_); break;   \
+    case 32: TT_SMB(V_, 32, LOG_); break;   \
+    case 64: TT_SMB(V_, 64, LOG_); break;   \
+    default: TT_SMB(V_, 256, LOG_); break;  \
+  }
+    if (vec) {
+      if (log_form) { TT_SMB_L(VEC, true) } else { TT_SMB_L(VEC, false) }
+    } else {
+      if (log_form) { TT_SMB_L(1, true) } else { TT_SMB_L(1, false) }
+    }
+#undef TT_SMB_L
+#undef TT_SMB
+    return (int)hipGetLastError();
+  }
+  const bool vec = inner % VEC == 0 && aligned16(g) && aligned16(y) && aligned16(out);
+  const long long groups = outer * (vec ? inner / VEC : inner);
+  const unsigned grid = (unsigned)((groups + 255) / 256);
+#define TT_SMBS(V_, LOG_) \
+  hipLaunchKernelGGL((softmax_backward_strided_kernel<T, V_, LOG_>), dim3(grid), dim3(256), 0, s, (const T*)g, (const T*)y, (T*)out, outer, dim, inner)
+  if (vec) {
+    if (log_form) TT_SMBS(VEC, true); else TT_SMBS(VEC, false);
+  } else {
+    if (log_form) TT_SMBS(1, true); else TT_SMBS(1, false);
+  }
+#undef TT_SMBS
+  return (int)hipGetLastError();
+}
+
 int check_common(int dtype, long long rows, long long dim) {
   if (dtype != TTSDPA_F32 && dtype != TTSDPA_F16 && dtype != TTSDPA_BF16) return TTSDPA_ERR_DTYPE;
   if (rows < 0 || dim < 0 || dim > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
@@ -506,6 +621,22 @@ int ttfused_softmax(int dtype, const void* x, void* out, int64_t outer, int64_t 
     case TTSDPA_F32: return softmax_dispatch<float>(x, out, outer, (int)dim, inner, log_form != 0, s);
     case TTSDPA_F16: return softmax_dispatch<_Float16>(x, out, outer, (int)dim, inner, log_form != 0, s);
     default: return softmax_dispatch<__bf16>(x, out, outer, (int)dim, inner, log_form != 0, s);
+  }
+}
+
+int ttfused_softmax_backward(int dtype, const void* grad, const void* output, void* out, int64_t outer, int64_t dim,
+                             int64_t inner, int log_form, void* stream) {
+  int rc = check_common(dtype, outer, dim);
+  if (rc != TTSDPA_OK) return rc;
+  if (inner < 0) return TTSDPA_ERR_SHAPE;
+  if (outer == 0 || dim == 0 || inner == 0) return TTSDPA_OK;
+  if (!grad || !output || !out) return TTSDPA_ERR_NULL;
+  if (inner > 0x7fffffffLL || !grid_ok(outer) || outer > (0x7fffffffLL * 256) / inner) return TTSDPA_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case TTSDPA_F32: return softmax_backward_dispatch<float>(grad, output, out, outer, (int)dim, inner, log_form != 0, s);
+    case TTSDPA_F16: return softmax_backward_dispatch<_Float16>(grad, output, out, outer, (int)dim, inner, log_form != 0, s);
+    default: return softmax_backward_dispatch<__bf16>(grad, output, out, outer, (int)dim, inner, log_form != 0, s);
   }
 }
 

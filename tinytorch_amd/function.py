@@ -333,6 +333,34 @@ def logSoftmax(x, dim=-1):
     return _softmax("logSoftmax", x, dim, True)
 
 
+def _softmax_backward(name, grad, output, dim, log):
+    _check_rowwise(name, grad, output)
+    if grad.shape != output.shape or grad.dim() == 0:
+        raise ValueError("%s: grad %s and output %s must have the same shape" % (name, tuple(grad.shape), tuple(output.shape)))
+    dim = dim % grad.dim()
+    grad, output = grad.contiguous(), output.contiguous()
+    out = torch.empty_like(grad)
+    outer = 1
+    for n in grad.shape[:dim]:
+        outer *= n
+    inner = 1
+    for n in grad.shape[dim + 1:]:
+        inner *= n
+    _launch("ttfused_softmax_backward", _capi.lib().ttfused_softmax_backward, grad.device, _DTYPES[grad.dtype],
+            grad.data_ptr(), output.data_ptr(), out.data_ptr(), outer, grad.shape[dim], inner, int(log))
+    return out
+
+
+def softmaxBackward(grad, output, dim=-1):
+    """output * (grad - sum(output * grad)) along `dim` (reference op::softmaxBackward, src/Operation/OpNNLayerCpu.h:79-109)."""
+    return _softmax_backward("softmaxBackward", grad, output, dim, False)
+
+
+def logSoftmaxBackward(grad, output, dim=-1):
+    """grad - exp(output) * sum(grad) along `dim` (reference op::logSoftmaxBackward, src/Operation/OpNNLayerCpu.h:123-150)."""
+    return _softmax_backward("logSoftmaxBackward", grad, output, dim, True)
+
+
 # ---- the linear layer (include/ttlinear.h) ------------------------------------------------------------------------------
 
 def linear(input, weight, bias=None):

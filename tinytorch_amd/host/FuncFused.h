@@ -1,7 +1,7 @@
 // function::siluMul / fusedAddRmsNorm / rmsNorm / softmax / logSoftmax with the reference's signatures and defaults
 // (src/Function/FuncFused.h:14-34, src/Function/FuncNNLayer.h:219-227,294-296, src/Function/FuncActivation.h:42-92).
 // Forward only: the reference's backward of siluMul, fusedAddRmsNorm and rmsNorm is NOT_IMPLEMENTED as well; the
-// softmax backward of the reference is not part of this inference path and fails the same loud way here.
+// softmax / logSoftmax backward is the reference's own (op::softmaxBackward / op::logSoftmaxBackward).
 #pragma once
 
 #include <vector>
@@ -40,13 +40,23 @@ class FuncRMSNorm : public Function<FuncRMSNorm> {
 template <bool LOG>
 class FuncSoftmaxT : public Function<FuncSoftmaxT<LOG>> {
  public:
+  // forward keeps its output and the axis; backward is the reference's (src/Function/FuncActivation.h:45-62, 68-85)
   static Tensor forward(AutogradContext* ctx, const Tensor& self, int64_t dim) {
-    (void)ctx;
-    return LOG ? op::logSoftmax(self, dim) : op::softmax(self, dim);
+    Tensor out = LOG ? op::logSoftmax(self, dim) : op::softmax(self, dim);
+    if (ctx && out.defined()) {
+      ctx->saveForBackward(out.detach());
+      ctx->dim = dim;
+    }
+    return out;
   }
   static void backward(AutogradContext* ctx, const Tensor& grad) {
-    (void)ctx, (void)grad;
-    NOT_IMPLEMENTED();
+    ASSERT(ctx && !ctx->savedInputs.empty() && ctx->savedForBackward.size() == 1);
+    if (!ctx || ctx->savedInputs.empty() || ctx->savedForBackward.size() != 1) return;
+    Tensor& self = ctx->savedInputs[0];
+    if (self.requiresGrad()) {
+      const Tensor& output = ctx->savedForBackward[0];
+      self.addGrad(LOG ? op::logSoftmaxBackward(grad, output, ctx->dim) : op::softmaxBackward(grad, output, ctx->dim));
+    }
   }
 };
 

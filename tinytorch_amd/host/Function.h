@@ -40,6 +40,7 @@ struct AutogradContext {
   // non-tensor arguments a backward needs (the reference keeps such values in an IValue list, src/Tensor/IValue.h)
   bool isCausal = false;
   float scale = 1.f;
+  int64_t dim = -1;
 };
 
 struct FunctionBase {

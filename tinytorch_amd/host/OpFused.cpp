@@ -95,6 +95,24 @@ Tensor softmaxGpuImpl(const Tensor& self, int64_t dim) {
   return out;
 }
 
+template <bool LOG>
+Tensor softmaxBackwardGpuImpl(const Tensor& grad, const Tensor& output, int64_t dim) {
+  ASSERT(grad.defined() && output.defined() && output.shape() == grad.shape() && output.dtype() == grad.dtype());
+  if (!grad.defined() || !output.defined() || output.shape() != grad.shape() || output.dtype() != grad.dtype() || grad.dim() < 1) return {};
+  if (dim < 0) dim += grad.dim();
+  ASSERT(dim >= 0 && dim < grad.dim());
+  if (dim < 0 || dim >= grad.dim()) return {};
+  int64_t outer = 1, inner = 1;
+  for (int64_t i = 0; i < dim; i++) outer *= grad.size(i);
+  for (int64_t i = dim + 1; i < grad.dim(); i++) inner *= grad.size(i);
+  Tensor out = Tensor::empty(grad.shape(), grad.options().noGrad());
+  if (!launched("ttfused_softmax_backward",
+                ttfused_softmax_backward(dtypeCode(grad.dtype()), grad.rawPtr(), output.rawPtr(), out.rawPtr(), outer, grad.size(dim),
+                                         inner, LOG ? 1 : 0, streamOf(grad))))
+    return {};
+  return out;
+}
+
 }  // namespace
 
 void registerFusedGpu() {
@@ -113,6 +131,12 @@ void registerFusedGpu() {
   REGISTER_OP_IMPL(logSoftmax, GPU, Float32, &softmaxGpuImpl<true>);
   REGISTER_OP_IMPL(logSoftmax, GPU, Float16, &softmaxGpuImpl<true>);
   REGISTER_OP_IMPL(logSoftmax, GPU, BFloat16, &softmaxGpuImpl<true>);
+  REGISTER_OP_IMPL(softmaxBackward, GPU, Float32, &softmaxBackwardGpuImpl<false>);
+  REGISTER_OP_IMPL(softmaxBackward, GPU, Float16, &softmaxBackwardGpuImpl<false>);
+  REGISTER_OP_IMPL(softmaxBackward, GPU, BFloat16, &softmaxBackwardGpuImpl<false>);
+  REGISTER_OP_IMPL(logSoftmaxBackward, GPU, Float32, &softmaxBackwardGpuImpl<true>);
+  REGISTER_OP_IMPL(logSoftmaxBackward, GPU, Float16, &softmaxBackwardGpuImpl<true>);
+  REGISTER_OP_IMPL(logSoftmaxBackward, GPU, BFloat16, &softmaxBackwardGpuImpl<true>);
 }
 
 }  // namespace tinytorch::op

@@ -26,6 +26,11 @@ DEFINE_OP(fusedAddRmsNorm, FusedAddRmsNormOpFn)
 DEFINE_OP(rmsNorm, RMSNormOpFn)
 DEFINE_OP(softmax, SoftmaxOpFn)
 DEFINE_OP(logSoftmax, SoftmaxOpFn)
+// gradient of softmax / logSoftmax along dim from the upstream gradient and the forward's output (reference
+// src/Operation/OpNNLayer.h:46-51)
+using SoftmaxOpBackwardFn = Tensor (*)(const Tensor& grad, const Tensor& output, int64_t dim);
+DEFINE_OP(softmaxBackward, SoftmaxOpBackwardFn)
+DEFINE_OP(logSoftmaxBackward, SoftmaxOpBackwardFn)
 
 void registerFusedGpu();
 STATIC_CALL(registerFusedGpu);
