@@ -185,7 +185,7 @@ typedef struct ttsdpa_backward_params {
 /* Fill *p for dense tensors (ttsdpa_params_init for fwd, dense gradient strides); pointers NULL. */
 void ttsdpa_backward_params_init(ttsdpa_backward_params* p, int dtype, int B, int Hq, int Hkv, int L, int S, int D);
 /* Validate and report the kernels ttsdpa_backward would use: TTSDPA_ROUTE_PREFILL = the MFMA backward kernels
- * (fp16/bf16, head_dim 64 or 128, no attnMask), TTSDPA_ROUTE_GENERAL = the vector-ALU kernels,
+ * (fp16/bf16, head_dim 64 or 128; an attnMask must have contiguous, 4-aligned keys), TTSDPA_ROUTE_GENERAL = the vector-ALU kernels,
  * TTSDPA_ROUTE_NONE = nothing to compute.  Needs no GPU. */
 int ttsdpa_backward_plan(const ttsdpa_backward_params* p, int* route);
 size_t ttsdpa_backward_workspace_bytes(const ttsdpa_backward_params* p);

@@ -138,6 +138,49 @@ def test_backward_with_masks(dtype, kind):
     check("mask-%s-%s" % (kind, dtype), host, dev, dtype, mask_h=m, mask_d=md, route="general")
 
 
+@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64)])
+@pytest.mark.parametrize("kind", ["bool", "add", "keypad", "perhead", "hiddenrow"])
+def test_backward_mfma_with_masks(dtype, D, kind):
+    """attnMasks the MFMA pair takes (contiguous keys, S a multiple of 4): Bool [L,S], additive [L,S], key padding
+    [B,1,1,S], per-head [Hq,L,S]; and a mask with one fully hidden query row, whose dq is 0 and which adds nothing to dk / dv
+    (the oracle, like the forward, has NaN there: that row is left out of the comparison)."""
+    B, Hq, Hkv, L, S = 2, 4, 2, 70, 132
+    host, dev = make_inputs(4500 + D, B, Hq, Hkv, L, S, D, dtype)
+    rng = np.random.default_rng(4)
+    if kind == "bool" or kind == "hiddenrow":
+        m = rng.random((L, S)) < 0.7
+        m[:, 0] = True
+        if kind == "hiddenrow":
+            m[5, :] = False
+    elif kind == "add":
+        m = oracle.round_to(rng.standard_normal((L, S)).astype(np.float32), dtype)[0]
+    elif kind == "keypad":
+        m = np.arange(S)[None, None, None, :] < np.array([S, 77])[:, None, None, None]
+    else:
+        m = rng.random((Hq, L, S)) < 0.7
+        m[..., 0] = True
+    md = torch.from_numpy(np.ascontiguousarray(m)).cuda()
+    if md.dtype != torch.bool:
+        md = md.to(TORCH_DTYPE[dtype])
+    if kind != "hiddenrow":
+        check("mfma-mask-%s-%s" % (kind, dtype), host, dev, dtype, mask_h=m, mask_d=md, route="prefill")
+        return
+    say("backward mfma hidden row", dtype, D)
+    q, k, v = dev
+    go_h, go = upstream(9, q.shape, dtype)
+    rc, out = call("forward", q, k, v, mask=md)
+    assert rc == 0
+    out = torch.nan_to_num(out)   # the hidden row's forward output is NaN; the backward must not depend on it
+    assert backward_route_of(q, k, v, out, go, False, md) == "prefill"
+    rc, (dq, dk, dv) = backward_call(q, k, v, out, go, mask=md)
+    assert rc == 0 and torch.all(dq[:, :, 5] == 0)
+    keep = np.ones(L, bool)
+    keep[5] = False
+    eq, ek, ev = oracle.sdpa_backward_f32(host[0][:, :, keep], host[1], host[2], go_h[:, :, keep], mask=m[keep])
+    assert grad_err(dq[:, :, torch.from_numpy(keep).cuda()], eq) <= TOL[dtype]
+    assert grad_err(dk, ek) <= TOL[dtype] and grad_err(dv, ev) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 def test_backward_bottom_right_causal_and_key_counts(dtype):
     """Bottom-right alignment with per-batch key counts: the oracle sees it as a Bool mask per batch entry; rows of

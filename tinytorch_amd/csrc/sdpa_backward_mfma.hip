@@ -125,7 +125,8 @@ __device__ __forceinline__ vec8 regs_to_operand(const f32x16& acc, int t) {
 // ---- kernel 1: dq, lse, delta ----------------------------------------------------------------------------------------
 // BN: keys per streamed tile.  64 for head_dim 64; 32 for head_dim 128, which keeps a wavefront under 256 registers:
 // two wavefronts per SIMD (one's vector work overlaps the other's matrix work), accumulators in ordinary registers.
-template <typename TR, int D, bool CAUSAL>
+// MASKED: an attnMask (exclusive with CAUSAL) whose keys can be read four at a time, as in the forward kernels.
+template <typename TR, int D, bool CAUSAL, bool MASKED>
 __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
   constexpr int BN = DqTile<D>::BN;
   typedef typename TR::elem T;
@@ -277,6 +278,13 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
             if (key >= S || (CAUSAL && key > qi)) sacc[blk][r] = -INFINITY;
           }
       }
+      if (MASKED) {
+        int qi = qw0 + lq;
+        qi = qi < f.L ? qi : f.L - 1;
+        const long long mrow = b * f.ms[0] + h * f.ms[1] + qi * f.ms[2];
+#pragma unroll
+        for (int blk = 0; blk < NBLK; blk++) apply_attn_mask<T, true>(f, sacc[blk], mrow, kv0 + 32 * blk, lh, S, 1.f / f.scale);
+      }
       float mloc = sacc[0][0];
 #pragma unroll
       for (int blk = 0; blk < NBLK; blk++)
@@ -335,8 +343,10 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
   if (qi < f.L) {
     const long long row_id = ((long long)b * f.Hq + h) * f.L + qi;
     // log2 of the row's sum of exponentials, the unit the second kernel's exp2 wants
-    if (lh == 0) *(float2*)(a.stats + 2 * row_id) = make_float2(m_use * c + __log2f(l_tot), delta);
-    const float w = f.scale / l_tot;
+    // a row whose keys are all hidden (possible with an attnMask): dq = 0, and a statistic that gives it weight 0 below
+    const bool seen = l_tot > 0.f;
+    if (lh == 0) *(float2*)(a.stats + 2 * row_id) = make_float2(seen ? m_use * c + __log2f(l_tot) : 1e30f, delta);
+    const float w = seen ? f.scale / l_tot : 0.f;
     T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
 #pragma unroll
     for (int db = 0; db < DBLK; db++)
@@ -344,14 +354,14 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
       for (int rg = 0; rg < 4; rg++) {
         f32x4 x;
 #pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = dqacc[db][4 * rg + i] * w;
+        for (int i = 0; i < 4; i++) x[i] = seen ? dqacc[db][4 * rg + i] * w : 0.f;
         *(typename TR::vec4*)(dqp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
       }
   }
 }
 
 // ---- kernel 2: dk, dv ---------------------------------------------------------------------------------------------------
-template <typename TR, int D, bool CAUSAL>
+template <typename TR, int D, bool CAUSAL, bool MASKED>
 __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kernel(BwdArgs a) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
@@ -470,6 +480,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
       if (idx + 2 < total) load_tile(idx + 2);
     }
     const int i0 = (ntq - 1 - idx / f.G) * BQ;
+    const int h_of_tile = hk * f.G + idx % f.G;
     if (wave_live && (!CAUSAL || kw0 <= i0 + BQ - 1 + coff)) {
       const T* Qr = smem + cur * Lds::KV_STAGE;
       const T* Gr = Qr + BQ * RP;
@@ -497,7 +508,18 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 4 * rg + e;
-          const float p = fast_exp2(fmaf(sacc[r], c, -lse2[e]));
+          float bias2 = 0.f;  // attnMask: the additive bias in log2 units, or -inf for a hidden key
+          if (MASKED) {
+            int qrow = i0 + 8 * rg + 4 * lh + e;
+            qrow = qrow < f.L ? qrow : f.L - 1;
+            const long long at = b * f.ms[0] + h_of_tile * f.ms[1] + qrow * f.ms[2] + (key < S ? key : S - 1) * f.ms[3];
+            if (f.mask_kind == 1) {
+              bias2 = ((const uint8_t*)f.mask)[at] == 0 ? -INFINITY : 0.f;
+            } else {
+              bias2 = (float)((const T*)f.mask)[at] * kLog2e;
+            }
+          }
+          const float p = fast_exp2(fmaf(sacc[r], c, bias2 - lse2[e]));
           sacc[r] = p;
           dpacc[r] = p * (dpacc[r] - dl[e]);
         }
@@ -817,36 +839,44 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
   }
 }
 
-template <typename TR, int D, bool CAUSAL>
+template <typename TR, int D, bool CAUSAL, bool MASKED>
 int launch_k(const BwdArgs& a, hipStream_t stream) {
   typedef BwdLds<D> Lds;
+  // with an attnMask, head_dim 128 takes the register-staged dk/dv kernel: the mask's 16 values per tile do not fit the
+  // 256 registers of the direct-to-LDS one
+  constexpr bool DMA = D == 128 && !MASKED;
   static hipError_t state1[kMaxDevices], state2[kMaxDevices];
   static bool done1[kMaxDevices], done2[kMaxDevices];
-  hipError_t e = grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL>, DqTile<D>::BYTES, state1, done1);
+  hipError_t e = grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED>, DqTile<D>::BYTES, state1, done1);
   if (e != hipSuccess) return (int)e;
-  if (D == 128) {
+  if (DMA) {
     e = grant_dynamic_lds((const void*)backward_dkv128_kernel<TR, CAUSAL>, dkv128::LDS_BYTES, state2, done2);
   } else {
-    e = grant_dynamic_lds((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL>, Lds::KV_BYTES, state2, done2);
+    e = grant_dynamic_lds((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED>, Lds::KV_BYTES, state2, done2);
   }
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM);
-  hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g1), dim3(256), DqTile<D>::BYTES, stream, a);
+  hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED>), dim3((unsigned)g1), dim3(256), DqTile<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
-  if (D == 128) {
+  if (DMA) {
     hipLaunchKernelGGL((backward_dkv128_kernel<TR, CAUSAL>), dim3((unsigned)g2), dim3(512), dkv128::LDS_BYTES, stream, a);
   } else {
-    hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
+    hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
   }
   return (int)hipGetLastError();
 }
 
+template <typename TR, int D>
+int launch_d(const BwdArgs& a, hipStream_t stream) {
+  if (a.f.mask_kind != 0) return launch_k<TR, D, false, true>(a, stream);  // exclusive with causal (validated)
+  return a.f.causal ? launch_k<TR, D, true, false>(a, stream) : launch_k<TR, D, false, false>(a, stream);
+}
+
 template <typename TR>
 int launch_t(const BwdArgs& a, hipStream_t stream) {
-  if (a.f.D == 64) return a.f.causal ? launch_k<TR, 64, true>(a, stream) : launch_k<TR, 64, false>(a, stream);
-  return a.f.causal ? launch_k<TR, 128, true>(a, stream) : launch_k<TR, 128, false>(a, stream);
+  return a.f.D == 64 ? launch_d<TR, 64>(a, stream) : launch_d<TR, 128>(a, stream);
 }
 
 }  // namespace

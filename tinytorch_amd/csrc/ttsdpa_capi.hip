@@ -223,10 +223,10 @@ int validate_backward(const ttsdpa_backward_params* p, BwdArgs* a) {
 }
 
 // The MFMA backward kernels: 16-bit tensors they can read and write with 16-byte / 8-byte accesses, head_dim 64 or
-// 128, no attnMask.
+// 128, attnMasks the forward's 4-wavefront kernel takes (keys readable four at a time, no kv_len beside them).
 bool backward_mfma_ok(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
-  if (!fast_layout_ok(f) || (f->D != 64 && f->D != 128) || f->L < 1 || f->S < 1) return false;
+  if (!fast_layout_ok(f, true) || !simple_mask_ok(f) || (f->D != 64 && f->D != 128) || f->L < 1 || f->S < 1) return false;
   if (!dense_last_ok(p->dout_stride, 8) || !dense_last_ok(p->dq_stride, 8) || !dense_last_ok(p->dk_stride, 8) ||
       !dense_last_ok(p->dv_stride, 8))
     return false;
