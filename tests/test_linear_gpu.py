@@ -45,6 +45,10 @@ CASES = [
     (256, 256, 32, "f32", True, "mfma"),         # fp32 on the fp32 matrix cores: one tile, one k step
     (300, 260, 160, "f32", True, "mfma"),
     (1100, 520, 96, "f32", False, "mfma"),
+    (1, 4096, 512, "bf16", True, "mfma"),        # a handful of rows: the weight-streaming kernel
+    (7, 200, 128, "f16", False, "mfma"),         # ... a partial block of 32 columns
+    (33, 96, 192, "bf16", True, "mfma"),         # ... two row blocks, the second nearly empty
+    (64, 1536, 2048, "f16", True, "mfma"),
     (2, 3, 5, "f32", True, "general"),
     (70, 90, 100, "f32", True, "general"),
     (129, 65, 200, "bf16", True, "general"),     # K not a multiple of 64

@@ -230,6 +230,100 @@ __global__ __launch_bounds__(WN * WM * 64, 1) void linear_mfma_kernel(LinArgs a)
   }
 }
 
+// ---- few rows of x (a decode step's projections: M = the batch): the weight is read once at HBM speed ------------------
+// With M <= 64 the layer is a stream over w (N*K elements) against 64 rows of x that stay in L2: a workgroup owns 32
+// output columns and all rows of x; its four wavefronts take the 64-element k-blocks in turn (wavefront v: blocks v,
+// v+4, ...), so the four read neighbouring 128-byte lines of each weight row, and add their partial sums through LDS at
+// the end.  Per k-block a lane reads 64 contiguous bytes of its weight row (column lq, k-half lh) and of its x row(s)
+// straight from global memory into registers; MFMA j of the block contracts elements 8j..8j+7 of both lane halves' 32,
+// the same order on both operands.  out^T[n][m] accumulates with w as the A operand, so a lane ends up with four
+// consecutive n of one row m: 8-byte stores.
+template <typename TR, int MB>  // MB = 32-row blocks of x: 1 (M <= 32) or 2 (M <= 64)
+__global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
+  typedef typename TR::elem T;
+  typedef typename TR::vec8 vec8;
+  __shared__ float part[3][MB][16][64];  // the partial sums of wavefronts 1-3
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lq = lane & 31, lh = lane >> 5;
+  const long long n0 = (long long)blockIdx.x * 32;
+  const long long nrow = n0 + lq < a.N ? n0 + lq : a.N - 1;  // columns past the end re-read the last weight row (not stored)
+  const T* wr = (const T*)a.w + nrow * a.ldw + 32 * lh;
+  const T* xr[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++) {
+    const long long m = 32 * mb + lq < a.M ? 32 * mb + lq : a.M - 1;
+    xr[mb] = (const T*)a.x + m * a.ldx + 32 * lh;
+  }
+  f32x16 acc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[mb][r] = 0.f;
+  const long long nkb = a.K / 64;
+  for (long long kb = wave; kb < nkb; kb += 8) {  // two k-blocks of this wavefront per iteration: 128 bytes per lane in flight per operand
+    const bool two = kb + 4 < nkb;
+    vec8 wv[2][4], xv[2][MB][4];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      if (u == 1 && !two) break;
+      const long long k = (kb + 4 * u) * 64;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        wv[u][j] = __builtin_nontemporal_load((const vec8*)(wr + k + 8 * j));  // streamed once
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) xv[u][mb][j] = *(const vec8*)(xr[mb] + k + 8 * j);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      if (u == 1 && !two) break;
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) acc[mb] = TR::mfma32(wv[u][j], xv[u][mb][j], acc[mb]);
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) part[wave - 1][mb][r][lane] = acc[mb][r];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++) {
+    const long long m = 32 * mb + lq;
+#pragma unroll
+    for (int rg = 0; rg < 4; rg++) {
+      const long long n = n0 + 8 * rg + 4 * lh;
+      f32x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int r = 4 * rg + i;
+        float sum = acc[mb][r] + part[0][mb][r][lane] + part[1][mb][r][lane] + part[2][mb][r][lane];
+        if (a.bias && n + i < a.N) sum += load_as_float((const T*)a.bias + n + i);
+        v[i] = sum;
+      }
+      if (m < a.M && n < a.N) {  // N is a multiple of 4 on this route: a group of four is inside or outside
+        *(typename TR::vec4*)((T*)a.out + m * a.ldo + n) = __builtin_convertvector(v, typename TR::vec4);
+      }
+    }
+  }
+}
+
+template <typename TR>
+int launch_skinny(const LinArgs& a, hipStream_t stream) {
+  const long long nwg = (a.N + 31) / 32;
+  if (nwg > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
+  if (a.M <= 32) {
+    hipLaunchKernelGGL((linear_skinny_kernel<TR, 1>), dim3((unsigned)nwg), dim3(256), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((linear_skinny_kernel<TR, 2>), dim3((unsigned)nwg), dim3(256), 0, stream, a);
+  }
+  return (int)hipGetLastError();
+}
+
 // Any element type and shape: 64 x 64 output tile per workgroup, 4 x 4 outputs per lane, K in steps of 16 through LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void linear_general_kernel(LinArgs a) {
@@ -418,8 +512,11 @@ int ttlinear_forward(int dtype, const void* x, const void* w, const void* bias, 
   if (bias && !aligned(bias, esz)) return TTSDPA_ERR_STRIDE;
   LinArgs a{x, w, bias, out, M, N, K, ldx, ldw, ldo};
   hipStream_t s = (hipStream_t)stream;
-  if (route == TTLINEAR_ROUTE_MFMA)
+  if (route == TTLINEAR_ROUTE_MFMA) {
+    // a handful of rows (a decode step): stream the weight once instead of tiling for reuse
+    if (dtype != TTSDPA_F32 && M <= 64 && N >= 64) return dtype == TTSDPA_F16 ? launch_skinny<F16>(a, s) : launch_skinny<BF16>(a, s);
     return dtype == TTSDPA_F32 ? launch_mfma<F32>(a, s) : dtype == TTSDPA_F16 ? launch_mfma<F16>(a, s) : launch_mfma<BF16>(a, s);
+  }
   switch (dtype) {
     case TTSDPA_F32: return launch_general_linear<float>(a, s);
     case TTSDPA_F16: return launch_general_linear<_Float16>(a, s);
