@@ -233,61 +233,108 @@ __global__ __launch_bounds__(WN * WM * 64, 1) void linear_mfma_kernel(LinArgs a)
 // ---- few rows of x (a decode step's projections: M = the batch): the weight is read once at HBM speed ------------------
 // With M <= 64 the layer is a stream over w (N*K elements) against 64 rows of x that stay in L2: a workgroup owns 32
 // output columns and all rows of x; its four wavefronts take the 64-element k-blocks in turn (wavefront v: blocks v,
-// v+4, ...), so the four read neighbouring 128-byte lines of each weight row, and add their partial sums through LDS at
-// the end.  Per k-block a lane reads 64 contiguous bytes of its weight row (column lq, k-half lh) and of its x row(s)
-// straight from global memory into registers; MFMA j of the block contracts elements 8j..8j+7 of both lane halves' 32,
-// the same order on both operands.  out^T[n][m] accumulates with w as the A operand, so a lane ends up with four
-// consecutive n of one row m: 8-byte stores.
+// v+4, ...) and add their partial sums through LDS at the end.  Every wavefront has a ring of three k-blocks of its own in
+// LDS, filled by direct global->LDS loads (eight lanes fetch the 128 bytes of a row's k-block: whole cache lines) and
+// read back as MFMA operands, 16-byte chunk c of row r at slot c ^ ((r/2) % 8) (conflict-free b128 reads).  No
+// barriers inside the stream: a ring belongs to one wavefront.  out^T[n][m] accumulates with w as the A operand, so a
+// lane ends up with four consecutive n of one row m: 8-byte stores.
+template <int MB>
+struct Skinny {
+  static constexpr int NST = 3;                        // k-blocks of a wavefront in LDS
+  static constexpr int WT = 32 * 128;                  // bytes of a weight tile: 32 rows x 64 k
+  static constexpr int STG = WT + MB * 32 * 128;       // ... plus the x tile
+  static constexpr int LPB = 4 + 4 * MB;               // load instructions per k-block
+  static constexpr int LDS = 4 * NST * STG;
+  static_assert(LDS >= 3 * MB * 16 * 64 * 4, "the partial sums of three wavefronts reuse the rings");
+};
+
 template <typename TR, int MB>  // MB = 32-row blocks of x: 1 (M <= 32) or 2 (M <= 64)
 __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
-  __shared__ float part[3][MB][16][64];  // the partial sums of wavefronts 1-3
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  typedef Skinny<MB> SK;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lq = lane & 31, lh = lane >> 5;
   const long long n0 = (long long)blockIdx.x * 32;
-  const long long nrow = n0 + lq < a.N ? n0 + lq : a.N - 1;  // columns past the end re-read the last weight row (not stored)
-  const T* wr = (const T*)a.w + nrow * a.ldw + 32 * lh;
-  const T* xr[MB];
+  char* ring = smem + wave * SK::NST * SK::STG;
+  const unsigned ring_addr = (unsigned)(unsigned long)(lds_void_t*)ring;
+
+  auto dma16 = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+  };
+  // this lane's part of a load instruction: row 8i + lane/8 of a tile, slot lane%8
+  unsigned woff[4], xoff[MB][4];
 #pragma unroll
-  for (int mb = 0; mb < MB; mb++) {
-    const long long m = 32 * mb + lq < a.M ? 32 * mb + lq : a.M - 1;
-    xr[mb] = (const T*)a.x + m * a.ldx + 32 * lh;
+  for (int i = 0; i < 4; i++) {
+    const int row = 8 * i + (lane >> 3);
+    const unsigned chunk = (unsigned)((lane & 7) ^ ((row >> 1) & 7));
+    // columns past the end re-read the last weight row (not stored)
+    woff[i] = (unsigned)(((n0 + row < a.N ? row : (int)(a.N - 1 - n0)) * a.ldw + 8 * chunk) * 2);
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+      const int m = 32 * mb + row;
+      xoff[mb][i] = (unsigned)(((m < a.M ? m : (int)(a.M - 1)) * a.ldx + 8 * chunk) * 2);
+    }
   }
+  const char* wbase = (const char*)((const T*)a.w + n0 * a.ldw);
+  const char* xbase = (const char*)a.x;
+  auto issue = [&](long long kb, int stage) __attribute__((always_inline)) {
+    const unsigned at = ring_addr + stage * SK::STG;
+    const char* wk = wbase + kb * 128;
+    const char* xk = xbase + kb * 128;
+#pragma unroll
+    for (int i = 0; i < 4; i++) dma16(wk, woff[i], at + 8 * i * 128);
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) dma16(xk, xoff[mb][i], at + SK::WT + (32 * mb + 8 * i) * 128);
+  };
+  // operand (j): row lq, chunk 4*lh + j
+  unsigned rd[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) rd[j] = (unsigned)(lq * 128 + 16 * ((4 * lh + j) ^ ((lq >> 1) & 7)));
+
   f32x16 acc[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; mb++)
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[mb][r] = 0.f;
   const long long nkb = a.K / 64;
-  for (long long kb = wave; kb < nkb; kb += 8) {  // two k-blocks of this wavefront per iteration: 128 bytes per lane in flight per operand
-    const bool two = kb + 4 < nkb;
-    vec8 wv[2][4], xv[2][MB][4];
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-      if (u == 1 && !two) break;
-      const long long k = (kb + 4 * u) * 64;
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        wv[u][j] = __builtin_nontemporal_load((const vec8*)(wr + k + 8 * j));  // streamed once
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++) xv[u][mb][j] = *(const vec8*)(xr[mb] + k + 8 * j);
-      }
+  const long long nb = nkb > wave ? (nkb - wave + 3) / 4 : 0;  // k-blocks of this wavefront: wave, wave + 4, ...
+  if (nb > 0) issue(wave, 0);
+  if (nb > 1) issue(wave + 4, 1);
+  int cur = 0;
+  for (long long t = 0; t < nb; t++) {
+    const int nxt2 = cur == 0 ? 2 : cur - 1;  // (t + 2) % 3
+    if (t + 2 < nb) issue(wave + 4 * (t + 2), nxt2);
+    // block t has landed when only the loads of the blocks issued after it are outstanding
+    const long long later = nb - 1 - t < 2 ? nb - 1 - t : 2;
+    if (later == 2) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SK::LPB) : "memory");
+    } else if (later == 1) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SK::LPB) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
+    const char* wt = ring + cur * SK::STG;
+    const char* xt = wt + SK::WT;
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
-      if (u == 1 && !two) break;
+    for (int j = 0; j < 4; j++) {
+      const vec8 wv = *(const vec8*)(wt + rd[j]);
 #pragma unroll
-      for (int j = 0; j < 4; j++)
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++) acc[mb] = TR::mfma32(wv[u][j], xv[u][mb][j], acc[mb]);
+      for (int mb = 0; mb < MB; mb++) acc[mb] = TR::mfma32(wv, *(const vec8*)(xt + mb * 32 * 128 + rd[j]), acc[mb]);
     }
+    cur = cur == 2 ? 0 : cur + 1;
   }
+  __syncthreads();  // every ring is drained: the partial sums of wavefronts 1-3 take their place
+  float* part = (float*)smem;
   if (wave > 0) {
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) part[wave - 1][mb][r][lane] = acc[mb][r];
+      for (int r = 0; r < 16; r++) part[(((wave - 1) * MB + mb) * 16 + r) * 64 + lane] = acc[mb][r];
   }
   __syncthreads();
   if (wave != 0) return;
@@ -301,7 +348,9 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int r = 4 * rg + i;
-        float sum = acc[mb][r] + part[0][mb][r][lane] + part[1][mb][r][lane] + part[2][mb][r][lane];
+        float sum = acc[mb][r];
+#pragma unroll
+        for (int w = 0; w < 3; w++) sum += part[((w * MB + mb) * 16 + r) * 64 + lane];
         if (a.bias && n + i < a.N) sum += load_as_float((const T*)a.bias + n + i);
         v[i] = sum;
       }
@@ -312,16 +361,21 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
   }
 }
 
-template <typename TR>
-int launch_skinny(const LinArgs& a, hipStream_t stream) {
+template <typename TR, int MB>
+int launch_skinny_mb(const LinArgs& a, hipStream_t stream) {
+  static hipError_t state[kMaxDevices];
+  static bool done[kMaxDevices];
+  const hipError_t granted = grant_dynamic_lds((const void*)linear_skinny_kernel<TR, MB>, Skinny<MB>::LDS, state, done);
+  if (granted != hipSuccess) return (int)granted;
   const long long nwg = (a.N + 31) / 32;
   if (nwg > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
-  if (a.M <= 32) {
-    hipLaunchKernelGGL((linear_skinny_kernel<TR, 1>), dim3((unsigned)nwg), dim3(256), 0, stream, a);
-  } else {
-    hipLaunchKernelGGL((linear_skinny_kernel<TR, 2>), dim3((unsigned)nwg), dim3(256), 0, stream, a);
-  }
+  hipLaunchKernelGGL((linear_skinny_kernel<TR, MB>), dim3((unsigned)nwg), dim3(256), Skinny<MB>::LDS, stream, a);
   return (int)hipGetLastError();
+}
+
+template <typename TR>
+int launch_skinny(const LinArgs& a, hipStream_t stream) {
+  return a.M <= 32 ? launch_skinny_mb<TR, 1>(a, stream) : launch_skinny_mb<TR, 2>(a, stream);
 }
 
 // Any element type and shape: 64 x 64 output tile per workgroup, 4 x 4 outputs per lane, K in steps of 16 through LDS.
