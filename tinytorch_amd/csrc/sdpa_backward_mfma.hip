@@ -839,6 +839,225 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
   }
 }
 
+// ---- kernel 1 for head_dim 128 without an attnMask: the same products, K / V tiles by direct global->LDS loads ----------
+// As in backward_dkv128_kernel: unpadded 256-byte rows, chunk c of row r at slot c ^ f(r), so one copy of the K tile
+// serves the row-major reads (S^T = K.Q^T) and the transposed ones (dq^T += K^T.dS^T); a three-stage ring of 32-key tiles
+// per workgroup, the loads of tile j+2 in flight while tile j is computed; no staging registers.
+namespace dq128 {
+using dkv128::ROW_BYTES;
+using dkv128::swz;
+constexpr int BN = 32;                        // keys per tile
+constexpr int TILE_BYTES = BN * ROW_BYTES;    // one tile of K or V
+constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+constexpr int NSTAGE = 3;
+constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
+}  // namespace dq128
+
+template <typename TR, bool CAUSAL>
+__global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
+  using namespace dq128;
+  constexpr int D = 128;
+  typedef typename TR::elem T;
+  typedef typename TR::vec8 vec8;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  constexpr int KSTEPS = D / 16, DBLK = D / 32;
+  const KArgs& f = a.f;
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const unsigned smem_addr = (unsigned)(unsigned long)(lds_void*)smem;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, lh = lane >> 5;
+
+  const int ntile = (f.L + BM - 1) / BM;
+  int pair, in;
+  map_workgroup(blockIdx.x, f.B * f.Hq, ntile, &pair, &in);
+  const int h = pair % f.Hq, b = pair / f.Hq;
+  const int hk = h / f.G;
+  const int rt = CAUSAL ? ntile - 1 - in : in;  // longest rows first
+  const int q0 = rt * BM, qw0 = q0 + wave * 32;
+  const bool wave_live = qw0 < f.L;
+
+  // ---- this lane's query row: q and dout as B operands, delta = dout . out ------------------------------------------------
+  vec8 qreg[KSTEPS], greg[KSTEPS];
+  float delta;
+  {
+    int row = qw0 + lq;
+    row = row < f.L ? row : f.L - 1;
+    const T* qr = (const T*)f.q + b * f.qs[0] + h * f.qs[1] + row * f.qs[2] + 8 * lh;
+    const T* gr = (const T*)a.dout + b * a.dos[0] + h * a.dos[1] + row * a.dos[2] + 8 * lh;
+    const T* orow = (const T*)f.out + b * f.os[0] + h * f.os[1] + row * f.os[2] + 8 * lh;
+    float part = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      qreg[ks] = *(const vec8*)(qr + 16 * ks);
+      greg[ks] = *(const vec8*)(gr + 16 * ks);
+      const vec8 o = *(const vec8*)(orow + 16 * ks);
+#pragma unroll
+      for (int i = 0; i < 8; i++) part = fmaf((float)o[i], (float)greg[ks][i], part);
+    }
+    delta = part + __shfl_xor(part, 32);
+  }
+
+  f32x16 dqacc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dqacc[i][r] = 0.f;
+  const float c = f.scale * kLog2e;
+  const float lazy = kLazyExp / c;
+  float m_use = -1e30f, mc = m_use * c, l_run = 0.f;
+
+  const int S = keys_of_batch(f, b);
+  if (S == 0) {  // no keys (an empty cache entry): the output did not depend on q
+    const int qi = qw0 + lq;
+    if (qi < f.L) {
+      T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
+      typename TR::vec4 zero;
+#pragma unroll
+      for (int i = 0; i < 4; i++) zero[i] = (T)0.f;
+      for (int d = 4 * lh; d < D; d += 8) *(typename TR::vec4*)(dqp + d) = zero;
+    }
+    return;
+  }
+  const int coff = CAUSAL ? causal_offset(f, S) : 0;
+  int ntiles_kv = (S + BN - 1) / BN;
+  if (CAUSAL) {
+    const int last = (q0 + BM - 1 < f.L - 1 ? q0 + BM - 1 : f.L - 1) + coff;  // last key any row of the workgroup sees
+    const int lastkv = last < S - 1 ? last : S - 1;
+    ntiles_kv = lastkv / BN + 1;
+  }
+
+  auto dma16 = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+  };
+  const int drow = lane >> 4, dslot = lane & 15;
+  const T* kp = (const T*)f.k + b * f.ks[0] + hk * f.ks[1];
+  const T* vp = (const T*)f.v + b * f.vs[0] + hk * f.vs[1];
+  // wavefront w brings rows 8w .. 8w+7 of the K tile and of the V tile: two loads each
+  auto dma_tile = [&](int jt, int stage) __attribute__((always_inline)) {
+    const int kv0 = jt * BN;
+    const char* kb = (const char*)(kp + (long long)kv0 * f.ks[2]);
+    const char* vb = (const char*)(vp + (long long)kv0 * f.vs[2]);
+    const unsigned at = smem_addr + stage * STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const int row = 8 * wave + 4 * i + drow;
+      const int rowc = kv0 + row < S ? row : S - 1 - kv0;  // rows past the end re-read the last key (hidden below)
+      const unsigned chunk = (unsigned)(dslot ^ swz(row));
+      dma16(kb, ((unsigned)rowc * (unsigned)f.ks[2] + 8u * chunk) * 2u, at + (8 * wave + 4 * i) * ROW_BYTES);
+      dma16(vb, ((unsigned)rowc * (unsigned)f.vs[2] + 8u * chunk) * 2u, at + TILE_BYTES + (8 * wave + 4 * i) * ROW_BYTES);
+    }
+  };
+  const unsigned r_base = (unsigned)(lq * ROW_BYTES + 16 * (lh ^ swz(lq)));
+  unsigned t_base[2];
+  {
+    const int s = lane & 15, dhalf = (lane >> 4) & 1;
+#pragma unroll
+    for (int ld = 0; ld < 2; ld++) {
+      const int row = 8 * ld + 4 * lh + (s >> 2);
+      const int c0 = 2 * dhalf + ((s & 3) >> 1);
+      t_base[ld] = (unsigned)(row * ROW_BYTES + 16 * (c0 ^ swz(row)) + 8 * (s & 1));
+    }
+  }
+
+  dma_tile(0, 0);
+  if (1 < ntiles_kv) dma_tile(1, 1);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  int cur = 0;
+  for (int jt = 0; jt < ntiles_kv; jt++) {
+    const int kv0 = jt * BN;
+    const int nxt2 = cur == 0 ? 2 : cur - 1;  // (jt + 2) % 3: last read in iteration jt-1, which a barrier ended
+    const bool more = jt + 2 < ntiles_kv;
+    if (more) dma_tile(jt + 2, nxt2);
+    if (wave_live && (!CAUSAL || kv0 <= qw0 + 31 + coff)) {
+      const char* kt = smem + cur * STAGE_BYTES;
+      const char* vt = kt + TILE_BYTES;
+      f32x16 sacc, dpacc;
+#pragma unroll
+      for (int r = 0; r < 16; r++) sacc[r] = 0.f, dpacc[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) sacc = TR::mfma32(*(const vec8*)(kt + (r_base ^ (unsigned)(32 * ks))), qreg[ks], sacc);
+      if ((CAUSAL && kv0 + BN - 1 > qw0 + coff) || kv0 + BN > S) {
+        const int qi = qw0 + lq + coff;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          if (key >= S || (CAUSAL && key > qi)) sacc[r] = -INFINITY;
+        }
+      }
+      float mloc = sacc[0];
+#pragma unroll
+      for (int r = 1; r < 16; r++) mloc = fmaxf(mloc, sacc[r]);
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+      if (__builtin_amdgcn_ballot_w64(mloc > m_use + lazy) != 0) {
+        const float m_new = fmaxf(m_use, mloc);
+        const float alpha = fast_exp2((m_use - m_new) * c);
+        m_use = m_new;
+        mc = m_new * c;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DBLK; i++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) dqacc[i][r] *= alpha;
+      }
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) dpacc = TR::mfma32(*(const vec8*)(vt + (r_base ^ (unsigned)(32 * ks))), greg[ks], dpacc);
+      float psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float p = fast_exp2(fmaf(sacc[r], c, -mc));  // relative to m_use; normalised at the end
+        psum += p;
+        sacc[r] = p * (dpacc[r] - delta);
+      }
+      l_run += psum;
+      vec8 dsb[2];
+#pragma unroll
+      for (int t = 0; t < 2; t++) dsb[t] = regs_to_operand<vec8>(sacc, t);
+#pragma unroll
+      for (int db = 0; db < DBLK; db++)
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const unsigned lo = (t_base[0] ^ (unsigned)(64 * db)) + 16 * t * ROW_BYTES, hi = (t_base[1] ^ (unsigned)(64 * db)) + 16 * t * ROW_BYTES;
+          const s16x4 klo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(kt + lo));
+          const s16x4 khi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(kt + hi));
+          dqacc[db] = TR::mfma32(__builtin_bit_cast(vec8, __builtin_shufflevector(klo, khi, 0, 1, 2, 3, 4, 5, 6, 7)), dsb[t], dqacc[db]);
+        }
+    }
+    // tile jt+1 must have landed before the next iteration; the four loads of tile jt+2 may stay in flight
+    if (more) {
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    cur = cur == 2 ? 0 : cur + 1;
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const int qi = qw0 + lq;
+  if (qi < f.L) {
+    const long long row_id = ((long long)b * f.Hq + h) * f.L + qi;
+    if (lh == 0) *(float2*)(a.stats + 2 * row_id) = make_float2(m_use * c + __log2f(l_tot), delta);
+    const float w = f.scale / l_tot;
+    T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
+#pragma unroll
+    for (int db = 0; db < DBLK; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        f32x4 x;
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = dqacc[db][4 * rg + i] * w;
+        *(typename TR::vec4*)(dqp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
+      }
+  }
+}
+
 template <typename TR, int D, bool CAUSAL, bool MASKED>
 int launch_k(const BwdArgs& a, hipStream_t stream) {
   typedef BwdLds<D> Lds;
@@ -847,7 +1066,8 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   constexpr bool DMA = D == 128 && !MASKED;
   static hipError_t state1[kMaxDevices], state2[kMaxDevices];
   static bool done1[kMaxDevices], done2[kMaxDevices];
-  hipError_t e = grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED>, DqTile<D>::BYTES, state1, done1);
+  hipError_t e = DMA ? grant_dynamic_lds((const void*)backward_dq128_kernel<TR, CAUSAL>, dq128::LDS_BYTES, state1, done1)
+                     : grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED>, DqTile<D>::BYTES, state1, done1);
   if (e != hipSuccess) return (int)e;
   if (DMA) {
     e = grant_dynamic_lds((const void*)backward_dkv128_kernel<TR, CAUSAL>, dkv128::LDS_BYTES, state2, done2);
@@ -857,7 +1077,11 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM);
-  hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED>), dim3((unsigned)g1), dim3(256), DqTile<D>::BYTES, stream, a);
+  if (DMA) {
+    hipLaunchKernelGGL((backward_dq128_kernel<TR, CAUSAL>), dim3((unsigned)g1), dim3(256), dq128::LDS_BYTES, stream, a);
+  } else {
+    hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED>), dim3((unsigned)g1), dim3(256), DqTile<D>::BYTES, stream, a);
+  }
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   if (DMA) {

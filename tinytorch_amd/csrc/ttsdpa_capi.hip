@@ -231,7 +231,9 @@ bool backward_mfma_ok(const ttsdpa_backward_params* p) {
       !dense_last_ok(p->dv_stride, 8))
     return false;
   // the head_dim-128 dk/dv kernel addresses the rows of a tile with 32-bit byte offsets from the tile's first row
-  if (f->D == 128 && (f->q_stride[2] >= (1 << 24) || f->v_stride[2] >= (1 << 24) || p->dout_stride[2] >= (1 << 24))) return false;
+  if (f->D == 128 && (f->q_stride[2] >= (1 << 24) || f->k_stride[2] >= (1 << 24) || f->v_stride[2] >= (1 << 24) ||
+                      p->dout_stride[2] >= (1 << 24)))
+    return false;
   return ptr_aligned(p->dout, 16) && ptr_aligned(p->dq, 16) && ptr_aligned(p->dk, 16) && ptr_aligned(p->dv, 16);
 }
 
