@@ -369,7 +369,7 @@ def run_backward(steps, warmup, cpu=True):
            "route": _capi.ROUTE_NAMES[route.value], "ms_per_step": round(ms, 5), "value": round(tf, 1), "unit": "TFLOP/s",
            "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
                         "frac": round(tf / PEAK_TFLOPS["bf16"], 4), "traffic": measured_traffic("backward"),
-                        "algorithmic_flops": flops, "kernels": "backward_dq_mfma_kernel + backward_dkv128_kernel per step"}}
+                        "algorithmic_flops": flops, "kernels": "backward_dq128_kernel + backward_dkv128_kernel per step"}}
     if cpu:
         import oracle
         # the causal top-left corner is a problem of its own for dq: rows below n see keys below n only
