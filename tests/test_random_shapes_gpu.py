@@ -65,3 +65,66 @@ def test_random_shape(case):
     torch.cuda.synchronize()
     exp = oracle.sdpa_f32(*host, **kw_host)
     assert max_abs_err(out, exp) <= TOL[dtype], route_of(*dev, causal=extra == "causal")
+
+
+def _backward_cases():
+    rng = np.random.RandomState(20240911)
+    out = []
+    for i in range(40):
+        dtype = ["bf16", "f16", "f32"][rng.randint(3)]
+        D = [128, 128, 64, 64, 32, 80][rng.randint(6)]
+        Hkv = int(rng.randint(1, 3))
+        G = [1, 1, 2, 4, 3][rng.randint(5)]
+        B = int(rng.randint(1, 3))
+        L = int(rng.randint(1, 330))
+        S = L if rng.rand() < 0.4 else int(rng.randint(1, 400))
+        extra = ["none", "causal", "causal-br", "boolmask", "addmask", "kvlen", "boolmask4"][rng.randint(7)]
+        if extra == "boolmask4":
+            S = (S + 3) // 4 * 4   # keys readable four at a time: the MFMA pair's masks
+        out.append((i, dtype, B, Hkv * G, Hkv, L, S, D, extra))
+    return out
+
+
+@pytest.mark.parametrize("case", _backward_cases(), ids=lambda c: "%d-%s-B%d-H%d/%d-L%d-S%d-D%d-%s" % c)
+def test_random_backward_shape(case):
+    """The same idea for ttsdpa_backward: both kernel families, ragged tiles on both sides, grouped heads, both causal
+    alignments, masks, per-batch key counts — against the oracle's gradients."""
+    from gpu_util import backward_route_of, grad_err
+    from tinytorch_amd import sdpAttentionBackward
+    i, dtype, B, Hq, Hkv, L, S, D, extra = case
+    host, dev = make_inputs(5000 + i, B, Hq, Hkv, L, S, D, dtype)
+    go_h, go_b = oracle.round_to(oracle.randn(5000 + i, 9, host[0].shape), dtype)
+    go = to_device(go_h, go_b, dtype)
+    kw, mask_h, lens = {}, None, None
+    if extra == "causal":
+        kw["isCausal"] = True
+        mask_h = np.arange(S)[None, :] <= np.arange(L)[:, None]
+        if S < L:
+            mask_h = mask_h.copy()   # rows past S see every key: nothing to fix, the tril covers it
+    elif extra == "causal-br":
+        kw.update(isCausal=True, causalAlign="bottom-right")
+        mask_h = np.arange(S)[None, :] <= np.arange(L)[:, None] + max(0, S - L)
+    elif extra in ("boolmask", "boolmask4"):
+        mask_h = np.random.RandomState(i).rand(B, 1, L, S) > 0.4
+        mask_h[..., 0] = True
+        kw["attnMask"] = torch.from_numpy(mask_h).cuda()
+    elif extra == "addmask":
+        mask_h, bits = oracle.round_to(oracle.randn(6000 + i, 5, (Hq, 1, S)), dtype)
+        kw["attnMask"] = to_device(mask_h, bits, dtype)
+    elif extra == "kvlen":
+        lens = np.random.RandomState(i).randint(1, S + 1, size=B).astype(np.int32)
+        kw["kvLens"] = torch.from_numpy(lens).cuda()
+    out = sdpAttention(*dev, **kw)
+    dq, dk, dv = sdpAttentionBackward(go, *dev, out, **kw)
+    torch.cuda.synchronize()
+    if lens is not None:
+        for b in range(B):
+            n = int(lens[b])
+            eq, ek, ev = oracle.sdpa_backward_f32(host[0][b:b + 1], host[1][b:b + 1, :, :n], host[2][b:b + 1, :, :n], go_h[b:b + 1])
+            assert grad_err(dq[b:b + 1], eq) <= TOL[dtype] and grad_err(dk[b:b + 1, :, :n], ek) <= TOL[dtype]
+            assert grad_err(dv[b:b + 1, :, :n], ev) <= TOL[dtype]
+            assert torch.all(dk[b, :, n:] == 0) and torch.all(dv[b, :, n:] == 0)
+        return
+    eq, ek, ev = oracle.sdpa_backward_f32(*host, go_h, mask=mask_h)
+    for name, got, exp in (("dq", dq, eq), ("dk", dk, ek), ("dv", dv, ev)):
+        assert grad_err(got, exp) <= TOL[dtype], name
