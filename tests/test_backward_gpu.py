@@ -249,6 +249,25 @@ def test_backward_strided_views_and_scale():
         assert grad_err(got, exp) <= TOL["f32"]
 
 
+def test_backward_mfma_packed_projection_views():
+    """bf16 q/k/v as slices of one packed QKV projection output [B, N, 3, H, D] and the gradients written into slices of
+    one packed buffer: row strides of 3*H*D elements on the MFMA pair (head_dim 128, the direct-load kernels)."""
+    B, H, N, D = 2, 4, 300, 128
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    qkv = torch.randn(B, N, 3, H, D, device="cuda", generator=gen).bfloat16()
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    go = torch.randn(B, H, N, D, device="cuda", generator=gen).bfloat16()
+    out = sdpAttention(q, k, v, isCausal=True)
+    assert backward_route_of(q, k, v, out, go, True) == "prefill"
+    dqkv = torch.full_like(qkv, float("nan"))
+    grads = tuple(dqkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    rc, _ = backward_call(q, k, v, out, go, causal=True, grads=grads)
+    assert rc == 0 and torch.isfinite(dqkv).all()
+    eq, ek, ev = oracle.sdpa_backward_f32(to_host_f32(q), to_host_f32(k), to_host_f32(v), to_host_f32(go), causal=True)
+    for got, exp in zip(grads, (eq, ek, ev)):
+        assert grad_err(got, exp) <= TOL["bf16"]
+
+
 def test_backward_validation_and_empty_shapes():
     from tinytorch_amd import _capi
     q = torch.randn(1, 2, 4, 64, device="cuda")
