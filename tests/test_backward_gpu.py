@@ -51,6 +51,9 @@ GENERAL_CASES = [
     (2, 8, 2, 70, 130, 40, "f32", False),      # grouped heads, head_dim not a multiple of 64
     (1, 4, 2, 65, 20, 96, "f32", True),        # L > S, top-left causal: rows past S see every key
     (1, 2, 1, 17, 200, 256, "f32", False),     # the largest head_dim
+    (2, 4, 2, 70, 45, 160, "f32", True),       # head_dim in (128, 256]: eight lanes per row, 16-row tiles
+    (1, 6, 2, 40, 90, 136, "bf16", True),
+    (1, 2, 2, 33, 64, 256, "f16", False),
     (2, 4, 2, 50, 77, 64, "bf16", True),
     (2, 4, 2, 50, 77, 128, "f16", False),
     (1, 6, 3, 129, 64, 32, "bf16", False),
