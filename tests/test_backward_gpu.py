@@ -77,6 +77,15 @@ MFMA_CASES = [
     (1, 2, 2, 1, 129, 128, "bf16", False),        # one query row
     (1, 2, 1, 300, 17, 64, "f16", "br"),          # more queries than keys, bottom-right: offset 0
     (3, 4, 2, 33, 257, 128, "f16", False),
+    # fp32 tensors: the fp32 matrix-core pair
+    (2, 8, 2, 256, 256, 128, "f32", True),
+    (1, 4, 4, 200, 333, 64, "f32", False),
+    (2, 6, 2, 130, 70, 128, "f32", True),
+    (1, 8, 8, 64, 500, 128, "f32", "br"),
+    (2, 4, 1, 96, 96, 64, "f32", True),
+    (1, 2, 2, 1, 129, 128, "f32", False),
+    (1, 2, 1, 300, 17, 64, "f32", "br"),
+    (3, 4, 2, 33, 257, 128, "f32", False),
 ]
 
 
@@ -205,7 +214,7 @@ def test_backward_bottom_right_causal_and_key_counts(dtype):
         assert torch.all(dk[b, :, lens[b]:] == 0) and torch.all(dv[b, :, lens[b]:] == 0)
 
 
-@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64)])
+@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64), ("f32", 128), ("f32", 64)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_backward_mfma_per_batch_key_counts(dtype, D, causal):
     """kv_len on the MFMA pair: each batch entry against the oracle on its own key prefix (bottom-right causal when

@@ -42,15 +42,6 @@ __device__ __forceinline__ float biased_score(const KArgs& f, float dot, int i, 
   return hidden ? -INFINITY : x;
 }
 
-__device__ __forceinline__ int keys_of_batch(const KArgs& f, int b) {
-  int S = f.S;
-  if (f.kv_len) {
-    int len = f.kv_len[b];
-    S = len < 0 ? 0 : (len < S ? len : S);
-  }
-  return S;
-}
-
 // ---- 64 rows per workgroup with four adjacent lanes per row (head_dim <= 128), 32 rows with eight (<= 256) ----
 // The layout of the general forward kernel: lane s of the LPR holds head_dim elements s, s+LPR, s+2*LPR, ... of its
 // row's vectors in registers; the other side streams through LDS as fp32 tiles of 32 / 16 rows, read as broadcasts.

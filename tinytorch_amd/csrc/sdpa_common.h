@@ -178,7 +178,43 @@ struct BwdArgs {
   float* stats;
 };
 int launch_backward_general(const BwdArgs& a, int dtype, hipStream_t stream);
-int launch_backward_mfma(const BwdArgs& a, int dtype, hipStream_t stream);  // fp16/bf16, head_dim 64 or 128, no attnMask / kv_len
+int launch_backward_mfma(const BwdArgs& a, int dtype, hipStream_t stream);  // fp16/bf16, head_dim 64 or 128
+int launch_backward_f32(const BwdArgs& a, hipStream_t stream);              // fp32 on the fp32 matrix cores, head_dim 64 or 128, no attnMask
+
+// Workgroup n -> (pair, block) for npair (batch, head) pairs of nblk blocks each, block 0 the longest under a causal
+// mask.  Workgroups are handed to the 8 XCDs round-robin (n % 8) and start in order: every XCD gets whole pairs (a
+// contiguous range, so the heads of a group share its L2) and takes their blocks longest first across all its pairs,
+// which keeps the XCDs evenly loaded and the short blocks for the end.  Without a multiple of 8 pairs: longest first
+// over all pairs.
+__device__ __forceinline__ void map_workgroup(int n, int npair, int nblk, int* pair, int* blk) {
+  if ((npair & 7) == 0) {
+    const int xcd = n & 7, slot = n >> 3, ppx = npair >> 3;
+    *blk = slot / ppx;
+    *pair = xcd * ppx + slot % ppx;
+  } else {
+    *blk = n / npair;
+    *pair = n % npair;
+  }
+}
+
+// head_dim 128 needs more than 256 registers per lane: one wavefront per SIMD, the gradient accumulators in the
+// accumulation registers.  Pinning them there at the end of every iteration keeps the loop-carried values in that
+// register class, so the matrix instructions accumulate in place instead of being fed through copies (128 moves each
+// way per tile otherwise).
+template <bool PIN>
+__device__ __forceinline__ void pin_accumulator(f32x16& acc) {
+  if constexpr (PIN) asm volatile("" : "+a"(acc));
+}
+
+// Keys of batch entry b: all S of them, or the filled prefix of a cache / the unpadded length (kv_len).
+__device__ __forceinline__ int keys_of_batch(const KArgs& f, int b) {
+  int S = f.S;
+  if (f.kv_len) {
+    const int len = __builtin_amdgcn_readfirstlane(f.kv_len[b]);
+    S = len < 0 ? 0 : (len < S ? len : S);
+  }
+  return S;
+}
 
 // Host-side launchers (one per kernel family); each returns a hipError_t as int.
 int launch_general(const KArgs& a, int dtype, hipStream_t stream);

@@ -237,10 +237,23 @@ bool backward_mfma_ok(const ttsdpa_backward_params* p) {
   return ptr_aligned(p->dout, 16) && ptr_aligned(p->dq, 16) && ptr_aligned(p->dk, 16) && ptr_aligned(p->dv, 16);
 }
 
+// The fp32 matrix-core backward kernels: fp32 tensors with 16-byte aligned rows, head_dim 64 or 128, no attnMask.
+bool backward_f32_ok(const ttsdpa_backward_params* p) {
+  const ttsdpa_params* f = &p->fwd;
+  if (f->dtype != TTSDPA_F32 || f->block_table || f->mask_kind != TTSDPA_MASK_NONE || (f->D != 64 && f->D != 128)) return false;
+  if (!(f->scale > 0.f) || !isfinite(f->scale) || f->L < 1 || f->S < 1) return false;  // the row maximum is taken on unscaled scores
+  if (!dense_last_ok(f->q_stride, 4) || !dense_last_ok(f->k_stride, 4) || !dense_last_ok(f->v_stride, 4) ||
+      !dense_last_ok(f->o_stride, 4) || !dense_last_ok(p->dout_stride, 4) || !dense_last_ok(p->dq_stride, 4) ||
+      !dense_last_ok(p->dk_stride, 4) || !dense_last_ok(p->dv_stride, 4))
+    return false;
+  return ptr_aligned(f->q, 16) && ptr_aligned(f->k, 16) && ptr_aligned(f->v, 16) && ptr_aligned(f->out, 16) &&
+         ptr_aligned(p->dout, 16) && ptr_aligned(p->dq, 16) && ptr_aligned(p->dk, 16) && ptr_aligned(p->dv, 16);
+}
+
 int pick_backward_route(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
   if (f->B == 0 || (f->L == 0 && f->S == 0)) return TTSDPA_ROUTE_NONE;
-  return backward_mfma_ok(p) ? TTSDPA_ROUTE_PREFILL : TTSDPA_ROUTE_GENERAL;
+  return backward_mfma_ok(p) || backward_f32_ok(p) ? TTSDPA_ROUTE_PREFILL : TTSDPA_ROUTE_GENERAL;
 }
 
 size_t backward_stats_bytes(const ttsdpa_backward_params* p) {
@@ -411,6 +424,7 @@ int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t wor
   if (route == TTSDPA_ROUTE_PREFILL) {
     const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + 127) / 128), g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + 127) / 128);
     if (check_grid(g1) != TTSDPA_OK || check_grid(g2) != TTSDPA_OK) return TTSDPA_ERR_SHAPE;
+    if (p->fwd.dtype == TTSDPA_F32) return launch_backward_f32(a, (hipStream_t)stream);
     return launch_backward_mfma(a, p->fwd.dtype, (hipStream_t)stream);
   }
   return launch_backward_general(a, p->fwd.dtype, (hipStream_t)stream);
