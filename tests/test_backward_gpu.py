@@ -150,7 +150,7 @@ def test_backward_with_masks(dtype, kind):
     check("mask-%s-%s" % (kind, dtype), host, dev, dtype, mask_h=m, mask_d=md, route="general")
 
 
-@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64)])
+@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64), ("f32", 128), ("f32", 64)])
 @pytest.mark.parametrize("kind", ["bool", "add", "keypad", "perhead", "hiddenrow"])
 def test_backward_mfma_with_masks(dtype, D, kind):
     """attnMasks the MFMA pair takes (contiguous keys, S a multiple of 4): Bool [L,S], additive [L,S], key padding

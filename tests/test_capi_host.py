@@ -320,8 +320,16 @@ def test_backward_params_layout_routes_and_validation():
     bp.fwd.block_table = None
     bp.struct_size -= 8
     assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == _capi.ERR_ABI
-    # fp32 and masks: the vector-ALU kernels
+    # fp32: the fp32 matrix-core pair at head_dim 64 / 128 with 16-byte aligned rows, else the vector-ALU kernels
     L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.F32, 1, 4, 4, 32, 32, 64)
+    bp.fwd.q = bp.fwd.k = bp.fwd.v = bp.fwd.out = bp.dout = bp.dq = bp.dk = bp.dv = FAKE
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_PREFILL
+    bp.dq_stride[2] = 66
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_GENERAL
+    bp.dq_stride[2] = 64
+    bp.fwd.k = FAKE + 4
+    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_GENERAL
+    L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.F32, 1, 4, 4, 32, 32, 96)
     bp.fwd.q = bp.fwd.k = bp.fwd.v = bp.fwd.out = bp.dout = bp.dq = bp.dk = bp.dv = FAKE
     assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_GENERAL
     L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.F32, 0, 4, 4, 32, 32, 64)

@@ -1,7 +1,7 @@
 // Attention backward for fp32 tensors on the gfx950 fp32 matrix cores (v_mfma_f32_32x32x2_f32: full fp32 products and
-// sums), head_dim 64 or 128, optional causal mask (either alignment), per-batch key counts, grouped heads.  fp32 is the
-// reference's default dtype.  The reference has no attention backward (reference src/Function/FuncNNLayer.h:267 is
-// NOT_IMPLEMENTED); this is the chain rule through its forward chain matmul -> scale -> softmax -> matmul
+// sums), head_dim 64 or 128, optional causal mask (either alignment) or attnMask, per-batch key counts, grouped heads.
+// fp32 is the reference's default dtype.  The reference has no attention backward (reference
+// src/Function/FuncNNLayer.h:267 is NOT_IMPLEMENTED); this is the chain rule through its forward chain matmul -> scale -> bias -> softmax -> matmul
 // (src/Function/FuncNNLayer.h:237-265, softmax step as src/Operation/OpNNLayerCpu.h:79-109):
 //   P_ij = exp(scale * q_i.k_j - lse_i)    dP_ij = dout_i.v_j    delta_i = dout_i.out_i    dS_ij = P_ij (dP_ij - delta_i)
 //   dq_i = scale * sum_j dS_ij k_j         dk_j = scale * sum_i dS_ij q_i                  dv_j = sum_i P_ij dout_i
@@ -76,7 +76,8 @@ __device__ __forceinline__ void load_half_row(const float* row, int lh, float (&
 }
 
 // ---- kernel 1: dq, lse, delta -------------------------------------------------------------------------------------
-template <int D, bool CAUSAL>
+// MASKED: an attnMask (exclusive with CAUSAL) whose keys can be read four at a time, as in the forward kernel.
+template <int D, bool CAUSAL, bool MASKED>
 __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(BwdArgs a) {
   typedef BwdF32Lds<D> Lds;
   constexpr int PITCH = Lds::PITCH, NLD = Lds::NLD, DBLK = D / 32;
@@ -202,6 +203,11 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
           if (key >= S || (CAUSAL && key > qi)) s[r] = -INFINITY;
         }
       }
+      if (MASKED) {
+        int qi = qw0 + lq;
+        qi = qi < f.L ? qi : f.L - 1;
+        apply_attn_mask<float, true>(f, s, b * f.ms[0] + h * f.ms[1] + qi * f.ms[2], kv0, lh, S, 1.f / f.scale);
+      }
       float mloc = s[0];
 #pragma unroll
       for (int r = 1; r < 16; r++) mloc = fmaxf(mloc, s[r]);
@@ -244,8 +250,10 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
   if (qi < f.L) {
     const long long row_id = ((long long)b * f.Hq + h) * f.L + qi;
     // log2 of the row's sum of exponentials, the unit the second kernel's exp2 wants
-    if (lh == 0) *(float2*)(a.stats + 2 * row_id) = make_float2(m_use * c + __log2f(l_tot), delta);
-    const float w = f.scale / l_tot;
+    // a row whose keys are all hidden (possible with an attnMask): dq = 0, and a statistic that gives it weight 0 below
+    const bool seen = l_tot > 0.f;
+    if (lh == 0) *(float2*)(a.stats + 2 * row_id) = make_float2(seen ? m_use * c + __log2f(l_tot) : 1e30f, delta);
+    const float w = seen ? f.scale / l_tot : 0.f;
     float* dqp = (float*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
 #pragma unroll
     for (int db = 0; db < DBLK; db++)
@@ -253,15 +261,17 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
       for (int rg = 0; rg < 4; rg++) {
         f32x4 x;
 #pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = dqacc[db][4 * rg + i] * w;
+        for (int i = 0; i < 4; i++) x[i] = seen ? dqacc[db][4 * rg + i] * w : 0.f;
         *(f32x4*)(dqp + 32 * db + 8 * rg + 4 * lh) = x;
       }
   }
 }
 
 // ---- kernel 2: dk, dv -----------------------------------------------------------------------------------------------
-template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_f32_kernel(BwdArgs a) {
+// MASKED reads one mask value per score (a key is a lane column here, the mask's rows run across registers); with its
+// addressing the head_dim-64 variant no longer fits two wavefronts per SIMD either.
+template <int D, bool CAUSAL, bool MASKED>
+__global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_f32_kernel(BwdArgs a) {
   typedef BwdF32Lds<D> Lds;
   constexpr int PITCH = Lds::PITCH, NLD = Lds::NLD, DBLK = D / 32;
   const KArgs& f = a.f;
@@ -370,6 +380,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_f32_kernel
       if (idx + 2 < total) load_tile(idx + 2);
     }
     const int i0 = (ntq - 1 - idx / f.G) * BT;
+    const int h_of_tile = hk * f.G + idx % f.G;
     if (wave_live && (!CAUSAL || kw0 <= i0 + BT - 1 + coff)) {
       const float* Qs = smem + cur * Lds::STAGE;
       const float* Gs = Qs + Lds::TILE;
@@ -388,7 +399,18 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_f32_kernel
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 4 * rg + e;
-          const float p = fast_exp2(fmaf(s[r], c, -lse2[e]));
+          float bias2 = 0.f;  // attnMask: the additive bias in log2 units, or -inf for a hidden key
+          if (MASKED) {
+            int qrow = i0 + 8 * rg + 4 * lh + e;
+            qrow = qrow < f.L ? qrow : f.L - 1;
+            const long long at = b * f.ms[0] + h_of_tile * f.ms[1] + qrow * f.ms[2] + (key < S ? key : S - 1) * f.ms[3];
+            if (f.mask_kind == 1) {
+              bias2 = ((const uint8_t*)f.mask)[at] == 0 ? -INFINITY : 0.f;
+            } else {
+              bias2 = ((const float*)f.mask)[at] * kLog2e;
+            }
+          }
+          const float p = fast_exp2(fmaf(s[r], c, bias2 - lse2[e]));
           s[r] = p;
           dp[r] = p * (dp[r] - dl[e]);
         }
@@ -413,7 +435,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_f32_kernel
         }
     }
 #pragma unroll
-    for (int db = 0; db < DBLK; db++) pin_accumulator<(D > 64)>(dkacc[db]), pin_accumulator<(D > 64)>(dvacc[db]);
+    for (int db = 0; db < DBLK; db++) pin_accumulator<(D > 64 || MASKED)>(dkacc[db]), pin_accumulator<(D > 64 || MASKED)>(dvacc[db]);
     __syncthreads();
   }
 
@@ -431,28 +453,30 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_f32_kernel
   }
 }
 
-template <int D, bool CAUSAL>
+template <int D, bool CAUSAL, bool MASKED>
 int launch_k(const BwdArgs& a, hipStream_t stream) {
   static hipError_t state1[kMaxDevices], state2[kMaxDevices];
   static bool done1[kMaxDevices], done2[kMaxDevices];
-  hipError_t e = grant_dynamic_lds((const void*)backward_dq_f32_kernel<D, CAUSAL>, BwdF32Lds<D>::BYTES, state1, done1);
+  hipError_t e = grant_dynamic_lds((const void*)backward_dq_f32_kernel<D, CAUSAL, MASKED>, BwdF32Lds<D>::BYTES, state1, done1);
   if (e != hipSuccess) return (int)e;
-  e = grant_dynamic_lds((const void*)backward_dkv_f32_kernel<D, CAUSAL>, BwdF32Lds<D>::BYTES, state2, done2);
+  e = grant_dynamic_lds((const void*)backward_dkv_f32_kernel<D, CAUSAL, MASKED>, BwdF32Lds<D>::BYTES, state2, done2);
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM);
-  hipLaunchKernelGGL((backward_dq_f32_kernel<D, CAUSAL>), dim3((unsigned)g1), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
+  hipLaunchKernelGGL((backward_dq_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g1), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
-  hipLaunchKernelGGL((backward_dkv_f32_kernel<D, CAUSAL>), dim3((unsigned)g2), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
+  hipLaunchKernelGGL((backward_dkv_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g2), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
   return (int)hipGetLastError();
 }
 
 }  // namespace
 
 int launch_backward_f32(const BwdArgs& a, hipStream_t stream) {
-  if (a.f.D == 128) return a.f.causal ? launch_k<128, true>(a, stream) : launch_k<128, false>(a, stream);
-  return a.f.causal ? launch_k<64, true>(a, stream) : launch_k<64, false>(a, stream);
+  if (a.f.mask_kind != 0)  // exclusive with causal (validated by the caller, as the reference asserts)
+    return a.f.D == 128 ? launch_k<128, false, true>(a, stream) : launch_k<64, false, true>(a, stream);
+  if (a.f.D == 128) return a.f.causal ? launch_k<128, true, false>(a, stream) : launch_k<128, false, false>(a, stream);
+  return a.f.causal ? launch_k<64, true, false>(a, stream) : launch_k<64, false, false>(a, stream);
 }
 
 }  // namespace ttsdpa

@@ -179,7 +179,7 @@ struct BwdArgs {
 };
 int launch_backward_general(const BwdArgs& a, int dtype, hipStream_t stream);
 int launch_backward_mfma(const BwdArgs& a, int dtype, hipStream_t stream);  // fp16/bf16, head_dim 64 or 128
-int launch_backward_f32(const BwdArgs& a, hipStream_t stream);              // fp32 on the fp32 matrix cores, head_dim 64 or 128, no attnMask
+int launch_backward_f32(const BwdArgs& a, hipStream_t stream);              // fp32 on the fp32 matrix cores, head_dim 64 or 128
 
 // Workgroup n -> (pair, block) for npair (batch, head) pairs of nblk blocks each, block 0 the longest under a causal
 // mask.  Workgroups are handed to the 8 XCDs round-robin (n % 8) and start in order: every XCD gets whole pairs (a
