@@ -325,9 +325,10 @@ def run_linear(steps, warmup, cpu=True):
     return res
 
 
-def run_backward(steps, warmup, cpu=True):
-    """Attention backward (ttsdpa_backward) at config 3's shape, bf16, causal: dq, dk, dv per launch pair.  Flop count:
-    the textbook five matrix products (2.5 x the forward's), halved by the causal mask; the two kernels execute seven."""
+def run_backward(steps, warmup, cpu=True, dtype="bf16"):
+    """Attention backward (ttsdpa_backward) at config 3's shape, causal, bf16 or fp32 (the reference's default dtype, on
+    the fp32 matrix cores): dq, dk, dv per launch pair.  Flop count: the textbook five matrix products (2.5 x the
+    forward's), halved by the causal mask; the two kernels execute seven."""
     import ctypes
     import numpy as np
     import torch
@@ -337,10 +338,11 @@ def run_backward(steps, warmup, cpu=True):
     lib = _capi.lib()
     stream = torch.cuda.current_stream()
     gen = torch.Generator(device="cuda").manual_seed(0x5EED)
-    q = torch.randn(B, Hq, L, D, device="cuda", generator=gen).bfloat16()
-    k = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).bfloat16()
-    v = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).bfloat16()
-    go = torch.randn(B, Hq, L, D, device="cuda", generator=gen).bfloat16()
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    q = torch.randn(B, Hq, L, D, device="cuda", generator=gen).to(td)
+    k = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).to(td)
+    v = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).to(td)
+    go = torch.randn(B, Hq, L, D, device="cuda", generator=gen).to(td)
     out = sdpAttention(q, k, v, isCausal=True)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     bp = build_backward_params(q, k, v, out, go, dq, dk, dv, True)
@@ -365,11 +367,13 @@ def run_backward(steps, warmup, cpu=True):
     ms = e0.elapsed_time(e1) / steps
     flops = 2.5 * 4.0 * B * Hq * L * S * D * 0.5
     tf = flops / (ms * 1e-3) / 1e12
-    res = {"workload": "attention backward bf16 B%d %dq/%dkv L=S=%d D%d causal" % (B, Hq, Hkv, L, D), "dtype": "bf16",
+    kernels = "backward_dq128_kernel + backward_dkv128_kernel" if dtype == "bf16" else "backward_dq_f32_kernel + backward_dkv_f32_kernel"
+    res = {"workload": "attention backward %s B%d %dq/%dkv L=S=%d D%d causal" % (dtype, B, Hq, Hkv, L, D), "dtype": dtype,
            "route": _capi.ROUTE_NAMES[route.value], "ms_per_step": round(ms, 5), "value": round(tf, 1), "unit": "TFLOP/s",
-           "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
-                        "frac": round(tf / PEAK_TFLOPS["bf16"], 4), "traffic": measured_traffic("backward"),
-                        "algorithmic_flops": flops, "kernels": "backward_dq128_kernel + backward_dkv128_kernel per step"}}
+           "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_TFLOPS[dtype], "unit": "TFLOP/s",
+                        "frac": round(tf / PEAK_TFLOPS[dtype], 4),
+                        "traffic": measured_traffic("backward" if dtype == "bf16" else "backward_f32"),
+                        "algorithmic_flops": flops, "kernels": kernels + " per step"}}
     if cpu:
         import oracle
         # the causal top-left corner is a problem of its own for dq: rows below n see keys below n only
@@ -442,6 +446,7 @@ def main():
                     help="measure one row-wise op only and print its line (for profiling)")
     ap.add_argument("--linear-only", action="store_true", help="measure the linear layer only and print its line (for profiling)")
     ap.add_argument("--backward-only", action="store_true", help="measure the attention backward only and print its line (for profiling)")
+    ap.add_argument("--backward-dtype", choices=["bf16", "f32"], default="bf16", help="element type for --backward-only")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one device-to-device copy of 1 GiB (a kernel of known traffic that calibrates "
                          "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc)")
@@ -466,7 +471,8 @@ def main():
         print(json.dumps(run_linear(args.steps, args.warmup, cpu=not args.no_cpu)), flush=True)
         return
     if args.backward_only:
-        print(json.dumps(run_backward(args.steps, args.warmup, cpu=not args.no_cpu)), flush=True)
+        print(json.dumps(run_backward(args.steps, args.warmup, cpu=not args.no_cpu and args.backward_dtype == "bf16",
+                                      dtype=args.backward_dtype)), flush=True)
         return
     main_res, tensors = run_gpu(args.workload, args.steps, args.warmup)
     ceilings = None if args.no_probes else run_probes()
@@ -500,6 +506,7 @@ def main():
         line["linear"] = run_linear(max(1, min(args.steps, 100)), min(args.warmup, 50), cpu=not args.no_cpu)
         torch.cuda.empty_cache()
         line["backward"] = run_backward(max(1, min(args.steps, 50)), min(args.warmup, 20), cpu=not args.no_cpu)
+        line["backward"]["fp32"] = run_backward(max(1, min(args.steps, 10)), min(args.warmup, 3), cpu=False, dtype="f32")
     print(json.dumps(line), flush=True)
 
 
