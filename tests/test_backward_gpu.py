@@ -4,6 +4,8 @@ The reference has no attention backward (reference src/Function/FuncNNLayer.h:26
 gradients are pinned by differences, closed forms and invariants (tests/test_oracle_backward.py) rather than against
 reference vectors.  Bars: the forward's (fp32 1e-4, fp16/bf16 2e-2), in units of max(1, largest expected magnitude) —
 gradient entries are sums over many rows.  `out` handed to the backward is what the GPU forward produced."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -11,7 +13,7 @@ import torch
 import oracle
 from gpu_util import (TOL, TORCH_DTYPE, backward_call, backward_route_of, call, grad_err, make_inputs, to_device,
                       to_host_f32)
-from tinytorch_amd import sdpAttention, sdpAttentionBackward
+from tinytorch_amd import _capi, build_backward_params, sdpAttention, sdpAttentionBackward
 
 pytestmark = pytest.mark.gpu
 
@@ -244,6 +246,35 @@ def test_backward_mfma_per_batch_key_counts(dtype, D, causal):
         assert torch.all(dk[b, :, n:] == 0) and torch.all(dv[b, :, n:] == 0)
 
 
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("mode", ["causal", "full", "kvlen", "mask"])
+def test_backward_f32_split_query_stream(D, mode):
+    """fp32 matrix-core pair with few key blocks and a long query stream (4 heads x 17 tiles per KV head): the dk/dv
+    kernel deals the stream out to four workgroups per key block and a third kernel adds their partial sums.  The
+    scratch the library asks for holds the partials (more than the 8 bytes per query row of the statistics)."""
+    B, Hq, Hkv, L, S = 2, 8, 2, 520, 300
+    host, dev = make_inputs(4700 + D, B, Hq, Hkv, L, S, D, "f32")
+    q, k, v = dev
+    go = upstream(9, q.shape, "f32")[1]
+    out = sdpAttention(q, k, v, isCausal=(mode == "causal"))
+    bp = build_backward_params(q, k, v, out, go, torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), mode == "causal")
+    assert _capi.lib().ttsdpa_backward_workspace_bytes(ctypes.byref(bp)) >= B * Hq * L * 8 + 4 * 2 * B * Hkv * S * D * 4
+    if mode == "kvlen":
+        lens = [300, 129]
+        kv = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        m = np.zeros((B, 1, L, S), dtype=bool)
+        for b in range(B):
+            m[b, 0] = np.arange(S)[None, :] <= np.arange(L)[:, None] + max(0, lens[b] - L)
+            m[b, 0, :, lens[b]:] = False
+        check("split-kvlen-%d" % D, host, dev, "f32", causal=True, kv_lens=kv, align="bottom-right", oracle_mask=m, route="prefill")
+    elif mode == "mask":
+        m = np.random.default_rng(6).random((Hq, L, S)) < 0.6
+        m[..., 0] = True
+        check("split-mask-%d" % D, host, dev, "f32", mask_h=m, mask_d=torch.from_numpy(m).cuda(), route="prefill")
+    else:
+        check("split-%s-%d" % (mode, D), host, dev, "f32", causal=(mode == "causal"), route="prefill")
+
+
 def test_backward_strided_views_and_scale():
     """q/k/v as slices of one packed projection output, gradients into slices of one packed buffer."""
     B, H, N, D = 2, 4, 40, 64
@@ -281,7 +312,6 @@ def test_backward_mfma_packed_projection_views():
 
 
 def test_backward_validation_and_empty_shapes():
-    from tinytorch_amd import _capi
     q = torch.randn(1, 2, 4, 64, device="cuda")
     k = torch.randn(1, 2, 6, 64, device="cuda")
     v = torch.randn(1, 2, 6, 64, device="cuda")

@@ -14,7 +14,10 @@
 //      dP^T = V.dout^T, dS^T, dq^T += K^T.dS^T; at the end dq = scale/l * accumulator, (lse, delta) to scratch.
 //   2. backward_dkv_f32_kernel — a workgroup owns 128 keys of one (batch, kv head), a wavefront 32 of them, and streams
 //      the query rows of every head of the group in tiles of 32: S = Q.K^T, P from lse, dP = dout.V^T, dS,
-//      dv^T += dout^T.P, dk^T += Q^T.dS.
+//      dv^T += dout^T.P, dk^T += Q^T.dS.  When the launch has too few key blocks to fill and balance the chip (under a
+//      causal mask the first key block sees every query tile, the last one a few), the tiles of a key block's query
+//      stream are dealt out to 2-4 workgroups, which leave partial dk / dv in scratch, and
+//   3. backward_dkv_f32_sum_kernel adds the partials in a fixed order.
 // In the score products MFMA ks contracts head_dim elements ks (lanes 0-31) and ks + D/2 (lanes 32-63): the operand a
 // lane keeps in registers is one contiguous half of its row.  In the gradient products MFMA t contracts the two rows
 // that the lane halves hold in accumulator register t, so P and dS feed the matrix cores straight from registers.
@@ -285,14 +288,20 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
   const int lq = lane & 31, lh = lane >> 5;
 
   const int nkb = (f.S + BM - 1) / BM;
+  const int nsplit = a.dkv_splits, split = blockIdx.x % nsplit;  // this workgroup takes tiles split, split + nsplit, ...
   int pair, kb;  // the first key block is seen by every query row: the longest
-  map_workgroup(blockIdx.x, f.B * f.Hkv, nkb, &pair, &kb);
+  map_workgroup(blockIdx.x / nsplit, f.B * f.Hkv, nkb, &pair, &kb);
   const int hk = pair % f.Hkv, b = pair / f.Hkv;
   const int k0 = kb * BM, kw0 = k0 + wave * 32;
   const int S = keys_of_batch(f, b);
   const int key = kw0 + lq;
   float* dkp = (float*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
   float* dvp = (float*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
+  if (nsplit > 1) {  // partial sums: dense [split][dk | dv][B][Hkv][S][D]
+    const long long plane = (long long)f.B * f.Hkv * f.S * D;
+    dkp = a.partial + 2 * split * plane + (((long long)b * f.Hkv + hk) * f.S + key) * D;
+    dvp = dkp + plane;
+  }
   if (k0 >= S) {  // keys no query row attends to (at or beyond the batch entry's key count): zeros
     if (key < f.S)
       for (int d = 4 * lh; d < D; d += 8) {
@@ -366,18 +375,18 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
   const int s_lane = lq * PITCH + lh * (D / 2);
   const int g_lane = 4 * lh * PITCH + lq;
 
-  if (total > 0) {
-    load_tile(0);
+  if (split < total) {
+    load_tile(split);
     store_tile(0);
-    if (1 < total) load_tile(1);
+    if (split + nsplit < total) load_tile(split + nsplit);
   }
   __syncthreads();
 
-  for (int idx = 0; idx < total; idx++) {
-    const int cur = idx & 1;
-    if (idx + 1 < total) {
+  int cur = 0;
+  for (int idx = split; idx < total; idx += nsplit, cur ^= 1) {
+    if (idx + nsplit < total) {
       store_tile(cur ^ 1);
-      if (idx + 2 < total) load_tile(idx + 2);
+      if (idx + 2 * nsplit < total) load_tile(idx + 2 * nsplit);
     }
     const int i0 = (ntq - 1 - idx / f.G) * BT;
     const int h_of_tile = hk * f.G + idx % f.G;
@@ -453,6 +462,28 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
   }
 }
 
+// ---- kernel 3: dk / dv = sum of the partials, split 0 first ------------------------------------------------------------
+__global__ __launch_bounds__(256) void backward_dkv_f32_sum_kernel(BwdArgs a, long long nvec) {
+  const KArgs& f = a.f;
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // one float4 of dk and one of dv
+  if (i >= nvec) return;
+  const int dvec = f.D / 4;
+  const int d = 4 * (int)(i % dvec);
+  long long row = i / dvec;
+  const int key = (int)(row % f.S);
+  row /= f.S;
+  const int hk = (int)(row % f.Hkv), b = (int)(row / f.Hkv);
+  const long long plane = (long long)f.B * f.Hkv * f.S * f.D;
+  const float* p = a.partial + 4 * i;
+  f32x4 x = *(const f32x4*)p, y = *(const f32x4*)(p + plane);
+  for (int s = 1; s < a.dkv_splits; s++) {
+    x += *(const f32x4*)(p + 2 * s * plane);
+    y += *(const f32x4*)(p + (2 * s + 1) * plane);
+  }
+  *(f32x4*)((float*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2] + d) = x;
+  *(f32x4*)((float*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2] + d) = y;
+}
+
 template <int D, bool CAUSAL, bool MASKED>
 int launch_k(const BwdArgs& a, hipStream_t stream) {
   static hipError_t state1[kMaxDevices], state2[kMaxDevices];
@@ -462,15 +493,32 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   e = grant_dynamic_lds((const void*)backward_dkv_f32_kernel<D, CAUSAL, MASKED>, BwdF32Lds<D>::BYTES, state2, done2);
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
-  const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM);
+  const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM) * a.dkv_splits;
   hipLaunchKernelGGL((backward_dq_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g1), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL((backward_dkv_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g2), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
+  e = hipGetLastError();
+  if (e != hipSuccess || a.dkv_splits == 1) return (int)e;
+  const long long nvec = (long long)a.f.B * a.f.Hkv * a.f.S * (D / 4);
+  hipLaunchKernelGGL(backward_dkv_f32_sum_kernel, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, stream, a, nvec);
   return (int)hipGetLastError();
 }
 
 }  // namespace
+
+// One workgroup runs per CU at head_dim 128, and its length varies 1 : (number of key blocks) under a causal mask: below
+// about four workgroups per CU the longest ones set the time.  Without a causal mask all are equally long, and splitting
+// only serves to give every CU one (measured: splitting 256 equal workgroups further costs 1 %, 13-20 % with an
+// attnMask).  Splits are only worth it if each still gets a few tiles.
+int backward_f32_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal) {
+  const long long wgs = (long long)B * Hkv * ((S + BM - 1) / BM);
+  const long long tiles = (long long)(Hq / Hkv) * ((L + BT - 1) / BT);  // the longest query stream
+  const long long enough = causal ? 1024 : 256;
+  int n = 1;
+  while (n < 4 && wgs * n < enough && tiles >= 16 * n) n *= 2;
+  return n;
+}
 
 int launch_backward_f32(const BwdArgs& a, hipStream_t stream) {
   if (a.f.mask_kind != 0)  // exclusive with causal (validated by the caller, as the reference asserts)

@@ -176,7 +176,13 @@ struct BwdArgs {
   void* dv;
   long long dos[3], dqs[3], dks[3], dvs[3];  // element strides: batch, head, sequence
   float* stats;
+  // fp32 matrix-core pair only: with dkv_splits > 1 the query stream of every key block is dealt out to that many
+  // workgroups, which leave partial dk / dv in `partial` ([split][dk | dv][B][Hkv][S][D] floats) for a second pass to add.
+  float* partial;
+  int dkv_splits;
 };
+// Workgroups that share a key block in the fp32 dk/dv kernel (1: none, the kernel writes dk / dv itself).
+int backward_f32_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal);
 int launch_backward_general(const BwdArgs& a, int dtype, hipStream_t stream);
 int launch_backward_mfma(const BwdArgs& a, int dtype, hipStream_t stream);  // fp16/bf16, head_dim 64 or 128
 int launch_backward_f32(const BwdArgs& a, hipStream_t stream);              // fp32 on the fp32 matrix cores, head_dim 64 or 128

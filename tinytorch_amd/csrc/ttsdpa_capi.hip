@@ -218,7 +218,7 @@ int validate_backward(const ttsdpa_backward_params* p, BwdArgs* a) {
   }
   if ((p->dout_stride[2] < f->D || p->dq_stride[2] < f->D) && f->L > 1) return TTSDPA_ERR_STRIDE;
   if ((p->dk_stride[2] < f->D || p->dv_stride[2] < f->D) && f->S > 1) return TTSDPA_ERR_STRIDE;
-  a->dout = p->dout, a->dq = p->dq, a->dk = p->dk, a->dv = p->dv, a->stats = nullptr;
+  a->dout = p->dout, a->dq = p->dq, a->dk = p->dk, a->dv = p->dv, a->stats = nullptr, a->partial = nullptr, a->dkv_splits = 1;
   return TTSDPA_OK;
 }
 
@@ -259,6 +259,19 @@ int pick_backward_route(const ttsdpa_backward_params* p) {
 
 size_t backward_stats_bytes(const ttsdpa_backward_params* p) {
   return (size_t)p->fwd.B * p->fwd.Hq * p->fwd.L * 2 * sizeof(float);
+}
+
+// Scratch layout: the statistics, then (fp32 matrix-core pair with a split query stream) the partial dk / dv, 256-byte aligned.
+int backward_dkv_splits(const ttsdpa_backward_params* p) {
+  const ttsdpa_params* f = &p->fwd;
+  if (f->B == 0 || f->L == 0 || !backward_f32_ok(p)) return 1;
+  return backward_f32_dkv_splits(f->B, f->Hkv, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE);
+}
+size_t backward_partial_offset(const ttsdpa_backward_params* p) { return (backward_stats_bytes(p) + 255) & ~(size_t)255; }
+size_t backward_scratch_bytes(const ttsdpa_backward_params* p) {
+  const int n = backward_dkv_splits(p);
+  if (n == 1) return backward_stats_bytes(p);
+  return backward_partial_offset(p) + (size_t)n * 2 * p->fwd.B * p->fwd.Hkv * p->fwd.S * p->fwd.D * sizeof(float);
 }
 
 int check_grid(long long nwg) { return nwg > 0x7fffffffLL ? TTSDPA_ERR_SHAPE : TTSDPA_OK; }
@@ -410,7 +423,7 @@ int ttsdpa_backward_plan(const ttsdpa_backward_params* p, int* route) {
 size_t ttsdpa_backward_workspace_bytes(const ttsdpa_backward_params* p) {
   BwdArgs a;
   if (validate_backward(p, &a) != TTSDPA_OK) return 0;
-  return backward_stats_bytes(p);
+  return backward_scratch_bytes(p);
 }
 
 int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t workspace_bytes, void* stream) {
@@ -419,9 +432,11 @@ int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t wor
   if (rc != TTSDPA_OK) return rc;
   const int route = pick_backward_route(p);
   if (route == TTSDPA_ROUTE_NONE) return TTSDPA_OK;
-  const size_t need = backward_stats_bytes(p);
+  const size_t need = backward_scratch_bytes(p);
   if (need > 0 && (!workspace || workspace_bytes < need || !ptr_aligned(workspace, 16))) return TTSDPA_ERR_WORKSPACE;
   a.stats = (float*)workspace;
+  a.dkv_splits = backward_dkv_splits(p);
+  a.partial = a.dkv_splits > 1 ? (float*)((char*)workspace + backward_partial_offset(p)) : nullptr;
   if (route == TTSDPA_ROUTE_PREFILL) {
     const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + 127) / 128), g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + 127) / 128);
     if (check_grid(g1) != TTSDPA_OK || check_grid(g2) != TTSDPA_OK) return TTSDPA_ERR_SHAPE;
