@@ -246,19 +246,21 @@ def test_backward_mfma_per_batch_key_counts(dtype, D, causal):
         assert torch.all(dk[b, :, n:] == 0) and torch.all(dv[b, :, n:] == 0)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("mode", ["causal", "full", "kvlen", "mask"])
-def test_backward_f32_split_query_stream(D, mode):
-    """fp32 matrix-core pair with few key blocks and a long query stream (4 heads x 17 tiles per KV head): the dk/dv
-    kernel deals the stream out to four workgroups per key block and a third kernel adds their partial sums.  The
-    scratch the library asks for holds the partials (more than the 8 bytes per query row of the statistics)."""
+def test_backward_split_query_stream(dtype, D, mode):
+    """Matrix-core pairs with few key blocks and a long query stream (4 heads x 17 tiles per KV head): the dk/dv kernel
+    deals the stream out to four workgroups per key block and a third kernel adds their fp32 partial sums.  The scratch
+    the library asks for holds the partials (more than the 8 bytes per query row of the statistics)."""
     B, Hq, Hkv, L, S = 2, 8, 2, 520, 300
-    host, dev = make_inputs(4700 + D, B, Hq, Hkv, L, S, D, "f32")
+    host, dev = make_inputs(4700 + D, B, Hq, Hkv, L, S, D, dtype)
     q, k, v = dev
-    go = upstream(9, q.shape, "f32")[1]
+    go = upstream(9, q.shape, dtype)[1]
     out = sdpAttention(q, k, v, isCausal=(mode == "causal"))
     bp = build_backward_params(q, k, v, out, go, torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), mode == "causal")
     assert _capi.lib().ttsdpa_backward_workspace_bytes(ctypes.byref(bp)) >= B * Hq * L * 8 + 4 * 2 * B * Hkv * S * D * 4
+    name = "split-%s-%s-%d" % (mode, dtype, D)
     if mode == "kvlen":
         lens = [300, 129]
         kv = torch.tensor(lens, dtype=torch.int32, device="cuda")
@@ -266,13 +268,16 @@ def test_backward_f32_split_query_stream(D, mode):
         for b in range(B):
             m[b, 0] = np.arange(S)[None, :] <= np.arange(L)[:, None] + max(0, lens[b] - L)
             m[b, 0, :, lens[b]:] = False
-        check("split-kvlen-%d" % D, host, dev, "f32", causal=True, kv_lens=kv, align="bottom-right", oracle_mask=m, route="prefill")
+        check(name, host, dev, dtype, causal=True, kv_lens=kv, align="bottom-right", oracle_mask=m, route="prefill")
+        _, dk, dv = sdpAttentionBackward(go, q, k, v, sdpAttention(q, k, v, isCausal=True, causalAlign="bottom-right", kvLens=kv),
+                                         isCausal=True, causalAlign="bottom-right", kvLens=kv)
+        assert torch.all(dk[1, :, 129:] == 0) and torch.all(dv[1, :, 129:] == 0)
     elif mode == "mask":
         m = np.random.default_rng(6).random((Hq, L, S)) < 0.6
         m[..., 0] = True
-        check("split-mask-%d" % D, host, dev, "f32", mask_h=m, mask_d=torch.from_numpy(m).cuda(), route="prefill")
+        check(name, host, dev, dtype, mask_h=m, mask_d=torch.from_numpy(m).cuda(), route="prefill")
     else:
-        check("split-%s-%d" % (mode, D), host, dev, "f32", causal=(mode == "causal"), route="prefill")
+        check(name, host, dev, dtype, causal=(mode == "causal"), route="prefill")
 
 
 def test_backward_strided_views_and_scale():

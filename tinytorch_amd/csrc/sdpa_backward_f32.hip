@@ -17,7 +17,7 @@
 //      dv^T += dout^T.P, dk^T += Q^T.dS.  When the launch has too few key blocks to fill and balance the chip (under a
 //      causal mask the first key block sees every query tile, the last one a few), the tiles of a key block's query
 //      stream are dealt out to 2-4 workgroups, which leave partial dk / dv in scratch, and
-//   3. backward_dkv_f32_sum_kernel adds the partials in a fixed order.
+//   3. backward_dkv_sum_kernel adds the partials in a fixed order.
 // In the score products MFMA ks contracts head_dim elements ks (lanes 0-31) and ks + D/2 (lanes 32-63): the operand a
 // lane keeps in registers is one contiguous half of its row.  In the gradient products MFMA t contracts the two rows
 // that the lane halves hold in accumulator register t, so P and dS feed the matrix cores straight from registers.
@@ -462,28 +462,6 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
   }
 }
 
-// ---- kernel 3: dk / dv = sum of the partials, split 0 first ------------------------------------------------------------
-__global__ __launch_bounds__(256) void backward_dkv_f32_sum_kernel(BwdArgs a, long long nvec) {
-  const KArgs& f = a.f;
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // one float4 of dk and one of dv
-  if (i >= nvec) return;
-  const int dvec = f.D / 4;
-  const int d = 4 * (int)(i % dvec);
-  long long row = i / dvec;
-  const int key = (int)(row % f.S);
-  row /= f.S;
-  const int hk = (int)(row % f.Hkv), b = (int)(row / f.Hkv);
-  const long long plane = (long long)f.B * f.Hkv * f.S * f.D;
-  const float* p = a.partial + 4 * i;
-  f32x4 x = *(const f32x4*)p, y = *(const f32x4*)(p + plane);
-  for (int s = 1; s < a.dkv_splits; s++) {
-    x += *(const f32x4*)(p + 2 * s * plane);
-    y += *(const f32x4*)(p + (2 * s + 1) * plane);
-  }
-  *(f32x4*)((float*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2] + d) = x;
-  *(f32x4*)((float*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2] + d) = y;
-}
-
 template <int D, bool CAUSAL, bool MASKED>
 int launch_k(const BwdArgs& a, hipStream_t stream) {
   static hipError_t state1[kMaxDevices], state2[kMaxDevices];
@@ -500,25 +478,10 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((backward_dkv_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g2), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess || a.dkv_splits == 1) return (int)e;
-  const long long nvec = (long long)a.f.B * a.f.Hkv * a.f.S * (D / 4);
-  hipLaunchKernelGGL(backward_dkv_f32_sum_kernel, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, stream, a, nvec);
-  return (int)hipGetLastError();
+  return launch_backward_dkv_sum<float>(a, stream);
 }
 
 }  // namespace
-
-// One workgroup runs per CU at head_dim 128, and its length varies 1 : (number of key blocks) under a causal mask: below
-// about four workgroups per CU the longest ones set the time.  Without a causal mask all are equally long, and splitting
-// only serves to give every CU one (measured: splitting 256 equal workgroups further costs 1 %, 13-20 % with an
-// attnMask).  Splits are only worth it if each still gets a few tiles.
-int backward_f32_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal) {
-  const long long wgs = (long long)B * Hkv * ((S + BM - 1) / BM);
-  const long long tiles = (long long)(Hq / Hkv) * ((L + BT - 1) / BT);  // the longest query stream
-  const long long enough = causal ? 1024 : 256;
-  int n = 1;
-  while (n < 4 && wgs * n < enough && tiles >= 16 * n) n *= 2;
-  return n;
-}
 
 int launch_backward_f32(const BwdArgs& a, hipStream_t stream) {
   if (a.f.mask_kind != 0)  // exclusive with causal (validated by the caller, as the reference asserts)

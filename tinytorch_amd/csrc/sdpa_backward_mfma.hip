@@ -63,20 +63,52 @@ __device__ __forceinline__ vec8 transposed_operand(const void* lane_base, int by
   return __builtin_bit_cast(vec8, r);
 }
 
-// dk and dv rows of a key no query row attends to (at or beyond the batch entry's key count): zeros.
+// A lane's share of the dk / dv rows of key `key` (accumulator layout: registers 4rg .. 4rg+3 of block db are elements
+// 32db + 8rg + 4lh .. +3) goes to the gradient tensors, or — when the key block's query stream is split over several
+// workgroups — as fp32 to this split's partial sums, dense [split][dk | dv][B][Hkv][S][D].
 template <typename TR, int D>
-__device__ __forceinline__ void zero_key_rows(const BwdArgs& a, int b, int hk, int key, int lh) {
+__device__ __forceinline__ void store_key_grads(const BwdArgs& a, int split, int b, int hk, int key, int lh,
+                                                const f32x16 (&dkacc)[D / 32], const f32x16 (&dvacc)[D / 32], float scale) {
   typedef typename TR::elem T;
   if (key >= a.f.S) return;
+  if (a.dkv_splits > 1) {
+    const long long plane = (long long)a.f.B * a.f.Hkv * a.f.S * D;
+    float* dkp = a.partial + 2 * split * plane + (((long long)b * a.f.Hkv + hk) * a.f.S + key) * D;
+#pragma unroll
+    for (int db = 0; db < D / 32; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        f32x4 x, y;
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = dkacc[db][4 * rg + i] * scale, y[i] = dvacc[db][4 * rg + i];
+        *(f32x4*)(dkp + 32 * db + 8 * rg + 4 * lh) = x;
+        *(f32x4*)(dkp + plane + 32 * db + 8 * rg + 4 * lh) = y;
+      }
+    return;
+  }
   T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
   T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
-  typename TR::vec4 zero;
 #pragma unroll
-  for (int i = 0; i < 4; i++) zero[i] = (T)0.f;
-  for (int d = 4 * lh; d < D; d += 8) {
-    *(typename TR::vec4*)(dkp + d) = zero;
-    *(typename TR::vec4*)(dvp + d) = zero;
-  }
+  for (int db = 0; db < D / 32; db++)
+#pragma unroll
+    for (int rg = 0; rg < 4; rg++) {
+      f32x4 x, y;
+#pragma unroll
+      for (int i = 0; i < 4; i++) x[i] = dkacc[db][4 * rg + i] * scale, y[i] = dvacc[db][4 * rg + i];
+      *(typename TR::vec4*)(dkp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
+      *(typename TR::vec4*)(dvp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(y, typename TR::vec4);
+    }
+}
+
+// dk and dv rows of a key no query row attends to (at or beyond the batch entry's key count): zeros.
+template <typename TR, int D>
+__device__ __forceinline__ void zero_key_rows(const BwdArgs& a, int split, int b, int hk, int key, int lh) {
+  f32x16 zero[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[i][r] = 0.f;
+  store_key_grads<TR, D>(a, split, b, hk, key, lh, zero, zero, 0.f);
 }
 
 template <typename vec8>
@@ -346,13 +378,14 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   const int lq = lane & 31, lh = lane >> 5;
 
   const int nkb = (f.S + BM - 1) / BM;
+  const int nsplit = a.dkv_splits, split = blockIdx.x % nsplit;  // this workgroup takes tiles split, split + nsplit, ...
   int pair, kb;  // the first key block is seen by every query row: the longest
-  map_workgroup(blockIdx.x, f.B * f.Hkv, nkb, &pair, &kb);
+  map_workgroup(blockIdx.x / nsplit, f.B * f.Hkv, nkb, &pair, &kb);
   const int hk = pair % f.Hkv, b = pair / f.Hkv;
   const int k0 = kb * BM, kw0 = k0 + wave * 32;
   const int S = keys_of_batch(f, b);  // rows of dk / dv from here to f.S are written as zeros
   if (k0 >= S) {
-    zero_key_rows<TR, D>(a, b, hk, kw0 + lq, lh);
+    zero_key_rows<TR, D>(a, split, b, hk, kw0 + lq, lh);
     return;
   }
   const bool wave_live = kw0 < S;
@@ -431,18 +464,18 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   const int r_lane = lq * RP + 8 * lh;
   const int t_lane = (4 * lh + ((lane & 15) >> 2)) * TP + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  if (total > 0) {
-    load_tile(0);
+  if (split < total) {
+    load_tile(split);
     store_tile(0);
-    if (1 < total) load_tile(1);
+    if (split + nsplit < total) load_tile(split + nsplit);
   }
   __syncthreads();
 
-  for (int idx = 0; idx < total; idx++) {
-    const int cur = idx & 1;
-    if (idx + 1 < total) {
+  int cur = 0;
+  for (int idx = split; idx < total; idx += nsplit, cur ^= 1) {
+    if (idx + nsplit < total) {
       store_tile(cur ^ 1);
-      if (idx + 2 < total) load_tile(idx + 2);
+      if (idx + 2 * nsplit < total) load_tile(idx + 2 * nsplit);
     }
     const int i0 = (ntq - 1 - idx / f.G) * BQ;
     const int h_of_tile = hk * f.G + idx % f.G;
@@ -518,21 +551,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
     __syncthreads();
   }
 
-  const int key = kw0 + lq;
-  if (key < f.S) {
-    T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
-    T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
-#pragma unroll
-    for (int db = 0; db < DBLK; db++)
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        f32x4 x, y;
-#pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = dkacc[db][4 * rg + i] * f.scale, y[i] = dvacc[db][4 * rg + i];
-        *(typename TR::vec4*)(dkp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
-        *(typename TR::vec4*)(dvp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(y, typename TR::vec4);
-      }
-  }
+  store_key_grads<TR, D>(a, split, b, hk, kw0 + lq, lh, dkacc, dvacc, f.scale);
 }
 
 // ---- kernel 2 for head_dim 128: the same products with the tiles brought in by direct global->LDS loads ----------------
@@ -580,13 +599,14 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
   const int lq = lane & 31, lh = lane >> 5;
 
   const int nkb = (f.S + BM - 1) / BM;
+  const int nsplit = a.dkv_splits, split = blockIdx.x % nsplit;  // this workgroup takes entries split, split + nsplit, ...
   int pair, kb;
-  map_workgroup(blockIdx.x, f.B * f.Hkv, nkb, &pair, &kb);
+  map_workgroup(blockIdx.x / nsplit, f.B * f.Hkv, nkb, &pair, &kb);
   const int hk = pair % f.Hkv, b = pair / f.Hkv;
   const int k0 = kb * BM, kw0 = k0 + gw * 32;
   const int S = keys_of_batch(f, b);  // rows of dk / dv from here to f.S are written as zeros
   if (k0 >= S) {
-    if (grp == 0) zero_key_rows<TR, D>(a, b, hk, kw0 + lq, lh);
+    if (grp == 0) zero_key_rows<TR, D>(a, split, b, hk, kw0 + lq, lh);
     return;
   }
   const int coff = CAUSAL ? causal_offset(f, S) : 0;
@@ -629,20 +649,22 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
   // Query tiles it0 .. ntq-1 of each of the G heads see keys of this workgroup.  They are taken from the last tile down,
   // the heads of a tile one after the other: every key block of a (batch, kv head) then starts at the same tile and walks
   // in step with the others (a block further down the causal triangle just stops earlier), so the tile one workgroup
-  // fetches from HBM is in the XCD's L2 for the others.  Entry idx of that list belongs to group idx % 2.
+  // fetches from HBM is in the XCD's L2 for the others.  This workgroup's entries are split, split + nsplit, ... of that
+  // list; entry idx of ITS list belongs to group idx % 2.
   const int ntq = (f.L + BQ - 1) / BQ;
   int it0 = 0;
   if (CAUSAL) it0 = (k0 - coff > 0 ? k0 - coff : 0) / BQ;
   const int nt = ntq > it0 ? ntq - it0 : 0;
-  const int total = f.G * nt;
+  const int total = split < f.G * nt ? (f.G * nt - split + nsplit - 1) / nsplit : 0;
   const int niter = (total + 1) / 2;  // iterations of either group (the second may have one entry less)
 
   // wavefront gw of a group brings rows 8gw .. 8gw+7 of the Q tile and of the dout tile (two loads each) into the
   // group's ring; its first wavefront the statistics as well
   const unsigned ring_addr = smem_addr + V_BYTES + grp * NSTAGE * STAGE_BYTES;
   auto dma_tile = [&](int idx, int stage) __attribute__((always_inline)) {
-    const int h = hk * f.G + idx % f.G;
-    const int i0 = (ntq - 1 - idx / f.G) * BQ;
+    const int entry = split + nsplit * idx;
+    const int h = hk * f.G + entry % f.G;
+    const int i0 = (ntq - 1 - entry / f.G) * BQ;
     const char* qb = (const char*)((const T*)f.q + b * f.qs[0] + h * f.qs[1] + (long long)i0 * f.qs[2]);
     const char* gb = (const char*)((const T*)a.dout + b * a.dos[0] + h * a.dos[1] + (long long)i0 * a.dos[2]);
     const unsigned at = ring_addr + stage * STAGE_BYTES;
@@ -695,7 +717,7 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
     const bool more = idx + 4 < total;
     if (more) dma_tile(idx + 4, nxt2);
     if (idx < total) {
-      const int i0 = (ntq - 1 - idx / f.G) * BQ;
+      const int i0 = (ntq - 1 - (split + nsplit * idx) / f.G) * BQ;
       const char* qt = ring + cur * STAGE_BYTES;
       const char* gt = qt + TILE_BYTES;
       const float* st = (const float*)(qt + 2 * TILE_BYTES);
@@ -788,20 +810,7 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
     __syncthreads();
   }
 
-  if (grp == 0 && key < f.S) {
-    T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2];
-    T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2];
-#pragma unroll
-    for (int db = 0; db < DBLK; db++)
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        f32x4 x, y;
-#pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = dkacc[db][4 * rg + i] * f.scale, y[i] = dvacc[db][4 * rg + i];
-        *(typename TR::vec4*)(dkp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
-        *(typename TR::vec4*)(dvp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(y, typename TR::vec4);
-      }
-  }
+  if (grp == 0) store_key_grads<TR, D>(a, split, b, hk, key, lh, dkacc, dvacc, f.scale);
 }
 
 // ---- kernel 1 for head_dim 128 without an attnMask: the same products, K / V tiles by direct global->LDS loads ----------
@@ -1041,7 +1050,7 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   }
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
-  const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM);
+  const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM) * a.dkv_splits;
   if (DMA) {
     hipLaunchKernelGGL((backward_dq128_kernel<TR, CAUSAL>), dim3((unsigned)g1), dim3(256), dq128::LDS_BYTES, stream, a);
   } else {
@@ -1054,7 +1063,9 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   } else {
     hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
   }
-  return (int)hipGetLastError();
+  e = hipGetLastError();
+  if (e != hipSuccess || a.dkv_splits == 1) return (int)e;
+  return launch_backward_dkv_sum<typename TR::elem>(a, stream);
 }
 
 template <typename TR, int D>

@@ -176,13 +176,57 @@ struct BwdArgs {
   void* dv;
   long long dos[3], dqs[3], dks[3], dvs[3];  // element strides: batch, head, sequence
   float* stats;
-  // fp32 matrix-core pair only: with dkv_splits > 1 the query stream of every key block is dealt out to that many
-  // workgroups, which leave partial dk / dv in `partial` ([split][dk | dv][B][Hkv][S][D] floats) for a second pass to add.
+  // matrix-core pairs only: with dkv_splits > 1 the query stream of every key block is dealt out to that many
+  // workgroups, which leave partial dk / dv in `partial` ([split][dk | dv][B][Hkv][S][D] floats) for a third kernel to add.
   float* partial;
   int dkv_splits;
 };
-// Workgroups that share a key block in the fp32 dk/dv kernel (1: none, the kernel writes dk / dv itself).
-int backward_f32_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal);
+
+// Workgroups that share a key block in the matrix-core dk/dv kernels (1: none, the kernel writes dk / dv itself).
+// A dk/dv workgroup owns 128 keys and about one runs per CU at a time; under a causal mask its length varies
+// 1 : (number of key blocks), and below about four workgroups per CU the longest ones set the time.  Without a causal
+// mask all are equally long and splitting only serves to give every CU one (splitting 256 equal workgroups further
+// measured 1 % slower, 13-20 % with an attnMask).  A split must still get a few tiles.  `groups`: wavefront groups
+// that already share a key block inside a workgroup (2 in the 16-bit head_dim-128 kernel, where splitting 512
+// workgroups of a causal call further measured 4 % slower, 256 of them 7-21 % faster).
+inline int backward_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal, int groups) {
+  const long long wgs = (long long)B * Hkv * ((S + 127) / 128) * groups;
+  const long long tiles = (long long)(Hq / Hkv) * ((L + 31) / 32) / groups;  // the longest query stream, in 32-row tiles
+  const long long enough = causal ? 1024 : 256;
+  int n = 1;
+  while (n < 4 && wgs * n < enough && tiles >= 16 * n) n *= 2;
+  return n;
+}
+
+// dk / dv = sum of the partials, split 0 first (a fixed order), converted to the tensors' element type.
+template <typename T>
+__global__ __launch_bounds__(256) void backward_dkv_sum_kernel(BwdArgs a, long long nvec) {
+  typedef T vec4t __attribute__((ext_vector_type(4)));
+  const KArgs& f = a.f;
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // one group of four elements of dk and of dv
+  if (i >= nvec) return;
+  const int dvec = f.D / 4;
+  const int d = 4 * (int)(i % dvec);
+  long long row = i / dvec;
+  const int key = (int)(row % f.S);
+  row /= f.S;
+  const int hk = (int)(row % f.Hkv), b = (int)(row / f.Hkv);
+  const long long plane = (long long)f.B * f.Hkv * f.S * f.D;
+  const float* p = a.partial + 4 * i;
+  f32x4 x = *(const f32x4*)p, y = *(const f32x4*)(p + plane);
+  for (int s = 1; s < a.dkv_splits; s++) {
+    x += *(const f32x4*)(p + 2 * s * plane);
+    y += *(const f32x4*)(p + (2 * s + 1) * plane);
+  }
+  *(vec4t*)((T*)a.dk + b * a.dks[0] + hk * a.dks[1] + key * a.dks[2] + d) = __builtin_convertvector(x, vec4t);
+  *(vec4t*)((T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + key * a.dvs[2] + d) = __builtin_convertvector(y, vec4t);
+}
+template <typename T>
+int launch_backward_dkv_sum(const BwdArgs& a, hipStream_t stream) {
+  const long long nvec = (long long)a.f.B * a.f.Hkv * a.f.S * (a.f.D / 4);
+  hipLaunchKernelGGL(backward_dkv_sum_kernel<T>, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, stream, a, nvec);
+  return (int)hipGetLastError();
+}
 int launch_backward_general(const BwdArgs& a, int dtype, hipStream_t stream);
 int launch_backward_mfma(const BwdArgs& a, int dtype, hipStream_t stream);  // fp16/bf16, head_dim 64 or 128
 int launch_backward_f32(const BwdArgs& a, hipStream_t stream);              // fp32 on the fp32 matrix cores, head_dim 64 or 128

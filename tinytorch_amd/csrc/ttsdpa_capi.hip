@@ -261,15 +261,16 @@ size_t backward_stats_bytes(const ttsdpa_backward_params* p) {
   return (size_t)p->fwd.B * p->fwd.Hq * p->fwd.L * 2 * sizeof(float);
 }
 
-// Scratch layout: the statistics, then (fp32 matrix-core pair with a split query stream) the partial dk / dv, 256-byte aligned.
-int backward_dkv_splits(const ttsdpa_backward_params* p) {
+// Scratch layout: the statistics, then (matrix-core pairs with a split query stream) the partial dk / dv, 256-byte aligned.
+int dkv_splits_of(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
-  if (f->B == 0 || f->L == 0 || !backward_f32_ok(p)) return 1;
-  return backward_f32_dkv_splits(f->B, f->Hkv, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE);
+  if (pick_backward_route(p) != TTSDPA_ROUTE_PREFILL) return 1;
+  const int groups = f->dtype != TTSDPA_F32 && f->D == 128 && f->mask_kind == TTSDPA_MASK_NONE ? 2 : 1;
+  return backward_dkv_splits(f->B, f->Hkv, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE, groups);
 }
 size_t backward_partial_offset(const ttsdpa_backward_params* p) { return (backward_stats_bytes(p) + 255) & ~(size_t)255; }
 size_t backward_scratch_bytes(const ttsdpa_backward_params* p) {
-  const int n = backward_dkv_splits(p);
+  const int n = dkv_splits_of(p);
   if (n == 1) return backward_stats_bytes(p);
   return backward_partial_offset(p) + (size_t)n * 2 * p->fwd.B * p->fwd.Hkv * p->fwd.S * p->fwd.D * sizeof(float);
 }
@@ -435,7 +436,7 @@ int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t wor
   const size_t need = backward_scratch_bytes(p);
   if (need > 0 && (!workspace || workspace_bytes < need || !ptr_aligned(workspace, 16))) return TTSDPA_ERR_WORKSPACE;
   a.stats = (float*)workspace;
-  a.dkv_splits = backward_dkv_splits(p);
+  a.dkv_splits = dkv_splits_of(p);
   a.partial = a.dkv_splits > 1 ? (float*)((char*)workspace + backward_partial_offset(p)) : nullptr;
   if (route == TTSDPA_ROUTE_PREFILL) {
     const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + 127) / 128), g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + 127) / 128);
