@@ -20,6 +20,9 @@
 // (ds_read_b64_tr_b16) are read from them, each copy with the row pitch that makes its reads conflict-free; the
 // head_dim-128 dk/dv kernel keeps one swizzled copy instead (see there).
 // Seven matrix products in all, against five in the textbook count (the scores are computed in both kernels).
+// When a call has too few key blocks to fill and balance the chip, the query stream of a key block is dealt out to 2-4
+// workgroups of kernel 2, which leave fp32 partial sums in scratch, and backward_dkv_sum_kernel (sdpa_common.h) adds
+// them in a fixed order.
 
 #include "sdpa_common.h"
 
