@@ -288,9 +288,11 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
   const int lq = lane & 31, lh = lane >> 5;
 
   const int nkb = (f.S + BM - 1) / BM;
-  const int nsplit = a.dkv_splits, split = blockIdx.x % nsplit;  // this workgroup takes tiles split, split + nsplit, ...
+  const int nsplit = a.dkv_splits;
+  int wg, split;  // this workgroup takes tiles split, split + nsplit, ... of key-block workgroup wg
+  split_of_workgroup(blockIdx.x, nsplit, f.B * f.Hkv, &wg, &split);
   int pair, kb;  // the first key block is seen by every query row: the longest
-  map_workgroup(blockIdx.x / nsplit, f.B * f.Hkv, nkb, &pair, &kb);
+  map_workgroup(wg, f.B * f.Hkv, nkb, &pair, &kb);
   const int hk = pair % f.Hkv, b = pair / f.Hkv;
   const int k0 = kb * BM, kw0 = k0 + wave * 32;
   const int S = keys_of_batch(f, b);

@@ -381,9 +381,11 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   const int lq = lane & 31, lh = lane >> 5;
 
   const int nkb = (f.S + BM - 1) / BM;
-  const int nsplit = a.dkv_splits, split = blockIdx.x % nsplit;  // this workgroup takes tiles split, split + nsplit, ...
+  const int nsplit = a.dkv_splits;
+  int wg, split;  // this workgroup takes tiles split, split + nsplit, ... of key-block workgroup wg
+  split_of_workgroup(blockIdx.x, nsplit, f.B * f.Hkv, &wg, &split);
   int pair, kb;  // the first key block is seen by every query row: the longest
-  map_workgroup(blockIdx.x / nsplit, f.B * f.Hkv, nkb, &pair, &kb);
+  map_workgroup(wg, f.B * f.Hkv, nkb, &pair, &kb);
   const int hk = pair % f.Hkv, b = pair / f.Hkv;
   const int k0 = kb * BM, kw0 = k0 + wave * 32;
   const int S = keys_of_batch(f, b);  // rows of dk / dv from here to f.S are written as zeros
@@ -602,9 +604,11 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
   const int lq = lane & 31, lh = lane >> 5;
 
   const int nkb = (f.S + BM - 1) / BM;
-  const int nsplit = a.dkv_splits, split = blockIdx.x % nsplit;  // this workgroup takes entries split, split + nsplit, ...
+  const int nsplit = a.dkv_splits;
+  int wg, split;  // this workgroup takes entries split, split + nsplit, ... of key-block workgroup wg
+  split_of_workgroup(blockIdx.x, nsplit, f.B * f.Hkv, &wg, &split);
   int pair, kb;
-  map_workgroup(blockIdx.x / nsplit, f.B * f.Hkv, nkb, &pair, &kb);
+  map_workgroup(wg, f.B * f.Hkv, nkb, &pair, &kb);
   const int hk = pair % f.Hkv, b = pair / f.Hkv;
   const int k0 = kb * BM, kw0 = k0 + gw * 32;
   const int S = keys_of_batch(f, b);  // rows of dk / dv from here to f.S are written as zeros

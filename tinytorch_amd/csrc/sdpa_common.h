@@ -198,6 +198,20 @@ inline int backward_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal
   return n;
 }
 
+// Workgroup id of a dk/dv launch with split query streams -> (key-block workgroup n, split).  The hardware hands
+// workgroup id to XCD id % 8 and map_workgroup places n by n % 8: the splits of eight consecutive n follow each other in
+// groups of eight, so that n % 8 == id % 8 and the order (longest key blocks first) is kept.
+__device__ __forceinline__ void split_of_workgroup(int id, int nsplit, int npair, int* n, int* split) {
+  if ((npair & 7) == 0) {
+    const int r = id % (8 * nsplit);
+    *split = r >> 3;
+    *n = (id / (8 * nsplit)) * 8 + (r & 7);
+  } else {
+    *split = id % nsplit;
+    *n = id / nsplit;
+  }
+}
+
 // dk / dv = sum of the partials, split 0 first (a fixed order), converted to the tensors' element type.
 template <typename T>
 __global__ __launch_bounds__(256) void backward_dkv_sum_kernel(BwdArgs a, long long nvec) {
