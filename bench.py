@@ -10,7 +10,7 @@ same run and reported under "secondary", config 3's shape in fp32 (the reference
 on the fp32 MFMA kernel, against the 157.3 TFLOP/s fp32 peak) under "fp32", and the row-wise neighbour ops (rmsNorm,
 fusedAddRmsNorm, siluMul, softmax; HBM-bound) under "fused_ops" and the linear layer (QKV projection of the same
 token batch; MFMA-bound) under "linear", and the attention backward (dq, dk, dv at config 3's shape; MFMA-bound) under
-"backward".  One JSON line is printed.
+"backward" (bf16, and the same shape in fp32 on the fp32 matrix cores under "backward"."fp32").  One JSON line is printed.
 
 Algorithmic work per launch (what "achieved" divides by the measured launch time):
   prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)

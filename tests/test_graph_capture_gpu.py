@@ -80,20 +80,24 @@ def test_decode_step_in_a_graph(B, Hq, Hkv, Smax):
         assert torch.equal(kc[b, :, :cur[b]], kd[b, :, :cur[b]])
 
 
-def test_forward_and_backward_in_a_graph():
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_forward_and_backward_in_a_graph(dtype):
     """A training-style step (attention forward, then its backward) recorded once and replayed on new inputs: both
-    calls only enqueue kernels and use caller-provided scratch, so every replay reproduces the eager bits."""
+    calls only enqueue kernels and use caller-provided scratch, so every replay reproduces the eager bits.  At this
+    shape the dk/dv kernels split their query streams: the partial sums in scratch and the kernel that adds them are
+    part of the recorded step."""
     import ctypes
     from tinytorch_amd import _capi, build_backward_params, build_params
     B, Hq, Hkv, N, D = 2, 8, 2, 384, 128
     gen = torch.Generator(device="cuda").manual_seed(77)
-    mk = lambda *shape: torch.randn(*shape, device="cuda", generator=gen).bfloat16()
+    mk = lambda *shape: torch.randn(*shape, device="cuda", generator=gen).to(dtype)
     q, k, v, go = mk(B, Hq, N, D), mk(B, Hkv, N, D), mk(B, Hkv, N, D), mk(B, Hq, N, D)
     out, dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     L = _capi.lib()
     fp = build_params(q, k, v, out, True)
     bp = build_backward_params(q, k, v, out, go, dq, dk, dv, True)
     nbytes = L.ttsdpa_backward_workspace_bytes(ctypes.byref(bp))
+    assert nbytes > B * Hq * N * 8   # more than the statistics: partial dk / dv
     ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
 
     def step():
