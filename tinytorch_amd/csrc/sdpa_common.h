@@ -189,10 +189,13 @@ struct BwdArgs {
 // measured 1 % slower, 13-20 % with an attnMask).  A split must still get a few tiles.  `groups`: wavefront groups
 // that already share a key block inside a workgroup (2 in the 16-bit head_dim-128 kernel, where splitting 512
 // workgroups of a causal call further measured 4 % slower, 256 of them 7-21 % faster).
-inline int backward_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal, int groups) {
+// `per_cu`: workgroups of the kernel that fit a CU (2 at head_dim 64 without an attnMask, else 1); it counts for calls
+// without a causal mask only (head_dim 64, 256 equal workgroups: two splits +28 %; causal with 512: four splits instead
+// of two -2 to -5 %).
+inline int backward_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal, int groups, int per_cu) {
   const long long wgs = (long long)B * Hkv * ((S + 127) / 128) * groups;
   const long long tiles = (long long)(Hq / Hkv) * ((L + 31) / 32) / groups;  // the longest query stream, in 32-row tiles
-  const long long enough = causal ? 1024 : 256;
+  const long long enough = causal ? 1024 : 256 * per_cu;
   int n = 1;
   while (n < 4 && wgs * n < enough && tiles >= 16 * n) n *= 2;
   return n;

@@ -266,7 +266,8 @@ int dkv_splits_of(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
   if (pick_backward_route(p) != TTSDPA_ROUTE_PREFILL) return 1;
   const int groups = f->dtype != TTSDPA_F32 && f->D == 128 && f->mask_kind == TTSDPA_MASK_NONE ? 2 : 1;
-  return backward_dkv_splits(f->B, f->Hkv, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE, groups);
+  const int per_cu = f->D == 64 && f->mask_kind == TTSDPA_MASK_NONE ? 2 : 1;
+  return backward_dkv_splits(f->B, f->Hkv, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE, groups, per_cu);
 }
 size_t backward_partial_offset(const ttsdpa_backward_params* p) { return (backward_stats_bytes(p) + 255) & ~(size_t)255; }
 size_t backward_scratch_bytes(const ttsdpa_backward_params* p) {
