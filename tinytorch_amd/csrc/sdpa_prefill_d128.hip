@@ -46,6 +46,7 @@
 // query heads and row tiles that share a KV head on the same XCD so its L2 holds that K/V once.
 
 #include "sdpa_common.h"
+#include "prefill128_steps.inc"  // hand-ordered instruction streams of the steady state (gen_prefill128_steps.py)
 
 namespace ttsdpa {
 
@@ -62,6 +63,8 @@ constexpr int KSTAGES = 4, VSTAGES = 4;     // K and V tiles are requested three
 constexpr int LDS_BYTES = (KSTAGES + VSTAGES) * STAGE_BYTES;
 constexpr float kSumLimit = 1024.f;  // a lane's 16 probabilities of a half may sum to this much before the maximum is raised
 
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x32 __attribute__((ext_vector_type(32)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -142,41 +145,19 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     return;
   }
 
-  for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
-  const int rt = (CAUSAL && (part == 0) == long_first) ? ntile - 1 - slot_rt : slot_rt;
-  if (part == 1 && slot_rt >= ntile - 1 - slot_rt) break;  // odd count: the middle tile has no mirror
-  const int q0 = rt * BM;
-  const int qw0 = q0 + rowgroup * WM;
-
-  // Query row i sees keys up to i + coff (coff = 0: the reference's top-left aligned mask); qc0 is this wavefront's
-  // first row in key coordinates.
-  const int coff = CAUSAL ? causal_offset(a, S) : 0;
-  const int qc0 = qw0 + coff;
-  int ntiles_kv = (S + BN - 1) / BN;
-  if (CAUSAL) {
-    int last = (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1) + coff;
-    int lastkv = last < S - 1 ? last : S - 1;
-    ntiles_kv = lastkv / BN + 1;
-  }
-  // 32-key halves this wavefront computes on: under a causal mask those that start at or before its last row
-  int my_halves = 2 * ntiles_kv;
-  if (CAUSAL) {
-    int t = (qc0 + WM - 1) / 32 + 1;
-    my_halves = t < my_halves ? t : my_halves;
-  }
-  // Tiles j whose two steps take the fast form: halves up to 2j+3 are this wavefront's, tile j+1 is complete, and
-  // half 2j+2 (whose exponentials step 2j+1 takes) needs no mask.
-  int nfast = (my_halves - 2) / 2;
-  {
-    int f = S >= 96 ? (S - 32) / BN : 0;
-    nfast = f < nfast ? f : nfast;
+  // ---- geometry of a part: first query row of the workgroup's row tile and its KV tile count ----------------------
+  auto part_rows = [&](int part, int& q0, int& ntiles_kv) __attribute__((always_inline)) {
+    const int rt = (CAUSAL && (part == 0) == long_first) ? ntile - 1 - slot_rt : slot_rt;
+    q0 = rt * BM;
+    ntiles_kv = (S + BN - 1) / BN;
     if (CAUSAL) {
-      f = qc0 >= 95 ? (qc0 - 31) / BN : 0;
-      nfast = f < nfast ? f : nfast;
+      const int coff = causal_offset(a, S);
+      int last = (q0 + BM - 1 < a.L - 1 ? q0 + BM - 1 : a.L - 1) + coff;
+      int lastkv = last < S - 1 ? last : S - 1;
+      ntiles_kv = lastkv / BN + 1;
     }
-  }
-  if (nfast < 0) nfast = 0;
-  if (a.mask_kind != 0) nfast = 0;  // an attnMask is applied in the general form of a step
+  };
+  const bool two_parts = CAUSAL && slot_rt < ntile - 1 - slot_rt;  // odd count: the middle tile has no mirror
 
   // ---- global -> LDS: wavefront w moves rows 8w .. 8w+7 of a tile, 4 rows (1 KiB) per instruction --------------
   // lane l fills slot (row 4i + l/16, chunk slot l%16) and therefore fetches chunk (l%16) ^ f(row)
@@ -244,7 +225,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 
   // ---- LDS operand addresses (bytes), loop-invariant ---------------------------------------------------------------
   // K operand (half, ks): row 32*half + lq, chunk 2*ks + lh  ->  row*256 + 16*((2ks + lh) ^ f(row))
-  unsigned k_addr[8];
+  u32x8 k_addr;
   {
     unsigned base = (unsigned)(lq * ROW_BYTES + 16 * (lh ^ swz(lq)));  // f(32*half + lq) == f(lq)
 #pragma unroll
@@ -253,7 +234,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   // V operand part (db, ld) of k-step t via the transpose load: this lane points at row 16t + 8ld + 4lh + s/4,
   // elements 32db + 16*dhalf + 4*(s%4) .. +3 (s = lane%16, dhalf = (lane/16)%2) and receives
   // V[16t + 8ld + 4lh + 0..3][32db + lq]
-  unsigned v_addr[4][2];
+  u32x8 v_addr;  // index 2 * db + ld
   {
     const int s = lane & 15, dhalf = (lane >> 4) & 1;
 #pragma unroll
@@ -263,35 +244,71 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       for (int db = 0; db < 4; db++) {
         int chunk = 4 * db + 2 * dhalf + ((s & 3) >> 1);
         // the V region's base is folded in here so that stage and k-step offsets fit the 16-bit ds_read immediate
-        v_addr[db][ld] = (unsigned)(KSTAGES * STAGE_BYTES + row * ROW_BYTES + 16 * (chunk ^ swz(row)) + 8 * (s & 1));
+        v_addr[2 * db + ld] = (unsigned)(KSTAGES * STAGE_BYTES + row * ROW_BYTES + 16 * (chunk ^ swz(row)) + 8 * (s & 1));
       }
     }
   }
 
 
-  // ---- prologue: first tiles on their way, Q into registers ---------------------------------------------------------
+  // ---- first loads of a part ---------------------------------------------------------------------------------------------
   // K runs one tile ahead of V in consumption (scores are formed two halves before their P.V), so K is requested
   // four tiles ahead and V three: iteration j sends for K(j+4) (stage of K(j), last read in iteration j-1) and
-  // V(j+3) (stage of V(j-1)).
-  vec8 qreg[8];
-  {
-    int row = qw0 + lq;
-    row = row < a.L ? row : a.L - 1;
-    const T* qr = qp + row * a.qs[2] + 8 * lh;
-#pragma unroll
-    for (int ks = 0; ks < 8; ks++) qreg[ks] = *(const vec8*)(qr + 16 * ks);
-  }
-  // Order of need: K(0) for the first scores, then K(1), V(0), ...; with four tiles or more the waits below let the
-  // later ones land while the first scores are formed.
-  const bool staged_start = ntiles_kv >= 4;
-  dma_k(0, 0);
-  if (1 < ntiles_kv) dma_k(1, 1);
-  dma_v(0, 0);
-  if (2 < ntiles_kv) dma_k(2, 2);
-  if (1 < ntiles_kv) dma_v(1, 1);
-  if (3 < ntiles_kv) dma_k(3, 3);
-  if (2 < ntiles_kv) dma_v(2, 2);
+  // V(j+3) (stage of V(j-1)).  A part starts with K(0..3) and V(0..2) on their way.  For the second part they are sent
+  // for before the first part's output is written: all stages but the last V stage, which the output passes through,
+  // are free then.
+  auto issue_tiles = [&](int part) __attribute__((always_inline)) {
+    int q0, ntiles_kv;
+    part_rows(part, q0, ntiles_kv);
+    kpage[0] = -1, vpage[0] = -1;
+    dma_k(0, 0);
+    if (1 < ntiles_kv) dma_k(1, 1);
+    dma_v(0, 0);
+    if (2 < ntiles_kv) dma_k(2, 2);
+    if (1 < ntiles_kv) dma_v(1, 1);
+    if (3 < ntiles_kv) dma_k(3, 3);
+    if (2 < ntiles_kv) dma_v(2, 2);
+  };
+  issue_tiles(0);
+  u32x32 qv;  // the lane's Q operands, k-step ks in elements 4ks .. 4ks+3
 
+
+  for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
+  if (part == 1 && !two_parts) break;
+  int q0, ntiles_kv;
+  part_rows(part, q0, ntiles_kv);
+  const int qw0 = q0 + rowgroup * WM;
+
+  // Query row i sees keys up to i + coff (coff = 0: the reference's top-left aligned mask); qc0 is this wavefront's
+  // first row in key coordinates.
+  const int coff = CAUSAL ? causal_offset(a, S) : 0;
+  const int qc0 = qw0 + coff;
+  // 32-key halves this wavefront computes on: under a causal mask those that start at or before its last row
+  int my_halves = 2 * ntiles_kv;
+  if (CAUSAL) {
+    int t = (qc0 + WM - 1) / 32 + 1;
+    my_halves = t < my_halves ? t : my_halves;
+  }
+  // Tiles j whose two steps take the fast form: halves up to 2j+3 are this wavefront's, tile j+1 is complete, and
+  // half 2j+2 (whose exponentials step 2j+1 takes) needs no mask.
+  int nfast = (my_halves - 2) / 2;
+  {
+    int f = S >= 96 ? (S - 32) / BN : 0;
+    nfast = f < nfast ? f : nfast;
+    if (CAUSAL) {
+      f = qc0 >= 95 ? (qc0 - 31) / BN : 0;
+      nfast = f < nfast ? f : nfast;
+    }
+  }
+  if (nfast < 0) nfast = 0;
+  if (a.mask_kind != 0) nfast = 0;  // an attnMask is applied in the general form of a step
+
+  // ---- prologue: the part's first loads were sent for by issue_part ------------------------------------------------
+  auto q_of = [&](int ks) __attribute__((always_inline)) {
+    u32x4 w;
+#pragma unroll
+    for (int i = 0; i < 4; i++) w[i] = qv[4 * ks + i];
+    return __builtin_bit_cast(vec8, w);
+  };
   f32x16 oacc[4];
 #pragma unroll
   for (int db = 0; db < 4; db++)
@@ -309,7 +326,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #pragma unroll
     for (int ks = 0; ks < 8; ks++) {
       vec8 ka = *(const vec8*)(kh + k_addr[ks]);
-      s = TR::mfma32(ka, qreg[ks], s);
+      s = TR::mfma32(ka, q_of(ks), s);
     }
   };
 
@@ -384,8 +401,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     for (int t = 0; t < 2; t++)
 #pragma unroll
       for (int db = 0; db < 4; db++) {
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vh + v_addr[db][0] + 16 * t * ROW_BYTES));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vh + v_addr[db][1] + 16 * t * ROW_BYTES));
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vh + v_addr[2 * db] + 16 * t * ROW_BYTES));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vh + v_addr[2 * db + 1] + 16 * t * ROW_BYTES));
         vec8 va = __builtin_bit_cast(vec8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         oacc[db] = TR::mfma32(va, pb[t], oacc[db]);
       }
@@ -410,58 +427,70 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     }
   };
 
-  // ---- fast form: hand-ordered, one MFMA per slot, operands fetched PD slots ahead -------------------------------------
+  // ---- fast form: the 16 slots of a step as one statement of hand-ordered instructions (prefill128_steps.inc) ---------
   // A tile iteration has 32 slots (two steps of 16).  Even slot 2i of a step is the S^T MFMA of k-step i, odd slot
   // 2i+1 the P.V MFMA (t = i/4, db = i%4): the dependent S^T chain is spaced by independent P.V MFMAs.  Each slot
-  // also carries one score's scale/exp (and every second slot the pair's conversion), and requests the LDS operand
-  // of the slot PD places further on into a ring of RING operand registers.
-  constexpr int PD = 6, RING = 8;  // RING divides the 128 slots of the unrolled body
-  vec8 ring[RING];
-  auto fetch = [&](const int G) __attribute__((always_inline)) {  // G: slot index within the 4-tile unrolled body
-    const int u = (G >> 5) & 3, kind = (G >> 4) & 1, s = G & 15, i = s >> 1;
-    if ((s & 1) == 0) {
-      const char* base = smem + ((u + 1) & 3) * STAGE_BYTES + kind * 32 * ROW_BYTES;
-      ring[G % RING] = *(const vec8*)(base + k_addr[i]);
-    } else {
-      const int t = i >> 2, db = i & 3;
-      const char* base = smem + u * STAGE_BYTES + kind * 32 * ROW_BYTES + 16 * t * ROW_BYTES;
-      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + v_addr[db][0]));
-      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + v_addr[db][1]));
-      ring[G % RING] = __builtin_bit_cast(vec8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-    }
-  };
-  auto fast_step = [&](const int G0, f32x16& s_new, const f32x16& s_nxt, const vec8 (&p_cur)[2], vec8 (&p_nxt)[2]) __attribute__((always_inline)) {
-    float psum = 0.f;
-    f32x8 x;
+  // also carries one score's scale / exp2 / sum (and every second slot a pair's conversion), each issued a slot
+  // apart from the instruction it depends on, and requests the LDS operand of the slot 6 places further on into a
+  // ring of 8 operand registers.  The statements name fixed registers for everything a vector instruction touches
+  // piecewise (scores, probabilities, operand ring, Q, LDS addresses); the output accumulators are ordinary operands.
+  u32x32 ring;
 #pragma unroll
-    for (int s = 0; s < 16; s++) {
-      const int G = G0 + s, i = s >> 1;
-      fetch((G + PD) & 127);
-      if ((s & 1) == 0) {
-        if (i == 0) {
-#pragma unroll
-          for (int r = 0; r < 16; r++) s_new[r] = 0.f;
-        }
-        s_new = TR::mfma32(ring[G % RING], qreg[i], s_new);
-      } else {
-        oacc[i & 3] = TR::mfma32(ring[G % RING], p_cur[i >> 2], oacc[i & 3]);
-      }
-      x[s & 7] = fast_exp2(fmaf(s_nxt[s], c, -mc));
-      psum += x[s & 7];
-      if ((s & 7) == 7) p_nxt[s >> 3] = __builtin_convertvector(x, vec8);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    settle_half(s_nxt, p_nxt, psum);
-  };
+  for (int i = 0; i < 32; i++) ring[i] = 0u;
+#define TT_P128_RUN_STEP(TXT)                                                                                          \
+  asm volatile(TXT                                                                                                     \
+               : [o0] "+v"(oacc[0]), [o1] "+v"(oacc[1]), [o2] "+v"(oacc[2]), [o3] "+v"(oacc[3]), [ps] "=&v"(psum_step),  \
+                 "+{v[160:175]}"(sB), "+{v[176:191]}"(sC), "+{v[192:199]}"(pAv), "+{v[200:207]}"(pBv),                   \
+                 "+{v[208:239]}"(ring)                                                                                 \
+               : [c] "v"(c), [mc] "v"(mc), "{v[120:151]}"(qv), "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr)            \
+               : "v240", "v241", "v242", "v243", "v244", "v245", "memory")
+  constexpr bool kIsBf16 = sizeof(typename TR::elem) == 2 && __is_same(typename TR::elem, __bf16);
 
   f32x16 sB, sC;
   vec8 pA[2], pB[2];
-  if (staged_start) {
-    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // Q and K(0) are here; six tiles (12 loads) may be on their way
+  u32x8 pAv, pBv;  // P of a half as two MFMA B operands (k-steps of 16 keys), 4 registers each
+  float psum_step;
+  auto p_load = [&](const u32x8& pv, vec8 (&p)[2]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      u32x4 w;
+#pragma unroll
+      for (int i = 0; i < 4; i++) w[i] = pv[4 * t + i];
+      p[t] = __builtin_bit_cast(vec8, w);
+    }
+  };
+  auto p_store = [&](u32x8& pv, const vec8 (&p)[2]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      const u32x4 w = __builtin_bit_cast(u32x4, p[t]);
+#pragma unroll
+      for (int i = 0; i < 4; i++) pv[4 * t + i] = w[i];
+    }
+  };
+  // Q into its registers, and everything sent for so far in place.  One statement: the compiler takes a statement's
+  // results as valid when it ends, so the wait has to be part of it (and, not knowing of the tile loads, the compiler
+  // would place waits of its own for plain loads that in effect wait for every tile).
+  {
+    const int first = qw0 < a.L ? qw0 : a.L - 1;  // rows past the end re-read the last row (never stored)
+    int row = qw0 + lq;
+    row = row < a.L ? row : a.L - 1;
+    const char* qbase = (const char*)(qp + (long long)first * a.qs[2]);
+    const unsigned qoff = ((unsigned)(row - first) * (unsigned)a.qs[2] + 8u * lh) * 2u;  // the host checks that 32 rows fit 32 bits
+    asm volatile(
+        "global_load_dwordx4 v[120:123], %1, %2\n\t"
+        "global_load_dwordx4 v[124:127], %1, %2 offset:32\n\t"
+        "global_load_dwordx4 v[128:131], %1, %2 offset:64\n\t"
+        "global_load_dwordx4 v[132:135], %1, %2 offset:96\n\t"
+        "global_load_dwordx4 v[136:139], %1, %2 offset:128\n\t"
+        "global_load_dwordx4 v[140:143], %1, %2 offset:160\n\t"
+        "global_load_dwordx4 v[144:147], %1, %2 offset:192\n\t"
+        "global_load_dwordx4 v[148:151], %1, %2 offset:224\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "={v[120:151]}"(qv)
+        : "v"(qoff), "s"(qbase)
+        : "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-  } else {
-    dma_wait_and_sync(0);
   }
   {  // P(0) and the scores of half 1
     qk_half(sC, half_base(0));
@@ -472,7 +501,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }
   // Every wavefront has read K(0): iteration 0 may overwrite its stage.  K(1), V(0), K(2), V(1) must be visible
   // before iteration 0; K(3) and V(2) (4 loads) are waited for at its end.
-  dma_wait_and_sync(staged_start ? 4 : 0);
+  dma_wait_and_sync(0);
 
   auto tile_dma = [&](int j) __attribute__((always_inline)) {
     int keep = 0;
@@ -489,23 +518,40 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
   int j = 0;
   if (nfast >= 1) {
-#pragma unroll
-    for (int g = 0; g < PD; g++) fetch(g);
-    // Four tiles per trip so that the stage of a tile is a compile-time constant; the trip may end after any of them.
-    for (bool more = true; more;) {
-#pragma unroll
-      for (int u = 0; u < 4; u++) {
-        if (j >= nfast) {
-          more = false;
-          break;
-        }
-        const int keep = tile_dma(j);
-        fast_step(32 * u, sC, sB, pA, pB);
-        fast_step(32 * u + 16, sB, sC, pB, pA);
-        dma_wait_and_sync(keep);
-        j++;
-      }
+    auto settle_fast = [&](const f32x16& s, u32x8& pv) __attribute__((always_inline)) {
+      vec8 p[2];
+      p_load(pv, p);
+      settle_half(s, p, psum_step);
+      p_store(pv, p);
+    };
+    p_store(pAv, pA);
+    p_store(pBv, pB);
+    asm volatile(TT_P128_PREFETCH : "+{v[208:239]}"(ring) : "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr) : "memory");
+    // Four tiles per trip so that the stage of a tile is a constant of its statement; the trip may end after any of them.
+#define TT_P128_TILE(U)                                                                                  \
+    if (j >= nfast) break;                                                                                \
+    {                                                                                                    \
+      const int keep = tile_dma(j);                                                                      \
+      if constexpr (kIsBf16) TT_P128_RUN_STEP(TT_P128_STEP_BF16_U##U##_K0);                              \
+      else TT_P128_RUN_STEP(TT_P128_STEP_F16_U##U##_K0);                                                 \
+      settle_fast(sB, pBv);                                                                              \
+      if constexpr (kIsBf16) TT_P128_RUN_STEP(TT_P128_STEP_BF16_U##U##_K1);                              \
+      else TT_P128_RUN_STEP(TT_P128_STEP_F16_U##U##_K1);                                                 \
+      settle_fast(sC, pAv);                                                                              \
+      dma_wait_and_sync(keep);                                                                           \
+      j++;                                                                                               \
     }
+    for (;;) {
+      TT_P128_TILE(0)
+      TT_P128_TILE(1)
+      TT_P128_TILE(2)
+      TT_P128_TILE(3)
+    }
+#undef TT_P128_TILE
+    // the ring's last requests belong to a step that takes the general form: let them land before the registers are reused
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+{v[208:239]}"(ring) : : "memory");
+    p_load(pAv, pA);
+    p_load(pBv, pB);
   }
   for (; j < ntiles_kv; j++) {
     const int keep = tile_dma(j);
@@ -513,6 +559,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     slow_step(2 * j + 1, pB, sC, sB, pA);
     dma_wait_and_sync(keep);
   }
+
+  if (CAUSAL && part == 0 && two_parts) issue_tiles(1);
 
   // ---- normalise, transpose through LDS, store whole rows -----------------------------------------------------------------
   // A lane holds 4 consecutive head_dim elements per register group of its query row: stored directly, every store

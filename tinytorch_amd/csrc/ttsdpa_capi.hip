@@ -119,7 +119,8 @@ bool f32_prefill_ok(const ttsdpa_params* p) {
 }
 
 bool pipelined_ok(const ttsdpa_params* p) {
-  return p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
+  // the kernel addresses the 64 rows of a K / V tile and the 256 rows of a Q tile with 32-bit byte offsets
+  return p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22);
 }
 
 // Few query rows per head against many keys on the 4-wavefront kernel: the G heads of a KV head share one row tile
