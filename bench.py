@@ -12,6 +12,16 @@ fusedAddRmsNorm, siluMul, softmax; HBM-bound) under "fused_ops" and the linear l
 token batch; MFMA-bound) under "linear", and the attention backward (dq, dk, dv at config 3's shape; MFMA-bound) under
 "backward" (bf16, and the same shape in fp32 on the fp32 matrix cores under "backward"."fp32").  One JSON line is printed.
 
+Timing.  After the --warmup launches comes a declared, untimed settle phase (about SETTLE_SECONDS of back-to-back
+launches, its length reported as "settle_launches"): the core clock of this chip takes that long to reach its level under
+a kernel, and without it the first timed launches measure the ramp.  Then --steps launches are timed, each between its own
+pair of HIP events on the launch stream; "kernel_ms" is the median of the launches ("kernel_ms_mean" beside it), and
+"ms_per_step" / "value" come from the host clock around the same --steps launches (synchronised on both sides).
+Inputs are drawn by tinytorch_amd.synth (counter-based normal generator, seed 0x5EED0000 + config number, one stream
+per tensor), rounded to the workload's element type.
+The other configurations of the baseline (1, 2, 5) and config 3's shape at head_dim 64 are measured the same way and
+reported under "other_configs".
+
 Algorithmic work per launch (what "achieved" divides by the measured launch time):
   prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)
   prefill, full:    4 * B * Hq * L * S * D flop
@@ -30,6 +40,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}  # MI355X dense MFMA peaks
 PEAK_HBM_GBS = 8000.0
+SETTLE_SECONDS = 0.4   # untimed launches after the warm-up, until the core clock has settled under the kernel
+TRAFFIC_SOURCE = ("profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of the same "
+                  "command, scaled by a 1 GiB copy; not measured in this run")
 
 WORKLOADS = {
     # name: (B, Hq, Hkv, L, S, D, dtype, causal, input multiplier, bound)
@@ -39,7 +52,10 @@ WORKLOADS = {
     "config4": (64, 32, 8, 1, 8192, 128, "bf16", False, 1.0, "hbm"),
     "config5": (1, 28, 4, 16384, 16384, 128, "bf16", True, 1.0, "mfma"),
     "config3_f32": (2, 32, 8, 4096, 4096, 128, "f32", True, 1.0, "mfma"),  # config 3's shape in the reference's default dtype
+    "config3_d64": (2, 32, 8, 4096, 4096, 64, "bf16", True, 1.0, "mfma"),   # config 3's shape at head_dim 64
 }
+SEEDS = {"config1": 0x5EED0001, "config2": 0x5EED0002, "config3": 0x5EED0003, "config4": 0x5EED0004, "config5": 0x5EED0005,
+         "config3_f32": 0x5EED0003, "config3_d64": 0x5EED0006}
 DESCR = {
     "config1": "fp32 causal SDPA B1 H4 S128 D64",
     "config2": "fp16 causal MHA prefill B4 H32 S2048 D128",
@@ -47,6 +63,7 @@ DESCR = {
     "config4": "bf16 decode B64 32q/8kv L1 KV8192 D128 (isCausal=false)",
     "config5": "bf16 causal GQA prefill B1 28q/4kv S16384 D128",
     "config3_f32": "fp32 causal GQA prefill B2 32q/8kv S4096 D128",
+    "config3_d64": "bf16 causal GQA prefill B2 32q/8kv S4096 D64",
 }
 
 
@@ -71,16 +88,58 @@ def measured_traffic(name):
         return json.load(f).get(name, {}).get("hbm_bytes_per_launch")
 
 
+def time_launches(step, stream, steps, warmup, settle_seconds=SETTLE_SECONDS):
+    """warmup untimed launches, a declared untimed settle phase, then `steps` launches each between its own pair of HIP
+    events on `stream`.  Returns per-launch device times (median, mean, min; ms), the host-clock time per step around
+    the timed launches, and the number of settle launches."""
+    import torch
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    settle = 0
+    if settle_seconds > 0:
+        t_end = time.perf_counter() + settle_seconds
+        while time.perf_counter() < t_end:
+            for _ in range(16):
+                step()
+            settle += 16
+            if settle % 256 == 0:
+                torch.cuda.synchronize()  # keeps the launch queue (and the phase's length) bounded
+        torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for e0, e1 in events:
+        e0.record(stream)
+        step()
+        e1.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms = sorted(e0.elapsed_time(e1) for e0, e1 in events)
+    return {"median_ms": ms[len(ms) // 2], "mean_ms": sum(ms) / len(ms), "min_ms": ms[0], "wall_ms": wall_ms,
+            "settle_launches": settle}
+
+
+def synth_qkv(name):
+    """The workload's Q, K, V on the device: N(0,1) * multiplier from the repository's generator, rounded to its dtype."""
+    import torch
+    from tinytorch_amd import synth
+
+    B, Hq, Hkv, L, S, D, dtype, causal, mul, bound = WORKLOADS[name]
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    seed = SEEDS[name]
+    q = synth.randn(seed, 0, (B, Hq, L, D), mul).to(td)
+    k = synth.randn(seed, 1, (B, Hkv, S, D), mul).to(td)
+    v = synth.randn(seed, 2, (B, Hkv, S, D), mul).to(td)
+    return q, k, v
+
+
 def run_gpu(name, steps, warmup):
     import torch
     from tinytorch_amd import _capi, build_params
 
     B, Hq, Hkv, L, S, D, dtype, causal, mul, bound = WORKLOADS[name]
-    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
-    gen = torch.Generator(device="cuda").manual_seed(0x5EED)
-    q = (torch.randn(B, Hq, L, D, device="cuda", generator=gen) * mul).to(td)
-    k = (torch.randn(B, Hkv, S, D, device="cuda", generator=gen) * mul).to(td)
-    v = (torch.randn(B, Hkv, S, D, device="cuda", generator=gen) * mul).to(td)
+    q, k, v = synth_qkv(name)
     out = torch.empty_like(q)
     p = build_params(q, k, v, out, causal)
     lib = _capi.lib()
@@ -95,18 +154,8 @@ def run_gpu(name, steps, warmup):
         if rc != 0:
             raise RuntimeError("ttsdpa_forward: %s" % _capi.status_string(rc))
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record(stream)
-    for _ in range(steps):
-        step()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    dev_ms = e0.elapsed_time(e1) / steps  # HIP events on the launch stream: average duration per launch
+    t = time_launches(step, stream, steps, warmup)
+    wall_ms, dev_ms = t["wall_ms"], t["median_ms"]  # HIP events on the launch stream, one pair per launch: the median
 
     flops, abytes = algorithmic_work(B, Hq, Hkv, L, S, D, dtype, causal)
     if bound == "mfma":
@@ -120,7 +169,10 @@ def run_gpu(name, steps, warmup):
         "value": round(value, 3), "unit": unit, "ms_per_step": round(wall_ms, 5),
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
                      "frac": round(achieved / peak, 4), "traffic": measured_traffic(name),
-                     "kernel_ms": round(dev_ms, 5), "algorithmic_flops": flops, "algorithmic_bytes": abytes},
+                     "traffic_source": TRAFFIC_SOURCE if measured_traffic(name) is not None else None,
+                     "kernel_ms": round(dev_ms, 5), "kernel_ms_mean": round(t["mean_ms"], 5),
+                     "kernel_ms_min": round(t["min_ms"], 5), "timing": "median of %d launches, one HIP event pair each" % steps,
+                     "settle_launches": t["settle_launches"], "algorithmic_flops": flops, "algorithmic_bytes": abytes},
     }
     return res, (q, k, v, out)
 
@@ -212,20 +264,14 @@ def run_fused(name, steps, warmup, cpu=True):
     first = None
     if op == "add_rms_norm":
         first = (x[:64].float().cpu().numpy(), res[:64].float().cpu().numpy())  # before further in-place passes
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(steps):
-        step()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / steps
+    t = time_launches(step, stream, steps, warmup)
+    ms = t["median_ms"]
     res_line = {"workload": "%s bf16 [%d, %d]" % (name, rows, cols), "dtype": "bf16", "ms_per_step": round(ms, 5),
+                "kernel_ms_mean": round(t["mean_ms"], 5), "settle_launches": t["settle_launches"],
                 "roofline": {"bound": "hbm", "achieved": round(abytes / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                              "unit": "GB/s", "frac": round(abytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                             "traffic": measured_traffic(name), "algorithmic_bytes": abytes}}
+                             "traffic": measured_traffic(name), "traffic_source": TRAFFIC_SOURCE,
+                             "algorithmic_bytes": abytes}}
     if cpu:
         import oracle
         kind = "reference" if oracle.have_ref() else "port"
@@ -284,21 +330,14 @@ def run_linear(steps, warmup, cpu=True):
                                   stream.cuda_stream)
         if rc != 0:
             raise RuntimeError("ttlinear_forward: %s" % _capi.status_string(rc))
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(steps):
-        step()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / steps
+    t = time_launches(step, stream, steps, warmup)
+    ms = t["median_ms"]
     flops = 2 * M * N * K
     res = {"workload": "linear bf16 x[%d,%d] . w[%d,%d]^T + bias" % (M, K, N, K), "dtype": "bf16", "ms_per_step": round(ms, 5),
+           "kernel_ms_mean": round(t["mean_ms"], 5), "settle_launches": t["settle_launches"],
            "roofline": {"bound": "mfma", "achieved": round(flops / (ms * 1e-3) / 1e12, 1), "peak": PEAK_TFLOPS["bf16"],
                         "unit": "TFLOP/s", "frac": round(flops / (ms * 1e-3) / 1e12 / PEAK_TFLOPS["bf16"], 4),
-                        "traffic": measured_traffic("linear"), "algorithmic_flops": flops,
+                        "traffic": measured_traffic("linear"), "traffic_source": TRAFFIC_SOURCE, "algorithmic_flops": flops,
                         "algorithmic_bytes": 2 * (M * K + N * K + M * N + N)}}
     if cpu:
         import oracle
@@ -337,12 +376,12 @@ def run_backward(steps, warmup, cpu=True, dtype="bf16"):
     B, Hq, Hkv, L, S, D = 2, 32, 8, 4096, 4096, 128
     lib = _capi.lib()
     stream = torch.cuda.current_stream()
-    gen = torch.Generator(device="cuda").manual_seed(0x5EED)
+    from tinytorch_amd import synth
     td = torch.bfloat16 if dtype == "bf16" else torch.float32
-    q = torch.randn(B, Hq, L, D, device="cuda", generator=gen).to(td)
-    k = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).to(td)
-    v = torch.randn(B, Hkv, S, D, device="cuda", generator=gen).to(td)
-    go = torch.randn(B, Hq, L, D, device="cuda", generator=gen).to(td)
+    q = synth.randn(0x5EED0003, 0, (B, Hq, L, D)).to(td)
+    k = synth.randn(0x5EED0003, 1, (B, Hkv, S, D)).to(td)
+    v = synth.randn(0x5EED0003, 2, (B, Hkv, S, D)).to(td)
+    go = synth.randn(0x5EED0003, 3, (B, Hq, L, D)).to(td)
     out = sdpAttention(q, k, v, isCausal=True)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     bp = build_backward_params(q, k, v, out, go, dq, dk, dv, True)
@@ -355,24 +394,17 @@ def run_backward(steps, warmup, cpu=True, dtype="bf16"):
         rc = lib.ttsdpa_backward(ctypes.byref(bp), ws.data_ptr(), nbytes, stream.cuda_stream)
         if rc != 0:
             raise RuntimeError("ttsdpa_backward: %s" % _capi.status_string(rc))
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(steps):
-        step()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / steps
+    t = time_launches(step, stream, steps, warmup)
+    ms = t["median_ms"]
     flops = 2.5 * 4.0 * B * Hq * L * S * D * 0.5
     tf = flops / (ms * 1e-3) / 1e12
     kernels = "backward_dq128_kernel + backward_dkv128_kernel" if dtype == "bf16" else "backward_dq_f32_kernel + backward_dkv_f32_kernel"
     res = {"workload": "attention backward %s B%d %dq/%dkv L=S=%d D%d causal" % (dtype, B, Hq, Hkv, L, D), "dtype": dtype,
-           "route": _capi.ROUTE_NAMES[route.value], "ms_per_step": round(ms, 5), "value": round(tf, 1), "unit": "TFLOP/s",
+           "route": _capi.ROUTE_NAMES[route.value], "ms_per_step": round(ms, 5), "kernel_ms_mean": round(t["mean_ms"], 5),
+           "settle_launches": t["settle_launches"], "value": round(tf, 1), "unit": "TFLOP/s",
            "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_TFLOPS[dtype], "unit": "TFLOP/s",
                         "frac": round(tf / PEAK_TFLOPS[dtype], 4),
-                        "traffic": measured_traffic("backward" if dtype == "bf16" else "backward_f32"),
+                        "traffic": measured_traffic("backward" if dtype == "bf16" else "backward_f32"), "traffic_source": TRAFFIC_SOURCE,
                         "algorithmic_flops": flops, "kernels": kernels + " per step"}}
     if cpu:
         import oracle
@@ -391,9 +423,11 @@ def run_backward(steps, warmup, cpu=True, dtype="bf16"):
     return res
 
 
-def run_cpu_baseline(name, tensors, budget_s=20.0):
+def run_cpu_baseline(name, tensors, budget_s=20.0, corner=None):
     """The reference CPU path (compiled reference if oracle/_ref is present, else this repository's C restatement)
-    on one host core, over as many (batch, head) slices of the same inputs as fit the time budget."""
+    on one host core, over as many (batch, head) slices of the same inputs as fit the time budget.  corner=n (causal
+    workloads with L == S): only the first n queries against the first n keys of a slice, which under the top-left
+    aligned mask is an attention problem of its own (rows below n see keys below n only)."""
     import numpy as np
     import oracle
 
@@ -402,17 +436,20 @@ def run_cpu_baseline(name, tensors, budget_s=20.0):
     kind = "reference" if oracle.have_ref() else "port"
     fn = oracle.ref_sdpa_f32 if kind == "reference" else (lambda *a, **kw: oracle.sdpa_f32(*a, nthreads=1, **kw))
     G = Hq // Hkv
+    if corner is not None:
+        assert causal and L == S
+        L = S = min(corner, L)
     flops_slice, _ = algorithmic_work(1, 1, 1, L, S, D, dtype, causal)
     done, spent, worst = 0, 0.0, 0.0
     slices = [(b, h) for b in range(B) for h in range(Hq)]
     for (b, h) in slices:
-        qs = q[b:b + 1, h:h + 1].float().cpu().numpy()
-        ks = k[b:b + 1, h // G:h // G + 1].float().cpu().numpy()
-        vs = v[b:b + 1, h // G:h // G + 1].float().cpu().numpy()
+        qs = q[b:b + 1, h:h + 1, :L].float().cpu().numpy()
+        ks = k[b:b + 1, h // G:h // G + 1, :S].float().cpu().numpy()
+        vs = v[b:b + 1, h // G:h // G + 1, :S].float().cpu().numpy()
         t0 = time.perf_counter()
         ref = fn(qs, ks, vs, causal=causal)
         dt = time.perf_counter() - t0
-        err = float(np.abs(ref - out[b:b + 1, h:h + 1].float().cpu().numpy()).max())
+        err = float(np.abs(ref - out[b:b + 1, h:h + 1, :L].float().cpu().numpy()).max())
         worst = max(worst, err)
         done += 1
         spent += dt
@@ -425,22 +462,24 @@ def run_cpu_baseline(name, tensors, budget_s=20.0):
         slice_bytes = (2 * S * D * esz) / G + 2 * L * D * esz  # a query head's share of its KV head + q + out
         val, unit = slice_bytes * done / spent / 1e9, "GB/s"
     return {"value": float("%.4g" % val), "unit": unit, "cores": 1, "host_cores": os.cpu_count(), "kind": kind,
-            "sample": "%d of %d (batch, head) slices of the same inputs, %.1f s, one thread; whole-job estimate %.1f s"
-                      % (done, len(slices), spent, spent / done * len(slices)),
+            "sample": "%d of %d (batch, head) slices of the same inputs%s, %.1f s, one thread%s"
+                      % (done, len(slices), "" if corner is None else " (their first %d queries x %d keys)" % (L, S), spent,
+                         "; whole-job estimate %.1f s" % (spent / done * len(slices)) if corner is None else ""),
             "max_abs_err_gpu_vs_cpu": float("%.3g" % worst)}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=500)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS))
     ap.add_argument("--secondary", default="config4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-probes", action="store_true", help="skip the hardware ceiling probes")
+    ap.add_argument("--no-other", action="store_true", help="skip the baseline's other configurations (1, 2, 5) and head_dim 64")
     ap.add_argument("--no-fused", action="store_true", help="skip the row-wise neighbour ops (rmsNorm, siluMul, ...)")
     ap.add_argument("--fused-only", default=None, choices=sorted(FUSED_WORKLOADS),
                     help="measure one row-wise op only and print its line (for profiling)")
@@ -483,7 +522,7 @@ def main():
         "metric": "attn prefill TFLOP/s + decode KV GB/s on 1 MI355X (% of roofline)",
         "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": main_res["dtype"], "data": "synthetic (torch.randn on device, seed 0x5EED)",
+        "vs_baseline": None, "dtype": main_res["dtype"], "data": "synthetic (tinytorch_amd.synth: counter-based N(0,1), seed 0x5EED0000 + config number, a stream per tensor)",
         "config": {"workload": "%s: %s" % (args.workload, main_res["description"]), "route": main_res["route"]},
         "roofline": main_res["roofline"], "cpu_baseline": cpu,
     }
@@ -498,6 +537,17 @@ def main():
             f32, tensors = run_gpu("config3_f32", max(1, min(args.steps, 100)), min(args.warmup, 20))
             del tensors
             line["fp32"] = f32
+    if not args.no_other and args.workload == "config3":
+        # the baseline's other configurations (config 1: launch-sized, its time is the figure) and head_dim 64
+        line["other_configs"] = []
+        for name, corner, budget in (("config1", None, 2.0), ("config2", None, 4.0), ("config5", 4096, 4.0),
+                                     ("config3_d64", 2048, 3.0)):
+            torch.cuda.empty_cache()
+            res, tensors = run_gpu(name, max(1, min(args.steps, 50)), min(args.warmup, 20))
+            if not args.no_cpu:
+                res["cpu_baseline"] = run_cpu_baseline(name, tensors, budget, corner)
+            del tensors
+            line["other_configs"].append(res)
     if not args.no_fused:
         torch.cuda.empty_cache()
         line["fused_ops"] = [run_fused(n, max(1, min(args.steps, 100)), min(args.warmup, 20), cpu=not args.no_cpu)

@@ -334,3 +334,20 @@ def test_backward_params_layout_routes_and_validation():
     assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_GENERAL
     L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.F32, 0, 4, 4, 32, 32, 64)
     assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_NONE
+
+
+def test_build_params_refuses_a_mask_on_another_device():
+    """The mask's address goes to the kernels as it is: a mask that does not live with the tensors must be refused on
+    the host (a host pointer dereferenced by a kernel is a GPU memory fault)."""
+    import torch
+    import tinytorch_amd
+
+    q = torch.zeros(1, 2, 4, 8)
+    k = torch.zeros(1, 2, 6, 8)
+    out = torch.empty_like(q)
+    mask = torch.ones(4, 6, dtype=torch.bool, device="meta")
+    with pytest.raises(RuntimeError, match="attnMask must live on the device"):
+        tinytorch_amd.build_params(q, k, k, out, False, mask)
+    p = tinytorch_amd.build_params(q, k, k, out, False, torch.ones(4, 6, dtype=torch.bool))  # same device: accepted
+    assert p.mask_kind == 1
+

@@ -171,7 +171,10 @@ bool prefill_ok(const ttsdpa_params* p) {
   // the pipelined head_dim-128 kernel takes any attnMask; the 4-wavefront kernel those it can read four keys at a time
   const bool mfma_head_dim = p->D == 32 || p->D == 64 || p->D == 96 || p->D == 128 || p->D == 256;
   if (p->block_table && p->page_size < kPrefillMinPage) return false;
-  return fast_layout_ok(p, true, true) && mfma_head_dim && p->S >= 1 && p->L >= 1 && (pipelined_ok(p) || simple_mask_ok(p));
+  // the 16-bit kernels address the rows of a K / V tile with 32-bit byte offsets (the fp32 kernel returned above does not)
+  const bool tile_offsets_ok = p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
+  return fast_layout_ok(p, true, true) && mfma_head_dim && p->S >= 1 && p->L >= 1 && tile_offsets_ok &&
+         (pipelined_ok(p) || simple_mask_ok(p));
 }
 
 bool decode_ok(const ttsdpa_params* p) {
@@ -445,6 +448,11 @@ int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t wor
     if (check_grid(g1) != TTSDPA_OK || check_grid(g2) != TTSDPA_OK) return TTSDPA_ERR_SHAPE;
     if (p->fwd.dtype == TTSDPA_F32) return launch_backward_f32(a, (hipStream_t)stream);
     return launch_backward_mfma(a, p->fwd.dtype, (hipStream_t)stream);
+  }
+  {  // the vector-ALU pair: 64 rows per workgroup up to head_dim 128, 32 beyond
+    const int rows = a.f.D <= 128 ? 64 : 32;
+    const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + rows - 1) / rows), g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + rows - 1) / rows);
+    if (check_grid(g1) != TTSDPA_OK || check_grid(g2) != TTSDPA_OK) return TTSDPA_ERR_SHAPE;
   }
   return launch_backward_general(a, p->fwd.dtype, (hipStream_t)stream);
 }

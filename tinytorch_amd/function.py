@@ -13,17 +13,14 @@ import torch
 from . import _capi
 
 _DTYPES = {torch.float32: _capi.F32, torch.float16: _capi.F16, torch.bfloat16: _capi.BF16}
-_workspaces = {}
 
 
 def _workspace(device, nbytes):
-    """Device scratch for the decode route, grown on demand and kept per device (the reference's ops take such
-    scratch from the caching allocator, src/Operation/OpNNLayerCuda.cuh:415)."""
-    buf = _workspaces.get(device)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[device] = buf
-    return buf
+    """Device scratch of one call, taken from torch's caching allocator as the reference's ops take theirs from its own
+    (src/Operation/OpNNLayerCuda.cuh:415).  A buffer per call, not one kept per device: the allocator orders reuse by
+    stream and keeps allocations made under graph capture in the graph's pool, so a captured call keeps its scratch for
+    every replay and calls on different streams never share partial results."""
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
 
 
 def _strides3(t):
@@ -71,6 +68,9 @@ def build_params(query, key, value, out, isCausal=False, attnMask=None, scale=No
     if attnMask is not None:
         if isCausal:
             raise ValueError("sdpAttention: isCausal and attnMask are exclusive")  # reference FuncNNLayer.h:242
+        if attnMask.device != query.device:  # its address goes to the kernels as is: a host pointer would fault the GPU
+            raise RuntimeError("sdpAttention: attnMask must live on the device of the tensors (got %s, tensors on %s)"
+                               % (attnMask.device, query.device))
         if attnMask.dim() > 4:
             raise ValueError("sdpAttention: attnMask must broadcast to [B, H, L, S]")
         try:  # the reference adds the mask with a broadcasting add (FuncNNLayer.h:249-260)
