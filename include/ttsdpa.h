@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TTSDPA_ABI_VERSION 6
+#define TTSDPA_ABI_VERSION 7
 
 /* Element types; numbering is the reference's DType enum (reference src/Tensor/DType.h:20-28). */
 enum ttsdpa_dtype { TTSDPA_F32 = 0, TTSDPA_F16 = 1, TTSDPA_BF16 = 2 };
@@ -50,7 +50,8 @@ enum ttsdpa_status {
   TTSDPA_ERR_MASK = -5,        /* mask_kind invalid, or causal together with a mask (the reference asserts) */
   TTSDPA_ERR_WORKSPACE = -6,   /* workspace NULL or smaller than ttsdpa_workspace_bytes() */
   TTSDPA_ERR_UNSUPPORTED = -7, /* valid call, but not for the kernel asked for (e.g. ttsdpa_decode with L > limit) */
-  TTSDPA_ERR_ABI = -8          /* struct_size does not match this library */
+  TTSDPA_ERR_ABI = -8,         /* struct_size does not match this library */
+  TTSDPA_ERR_STATIC_SCRATCH = -9 /* ttsdpa_decode_static: the call needs more than TTSDPA_STATIC_SCRATCH_BYTES of scratch */
 };
 
 /* Which kernel a call maps to (ttsdpa_plan). */
@@ -151,6 +152,17 @@ int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_byt
  * ttsdpa_general covers everything else the reference op accepts (other head sizes, unaligned rows, masks on fp32 or short inputs). */
 int ttsdpa_prefill(const ttsdpa_params* p, void* stream);
 int ttsdpa_decode(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ttsdpa_decode for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference.  Same kernels and results as ttsdpa_decode, but the split-KV
+ * partial records live in a buffer of TTSDPA_STATIC_SCRATCH_BYTES that is part of the library's device image (each GPU
+ * the library runs on holds one until the process ends), so the call takes no workspace and allocates nothing; a
+ * call whose ttsdpa_workspace_bytes() exceeds that size is refused with TTSDPA_ERR_STATIC_SCRATCH and launches
+ * nothing.  The first call on a device looks the buffer's address up (make it outside graph capture).  All calls on
+ * one GPU share the buffer: calls that may overlap on that GPU (different streams, several host threads) race on
+ * it; calls on one stream are ordered and safe. */
+#define TTSDPA_STATIC_SCRATCH_BYTES (2u << 20)
+int ttsdpa_decode_static(const ttsdpa_params* p, void* stream);
 int ttsdpa_general(const ttsdpa_params* p, void* stream);
 
 /*

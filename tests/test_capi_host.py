@@ -351,3 +351,22 @@ def test_build_params_refuses_a_mask_on_another_device():
     p = tinytorch_amd.build_params(q, k, k, out, False, torch.ones(4, 6, dtype=torch.bool))  # same device: accepted
     assert p.mask_kind == 1
 
+
+def test_static_scratch_decode_refuses_what_does_not_fit():
+    """ttsdpa_decode_static holds TTSDPA_STATIC_SCRATCH_BYTES of split-KV records: a call that needs more is refused
+    before anything is launched or looked up (so this needs no GPU), with a status of its own."""
+    lib = _capi.lib()
+    header = open(os.path.join(ROOT, "include", "ttsdpa.h")).read()
+    assert "#define TTSDPA_STATIC_SCRATCH_BYTES (2u << 20)" in header and _capi.STATIC_SCRATCH_BYTES == 2 << 20
+    # 16 rows per KV head against a very long cache, few (batch, head) pairs: 64 splits of 16 x 130 floats per pair
+    p = _capi.make_params(_capi.BF16, 4, 64, 4, 1, 1 << 20, 128)
+    p.q = p.k = p.v = p.out = 0x1000  # never dereferenced
+    need = lib.ttsdpa_workspace_bytes(ctypes.byref(p))
+    assert need > _capi.STATIC_SCRATCH_BYTES
+    assert lib.ttsdpa_decode_static(ctypes.byref(p), None) == _capi.ERR_STATIC_SCRATCH
+    assert "static" in _capi.status_string(_capi.ERR_STATIC_SCRATCH)
+    # outside the decode kernel's domain: the same answer as ttsdpa_decode
+    fp32 = _capi.make_params(_capi.F32, 1, 4, 4, 1, 1024, 128)
+    fp32.q = fp32.k = fp32.v = fp32.out = 0x1000
+    assert lib.ttsdpa_decode_static(ctypes.byref(fp32), None) == _capi.ERR_UNSUPPORTED
+    assert lib.ttsdpa_decode_static(None, None) == _capi.ERR_NULL

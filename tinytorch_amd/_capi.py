@@ -15,11 +15,12 @@ ROUTE_NONE, ROUTE_GENERAL, ROUTE_PREFILL, ROUTE_DECODE, ROUTE_ZERO = 0, 1, 2, 3,
 ROUTE_NAMES = {0: "none", 1: "general", 2: "prefill", 3: "decode", 4: "zero"}
 
 OK = 0
-ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_STRIDE, ERR_MASK, ERR_WORKSPACE, ERR_UNSUPPORTED, ERR_ABI = range(-1, -9, -1)
+ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_STRIDE, ERR_MASK, ERR_WORKSPACE, ERR_UNSUPPORTED, ERR_ABI, ERR_STATIC_SCRATCH = range(-1, -10, -1)
+STATIC_SCRATCH_BYTES = 2 << 20
 
 EXPORTS = [
     "ttsdpa_abi_version", "ttsdpa_status_string", "ttsdpa_params_init", "ttsdpa_plan", "ttsdpa_workspace_bytes",
-    "ttsdpa_forward", "ttsdpa_prefill", "ttsdpa_decode", "ttsdpa_general",
+    "ttsdpa_forward", "ttsdpa_prefill", "ttsdpa_decode", "ttsdpa_decode_static", "ttsdpa_general",
     "ttsdpa_kv_append_params_init", "ttsdpa_kv_append", "ttsdpa_probe",
     "ttsdpa_backward_params_init", "ttsdpa_backward_plan", "ttsdpa_backward_workspace_bytes", "ttsdpa_backward",
     # include/ttfused.h
@@ -127,6 +128,8 @@ def lib():
         L.ttsdpa_prefill.restype = ctypes.c_int
         L.ttsdpa_decode.argtypes = [P, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         L.ttsdpa_decode.restype = ctypes.c_int
+        L.ttsdpa_decode_static.argtypes = [P, ctypes.c_void_p]
+        L.ttsdpa_decode_static.restype = ctypes.c_int
         L.ttsdpa_general.argtypes = [P, ctypes.c_void_p]
         L.ttsdpa_general.restype = ctypes.c_int
         L.ttsdpa_kv_append_params_init.argtypes = [ctypes.POINTER(KvAppendParams)] + [ctypes.c_int] * 6
@@ -165,7 +168,7 @@ def lib():
         L.ttlinear_matmul.argtypes = [ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, ctypes.c_int, ctypes.c_int, i64, i64, i64,
                                       vp, ctypes.c_size_t, vp]
         L.ttlinear_matmul.restype = ctypes.c_int
-        if L.ttsdpa_abi_version() != 6:
+        if L.ttsdpa_abi_version() != 7:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L
     return _lib

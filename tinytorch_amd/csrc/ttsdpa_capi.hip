@@ -282,6 +282,33 @@ size_t backward_scratch_bytes(const ttsdpa_backward_params* p) {
 
 int check_grid(long long nwg) { return nwg > 0x7fffffffLL ? TTSDPA_ERR_SHAPE : TTSDPA_OK; }
 
+// Scratch of ttsdpa_decode_static: the split-KV partial records of one decode call.  Every GPU the library runs on holds
+// its own copy of this array, at its own address, until the process ends.  In host code the array's name is only a
+// handle for hipGetSymbolAddress: kernels and memory calls get the address that call returns, never the name.
+constexpr size_t kStaticScratchBytes = TTSDPA_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Address of the current device's copy of `scratch`, looked up once per device (with that device current) and kept.
+// Safe from several host threads: the worst case is two identical look-ups.
+int static_scratch_of_current_device(void** out) {
+  static void* ptr[kMaxDevices];
+  static bool done[kMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+  if (!__atomic_load_n(&done[dev], __ATOMIC_ACQUIRE)) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    __atomic_store_n(&ptr[dev], p, __ATOMIC_RELAXED);
+    __atomic_store_n(&done[dev], true, __ATOMIC_RELEASE);
+  }
+  *out = __atomic_load_n(&ptr[dev], __ATOMIC_RELAXED);
+  return TTSDPA_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -299,6 +326,7 @@ const char* ttsdpa_status_string(int status) {
     case TTSDPA_ERR_WORKSPACE: return "workspace missing or too small";
     case TTSDPA_ERR_UNSUPPORTED: return "arguments outside this kernel's domain";
     case TTSDPA_ERR_ABI: return "ttsdpa_params.struct_size mismatch";
+    case TTSDPA_ERR_STATIC_SCRATCH: return "call needs more scratch than the library's static buffer holds (TTSDPA_STATIC_SCRATCH_BYTES)";
     default: return status > 0 ? hipGetErrorString((hipError_t)status) : "unknown status";
   }
 }
@@ -393,6 +421,22 @@ int ttsdpa_decode(const ttsdpa_params* p, void* workspace, size_t workspace_byte
     return TTSDPA_ERR_WORKSPACE;
   if ((rc = check_grid((long long)a.B * a.Hkv * pl.splits)) != TTSDPA_OK) return rc;
   return launch_decode(a, p->dtype, workspace, (hipStream_t)stream);
+}
+
+int ttsdpa_decode_static(const ttsdpa_params* p, void* stream) {
+  KArgs a;
+  int rc = validate(p, &a);
+  if (rc != TTSDPA_OK) return rc;
+  if (p->B == 0 || p->L == 0) return TTSDPA_OK;
+  if (!decode_ok(p)) return TTSDPA_ERR_UNSUPPORTED;
+  const DecodePlan pl = plan_decode(a);
+  if (pl.ws_bytes > kStaticScratchBytes) return TTSDPA_ERR_STATIC_SCRATCH;
+  if ((rc = check_grid((long long)a.B * a.Hkv * pl.splits)) != TTSDPA_OK) return rc;
+  void* ws = nullptr;
+  if ((rc = static_scratch_of_current_device(&ws)) != TTSDPA_OK) return rc;
+  // Nothing in the records has to start at zero: every split writes its whole record (an empty split a weight of
+  // zero) before the merge kernel, later on the same stream, reads it.
+  return launch_decode(a, p->dtype, ws, (hipStream_t)stream);
 }
 
 int ttsdpa_forward(const ttsdpa_params* p, void* workspace, size_t workspace_bytes, void* stream) {
