@@ -89,9 +89,9 @@ __device__ __forceinline__ float row_reduce(float v, float* lds, int slot) {
 
 // Walk the part of a row that a lane does not keep in registers (vectors lr + CACHE*LPR, + LPR, ...), four loads in
 // flight: `load(i)` fetches vector i, `use(i, v)` consumes it.
-template <int LPR, typename Load, typename Use>
+template <int LPR, typename Load, typename Use, int KEPT = CACHE>
 __device__ __forceinline__ void walk_rest(int lr, int nvec, Load load, Use use) {
-  for (int i0 = lr + CACHE * LPR; i0 < nvec; i0 += 4 * LPR) {
+  for (int i0 = lr + KEPT * LPR; i0 < nvec; i0 += 4 * LPR) {
     decltype(load(0)) v[4];
 #pragma unroll
     for (int u = 0; u < 4; u++)
@@ -186,7 +186,9 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const T* x, T* res, const
 // One reading pass: every lane keeps a running maximum and the sum of exponentials relative to it (rescaled when the
 // maximum grows), the lanes' pairs are merged after the row maximum is known, then the row is written from the
 // registers (and from a second read for the part of a very long row that was not kept).
-template <typename T, int VEC, int LPR, bool LOG>
+// KEEP: vectors of its row a lane holds in registers between the statistics and the write (16 for rows of one workgroup
+// that would otherwise be read twice: up to 32768 16-bit elements are then read once).
+template <typename T, int VEC, int LPR, bool LOG, int KEEP>
 __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* out, long long rows, int dim) {  // out may be x
   typedef typename Pack<T, VEC>::type V;
   __shared__ float lds[8];
@@ -198,7 +200,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* out, l
   const T* xr = x + row * dim;
   T* orow = out + row * dim;
 
-  V keep[CACHE];
+  V keep[KEEP];
   float mx = -3.402823466e+38f;  // the reference starts from the lowest finite float
   float sum = 0.f;
   auto absorb = [&](int, const V& a) __attribute__((always_inline)) {
@@ -211,14 +213,15 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* out, l
     for (int e = 0; e < VEC; e++) sum += __expf((float)a[e] - mn);
     mx = mn;
   };
+  auto reload = [&](int i) __attribute__((always_inline)) { return load_plain<T, VEC>(xr + (long long)i * VEC); };
   if (live) {
 #pragma unroll
-    for (int c = 0; c < CACHE; c++)
+    for (int c = 0; c < KEEP; c++)
       if (lr + c * LPR < nvec) keep[c] = load_stream<T, VEC>(xr + (long long)(lr + c * LPR) * VEC);
 #pragma unroll
-    for (int c = 0; c < CACHE; c++)
+    for (int c = 0; c < KEEP; c++)
       if (lr + c * LPR < nvec) absorb(0, keep[c]);
-    walk_rest<LPR>(lr, nvec, [&](int i) __attribute__((always_inline)) { return load_plain<T, VEC>(xr + (long long)i * VEC); }, absorb);
+    walk_rest<LPR, decltype(reload), decltype(absorb), KEEP>(lr, nvec, reload, absorb);
   }
   const float rmax = row_reduce<LPR, MaxOp>(mx, lds, 0);
   sum = row_reduce<LPR, SumOp>(sum * __expf(mx - rmax), lds, 1);
@@ -235,9 +238,9 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* out, l
     store_pack<T, VEC>(orow + (long long)i * VEC, o);
   };
 #pragma unroll
-  for (int c = 0; c < CACHE; c++)
+  for (int c = 0; c < KEEP; c++)
     if (lr + c * LPR < nvec) give(lr + c * LPR, keep[c]);
-  walk_rest<LPR>(lr, nvec, [&](int i) __attribute__((always_inline)) { return load_plain<T, VEC>(xr + (long long)i * VEC); }, give);
+  walk_rest<LPR, decltype(reload), decltype(give), KEEP>(lr, nvec, reload, give);
 }
 
 // ---- softmax / logSoftmax over an inner axis: a lane owns VEC neighbouring (outer, inner) columns, lanes run along the
@@ -372,13 +375,18 @@ int launch_softmax_rows(const void* x, void* out, long long rows, int dim, hipSt
   const long long rpb = 256 / lpr;
   const unsigned grid = (unsigned)((rows + rpb - 1) / rpb);
 #define TT_SM(LPR) \
-  hipLaunchKernelGGL((softmax_rows_kernel<T, VEC, LPR, LOG>), dim3(grid), dim3(256), 0, s, (const T*)x, (T*)out, rows, dim)
+  hipLaunchKernelGGL((softmax_rows_kernel<T, VEC, LPR, LOG, CACHE>), dim3(grid), dim3(256), 0, s, (const T*)x, (T*)out, rows, dim)
   switch (lpr) {
     case 8: TT_SM(8); break;
     case 16: TT_SM(16); break;
     case 32: TT_SM(32); break;
     case 64: TT_SM(64); break;
-    default: TT_SM(256); break;
+    default:
+      if (dim / VEC > CACHE * 256 && dim / VEC <= 2 * CACHE * 256)  // a row of 8 to 16 vectors per lane: keep all of it
+        hipLaunchKernelGGL((softmax_rows_kernel<T, VEC, 256, LOG, 2 * CACHE>), dim3(grid), dim3(256), 0, s, (const T*)x, (T*)out, rows, dim);
+      else
+        TT_SM(256);
+      break;
   }
 #undef TT_SM
   return (int)hipGetLastError();

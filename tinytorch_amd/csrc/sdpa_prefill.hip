@@ -18,8 +18,11 @@
 //                                                 load ds_read_b64_tr_b16; B = P^T taken straight from the S^T
 //                                                 accumulator registers (the V side applies the same permutation
 //                                                 of the contraction index, see v_operand)
-// The running maximum m is only raised when a tile's maximum exceeds it by more than 2^8 in the exponent (the
-// probabilities stay <= 256, exact in fp32 sums and within bf16/fp16 range), so the accumulator rescale is rare.
+// The maximum m the exponentials are taken against is raised lazily: a lane's 32 probabilities of a tile are summed
+// anyway, and only when such a sum leaves [0, 1024] (which includes the first tile of a row, taken against -1e30) is
+// the true row maximum formed, sum and accumulator rescaled and the tile's exponentials redone.  No per-tile row
+// maximum: at small head sizes the vector ALUs, not the matrix pipe, bound this kernel (a score costs the same vector
+// work whatever head_dim is).
 // Causal masking (key j visible to query i iff j <= i, reference src/Operation/OpTransformCpu.h:202-209) skips
 // tiles above the diagonal and applies the predicate only on tiles that straddle it.
 // Grouped-query attention: kv head = query head / (Hq/Hkv), resolved in the kernel; the workgroup order puts the
@@ -33,7 +36,7 @@ namespace {
 
 constexpr int BM = 128;  // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
-constexpr float kLazyExp = 8.f;  // raise the running maximum only when exceeded by 2^8 in the exponent
+constexpr float kSumLimit = 1024.f;  // a lane's 32 probabilities of a tile may sum to this much before the maximum is raised
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -125,7 +128,6 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
 #pragma unroll
     for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
   const float c = a.scale * kLog2e;
-  const float lazy = kLazyExp / c;  // the same margin in raw-score units
   float m_use = -1e30f;  // maximum the exponentials are taken against (raw scores); finite: no inf - inf
   float mc = m_use * c;
   float l_run = 0.f;     // this lane's share of the running row sum
@@ -267,13 +269,22 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
       }
 
       // ---- online softmax with a lazily raised maximum ---------------------------------------------------------------
-      float mloc = sacc[0][0];
+      float psum = 0.f;
+      f32x16 pr[2];
 #pragma unroll
       for (int blk = 0; blk < 2; blk++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, sacc[blk][r]);
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-      if (__builtin_amdgcn_ballot_w64(mloc > m_use + lazy) != 0) {  // some row of the wavefront must move its maximum
+        for (int r = 0; r < 16; r++) {
+          pr[blk][r] = fast_exp2(fmaf(sacc[blk][r], c, -mc));
+          psum += pr[blk][r];
+        }
+      if (__builtin_amdgcn_ballot_w64(!(psum <= kSumLimit)) != 0) {  // some row of the wavefront outgrew its maximum
+        float mloc = sacc[0][0];
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, sacc[blk][r]);
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
         const float m_new = fmaxf(m_use, mloc);
         const float alpha = fast_exp2((m_use - m_new) * c);
         m_use = m_new;
@@ -283,16 +294,15 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
         for (int i = 0; i < DBLK; i++)
 #pragma unroll
           for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+        psum = 0.f;
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            pr[blk][r] = fast_exp2(fmaf(sacc[blk][r], c, -mc));
+            psum += pr[blk][r];
+          }
       }
-      float psum = 0.f;
-#pragma unroll
-      for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          float p = fast_exp2(fmaf(sacc[blk][r], c, -mc));
-          sacc[blk][r] = p;
-          psum += p;
-        }
       l_run += psum;
 
       // ---- P^T as B operands: MFMA t consumes accumulator registers 8*(t%2) .. +7 of block t/2 ------------------------
@@ -301,7 +311,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
       for (int t = 0; t < 4; t++) {
         f32x8 x;
 #pragma unroll
-        for (int i = 0; i < 8; i++) x[i] = sacc[t >> 1][8 * (t & 1) + i];
+        for (int i = 0; i < 8; i++) x[i] = pr[t >> 1][8 * (t & 1) + i];
         pb[t] = __builtin_convertvector(x, vec8);
       }
 
