@@ -88,12 +88,14 @@ def measured_traffic(name):
         return json.load(f).get(name, {}).get("hbm_bytes_per_launch")
 
 
-def time_launches(step, stream, steps, warmup, settle_seconds=SETTLE_SECONDS):
+def time_launches(step, stream, steps, warmup, settle_seconds=None):
     """warmup untimed launches, a declared untimed settle phase, then `steps` launches each between its own pair of HIP
     events on `stream`.  Returns per-launch device times (median, mean, min; ms), the host-clock time per step around
     the timed launches, and the number of settle launches."""
     import torch
 
+    if settle_seconds is None:
+        settle_seconds = SETTLE_SECONDS
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -479,6 +481,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-probes", action="store_true", help="skip the hardware ceiling probes")
+    ap.add_argument("--settle", type=float, default=None,
+                    help="seconds of untimed launches after the warm-up (default %.1f; 0 for counter runs that only need a few dispatches)" % SETTLE_SECONDS)
     ap.add_argument("--no-other", action="store_true", help="skip the baseline's other configurations (1, 2, 5) and head_dim 64")
     ap.add_argument("--no-fused", action="store_true", help="skip the row-wise neighbour ops (rmsNorm, siluMul, ...)")
     ap.add_argument("--fused-only", default=None, choices=sorted(FUSED_WORKLOADS),
@@ -490,6 +494,8 @@ def main():
                     help="also run one device-to-device copy of 1 GiB (a kernel of known traffic that calibrates "
                          "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc)")
     args = ap.parse_args()
+    if args.settle is not None:
+        globals()["SETTLE_SECONDS"] = max(0.0, args.settle)
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the attention path shards by batch / KV head with no "
                  "exchange; no multi-GPU figure is produced). Run with --gpus 1.")

@@ -97,15 +97,19 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   const int npair = a.B * a.Hkv;
   int pair, in;
   {
-    int n = blockIdx.x;
-    if ((npair & 7) == 0) {  // workgroup n runs on XCD n % 8: keep a (batch, kv head) on one XCD
-      int xcd = n & 7, slot = n >> 3;
-      pair = (slot / inner) * 8 + xcd;
-      in = slot % inner;
-    } else {
-      pair = n / inner;
-      in = n % inner;
-    }
+    // Workgroup n runs on XCD n % 8, and the workgroups of one (batch, kv head) share its K/V through an XCD's L2: with
+    // g = gcd(pairs, 8) the XCDs form g classes of 8/g, class x % g serves the pairs congruent to it and deals the
+    // work items (heads x row tiles) of those pairs out to its XCDs in turn.  A multiple of 8 pairs puts every pair on
+    // one XCD; 4 pairs (config 5) give each pair two XCDs instead of all eight streaming all four.
+    const int n = blockIdx.x;
+    const int gq = (npair & 7) == 0 ? 8 : ((npair & 3) == 0 ? 4 : ((npair & 1) == 0 ? 2 : 1));
+    const int xcd = n & 7, slot = n >> 3;
+    const int cls = xcd % gq, sub = xcd / gq;
+    const long long item = (long long)slot * (8 / gq) + sub;  // work item of the class
+    const long long items = (long long)(npair / gq) * inner;
+    if (item >= items) return;  // the grid is rounded up to a multiple of 8
+    pair = cls + gq * (int)(item / inner);
+    in = (int)(item % inner);
   }
   const int b = pair / a.Hkv, hk = pair % a.Hkv;
   const int g = in % a.G;
@@ -626,6 +630,14 @@ int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
 int launch_prefill_d128(const KArgs& a, int dtype, hipStream_t stream) {
   const int ntile = (a.L + BM - 1) / BM;
   long long nwg = (long long)a.B * a.Hq * (a.causal ? (ntile + 1) / 2 : ntile);
+  // the kernel's XCD-aware numbering addresses workgroups in groups of 8 (classes of XCDs): round up, the extras return
+  {
+    const int npair = a.B * a.Hkv;
+    const int gq = (npair & 7) == 0 ? 8 : ((npair & 3) == 0 ? 4 : ((npair & 1) == 0 ? 2 : 1));
+    const long long per_class = nwg / gq;                       // work items of one class of XCDs
+    const long long slots = (per_class + 8 / gq - 1) / (8 / gq);  // per XCD of the class
+    nwg = slots * 8;
+  }
   dim3 grid((unsigned)nwg);
   if (dtype == 1) return a.causal ? launch_k<F16, true>(a, grid, stream) : launch_k<F16, false>(a, grid, stream);
   return a.causal ? launch_k<BF16, true>(a, grid, stream) : launch_k<BF16, false>(a, grid, stream);
