@@ -53,6 +53,20 @@ int ttlinear_matmul(int dtype, const void* a, const void* b, const void* bias, v
                     int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldo, void* workspace,
                     size_t workspace_bytes, void* stream);
 
+/* op::matmul with batch dimensions (reference src/Operation/OpLinalg.cpp:107-223: leading dimensions of the two
+ * operands broadcast against each other; its device path is a strided-batched or pointer-array GEMM, its CPU path a
+ * loop over the batch with per-operand offsets, :205-223).  The batch is described as up to TTLINEAR_MAX_BATCH_DIMS
+ * dimensions batch_shape[0..nbatch_dims) with element strides a_batch_stride[d] / b_batch_stride[d] (0 broadcasts the
+ * operand along d); batch entry i of the output, numbered row-major over batch_shape, starts at out + i * out_batch_stride.
+ * Every batch entry is one ttlinear_matmul of the same M, N, K, flags and leading dimensions, enqueued in order on
+ * `stream`; the workspace (ttlinear_matmul_workspace_bytes of one entry) is shared by the entries.  bias ([N] or NULL)
+ * joins every entry. */
+#define TTLINEAR_MAX_BATCH_DIMS 8
+int ttlinear_matmul_batched(int dtype, const void* a, const void* b, const void* bias, void* out, int64_t M, int64_t N,
+                            int64_t K, int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldo, int nbatch_dims,
+                            const int64_t* batch_shape, const int64_t* a_batch_stride, const int64_t* b_batch_stride,
+                            int64_t out_batch_stride, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -404,6 +404,33 @@ def matmul(a, b, transA=False, transB=False, bias=None, dtype="f32"):
     return out
 
 
+def matmul_nd(a, b, transA=False, transB=False, bias=None, dtype="f32"):
+    """op::matmul with the reference's batch and 1-D rules (src/Operation/OpLinalg.cpp:52-241): a 1-D a is a row vector,
+    a 1-D b a column vector (their flags ignored, :63-72); leading dimensions broadcast (:84-89); every batch entry is
+    the 2-D product of the operands' slices at that index (the CPU path's loop, :205-223: an operand whose dimension is 1
+    stays at its only slice); the added dimensions are dropped from a 2-D result (:221-239)."""
+    a, b = _f32(a), _f32(b)
+    assert a.ndim >= 1 and b.ndim >= 1
+    prepend_a, append_b = a.ndim == 1, b.ndim == 1
+    if prepend_a:
+        a, transA = a[None, :], False
+    if append_b:
+        b, transB = b[:, None], False
+    batch = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+    M = a.shape[-1] if transA else a.shape[-2]
+    N = b.shape[-2] if transB else b.shape[-1]
+    ea = np.broadcast_to(a, batch + a.shape[-2:])
+    eb = np.broadcast_to(b, batch + b.shape[-2:])
+    out = np.empty(batch + (M, N), dtype=np.float32)
+    for idx in np.ndindex(*batch):
+        out[idx] = matmul(np.ascontiguousarray(ea[idx]), np.ascontiguousarray(eb[idx]), transA, transB, bias, dtype)
+    if append_b:
+        out = out.reshape(() if prepend_a else (M,))
+    elif prepend_a and not batch:
+        out = out.reshape(N)
+    return out
+
+
 def ref_matmul(a, b, transA=False, transB=False, bias=None):
     """op::matmul of the compiled reference (fp32, CPU)."""
     a, b = _f32(a), _f32(b)

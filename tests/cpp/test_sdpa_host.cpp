@@ -554,6 +554,62 @@ static void test_row_wise_ops() {
   setAssertHandler(old);
 }
 
+
+// op::matmul with batch dimensions, broadcasting and 1-D operands: the reference's own vectors
+// (reference test/test_operation.cpp:1223-1396), tensors on the accelerator.
+static void test_matmul_batched_reference_vectors() {
+  std::printf("op::matmul: batch / broadcast / 1-D vectors of the reference\n");
+  const Options gpu = options::device(DeviceType::GPU);
+  auto ar = [&](std::vector<int64_t> shape) {
+    int64_t n = 1;
+    for (int64_t d : shape) n *= d;
+    std::vector<float> v(static_cast<size_t>(n));
+    for (int64_t i = 0; i < n; i++) v[static_cast<size_t>(i)] = static_cast<float>(i);
+    return Tensor(v, shape, gpu);
+  };
+  auto is = [&](const Tensor& y, std::vector<int64_t> shape, std::vector<float> vals) {
+    return y.defined() && y.shape() == shape && vectorNear(y.toList<float>(), vals, 1e-4f);
+  };
+  Tensor d5(std::vector<float>{1, 0, 0, 1}, {2, 2}, gpu), d6(std::vector<float>{1, 2}, {2}, gpu), d7(std::vector<float>{2}, {1}, gpu);
+  EXPECT_TRUE(is(op::matmul(d5, d6, false, false, Tensor{}), {2}, {1, 2}));
+  EXPECT_TRUE(is(op::matmul(d6, d5, false, false, Tensor{}), {2}, {1, 2}));
+  EXPECT_TRUE(is(op::matmul(d7, d7, false, false, Tensor{}), {}, {4}));
+  EXPECT_TRUE(is(op::matmul(ar({2, 2, 4}), ar({1, 2, 4, 2}), false, false, Tensor{}), {1, 2, 2, 2}, {28, 34, 76, 98, 428, 466, 604, 658}));
+  EXPECT_TRUE(is(op::matmul(ar({2, 2, 4}), ar({1, 4, 2}), false, false, Tensor{}), {2, 2, 2}, {28, 34, 76, 98, 124, 162, 172, 226}));
+  EXPECT_TRUE(is(op::matmul(ar({2, 3, 4}), ar({2, 4, 2}), false, false, Tensor{}), {2, 3, 2},
+                 {28, 34, 76, 98, 124, 162, 604, 658, 780, 850, 956, 1042}));
+  EXPECT_TRUE(is(op::matmul(ar({3, 4}), ar({2, 4, 2}), false, false, Tensor{}), {2, 3, 2},
+                 {28, 34, 76, 98, 124, 162, 76, 82, 252, 274, 428, 466}));
+  EXPECT_TRUE(is(op::matmul(ar({2, 3, 4}), ar({1, 4, 2}), false, false, Tensor{}), {2, 3, 2},
+                 {28, 34, 76, 98, 124, 162, 172, 226, 220, 290, 268, 354}));
+  EXPECT_TRUE(is(op::matmul(ar({2, 3, 4}), ar({2, 2, 4}), false, true, Tensor{}), {2, 3, 2},
+                 {14, 38, 38, 126, 62, 214, 518, 734, 670, 950, 822, 1166}));
+  EXPECT_TRUE(is(op::matmul(ar({2, 4, 3}), ar({2, 4, 2}), true, false, Tensor{}), {2, 3, 2},
+                 {84, 102, 96, 118, 108, 134, 756, 822, 800, 870, 844, 918}));
+  EXPECT_TRUE(is(op::matmul(ar({2, 1, 3, 4}), ar({2, 1, 4, 2}), false, false, Tensor{}), {2, 1, 3, 2},
+                 {28, 34, 76, 98, 124, 162, 604, 658, 780, 850, 956, 1042}));
+  EXPECT_TRUE(is(op::matmul(ar({1, 2, 3}), ar({6, 3, 2}), false, false, Tensor{}), {6, 2, 2},
+                 {10, 13, 28, 40, 28, 31, 100, 112, 46, 49, 172, 184, 64, 67, 244, 256, 82, 85, 316, 328, 100, 103, 388, 400}));
+  // attention's own products as batched matmuls: scores [B,H,L,S] = q . k^T, and a grouped-query broadcast over a 5-D view
+  {
+    const int B = 2, H = 3, L = 40, S = 72, D = 64;
+    const Options o = options::device(DeviceType::GPU).dtype(DType::BFloat16);
+    Tensor q(pseudoRandom(static_cast<size_t>(B) * H * L * D, 81), {B, H, L, D}, o), k(pseudoRandom(static_cast<size_t>(B) * H * S * D, 82), {B, H, S, D}, o);
+    Tensor s = op::matmul(q, k, false, true, Tensor{});
+    EXPECT_TRUE(s.defined() && s.shape() == std::vector<int64_t>({B, H, L, S}));
+    const std::vector<float> qs = q.toList<float>(), ks = k.toList<float>(), got = s.toList<float>();
+    std::vector<float> ref(got.size());
+    for (int bh = 0; bh < B * H; bh++)
+      for (int i = 0; i < L; i++)
+        for (int j = 0; j < S; j++) {
+          double acc = 0;
+          for (int d = 0; d < D; d++) acc += static_cast<double>(qs[(static_cast<size_t>(bh) * L + i) * D + d]) * ks[(static_cast<size_t>(bh) * S + j) * D + d];
+          ref[(static_cast<size_t>(bh) * L + i) * S + j] = static_cast<float>(acc);
+        }
+    EXPECT_TRUE(vectorNear(got, ref, 2e-2f * std::sqrt(static_cast<float>(D))));
+  }
+}
+
 int main() {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
@@ -565,6 +621,7 @@ int main() {
   test_broadcast_masks();
   test_kv_cache();
   test_row_wise_ops();
+  test_matmul_batched_reference_vectors();
   test_backward();
   test_grad_bookkeeping_and_errors();
   std::printf(g_failures == 0 ? "ALL PASSED\n" : "%d FAILURES\n", g_failures);

@@ -183,3 +183,62 @@ def test_linear_backward_against_torch_autograd():
     for got, exp, k in ((gi, xf.grad, N), (gw, wf.grad, M), (gb, bf.grad, M)):
         err = (got.float() - exp).abs().max().item()
         assert err <= 2e-2 * max(1.0, k ** 0.5), err
+
+
+def test_matmul_batch_rules_reference_vectors():
+    """op::matmul with batch dimensions, broadcasting and 1-D operands: the reference's own vectors
+    (reference test/test_operation.cpp:1223-1396) through the Python mirror, exact in fp32."""
+    import tinytorch_amd
+
+    ar = lambda *shape: torch.arange(int(np.prod(shape)), dtype=torch.float32, device="cuda").reshape(shape)
+    t = lambda v: torch.tensor(v, dtype=torch.float32, device="cuda")
+
+    def check(y, shape, vals):
+        assert tuple(y.shape) == tuple(shape), (tuple(y.shape), shape)
+        assert np.array_equal(y.cpu().numpy().ravel(), np.array(vals, np.float32))
+
+    mm = tinytorch_amd.matmul
+    check(mm(t([[1, 0], [0, 1]]), t([1, 2])), (2,), [1, 2])
+    check(mm(t([1, 2]), t([[1, 0], [0, 1]])), (2,), [1, 2])
+    check(mm(t([2]), t([2])), (), [4])
+    check(mm(ar(2, 2, 4), ar(1, 2, 4, 2)), (1, 2, 2, 2), [28, 34, 76, 98, 428, 466, 604, 658])
+    check(mm(ar(2, 2, 4), ar(1, 4, 2)), (2, 2, 2), [28, 34, 76, 98, 124, 162, 172, 226])
+    check(mm(ar(2, 3, 4), ar(2, 4, 2)), (2, 3, 2), [28, 34, 76, 98, 124, 162, 604, 658, 780, 850, 956, 1042])
+    check(mm(ar(2, 3, 4), ar(4, 2)), (2, 3, 2), [28, 34, 76, 98, 124, 162, 172, 226, 220, 290, 268, 354])
+    check(mm(ar(3, 4), ar(2, 4, 2)), (2, 3, 2), [28, 34, 76, 98, 124, 162, 76, 82, 252, 274, 428, 466])
+    check(mm(ar(1, 3, 4), ar(2, 4, 2)), (2, 3, 2), [28, 34, 76, 98, 124, 162, 76, 82, 252, 274, 428, 466])
+    check(mm(ar(2, 3, 4), ar(2, 2, 4), False, True), (2, 3, 2), [14, 38, 38, 126, 62, 214, 518, 734, 670, 950, 822, 1166])
+    check(mm(ar(2, 4, 3), ar(2, 4, 2), True, False), (2, 3, 2), [84, 102, 96, 118, 108, 134, 756, 822, 800, 870, 844, 918])
+    check(mm(ar(2, 1, 3, 4), ar(2, 1, 4, 2)), (2, 1, 3, 2), [28, 34, 76, 98, 124, 162, 604, 658, 780, 850, 956, 1042])
+    check(mm(ar(1, 2, 3), ar(6, 3, 2)), (6, 2, 2), [10, 13, 28, 40, 28, 31, 100, 112, 46, 49, 172, 184, 64, 67, 244, 256, 82, 85,
+                                                  316, 328, 100, 103, 388, 400])
+    check(mm(ar(8, 2, 3), ar(1, 3, 2)), (8, 2, 2), [10, 13, 28, 40, 46, 67, 64, 94, 82, 121, 100, 148, 118, 175, 136, 202, 154, 229,
+                                                  172, 256, 190, 283, 208, 310, 226, 337, 244, 364, 262, 391, 280, 418])
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", [
+    # a shape, b shape, transA, transB, bias
+    ((3, 40, 72), (3, 72, 24), False, False, False),
+    ((2, 3, 130, 128), (2, 3, 200, 128), False, True, False),      # q . k^T of an attention call: the MFMA kernel per entry
+    ((2, 1, 64, 130), (1, 4, 64, 40), True, False, True),         # both operands broadcast, transposed first operand
+    ((5, 33, 128), (128, 48), False, False, True),                 # a batch against one matrix
+    ((2, 2, 1, 256, 256), (2, 1, 3, 256, 256), False, True, False),  # two broadcast axes, tile-sized entries
+])
+def test_matmul_batched_against_oracle(dtype, case):
+    import tinytorch_amd
+
+    sa, sb, ta, tb, with_bias = case
+    N = sb[-2] if tb else sb[-1]
+    K = sa[-2] if ta else sa[-1]
+    a_h, a_bits = oracle.round_to(oracle.randn(61, 0, sa, K ** -0.5), dtype)
+    b_h, b_bits = oracle.round_to(oracle.randn(61, 1, sb), dtype)
+    bias_h, bias_bits = oracle.round_to(oracle.randn(61, 2, (N,)), dtype)
+    a, b, bias = to_device(a_h, a_bits, dtype), to_device(b_h, b_bits, dtype), to_device(bias_h, bias_bits, dtype)
+    y = tinytorch_amd.matmul(a, b, ta, tb, bias if with_bias else None)
+    exp = oracle.matmul_nd(a_h, b_h, ta, tb, bias_h if with_bias else None)
+    assert tuple(y.shape) == exp.shape
+    tol = (1e-4 if dtype == "f32" else 2e-2) * max(1.0, float(np.sqrt(K)) / 4)
+    err = float(np.abs(y.float().cpu().numpy() - exp).max())
+    print("matmul batched %s %s x %s: max-abs-err %.3e" % (dtype, sa, sb, err), flush=True)
+    assert err <= tol

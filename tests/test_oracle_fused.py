@@ -201,3 +201,39 @@ def test_softmax_backward_reference_and_differences(oracle_mod):
     y16, _ = o.round_to(o.softmax(x, -1), "bf16")
     d16 = o.softmax_backward(g16, y16, -1, False, "bf16")
     assert np.array_equal(d16, o.round_to(o.softmax_backward(g16, y16, -1), "bf16")[0])
+
+
+def test_matmul_nd_against_the_references_vectors(oracle_mod):
+    """The batch / broadcast / 1-D rules of op::matmul, pinned by the reference's own known answers
+    (test/test_operation.cpp:1223-1396): the entries of a batch are the 2-D products the tests above hold bit-exact
+    against the compiled reference; these vectors fix which slices meet and what shape comes out."""
+    ar = lambda *shape: np.arange(int(np.prod(shape)), dtype=np.float32).reshape(shape)
+    oracle = oracle_mod
+    mm = oracle.matmul_nd
+    eq = lambda got, shape, vals: got.shape == tuple(shape) and np.array_equal(got.ravel(), np.array(vals, np.float32))
+    # :1223-1262
+    assert eq(mm(np.array([[1, 2], [3, 4]], np.float32), np.array([[2, 3], [4, 5]], np.float32)), (2, 2), [10, 13, 22, 29])
+    assert eq(mm(np.eye(2, dtype=np.float32), np.array([1, 2], np.float32)), (2,), [1, 2])
+    assert eq(mm(np.array([1, 2], np.float32), np.eye(2, dtype=np.float32)), (2,), [1, 2])
+    assert eq(mm(np.array([2], np.float32), np.array([2], np.float32)), (), [4])
+    assert eq(mm(ar(2, 2, 4), ar(1, 2, 4, 2)), (1, 2, 2, 2), [28, 34, 76, 98, 428, 466, 604, 658])
+    assert eq(mm(ar(2, 2, 4), ar(1, 4, 2)), (2, 2, 2), [28, 34, 76, 98, 124, 162, 172, 226])
+    # :1264-1277 (transposed second operand)
+    assert eq(mm(np.array([[1, 2], [3, 4]], np.float32), np.array([[2, 3], [4, 5]], np.float32), False, True), (2, 2), [8, 14, 18, 32])
+    # :1279-1372
+    assert eq(mm(ar(2, 3, 4), ar(2, 4, 2)), (2, 3, 2), [28, 34, 76, 98, 124, 162, 604, 658, 780, 850, 956, 1042])
+    assert eq(mm(ar(2, 3, 4), ar(4, 2)), (2, 3, 2), [28, 34, 76, 98, 124, 162, 172, 226, 220, 290, 268, 354])
+    assert eq(mm(ar(3, 4), ar(2, 4, 2)), (2, 3, 2), [28, 34, 76, 98, 124, 162, 76, 82, 252, 274, 428, 466])
+    assert eq(mm(ar(1, 3, 4), ar(2, 4, 2)), (2, 3, 2), [28, 34, 76, 98, 124, 162, 76, 82, 252, 274, 428, 466])
+    assert eq(mm(ar(2, 3, 4), ar(1, 4, 2)), (2, 3, 2), [28, 34, 76, 98, 124, 162, 172, 226, 220, 290, 268, 354])
+    assert eq(mm(ar(2, 3, 4), ar(2, 2, 4), False, True), (2, 3, 2), [14, 38, 38, 126, 62, 214, 518, 734, 670, 950, 822, 1166])
+    assert eq(mm(ar(2, 4, 3), ar(2, 4, 2), True, False), (2, 3, 2), [84, 102, 96, 118, 108, 134, 756, 822, 800, 870, 844, 918])
+    assert eq(mm(ar(2, 1, 3, 4), ar(2, 1, 4, 2)), (2, 1, 3, 2), [28, 34, 76, 98, 124, 162, 604, 658, 780, 850, 956, 1042])
+    # :1374-1396 (more than four batch entries)
+    assert eq(mm(ar(1, 2, 3), ar(6, 3, 2)), (6, 2, 2), [10, 13, 28, 40, 28, 31, 100, 112, 46, 49, 172, 184, 64, 67, 244, 256, 82,
+                                                      85, 316, 328, 100, 103, 388, 400])
+    assert eq(mm(ar(8, 2, 3), ar(1, 3, 2)), (8, 2, 2), [10, 13, 28, 40, 46, 67, 64, 94, 82, 121, 100, 148, 118, 175, 136, 202, 154,
+                                                      229, 172, 256, 190, 283, 208, 310, 226, 337, 244, 364, 262, 391, 280, 418])
+    # against numpy's own broadcasting product on a shape none of the vectors has
+    a, b = oracle.randn(5, 0, (2, 1, 3, 7, 5)), oracle.randn(5, 1, (4, 1, 5, 6))
+    assert np.allclose(mm(a, b), np.matmul(a.astype(np.float64), b.astype(np.float64)), atol=1e-5)

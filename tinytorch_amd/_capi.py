@@ -26,7 +26,7 @@ EXPORTS = [
     # include/ttfused.h
     "ttfused_rms_norm", "ttfused_add_rms_norm", "ttfused_silu_mul", "ttfused_softmax", "ttfused_softmax_backward",
     # include/ttlinear.h
-    "ttlinear_forward", "ttlinear_plan", "ttlinear_matmul", "ttlinear_matmul_workspace_bytes",
+    "ttlinear_forward", "ttlinear_plan", "ttlinear_matmul", "ttlinear_matmul_batched", "ttlinear_matmul_workspace_bytes",
 ]
 LINEAR_ROUTE_NAMES = {0: "none", 1: "mfma", 2: "general"}
 
@@ -168,6 +168,10 @@ def lib():
         L.ttlinear_matmul.argtypes = [ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, ctypes.c_int, ctypes.c_int, i64, i64, i64,
                                       vp, ctypes.c_size_t, vp]
         L.ttlinear_matmul.restype = ctypes.c_int
+        i64p = ctypes.POINTER(ctypes.c_int64)
+        L.ttlinear_matmul_batched.argtypes = [ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, ctypes.c_int, ctypes.c_int, i64, i64,
+                                              i64, ctypes.c_int, i64p, i64p, i64p, i64, vp, ctypes.c_size_t, vp]
+        L.ttlinear_matmul_batched.restype = ctypes.c_int
         if L.ttsdpa_abi_version() != 7:
             raise ImportError("tinytorch_amd: libttsdpa.so ABI version mismatch")
         _lib = L

@@ -639,4 +639,35 @@ int ttlinear_matmul(int dtype, const void* a, const void* b, const void* bias, v
   }
 }
 
+int ttlinear_matmul_batched(int dtype, const void* a, const void* b, const void* bias, void* out, int64_t M, int64_t N,
+                            int64_t K, int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldo, int nbatch_dims,
+                            const int64_t* batch_shape, const int64_t* a_batch_stride, const int64_t* b_batch_stride,
+                            int64_t out_batch_stride, void* workspace, size_t workspace_bytes, void* stream) {
+  if (dtype != TTSDPA_F32 && dtype != TTSDPA_F16 && dtype != TTSDPA_BF16) return TTSDPA_ERR_DTYPE;
+  if (nbatch_dims < 0 || nbatch_dims > TTLINEAR_MAX_BATCH_DIMS) return TTSDPA_ERR_SHAPE;
+  if (nbatch_dims > 0 && (!batch_shape || !a_batch_stride || !b_batch_stride)) return TTSDPA_ERR_NULL;
+  long long entries = 1;
+  for (int d = 0; d < nbatch_dims; d++) {
+    if (batch_shape[d] < 0 || a_batch_stride[d] < 0 || b_batch_stride[d] < 0) return TTSDPA_ERR_SHAPE;
+    entries *= batch_shape[d];
+  }
+  if (out_batch_stride < 0) return TTSDPA_ERR_STRIDE;
+  const size_t esz = dtype == TTSDPA_F32 ? 4 : 2;
+  for (long long i = 0; i < entries; i++) {
+    // offsets of entry i: the reference's index walk from the innermost batch dimension outwards
+    long long ao = 0, bo = 0, rest = i;
+    for (int d = nbatch_dims - 1; d >= 0; d--) {
+      const long long idx = rest % batch_shape[d];
+      rest /= batch_shape[d];
+      ao += idx * a_batch_stride[d];
+      bo += idx * b_batch_stride[d];
+    }
+    const int rc = ttlinear_matmul(dtype, a ? (const char*)a + ao * esz : nullptr, b ? (const char*)b + bo * esz : nullptr, bias,
+                                   out ? (char*)out + i * out_batch_stride * esz : nullptr, M, N, K, trans_a, trans_b, lda, ldb,
+                                   ldo, workspace, workspace_bytes, stream);
+    if (rc != 0) return rc;
+  }
+  return TTSDPA_OK;
+}
+
 }  // extern "C"

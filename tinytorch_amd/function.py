@@ -389,34 +389,65 @@ def linear(input, weight, bias=None):
 
 
 def matmul(a, b, transA=False, transB=False, bias=None):
-    """op(a) . op(b) + bias for 2-D tensors with the reference's transpose flags (op::matmul, reference
-    src/Operation/OpLinalg.cpp:244-276): a is [M, K], or [K, M] with transA; b is [K, N], or [N, K] with transB.
-    (False, True) is the linear layer; (False, False) and (True, False) are what FuncLinear::backward calls for the
-    input and the weight gradient (reference src/Function/FuncNNLayer.h:20-33)."""
+    """op(a) . op(b) + bias with the reference's transpose flags and batch rules (op::matmul, reference
+    src/Operation/OpLinalg.cpp:52-241): a is [..., M, K], or [..., K, M] with transA; b is [..., K, N], or [..., N, K]
+    with transB; leading dimensions broadcast against each other (:84-89, :205-223).  A 1-D a is a row vector, a 1-D b
+    a column vector (their transpose flags are ignored, :63-72), and the added dimension is dropped from the result.
+    For 2-D operands (False, True) is the linear layer; (False, False) and (True, False) are what
+    FuncLinear::backward calls for the input and the weight gradient (reference src/Function/FuncNNLayer.h:20-33)."""
     _check_rowwise("matmul", a, b, bias)
-    if a.dim() != 2 or b.dim() != 2:
-        raise ValueError("matmul: expected 2-D tensors")
-    K, M = a.shape if transA else (a.shape[1], a.shape[0])
-    Kb, N = (b.shape[1], b.shape[0]) if transB else b.shape
+    if a.dim() == 0 or b.dim() == 0:
+        raise ValueError("matmul: invalid shape")  # reference :54-57
+    prepend_a, append_b = a.dim() == 1, b.dim() == 1
+    if prepend_a:
+        a, transA = a.unsqueeze(0), False
+    if append_b:
+        b, transB = b.unsqueeze(-1), False
+    K, M = (a.shape[-2], a.shape[-1]) if transA else (a.shape[-1], a.shape[-2])
+    Kb, N = (b.shape[-1], b.shape[-2]) if transB else (b.shape[-2], b.shape[-1])
     if K != Kb:
         raise ValueError("matmul: inner sizes differ: %s (transA=%s), %s (transB=%s)" % (tuple(a.shape), transA, tuple(b.shape), transB))
     if bias is not None and tuple(bias.shape) != (N,):
         raise ValueError("matmul: bias must have shape [%d]" % N)
-    a = a if (a.stride(-1) == 1 or a.shape[-1] == 1) else a.contiguous()
-    b = b if (b.stride(-1) == 1 or b.shape[-1] == 1) else b.contiguous()
+    try:
+        batch = tuple(torch.broadcast_shapes(a.shape[:-2], b.shape[:-2]))
+    except RuntimeError:
+        raise ValueError("matmul: batch dimensions %s and %s do not broadcast" % (tuple(a.shape[:-2]), tuple(b.shape[:-2])))
+    if len(batch) > 8:
+        raise ValueError("matmul: more than 8 batch dimensions")
+    dense = lambda t: t if (t.stride(-1) == 1 or t.shape[-1] == 1) and (t.shape[-2] == 1 or t.stride(-2) >= max(t.shape[-1], 1)) else t.contiguous()
+    a, b = dense(a), dense(b)
     bs = bias.contiguous() if bias is not None else None
-    out = torch.empty(M, N, dtype=a.dtype, device=a.device)
+    out = torch.empty(batch + (M, N), dtype=a.dtype, device=a.device)
     L = _capi.lib()
     nbytes = L.ttlinear_matmul_workspace_bytes(_DTYPES[a.dtype], M, N, K, int(transA), int(transB))
     ws = _workspace(a.device, nbytes) if nbytes else None
-    lda = a.stride(0) if a.shape[0] > 1 else max(a.shape[1], 1)
-    ldb = b.stride(0) if b.shape[0] > 1 else max(b.shape[1], 1)
+    lda = a.stride(-2) if a.shape[-2] > 1 else max(a.shape[-1], 1)
+    ldb = b.stride(-2) if b.shape[-2] > 1 else max(b.shape[-1], 1)
+    common = (_DTYPES[a.dtype], a.data_ptr(), b.data_ptr(), bs.data_ptr() if bs is not None else None, out.data_ptr(), M, N, K,
+              int(transA), int(transB), lda, ldb, N)
+    tail = (ws.data_ptr() if ws is not None else None, nbytes, torch.cuda.current_stream(a.device).cuda_stream)
     with torch.cuda.device(a.device):
-        rc = L.ttlinear_matmul(_DTYPES[a.dtype], a.data_ptr(), b.data_ptr(), bs.data_ptr() if bs is not None else None,
-                               out.data_ptr(), M, N, K, int(transA), int(transB), lda, ldb, N,
-                               ws.data_ptr() if ws is not None else None, nbytes, torch.cuda.current_stream().cuda_stream)
+        if not batch:
+            rc = L.ttlinear_matmul(*common, *tail)
+        else:
+            ea = a.expand(batch + tuple(a.shape[-2:]))  # views: broadcast axes get stride 0
+            eb = b.expand(batch + tuple(b.shape[-2:]))
+            nb = len(batch)
+            arr = ctypes.c_int64 * nb
+            sa = arr(*[ea.stride(d) if batch[d] > 1 else 0 for d in range(nb)])
+            sb = arr(*[eb.stride(d) if batch[d] > 1 else 0 for d in range(nb)])
+            rc = L.ttlinear_matmul_batched(*common, nb, arr(*batch), sa, sb, M * N, *tail)
     if rc != 0:
         raise RuntimeError("ttlinear_matmul failed: %d (%s)" % (rc, _capi.status_string(rc)))
+    # the added dimensions are dropped as the reference drops them (:221-239): for 2-D results only — with batch
+    # dimensions a 1-D a keeps its row ([..., 1, N]) and a 1-D b has no defined result there (its reshape to [M] would not fit)
+    if append_b:
+        if batch and out.numel() != (1 if prepend_a else M):
+            raise ValueError("matmul: a 1-D second operand against a batched first operand has no result shape in the reference")
+        out = out.reshape(() if prepend_a else (M,))
+    elif prepend_a and not batch:
+        out = out.reshape(N)
     return out
 
 
