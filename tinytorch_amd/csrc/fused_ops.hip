@@ -214,6 +214,48 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* out, l
     mx = mn;
   };
   auto reload = [&](int i) __attribute__((always_inline)) { return load_plain<T, VEC>(xr + (long long)i * VEC); };
+  if (!LOG && nvec <= KEEP * LPR) {
+    // The whole row sits in the lanes' registers: the reference's own three steps (maximum, exponentials and their
+    // sum, scaling: reference src/Operation/OpNNLayerCpu.h:27-54) with one exponential per element — they are kept
+    // as fp32 between the sum and the write.  (The running form below spends two per element: one for the statistics
+    // and one for the result.)
+    if (live) {
+#pragma unroll
+      for (int c = 0; c < KEEP; c++)
+        if (lr + c * LPR < nvec) keep[c] = load_stream<T, VEC>(xr + (long long)(lr + c * LPR) * VEC);
+#pragma unroll
+      for (int c = 0; c < KEEP; c++)
+        if (lr + c * LPR < nvec) {
+#pragma unroll
+          for (int e = 0; e < VEC; e++) mx = fmaxf(mx, (float)keep[c][e]);
+        }
+    }
+    const float rmax = row_reduce<LPR, MaxOp>(mx, lds, 0);
+    float ex[KEEP][VEC];
+    if (live) {
+#pragma unroll
+      for (int c = 0; c < KEEP; c++)
+        if (lr + c * LPR < nvec) {
+#pragma unroll
+          for (int e = 0; e < VEC; e++) {
+            ex[c][e] = __expf((float)keep[c][e] - rmax);
+            sum += ex[c][e];
+          }
+        }
+    }
+    sum = row_reduce<LPR, SumOp>(sum, lds, 1);
+    if (!live) return;
+    const float inv = 1.f / sum;
+#pragma unroll
+    for (int c = 0; c < KEEP; c++)
+      if (lr + c * LPR < nvec) {
+        V o;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) o[e] = (T)(ex[c][e] * inv);
+        store_pack<T, VEC>(orow + (long long)(lr + c * LPR) * VEC, o);
+      }
+    return;
+  }
   if (live) {
 #pragma unroll
     for (int c = 0; c < KEEP; c++)
