@@ -17,6 +17,7 @@
 //
 // linear_general_kernel: any element type and shape, fp32 arithmetic on the vector ALUs (64 x 64 tiles).
 
+#include <type_traits>
 #include "../../include/ttlinear.h"
 #include "sdpa_common.h"
 
@@ -227,6 +228,176 @@ __global__ __launch_bounds__(WN * WM * 64, 1) void linear_mfma_kernel(LinArgs a)
           *(typename G::out4*)(orow + n) = G::cvt(v);
         }
       }
+  }
+}
+
+// ---- 16-bit tensors, 256 x 256 tiles: four wavefronts with 128 x 128 each and the K loop as one hand-ordered stream ------
+// Same tiles, LDS layout and direct loads as linear_mfma_kernel<TR, 256, 256>; what differs is who owns what and who
+// orders the instructions.  A wavefront owns 4 x 4 blocks of 32 x 32 (256 accumulator registers, in AGPRs: one wavefront
+// per SIMD), so an operand read from LDS feeds four matrix instructions instead of 2.7 — LDS operand traffic is the
+// second consumer of power after the matrix pipe itself, and the clock of this kernel is power-managed.  The K loop is
+// a single asm statement (linear256_loop.inc, written by gen_linear256_loop.py): the compiler's version of the loop
+// requested the operands of a k-step in one burst behind seven matrix instructions and waited for them before the next,
+// and put the sixteen tile loads and the next operands between the barrier and the matrix instructions behind it.
+#include "linear256_loop.inc"
+
+typedef unsigned u32x8 __attribute__((ext_vector_type(8)));
+
+template <typename TR>
+struct Lin256Loop;
+template <>
+struct Lin256Loop<BF16> {
+#define TT_LIN256_TEXT TT_LIN256_LOOP_BF16
+  static __device__ __forceinline__ void run(f32x16 (&c)[16], u32x8& xoff, u32x8& woff, u32x8& raddr, unsigned long long& xp, unsigned long long& wp,
+                                             unsigned& m0base, unsigned& left, unsigned& adv) {
+#include "linear256_stmt.inc"
+  }
+#undef TT_LIN256_TEXT
+};
+template <>
+struct Lin256Loop<F16> {
+#define TT_LIN256_TEXT TT_LIN256_LOOP_F16
+  static __device__ __forceinline__ void run(f32x16 (&c)[16], u32x8& xoff, u32x8& woff, u32x8& raddr, unsigned long long& xp, unsigned long long& wp,
+                                             unsigned& m0base, unsigned& left, unsigned& adv) {
+#include "linear256_stmt.inc"
+  }
+#undef TT_LIN256_TEXT
+};
+
+template <typename TR>
+__global__ __launch_bounds__(256, 1) void linear256_kernel(LinArgs a) {
+  constexpr int TM = 256, TN = 256;
+  constexpr int XTILE = TM * ROWB;
+  constexpr int STAGE = (TM + TN) * ROWB;
+  typedef typename TR::elem T;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, lh = lane >> 5;
+
+  // workgroup -> tile: 4 x 8 tile blocks per XCD, as in linear_mfma_kernel
+  const int tiles_m = (int)((a.M + TM - 1) / TM), tiles_n = (int)((a.N + TN - 1) / TN);
+  const int super_n = (tiles_n + 7) / 8;
+  const int nsuper = ((tiles_m + 3) / 4) * super_n;
+  const int slot = blockIdx.x >> 3;
+  const int super = (slot >> 5) * 8 + (blockIdx.x & 7);
+  if (super >= nsuper) return;
+  const int tm = (super / super_n) * 4 + ((slot & 31) >> 3);
+  const int tn = (super % super_n) * 8 + (slot & 7);
+  if (tm >= tiles_m || tn >= tiles_n) return;
+  const long long m0 = (long long)tm * TM, n0 = (long long)tn * TN;
+
+  // global -> LDS: wavefront v moves rows 64v .. 64v+63 of both tiles, 8 rows (1 KB) per instruction; lane l fills
+  // (row l/8, chunk slot l%8) and fetches chunk (l%8) ^ ((row/2) % 8); rows past the end re-read the last row
+  const long long mlim = a.M - 1 - m0, nlim = a.N - 1 - n0;
+  u32x8 xoff, woff;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int row = 64 * wave + 8 * i + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    xoff[i] = (unsigned)(((row < mlim ? row : mlim) * a.ldx + 8 * chunk) * 2);
+    woff[i] = (unsigned)(((row < nlim ? row : nlim) * a.ldw + 8 * chunk) * 2);
+  }
+  // (the 64-bit products are formed on the vector ALUs; the loads want their base in scalar registers)
+  auto uniform = [](const void* p) __attribute__((always_inline)) {
+    const unsigned long long v = (unsigned long long)p;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return (const char*)(((unsigned long long)hi << 32) | lo);
+  };
+  const char* xbase = uniform((const T*)a.x + m0 * a.ldx);
+  const char* wbase = uniform((const T*)a.w + n0 * a.ldw);
+  const unsigned smem_addr = (unsigned)(unsigned long)(lds_void_t*)smem;
+  auto dma_tile = [&](long long t, int stage) __attribute__((always_inline)) {
+    const char* xs = xbase + t * ROWB;
+    const char* ws = wbase + t * ROWB;
+    const unsigned dst = smem_addr + stage * STAGE + wave * 8192;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(xoff[i]), "s"(xs), "s"(dst + 1024 * i) : "memory", "m0");
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(woff[i]), "s"(ws), "s"(dst + XTILE + 1024 * i) : "memory", "m0");
+  };
+
+  // this wavefront's part: n rows 128*wn .. of the w tile (A operand), m rows 128*wm .. of the x tile (B operand);
+  // operand (block, ks): row 32*block + lq, chunk 2*ks + lh at row*128 + 16 * (chunk ^ ((row/2) % 8))
+  const int wn = wave & 1, wm = wave >> 1;
+  const unsigned frag = (unsigned)(lq * ROWB + 16 * (lh ^ ((lq >> 1) & 7)));
+  u32x8 raddr;
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++) {
+    raddr[2 * ks] = smem_addr + ((128 * wm * ROWB + frag) ^ (unsigned)(32 * ks));
+    raddr[2 * ks + 1] = smem_addr + ((128 * wn * ROWB + frag) ^ (unsigned)(32 * ks));
+  }
+
+  f32x16 acc[16];  // block (i, j): n rows 32i .., m rows 32j .. of the wavefront's part
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const long long n = n0 + 128 * wn + 32 * i + 8 * (r >> 2) + 4 * lh + (r & 3);
+      const float b = (a.bias && n < a.N) ? (float)((const T*)a.bias)[n] : 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[4 * i + j][r] = b;
+    }
+
+  const long long ntk = a.K / 64;
+  if (ntk > 0) {
+    dma_tile(0, 0);
+    if (ntk > 1) {
+      dma_tile(1, 1);
+      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    // the loop's loads: k-tile min(t + 2, ntk - 1) while k-tile t is computed
+    const long long first = ntk > 2 ? 2 : ntk - 1;
+    unsigned long long xp = (unsigned long long)(xbase + first * ROWB), wp = (unsigned long long)(wbase + first * ROWB);
+    unsigned m0base = smem_addr + wave * 8192;
+    unsigned left = (unsigned)ntk, adv = ntk > 3 ? (unsigned)(ntk - 3) : 0u;
+    Lin256Loop<TR>::run(acc, xoff, woff, raddr, xp, wp, m0base, left, adv);
+  }
+
+  // store through LDS, so that a store instruction writes whole lines: written 8 bytes at a time the tile took 16 % of
+  // the kernel (every instruction touched 32 rows, 16 bytes each; the L2 takes a request per piece).  The wavefront's
+  // 128 x 128 part goes to its quarter of the (now idle) stages as rows of 256 bytes, the 16-byte chunks of row r at
+  // slot c ^ (r % 16); then 16 lanes read a row back and store its 256 bytes.
+  __builtin_amdgcn_s_barrier();  // every wavefront has taken its last operands
+  asm volatile("" ::: "memory");
+  char* mine = smem + wave * 32768;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int row = 32 * j + lq;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        f32x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = acc[4 * i + j][4 * rg + e];
+        *(typename TR::vec4*)(mine + row * 256 + 16 * ((4 * i + rg) ^ (row & 15)) + 8 * lh) = __builtin_convertvector(v, typename TR::vec4);
+      }
+  }
+  // (a wavefront reads back only what it wrote: no barrier)
+  const long long nbase = n0 + 128 * wn;
+#pragma unroll 8
+  for (int it = 0; it < 32; it++) {
+    const int row = 4 * it + (lane >> 4);
+    const int c = (lane & 15) ^ (row & 15);
+    const u32x4 v = *(const u32x4*)(mine + row * 256 + 16 * (lane & 15));
+    const long long m = m0 + 128 * wm + row, n = nbase + 8 * c;
+    if (m < a.M) {
+      T* dst = (T*)a.out + m * a.ldo + n;
+      if (n + 8 <= a.N) {
+        *(u32x4*)dst = v;
+      } else if (n + 4 <= a.N) {  // N is a multiple of 4 on this route
+        *(u32x2*)dst = u32x2{v[0], v[1]};
+      }
+    }
   }
 }
 
@@ -526,11 +697,31 @@ int launch_mfma_tile(const LinArgs& a, hipStream_t stream) {
 }
 
 template <typename TR>
+int launch_linear256(const LinArgs& a, hipStream_t stream) {
+  constexpr int lds = 2 * (256 + 256) * ROWB;
+  static hipError_t state[kMaxDevices];
+  static bool done[kMaxDevices];
+  const hipError_t granted = grant_dynamic_lds((const void*)linear256_kernel<TR>, lds, state, done);
+  if (granted != hipSuccess) return (int)granted;
+  const long long tiles_m = (a.M + 255) / 256, tiles_n = (a.N + 255) / 256;
+  const long long nsuper = ((tiles_m + 3) / 4) * ((tiles_n + 7) / 8);
+  const long long nwg = (nsuper + 7) / 8 * 8 * 32;
+  if (nwg > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
+  hipLaunchKernelGGL((linear256_kernel<TR>), dim3((unsigned)nwg), dim3(256), lds, stream, a);
+  return (int)hipGetLastError();
+}
+
+template <typename TR>
 int launch_mfma(const LinArgs& a, hipStream_t stream) {
   // 256 x 256 tiles once they fill the 256 CUs; smaller problems get four times as many 128 x 128 tiles
   const long long big = ((a.M + 255) / 256) * ((a.N + 255) / 256);
   // (four wavefronts with 128 x 128 each — accumulators in AGPRs, half the LDS operand reads — measured 2-10 % slower
   // than eight with 64 x 128: one wavefront per SIMD hides too little)
+  if constexpr (!std::is_same<TR, F32>::value) {
+    // 16-bit tensors: the hand-ordered kernel
+    // and it stores 16 bytes at a time
+    if (big >= 256 && a.ldo % 8 == 0 && ((uintptr_t)a.out & 15) == 0) return launch_linear256<TR>(a, stream);
+  }
   return big >= 256 ? launch_mfma_tile<TR, 256, 256, 4, 2>(a, stream) : launch_mfma_tile<TR, 128, 128, 4, 2>(a, stream);
 }
 
