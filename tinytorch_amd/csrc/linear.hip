@@ -231,37 +231,42 @@ __global__ __launch_bounds__(WN * WM * 64, 1) void linear_mfma_kernel(LinArgs a)
   }
 }
 
-// ---- 16-bit tensors, 256 x 256 tiles: four wavefronts with 128 x 128 each and the K loop as one hand-ordered stream ------
-// Same tiles, LDS layout and direct loads as linear_mfma_kernel<TR, 256, 256>; what differs is who owns what and who
-// orders the instructions.  A wavefront owns 4 x 4 blocks of 32 x 32 (256 accumulator registers, in AGPRs: one wavefront
-// per SIMD), so an operand read from LDS feeds four matrix instructions instead of 2.7 — LDS operand traffic is the
-// second consumer of power after the matrix pipe itself, and the clock of this kernel is power-managed.  The K loop is
-// a single asm statement (linear256_loop.inc, written by gen_linear256_loop.py): the compiler's version of the loop
-// requested the operands of a k-step in one burst behind seven matrix instructions and waited for them before the next,
-// and put the sixteen tile loads and the next operands between the barrier and the matrix instructions behind it.
+// ---- 16-bit tensors, 256 x 256 tiles: four wavefronts with 128 x 128 each and the tile's arithmetic as one hand-ordered stream
+// Same tiles, LDS layout and direct loads as linear_mfma_kernel<TR, 256, 256>; what differs is who owns what, the matrix
+// instruction and who orders the instructions.  The clock of these kernels is power-managed, so what a tile costs is
+// energy rather than issue slots:
+//  * a wavefront owns 128 x 128 of the tile (256 accumulator registers, in AGPRs: one wavefront per SIMD), so an operand
+//    read from LDS feeds eight matrix instructions — LDS operand traffic is the second consumer after the matrix pipe;
+//  * v_mfma_f32_16x16x32 instead of 32x32x16: with random operands the chip sustains 2.10 against 1.84 PFLOP/s of them;
+//  * the body of a tile (accumulators from the bias, K loop, conversion into LDS) is a single asm statement
+//    (linear256_loop.inc, written by gen_linear256_loop.py): the compiler's version of the loop requested the operands
+//    of a k-step in one burst behind the matrix instructions and waited for them before the next, and put the tile
+//    loads and the next operands between the barrier and the matrix instructions behind it;
+//  * the output leaves through LDS as whole lines: written 8 bytes at a time the tile's stores took 16 % of the kernel
+//    (every instruction touched 32 rows, 16 bytes each; the L2 takes a request per piece).
 #include "linear256_loop.inc"
 
 typedef unsigned u32x8 __attribute__((ext_vector_type(8)));
 
 template <typename TR>
-struct Lin256Loop;
+struct Lin256Body;
 template <>
-struct Lin256Loop<BF16> {
-#define TT_LIN256_TEXT TT_LIN256_LOOP_BF16
-  static __device__ __forceinline__ void run(f32x16 (&c)[16], u32x8& xoff, u32x8& woff, u32x8& raddr, unsigned long long& xp, unsigned long long& wp,
-                                             unsigned& m0base, unsigned& left, unsigned& adv) {
+struct Lin256Body<BF16> {
+  static __device__ __forceinline__ void run(f32x16 bias_lo, f32x16 bias_hi, u32x8 xoff, u32x8 woff, u32x4 raddr, u32x8 eaddr,
+                                             unsigned long long xp, unsigned long long wp, unsigned m0base, unsigned left, unsigned adv) {
+#define TT_LIN256_TEXT TT_LIN256_BODY_BF16
 #include "linear256_stmt.inc"
-  }
 #undef TT_LIN256_TEXT
+  }
 };
 template <>
-struct Lin256Loop<F16> {
-#define TT_LIN256_TEXT TT_LIN256_LOOP_F16
-  static __device__ __forceinline__ void run(f32x16 (&c)[16], u32x8& xoff, u32x8& woff, u32x8& raddr, unsigned long long& xp, unsigned long long& wp,
-                                             unsigned& m0base, unsigned& left, unsigned& adv) {
+struct Lin256Body<F16> {
+  static __device__ __forceinline__ void run(f32x16 bias_lo, f32x16 bias_hi, u32x8 xoff, u32x8 woff, u32x4 raddr, u32x8 eaddr,
+                                             unsigned long long xp, unsigned long long wp, unsigned m0base, unsigned left, unsigned adv) {
+#define TT_LIN256_TEXT TT_LIN256_BODY_F16
 #include "linear256_stmt.inc"
-  }
 #undef TT_LIN256_TEXT
+  }
 };
 
 template <typename TR>
@@ -275,7 +280,7 @@ __global__ __launch_bounds__(256, 1) void linear256_kernel(LinArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int lq = lane & 31, lh = lane >> 5;
+  const int lr = lane & 15, lg = lane >> 4;
 
   // workgroup -> tile: 4 x 8 tile blocks per XCD, as in linear_mfma_kernel
   const int tiles_m = (int)((a.M + TM - 1) / TM), tiles_n = (int)((a.N + TN - 1) / TN);
@@ -322,67 +327,52 @@ __global__ __launch_bounds__(256, 1) void linear256_kernel(LinArgs a) {
   };
 
   // this wavefront's part: n rows 128*wn .. of the w tile (A operand), m rows 128*wm .. of the x tile (B operand);
-  // operand (block, ks): row 32*block + lq, chunk 2*ks + lh at row*128 + 16 * (chunk ^ ((row/2) % 8))
+  // operand (block, s): row 16*block + lane%16, chunk 4*s + lane/16 at row*128 + 16 * (chunk ^ ((row/2) % 8))
   const int wn = wave & 1, wm = wave >> 1;
-  const unsigned frag = (unsigned)(lq * ROWB + 16 * (lh ^ ((lq >> 1) & 7)));
-  u32x8 raddr;
+  const unsigned frag = (unsigned)(lr * ROWB + 16 * (lg ^ ((lr >> 1) & 7)));
+  u32x4 raddr;
 #pragma unroll
-  for (int ks = 0; ks < 4; ks++) {
-    raddr[2 * ks] = smem_addr + ((128 * wm * ROWB + frag) ^ (unsigned)(32 * ks));
-    raddr[2 * ks + 1] = smem_addr + ((128 * wn * ROWB + frag) ^ (unsigned)(32 * ks));
+  for (int s = 0; s < 2; s++) {
+    raddr[2 * s] = smem_addr + ((128 * wm * ROWB + frag) ^ (unsigned)(64 * s));
+    raddr[2 * s + 1] = smem_addr + ((128 * wn * ROWB + frag) ^ (unsigned)(64 * s));
   }
-
-  f32x16 acc[16];  // block (i, j): n rows 32i .., m rows 32j .. of the wavefront's part
+  // block (i, j) leaves the lane with out[m = .. + 16j + lane%16][n = .. + 16i + 4(lane/16) .. +3]: 8 bytes of row 16j + lane%16
+  // of the wavefront's quarter of LDS (rows of 256 bytes, the 16-byte chunks of row r at slot c ^ (r % 16))
+  u32x8 eaddr;
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < 8; i++) eaddr[i] = smem_addr + wave * 32768 + lr * 256 + 16 * ((2 * i + (lg >> 1)) ^ lr) + 8 * (lg & 1);
+  // accumulators start from the bias (the reference writes the bias into C and accumulates onto it)
+  f32x16 bias_lo, bias_hi;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const long long n = n0 + 128 * wn + 32 * i + 8 * (r >> 2) + 4 * lh + (r & 3);
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const long long n = n0 + 128 * wn + 16 * i + 4 * lg + e;
       const float b = (a.bias && n < a.N) ? (float)((const T*)a.bias)[n] : 0.f;
-#pragma unroll
-      for (int j = 0; j < 4; j++) acc[4 * i + j][r] = b;
+      if (i < 4) bias_lo[4 * i + e] = b;
+      else bias_hi[4 * (i - 4) + e] = b;
     }
 
-  const long long ntk = a.K / 64;
-  if (ntk > 0) {
-    dma_tile(0, 0);
-    if (ntk > 1) {
-      dma_tile(1, 1);
-      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
+  const long long ntk = a.K / 64;  // > 0 on this route
+  dma_tile(0, 0);
+  if (ntk > 1) {
+    dma_tile(1, 1);
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  {
     // the loop's loads: k-tile min(t + 2, ntk - 1) while k-tile t is computed
     const long long first = ntk > 2 ? 2 : ntk - 1;
-    unsigned long long xp = (unsigned long long)(xbase + first * ROWB), wp = (unsigned long long)(wbase + first * ROWB);
-    unsigned m0base = smem_addr + wave * 8192;
-    unsigned left = (unsigned)ntk, adv = ntk > 3 ? (unsigned)(ntk - 3) : 0u;
-    Lin256Loop<TR>::run(acc, xoff, woff, raddr, xp, wp, m0base, left, adv);
+    Lin256Body<TR>::run(bias_lo, bias_hi, xoff, woff, raddr, eaddr, (unsigned long long)(xbase + first * ROWB),
+                        (unsigned long long)(wbase + first * ROWB), smem_addr + wave * 8192, (unsigned)ntk,
+                        ntk > 3 ? (unsigned)(ntk - 3) : 0u);
   }
 
-  // store through LDS, so that a store instruction writes whole lines: written 8 bytes at a time the tile took 16 % of
-  // the kernel (every instruction touched 32 rows, 16 bytes each; the L2 takes a request per piece).  The wavefront's
-  // 128 x 128 part goes to its quarter of the (now idle) stages as rows of 256 bytes, the 16-byte chunks of row r at
-  // slot c ^ (r % 16); then 16 lanes read a row back and store its 256 bytes.
-  __builtin_amdgcn_s_barrier();  // every wavefront has taken its last operands
-  asm volatile("" ::: "memory");
-  char* mine = smem + wave * 32768;
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const int row = 32 * j + lq;
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        f32x4 v;
-#pragma unroll
-        for (int e = 0; e < 4; e++) v[e] = acc[4 * i + j][4 * rg + e];
-        *(typename TR::vec4*)(mine + row * 256 + 16 * ((4 * i + rg) ^ (row & 15)) + 8 * lh) = __builtin_convertvector(v, typename TR::vec4);
-      }
-  }
-  // (a wavefront reads back only what it wrote: no barrier)
+  // 16 lanes read a row of the wavefront's quarter back and store its 256 bytes (a wavefront reads only what it wrote)
+  const char* mine = smem + wave * 32768;
   const long long nbase = n0 + 128 * wn;
 #pragma unroll 8
   for (int it = 0; it < 32; it++) {
