@@ -17,7 +17,14 @@ Register plan of a lane (fixed, named in the statements' constraints by the kern
     v[192:199]  probabilities "A" (2 k-steps x 4)      v[200:207]  probabilities "B"
     v[208:239]  operand ring, 8 x 4        v[240:247]  temporaries      v[248:255]  K operand addresses, one per k-step
 Named operands of the statement: o0-o3 the four output accumulators (read-write), ps the lane's sum of the step's
-probabilities (out), c = scale*log2(e), mc = maximum*scale*log2(e).
+probabilities (out), c = scale*log2(e) (scalar register), mc = maximum*scale*log2(e), and for the causal variant
+mk (scalar, 1 = take it), kvs (scalar, first key of the half whose exponentials the step takes) and rl (query row of
+the lane in key coordinates - 4*(lane/32)).
+
+Every string holds the step twice: as above, and with the causal predicate applied to each probability (a score's
+key is visible iff kvs + 8*(n/4) + n%4 <= rl: two more instructions per score, a compare through m0 and vcc and a
+select).  The second form serves the one or two tiles of a wavefront's row group that touch the diagonal; it sits out
+of line, in subsection 1 of the kernel's section, so that the steady state falls through without a taken branch.
 """
 import sys
 
@@ -49,7 +56,7 @@ def pending_after(G):
     return sum(len(fetch(g)) for g in range(G + 1, G + PD))
 
 
-def step(u, kind, elem):
+def step(u, kind, elem, masked=False):
     mfma = "v_mfma_f32_32x32x16_%s" % elem
     cvt = "v_cvt_pk_%s_f32" % elem
     G0 = 32 * u + 16 * kind
@@ -59,6 +66,11 @@ def step(u, kind, elem):
     T = [T0, T0 + 1, T0 + 2, T0 + 3]
     out = []
     fma = lambda n: "v_fma_f32 %s, %s, %%[c], -%%[mc]" % (vr(F[n & 1]), vr(s_nxt + n))
+
+    def hide(n):  # causal mask of score n: visible iff kvs + 8*(n/4) + n%4 <= rl (kvs: first key of the half, rl = query - 4*(lane/32))
+        return ["s_add_i32 m0, %%[kvs], %d" % (8 * (n >> 2) + (n & 3)), "v_cmp_le_i32 vcc, m0, %[rl]",
+                "v_cndmask_b32 %s, 0, %s, vcc" % (vr(T[n & 3]), vr(T[n & 3]))]
+
     out.append(fma(0))
     for n in range(16):
         G = G0 + n
@@ -75,6 +87,8 @@ def step(u, kind, elem):
         out.append("v_exp_f32 %s, %s" % (vr(T[n & 3]), vr(F[n & 1])))
         if n + 1 < 16:
             out.append(fma(n + 1))
+        if masked:
+            out += hide(n)
         if n == 2:  # the sum starts as (score 0) + (score 1): what 0 + x0 + x1 gives
             out.append("v_add_f32 %%[ps], %s, %s" % (vr(T[0]), vr(T[1])))
         elif n >= 3:
@@ -82,7 +96,8 @@ def step(u, kind, elem):
         if n % 2 == 0 and n >= 2:
             j = (n - 2) // 2  # scores n-2, n-1
             out.append("%s %s, %s, %s" % (cvt, vr(p_nxt + j), vr(T[(n - 2) & 3]), vr(T[(n - 1) & 3])))
-    out.append("s_nop 0")
+    if not masked:
+        out.append("s_nop 0")
     out.append("v_add_f32 %%[ps], %%[ps], %s" % vr(T[15 & 3]))
     out.append("%s %s, %s, %s" % (cvt, vr(p_nxt + 7), vr(T[14 & 3]), vr(T[15 & 3])))
     return out
@@ -103,13 +118,19 @@ def emit(name, lines):
 
 def main():
     print("// Generated by gen_prefill128_steps.py; do not edit.  Instruction streams of the pipelined prefill kernel's")
-    print("// steady state: TT_P128_STEP_<elem>_U<tile of the unrolled body>_K<step of the tile>.")
+    print("// steady state: TT_P128_STEP_<elem>_U<tile of the unrolled body>_K<step of the tile> (with the causal variant out of")
+    print("// line), TT_P128_PSTEP_... the plain step alone.")
     print()
     emit("TT_P128_PREFETCH", prefetch())
     for elem in ("bf16", "f16"):
         for u in range(4):
             for kind in range(2):
-                emit("TT_P128_STEP_%s_U%d_K%d" % (elem.upper(), u, kind), step(u, kind, elem))
+                # the variant with the causal predicate sits out of line (at the end of the kernel's section), so that the
+                # steady state runs through without a taken branch
+                both = (["s_cmp_eq_u32 %[mk], 0", "s_cbranch_scc0 .Ltt_p128_m%="] + step(u, kind, elem) + [".Ltt_p128_e%=:", ".subsection 1", ".Ltt_p128_m%=:"]
+                        + step(u, kind, elem, True) + ["s_branch .Ltt_p128_e%=", ".subsection 0"])
+                emit("TT_P128_STEP_%s_U%d_K%d" % (elem.upper(), u, kind), both)
+                emit("TT_P128_PSTEP_%s_U%d_K%d" % (elem.upper(), u, kind), step(u, kind, elem))  # calls without a causal mask
 
 
 if __name__ == "__main__":

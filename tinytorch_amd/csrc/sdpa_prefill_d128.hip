@@ -39,7 +39,11 @@
 // is the true row maximum formed, sum and accumulator rescaled, and the half redone.  The scores of a half stay in
 // their accumulator registers until that check has passed.
 // Causal masking (key j visible to query i iff j <= i, reference src/Operation/OpTransformCpu.h:202-209) skips
-// halves above the diagonal and applies the predicate only on halves that straddle it.
+// halves above the diagonal and applies the predicate only on halves that straddle it.  The tile of a row group that
+// touches the diagonal stays in the steady state's pipelined form: its streams exist a second time with the predicate
+// applied to each probability (selected by a scalar flag), so that only a row group's last one or two steps take the
+// general form.  The eight row groups of a workgroup reach the diagonal in eight different tiles, and with the
+// general form on every one of them each of the workgroup's last five tiles waited for one wavefront in that form.
 // Under a causal mask a workgroup takes a row tile and its mirror (equal work for every workgroup), and neighbouring
 // workgroups take the two in opposite order so their load/store bursts do not coincide.
 // Grouped-query attention: kv head = query head / (Hq/Hkv), resolved in the kernel; the workgroup order puts the
@@ -304,7 +308,20 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     }
   }
   if (nfast < 0) nfast = 0;
-  if (a.mask_kind != 0) nfast = 0;  // an attnMask is applied in the general form of a step
+  // Tiles in the fast form including those whose exponentials take the causal predicate (a variant of the streams):
+  // both steps of tile j accumulate a half of this wavefront's (2j+1 < my_halves) and half 2j+2 is complete.
+  int nfast_all = nfast;
+  if (CAUSAL) {
+    int t = my_halves / 2;
+    const int f = S >= 96 ? (S - 32) / BN : 0;
+    t = f < t ? f : t;
+    nfast_all = t > nfast ? t : nfast;
+  }
+  if (a.mask_kind != 0) nfast = 0, nfast_all = 0;  // an attnMask is applied in the general form of a step
+  if (CAUSAL) {  // scalar registers: operands of the step statements derive from them
+    nfast = __builtin_amdgcn_readfirstlane(nfast);
+    nfast_all = __builtin_amdgcn_readfirstlane(nfast_all);
+  }
 
   // ---- prologue: the part's first loads were sent for by issue_part ------------------------------------------------
   auto q_of = [&](int ks) __attribute__((always_inline)) {
@@ -319,6 +336,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
   const float c = a.scale * kLog2e;
+  // the same, in a scalar register (causal step statements: their predicate operands take the freed vector register)
+  const float c_s = CAUSAL ? __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, c))) : 0.f;
   float m_use = -1e30f;  // maximum the exponentials are taken against (raw scores)
   float mc = -1e30f * c;
   float l_run = 0.f;
@@ -383,8 +402,16 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   // some probability left the range [0, kSumLimit] (which includes the first half of a row, taken against -1e30):
   // then the true row maximum is formed, sum and accumulator are rescaled and the half is redone.  Every
   // probability that reaches the matrix pipe is therefore at most kSumLimit.
-  auto settle_half = [&](const f32x16& s, vec8 (&pb)[2], float psum) __attribute__((always_inline)) {
+  const int rl = CAUSAL ? qc0 + lq - 4 * lh : 0;  // the causal predicate's lane operand: key k of a score is visible iff k - 4*(lane/32) <= rl
+  auto settle_half = [&](f32x16& s, vec8 (&pb)[2], float psum, int masked_kv0 = -1) __attribute__((always_inline)) {
     if (__builtin_amdgcn_ballot_w64(!(psum <= kSumLimit)) != 0) {
+      // after a step whose exponentials took the causal predicate in the stream, the scores themselves are masked only
+      // here (hidden scores, or what a stage held beyond the workgroup's last tile, must not enter the maximum)
+      if (CAUSAL && masked_kv0 >= 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          if (masked_kv0 + 8 * (r >> 2) + (r & 3) > rl) s[r] = -INFINITY;  // the streams' predicate
+      }
       const float m_new = fmaxf(m_use, row_max(s));
       const float alpha = fast_exp2((m_use - m_new) * c);
       m_use = m_new;
@@ -442,6 +469,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #pragma unroll
   for (int i = 0; i < 32; i++) ring[i] = 0u;
 #define TT_P128_RUN_STEP(TXT)                                                                                          \
+  asm volatile(TXT                                                                                                     \
+               : [o0] "+v"(oacc[0]), [o1] "+v"(oacc[1]), [o2] "+v"(oacc[2]), [o3] "+v"(oacc[3]), [ps] "=&v"(psum_step),  \
+                 "+{v[160:175]}"(sB), "+{v[176:191]}"(sC), "+{v[192:199]}"(pAv), "+{v[200:207]}"(pBv),                   \
+                 "+{v[208:239]}"(ring)                                                                                 \
+               : [c] "s"(c_s), [mc] "v"(mc), [rl] "v"(rl), [mk] "s"(mk), [kvs] "s"(kvs), "{v[120:151]}"(qv), "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr) \
+               : "v240", "v241", "v242", "v243", "v244", "v245", "vcc", "scc", "m0", "memory")
+// the plain step alone (calls without a causal mask): no predicate operands
+#define TT_P128_RUN_PSTEP(TXT)                                                                                         \
   asm volatile(TXT                                                                                                     \
                : [o0] "+v"(oacc[0]), [o1] "+v"(oacc[1]), [o2] "+v"(oacc[2]), [o3] "+v"(oacc[3]), [ps] "=&v"(psum_step),  \
                  "+{v[160:175]}"(sB), "+{v[176:191]}"(sC), "+{v[192:199]}"(pAv), "+{v[200:207]}"(pBv),                   \
@@ -521,11 +556,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     return keep;
   };
   int j = 0;
-  if (nfast >= 1) {
-    auto settle_fast = [&](const f32x16& s, u32x8& pv) __attribute__((always_inline)) {
+  if (nfast_all >= 1) {
+    auto settle_fast = [&](f32x16& s, u32x8& pv, int masked_kv0) __attribute__((always_inline)) {
       vec8 p[2];
       p_load(pv, p);
-      settle_half(s, p, psum_step);
+      settle_half(s, p, psum_step, masked_kv0);
       p_store(pv, p);
     };
     p_store(pAv, pA);
@@ -533,15 +568,27 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     asm volatile(TT_P128_PREFETCH : "+{v[208:239]}"(ring) : "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr) : "memory");
     // Four tiles per trip so that the stage of a tile is a constant of its statement; the trip may end after any of them.
 #define TT_P128_TILE(U)                                                                                  \
-    if (j >= nfast) break;                                                                                \
+    if (j >= nfast_all) break;                                                                            \
     {                                                                                                    \
       const int keep = tile_dma(j);                                                                      \
-      if constexpr (kIsBf16) TT_P128_RUN_STEP(TT_P128_STEP_BF16_U##U##_K0);                              \
-      else TT_P128_RUN_STEP(TT_P128_STEP_F16_U##U##_K0);                                                 \
-      settle_fast(sB, pBv);                                                                              \
-      if constexpr (kIsBf16) TT_P128_RUN_STEP(TT_P128_STEP_BF16_U##U##_K1);                              \
-      else TT_P128_RUN_STEP(TT_P128_STEP_F16_U##U##_K1);                                                 \
-      settle_fast(sC, pAv);                                                                              \
+      /* mk = 1: the tile's exponentials take the causal predicate; kvs = first key of the half whose exponentials   \
+         the step takes; kvm = kvs on such a tile, else -1.  As scalar instructions: the compiler's own form of     \
+         these selects passes through vector registers. */                                                         \
+      int mk = 0, kvs = 64 * j + 32, kvm0 = -1, kvm1 = -1;                                               \
+      if constexpr (CAUSAL)                                                                              \
+        asm("s_cmp_ge_i32 %3, %4\n\ts_cselect_b32 %0, 1, 0\n\ts_cselect_b32 %1, %5, -1\n\ts_cselect_b32 %2, %6, -1"     \
+            : "=&s"(mk), "=&s"(kvm0), "=&s"(kvm1) : "s"(j), "s"(nfast), "s"(kvs), "s"(kvs + 32) : "scc"); \
+      if constexpr (kIsBf16 && CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_BF16_U##U##_K0);                    \
+      else if constexpr (CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_F16_U##U##_K0);                           \
+      else if constexpr (kIsBf16) TT_P128_RUN_PSTEP(TT_P128_PSTEP_BF16_U##U##_K0);                       \
+      else TT_P128_RUN_PSTEP(TT_P128_PSTEP_F16_U##U##_K0);                                               \
+      settle_fast(sB, pBv, kvm0);                                                                        \
+      kvs += 32;                                                                                         \
+      if constexpr (kIsBf16 && CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_BF16_U##U##_K1);                    \
+      else if constexpr (CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_F16_U##U##_K1);                           \
+      else if constexpr (kIsBf16) TT_P128_RUN_PSTEP(TT_P128_PSTEP_BF16_U##U##_K1);                       \
+      else TT_P128_RUN_PSTEP(TT_P128_PSTEP_F16_U##U##_K1);                                               \
+      settle_fast(sC, pAv, kvm1);                                                                        \
       dma_wait_and_sync(keep);                                                                           \
       j++;                                                                                               \
     }
