@@ -320,10 +320,10 @@ __global__ __launch_bounds__(256, 1) void linear256_kernel(LinArgs a) {
     const unsigned dst = smem_addr + stage * STAGE + wave * 8192;
 #pragma unroll
     for (int i = 0; i < 8; i++)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(xoff[i]), "s"(xs), "s"(dst + 1024 * i) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(xoff[i]), "s"(xs), "s"(dst + 1024 * i) : "memory", "m0");
 #pragma unroll
     for (int i = 0; i < 8; i++)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(woff[i]), "s"(ws), "s"(dst + XTILE + 1024 * i) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(woff[i]), "s"(ws), "s"(dst + XTILE + 1024 * i) : "memory", "m0");
   };
 
   // this wavefront's part: n rows 128*wn .. of the w tile (A operand), m rows 128*wm .. of the x tile (B operand);
@@ -423,7 +423,7 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
   const unsigned ring_addr = (unsigned)(unsigned long)(lds_void_t*)ring;
 
   auto dma16 = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   // this lane's part of a load instruction: row 8i + lane/8 of a tile, slot lane%8
   unsigned woff[4], xoff[MB][4];

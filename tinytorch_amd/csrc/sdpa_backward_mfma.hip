@@ -620,10 +620,10 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
 
   // Issued as asm so that the compiler does not see stores to LDS (it would make every LDS read wait for all loads).
   auto dma16 = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   auto dma4 = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   const int drow = lane >> 4, dslot = lane & 15;  // this lane's row and slot inside a 4-row group of a load
 
@@ -912,7 +912,7 @@ __global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
   }
 
   auto dma16 = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   const int drow = lane >> 4, dslot = lane & 15;
   const T* kp = (const T*)f.k + b * f.ks[0] + hk * f.ks[1];

@@ -179,8 +179,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }
   // Issued as asm so that the compiler does not see a store to LDS: it would otherwise make every later LDS read
   // wait for all outstanding loads (vmcnt(0)).  The waits are placed by hand in dma_wait_and_sync.
+  // s_nop 3: the compiler's hazard pass does not look into the statement, and a scalar base that it restored with a
+  // vector instruction (v_readlane of a spilled scalar register, v_readfirstlane) just before is only valid for a
+  // memory instruction five wait states later; s_mov + s_nop 3 make five.
   auto dma_issue = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   const unsigned smem_addr = (unsigned)(unsigned long)(lds_void*)smem;
   // Paged cache: the table entry of a tile is fetched while the previous tile of the same stream (K or V) is issued,
@@ -516,6 +519,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     const char* qbase = (const char*)(qp + (long long)first * a.qs[2]);
     const unsigned qoff = ((unsigned)(row - first) * (unsigned)a.qs[2] + 8u * lh) * 2u;  // the host checks that 32 rows fit 32 bits
     asm volatile(
+        "s_nop 4\n\t"  // the base may have been written by a vector instruction (a restored scalar register): 5 wait states
         "global_load_dwordx4 v[120:123], %1, %2\n\t"
         "global_load_dwordx4 v[124:127], %1, %2 offset:32\n\t"
         "global_load_dwordx4 v[128:131], %1, %2 offset:64\n\t"
