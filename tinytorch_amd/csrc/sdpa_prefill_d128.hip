@@ -8,7 +8,7 @@
 // Work split.  A workgroup of 8 wavefronts owns 256 query rows of one (batch, query head), 32 rows per wavefront,
 // two wavefronts per SIMD.  Keys/values are consumed in tiles of 64 rows shared by the 8 wavefronts.
 //
-// LDS.  Four K stages and four V stages of 16 KiB, filled by direct global->LDS loads (global_load_lds_dwordx4: no
+// LDS.  Four K stages and four V stages of 16 KiB (and 32 KiB through which the output leaves: the CU's 160 KiB), filled by direct global->LDS loads (global_load_lds_dwordx4: no
 // staging registers, no ds_write).  Such a load deposits the 64 lanes' 16-byte pieces contiguously, so rows cannot
 // be padded; instead the 16-byte chunk c of tile row r is stored at chunk slot c ^ f(r), f(r) = (r%4)*4 + (r/4)%4,
 // which makes both access patterns below bank-conflict free.  The swizzle is applied on the global side (a lane
@@ -64,7 +64,8 @@ constexpr int BN = 64;   // keys per tile
 constexpr int ROW_BYTES = D * 2;
 constexpr int STAGE_BYTES = BN * ROW_BYTES;  // 16 KiB
 constexpr int KSTAGES = 4, VSTAGES = 4;     // K and V tiles are requested three tiles before use
-constexpr int LDS_BYTES = (KSTAGES + VSTAGES) * STAGE_BYTES;
+constexpr int OUT_BYTES = NW * 16 * ROW_BYTES;  // output staging: 16 rows per wavefront (the rest of the CU's 160 KiB)
+constexpr int LDS_BYTES = (KSTAGES + VSTAGES) * STAGE_BYTES + OUT_BYTES;
 constexpr float kSumLimit = 1024.f;  // a lane's 16 probabilities of a half may sum to this much before the maximum is raised
 
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
@@ -265,8 +266,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   // K runs one tile ahead of V in consumption (scores are formed two halves before their P.V), so K is requested
   // four tiles ahead and V three: iteration j sends for K(j+4) (stage of K(j), last read in iteration j-1) and
   // V(j+3) (stage of V(j-1)).  A part starts with K(0..3) and V(0..2) on their way.  For the second part they are sent
-  // for before the first part's output is written: all stages but the last V stage, which the output passes through,
-  // are free then.
+  // for before the first part's output is written: every stage is free then (all wavefronts passed the closing barrier
+  // of the last tile; the output passes through a staging area of its own).
   auto issue_tiles = [&](int part) __attribute__((always_inline)) {
     int q0, ntiles_kv;
     part_rows(part, q0, ntiles_kv);
@@ -537,10 +538,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }
   {  // P(0) and the scores of half 1
     qk_half(sC, half_base(0));
+    if (1 < my_halves) qk_half(sB, half_base(1));
     if ((CAUSAL && 31 > qc0) || 32 > S) mask_half(sC, 0);
     if (!CAUSAL && a.mask_kind != 0) user_mask_half(sC, 0);
-    settle_half(sC, pA, exp_half(sC, pA));
-    if (1 < my_halves) qk_half(sB, half_base(1));
+    // first half of a row: the maximum is formed directly (what the lazy rule arrives at after exponentials against
+    // -1e30, with nothing to rescale yet); a fully hidden half keeps -1e30 and gives zeros
+    m_use = fmaxf(m_use, row_max(sC));
+    mc = m_use * c;
+    l_run = exp_half(sC, pA);
   }
   // Every wavefront has read K(0): iteration 0 may overwrite its stage.  K(1), V(0), K(2), V(1) must be visible
   // before iteration 0; K(3) and V(2) (4 loads) are waited for at its end.
@@ -619,10 +624,10 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 
   // ---- normalise, transpose through LDS, store whole rows -----------------------------------------------------------------
   // A lane holds 4 consecutive head_dim elements per register group of its query row: stored directly, every store
-  // instruction would touch 32 rows with 16 bytes each.  Instead each wavefront stages 8 of its rows at a time in its
-  // 2 KiB slice of the last V stage and writes them out as whole 256-byte rows.  That stage is free here: all
-  // wavefronts passed the closing barrier of the last tile, and the next part sends for V(3) only in its iteration 0,
-  // two barriers from now.  16-byte chunk c of staged row r sits at chunk slot c ^ r (no bank conflicts either way).
+  // instruction would touch 32 rows with 16 bytes each.  Instead each wavefront stages 16 of its rows at a time in its
+  // 4 KiB of the staging area behind the tile stages and writes them out as whole 256-byte rows (two rounds; with 8
+  // rows in a slice of the last V stage it was four, each with its LDS round trip).  16-byte chunk c of staged row r
+  // sits at chunk slot c ^ r (no bank conflicts either way).
   {
     float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv = 1.f / l_tot;
@@ -636,24 +641,29 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
         for (int i = 0; i < 4; i++) x[i] = oacc[db][4 * rg + i] * inv;
         y[db][rg] = __builtin_convertvector(x, typename TR::vec4);
       }
-    char* tbuf = smem + (KSTAGES + 3) * STAGE_BYTES + wave * 2048;
+    char* tbuf = smem + (KSTAGES + VSTAGES) * STAGE_BYTES + wave * (16 * ROW_BYTES);
     T* obase = (T*)a.out + b * a.os[0] + h * a.os[1];
-    const int rr = lq & 7;
-    const int cc = lane & 15;
+    // the lane number anew (as asm: the compiler would otherwise keep the values derived from it alive, or spilled,
+    // through the whole kernel)
+    int ln;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+    const int rr = ln & 15;
+    const int cc = ln & 15;
+    const int lho = ln >> 5;
 #pragma unroll
-    for (int r8 = 0; r8 < 4; r8++) {
-      if ((lq >> 3) == r8) {
+    for (int r16 = 0; r16 < 2; r16++) {
+      if (((ln >> 4) & 1) == r16) {
 #pragma unroll
         for (int db = 0; db < 4; db++)
 #pragma unroll
           for (int rg = 0; rg < 4; rg++)
-            *(typename TR::vec4*)(tbuf + rr * ROW_BYTES + (((4 * db + rg) ^ rr) << 4) + 8 * lh) = y[db][rg];
+            *(typename TR::vec4*)(tbuf + rr * ROW_BYTES + (((4 * db + rg) ^ rr) << 4) + 8 * lho) = y[db][rg];
       }
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
-        const int row = 4 * i + (lane >> 4);
+      for (int i = 0; i < 4; i++) {
+        const int row = 4 * i + (ln >> 4);
         vec8 v = *(const vec8*)(tbuf + row * ROW_BYTES + ((cc ^ row) << 4));
-        const int qi = qw0 + 8 * r8 + row;
+        const int qi = qw0 + 16 * r16 + row;
         if (qi < a.L) __builtin_nontemporal_store(v, (vec8*)(obase + qi * a.os[2] + 8 * cc));  // written once, not read here
       }
     }
