@@ -202,7 +202,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       if (nxt != want && kv0 + BN < S) pc[0] = nxt, pc[1] = __builtin_amdgcn_readfirstlane(table[nxt]);
     }
     const T* tile = base + toff;
-    if (kv0 + BN <= S) {
+    if (__builtin_expect(kv0 + BN <= S, 1)) {
       const char* src = (const char*)tile;
 #pragma unroll
       for (int i = 0; i < 2; i++) dma_issue(src, off[i], stage_addr + (8 * wave + 4 * i) * ROW_BYTES);
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   // Wait until at most `keep` of this wavefront's global->LDS loads are still in flight (they complete in issue
   // order), then meet the other wavefronts: what was issued before the newest `keep` loads is visible to all.
   auto dma_wait_and_sync = [&](int keep) __attribute__((always_inline)) {
-    if (keep >= 4) {
+    if (__builtin_expect(keep >= 4, 1)) {
       asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     } else if (keep >= 2) {
       asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
@@ -322,6 +322,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     nfast_all = t > nfast ? t : nfast;
   }
   if (a.mask_kind != 0) nfast = 0, nfast_all = 0;  // an attnMask is applied in the general form of a step
+  // The fast form requests its tiles without the ragged-tile case: iteration j sends for K(j+4) and V(j+3), which have to
+  // be whole tiles.
+  if (!PAGED && (S % BN) != 0) {
+    int lim = S / BN - 4;
+    lim = lim < 0 ? 0 : lim;
+    nfast_all = lim < nfast_all ? lim : nfast_all;
+    nfast = nfast_all < nfast ? nfast_all : nfast;
+  }
   if (CAUSAL) {  // scalar registers: operands of the step statements derive from them
     nfast = __builtin_amdgcn_readfirstlane(nfast);
     nfast_all = __builtin_amdgcn_readfirstlane(nfast_all);
@@ -408,7 +416,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   // probability that reaches the matrix pipe is therefore at most kSumLimit.
   const int rl = CAUSAL ? qc0 + lq - 4 * lh : 0;  // the causal predicate's lane operand: key k of a score is visible iff k - 4*(lane/32) <= rl
   auto settle_half = [&](f32x16& s, vec8 (&pb)[2], float psum, int masked_kv0 = -1) __attribute__((always_inline)) {
-    if (__builtin_amdgcn_ballot_w64(!(psum <= kSumLimit)) != 0) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(psum <= kSumLimit)) != 0, 0)) {
       // after a step whose exponentials took the causal predicate in the stream, the scores themselves are masked only
       // here (hidden scores, or what a stage held beyond the workgroup's last tile, must not enter the maximum)
       if (CAUSAL && masked_kv0 >= 0) {
@@ -553,8 +561,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 
   auto tile_dma = [&](int j) __attribute__((always_inline)) {
     int keep = 0;
-    if (j + 3 < ntiles_kv) {
-      if (j + 4 < ntiles_kv) {
+    if (__builtin_expect(j + 3 < ntiles_kv, 1)) {
+      if (__builtin_expect(j + 4 < ntiles_kv, 1)) {
         dma_k(j + 4, j & 3);
         keep = 4;
       } else {
@@ -562,6 +570,29 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       }
       dma_v(j + 3, (j + 3) & 3);
     }
+    return keep;
+  };
+  // The fast form's requests: whole tiles through two running pointers (the general form multiplies the tile number
+  // out and carries the ragged and paged cases); U = j % 4 makes the stages constants.
+  const char* kfast = (const char*)(kp + (long long)(4 * BN) * a.ks[2]);
+  const char* vfast = (const char*)(vp + (long long)(3 * BN) * a.vs[2]);
+  const long long kfast_step = (long long)BN * a.ks[2] * 2, vfast_step = (long long)BN * a.vs[2] * 2;
+  auto tile_dma_fast = [&](int j, int U) __attribute__((always_inline)) {
+    int keep = 0;
+    if (__builtin_expect(j + 3 < ntiles_kv, 1)) {
+      if (__builtin_expect(j + 4 < ntiles_kv, 1)) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) dma_issue(kfast, ld_koff[i], smem_addr + U * STAGE_BYTES + (8 * wave + 4 * i) * ROW_BYTES);
+        keep = 4;
+      } else {
+        keep = 2;
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+        dma_issue(vfast, ld_voff[i], smem_addr + (KSTAGES + ((U + 3) & 3)) * STAGE_BYTES + (8 * wave + 4 * i) * ROW_BYTES);
+    }
+    kfast += kfast_step;
+    vfast += vfast_step;
     return keep;
   };
   int j = 0;
@@ -577,9 +608,9 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     asm volatile(TT_P128_PREFETCH : "+{v[208:239]}"(ring) : "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr) : "memory");
     // Four tiles per trip so that the stage of a tile is a constant of its statement; the trip may end after any of them.
 #define TT_P128_TILE(U)                                                                                  \
-    if (j >= nfast_all) break;                                                                            \
+    if (__builtin_expect(j >= nfast_all, 0)) break;                                                       \
     {                                                                                                    \
-      const int keep = tile_dma(j);                                                                      \
+      const int keep = PAGED ? tile_dma(j) : tile_dma_fast(j, U);                                        \
       /* mk = 1: the tile's exponentials take the causal predicate; kvs = first key of the half whose exponentials   \
          the step takes; kvm = kvs on such a tile, else -1.  As scalar instructions: the compiler's own form of     \
          these selects passes through vector registers. */                                                         \
