@@ -291,7 +291,7 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, sacc[blk][r]);
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-      if (__builtin_amdgcn_ballot_w64(mloc > m_use + lazy) != 0) {
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(mloc > m_use + lazy) != 0, 0)) {
         const float m_new = fmaxf(m_use, mloc);
         const float alpha = fast_exp2((m_use - m_new) * c);
         m_use = m_new;
@@ -976,7 +976,7 @@ __global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
 #pragma unroll
       for (int r = 1; r < 16; r++) mloc = fmaxf(mloc, sacc[r]);
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-      if (__builtin_amdgcn_ballot_w64(mloc > m_use + lazy) != 0) {
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(mloc > m_use + lazy) != 0, 0)) {
         const float m_new = fmaxf(m_use, mloc);
         const float alpha = fast_exp2((m_use - m_new) * c);
         m_use = m_new;

@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
           pr[blk][r] = fast_exp2(fmaf(sacc[blk][r], c, -mc));
           psum += pr[blk][r];
         }
-      if (__builtin_amdgcn_ballot_w64(!(psum <= kSumLimit)) != 0) {  // some row of the wavefront outgrew its maximum
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(psum <= kSumLimit)) != 0, 0)) {  // some row of the wavefront outgrew its maximum
         float mloc = sacc[0][0];
 #pragma unroll
         for (int blk = 0; blk < 2; blk++)
