@@ -12,7 +12,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "tinytorch_amd", "csrc")
-SOURCES = ["sdpa_prefill_d128.hip", "sdpa_backward_mfma.hip", "linear.hip"]
+SOURCES = ["sdpa_prefill_d128.hip", "sdpa_prefill_d64.hip", "sdpa_backward_mfma.hip", "linear.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
@@ -26,7 +26,7 @@ def listing(src, out):
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
 def test_no_scalar_restore_hazard_before_asm_memory_instructions(tmp_path):
     outs = [str(tmp_path / (s + ".s")) for s in SOURCES]
-    with ThreadPoolExecutor(max_workers=3) as pool:
+    with ThreadPoolExecutor(max_workers=4) as pool:
         results = list(pool.map(lambda p: listing(*p), zip(SOURCES, outs)))
     for src, r in zip(SOURCES, results):
         assert r.returncode == 0, "%s did not compile:\n%s" % (src, r.stderr[-2000:])

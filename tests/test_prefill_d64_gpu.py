@@ -1,0 +1,89 @@
+"""The pipelined prefill kernel at head_dim 64 (csrc/sdpa_prefill_d64.hip) against the oracle: it takes calls without an
+attnMask or pages that fill the chip with 256-row workgroups, so its cases are larger than the other parity tests'
+(B * Hq * row tiles >= 256).  Smaller head_dim-64 calls keep running on the 4-wavefront kernel and are covered in
+test_parity_gpu.py; both kernels must agree with the oracle on the same inputs."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import TOL, call, make_inputs, max_abs_err, route_of, to_host_f32
+
+pytestmark = pytest.mark.gpu
+
+
+def sampled_rows_err(out_dev, host, causal, rows, align="top-left", kv_len=None):
+    """max-abs-error of the sampled (batch, head) slices against the oracle"""
+    q, k, v = host
+    B, Hq, L, D = q.shape
+    G = Hq // k.shape[1]
+    y = to_host_f32(out_dev)
+    worst = 0.0
+    for b, h in rows:
+        S = k.shape[2] if kv_len is None else int(kv_len[b])
+        kk, vv = k[b:b + 1, h // G:h // G + 1, :S], v[b:b + 1, h // G:h // G + 1, :S]
+        if align == "bottom-right" and causal:
+            i = np.arange(L)[:, None]
+            j = np.arange(S)[None, :]
+            mask = j <= i + max(0, S - L)
+            exp = oracle.sdpa_f32(q[b:b + 1, h:h + 1], kk, vv, causal=False, mask=mask)
+        else:
+            exp = oracle.sdpa_f32(q[b:b + 1, h:h + 1], kk, vv, causal=causal)
+        got = y[b:b + 1, h:h + 1]
+        assert np.isfinite(got).all()
+        worst = max(worst, float(np.abs(got.astype(np.float64) - exp.astype(np.float64)).max()))
+    return worst
+
+
+ROWS = [(0, 0), (0, 5), (1, 17), (1, 63), (3, 31)]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("causal,L,S", [(True, 500, 500), (True, 769, 769), (False, 320, 411), (False, 257, 64)])
+def test_head_dim_64_pipelined_against_oracle(dtype, causal, L, S):
+    B, Hq, Hkv, D = 4, 64, 16, 64
+    host, dev = make_inputs(640 + L, B, Hq, Hkv, L, S, D, dtype, 0.8)
+    assert route_of(*dev, causal=causal) == "prefill"
+    rc, out = call("forward", *dev, causal=causal)
+    assert rc == 0
+    assert sampled_rows_err(out, host, causal, ROWS) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_head_dim_64_pipelined_bottom_right_and_key_counts(dtype):
+    B, Hq, Hkv, L, S, D = 4, 64, 64, 300, 700, 64
+    host, dev = make_inputs(777, B, Hq, Hkv, L, S, D, dtype, 0.8)
+    rc, out = call("forward", *dev, causal=True, align="bottom-right")
+    assert rc == 0
+    assert sampled_rows_err(out, host, True, ROWS, align="bottom-right") <= TOL[dtype]
+    lens = np.array([700, 333, 64, 1], np.int32)
+    rc, out = call("forward", *dev, causal=False, kv_lens=torch.from_numpy(lens).cuda())
+    assert rc == 0
+    assert sampled_rows_err(out, host, False, ROWS, kv_len=lens) <= TOL[dtype]
+    rc, out = call("forward", *dev, causal=True, align="bottom-right", kv_lens=torch.from_numpy(lens).cuda())
+    assert rc == 0
+    assert sampled_rows_err(out, host, True, ROWS, align="bottom-right", kv_len=lens) <= TOL[dtype]
+
+
+def test_head_dim_64_pipelined_equals_the_4_wavefront_kernel_within_rounding():
+    # the same call through both kernels: a batch that fills the chip, and the same heads one batch entry at a time
+    # (which stays under the 256-workgroup bar and runs on the 4-wavefront kernel)
+    B, Hq, Hkv, L, S, D = 4, 64, 16, 512, 512, 64
+    host, dev = make_inputs(4242, B, Hq, Hkv, L, S, D, "bf16", 0.8)
+    rc, big = call("forward", *dev, causal=True)
+    assert rc == 0
+    rc, one = call("forward", dev[0][:1].contiguous(), dev[1][:1].contiguous(), dev[2][:1].contiguous(), causal=True)
+    assert rc == 0
+    d = (big[:1].float() - one.float()).abs().max().item()
+    assert d <= 2e-2
+    # causal row 0 is v[0] exactly on both
+    assert torch.equal(big[:, :, 0, :], dev[2][:, :, 0, :].repeat_interleave(Hq // Hkv, dim=1))
+
+
+def test_large_score_range_head_dim_64_pipelined():
+    # scores far apart: the lazily raised maximum must not lose the small probabilities nor overflow the large ones
+    B, Hq, Hkv, L, S, D = 4, 64, 16, 300, 300, 64
+    host, dev = make_inputs(99, B, Hq, Hkv, L, S, D, "bf16", 6.0)
+    rc, out = call("forward", *dev, causal=True)
+    assert rc == 0
+    assert sampled_rows_err(out, host, True, ROWS) <= 0.12

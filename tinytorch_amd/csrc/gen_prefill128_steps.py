@@ -2,7 +2,8 @@
 """Writes prefill128_steps.inc: the hand-ordered instruction streams of the pipelined prefill kernel's steady state
 (sdpa_prefill_d128.hip), one string per (tile of the 4-tile unrolled body, step of the tile, element type).
 
-    python3 gen_prefill128_steps.py > prefill128_steps.inc
+    python3 gen_prefill128_steps.py > prefill128_steps.inc         (head_dim 128, sdpa_prefill_d128.hip)
+    python3 gen_prefill128_steps.py 64 > prefill64_steps.inc       (head_dim 64, sdpa_prefill_d64.hip)
 
 A step is 16 slots, one matrix instruction each (even slot: S^T k-step, odd slot: P.V product), with the vector work
 of one score (scale/shift, exp2, running sum, conversion of a pair) spread over the slots so that no instruction
@@ -29,8 +30,22 @@ of line, in subsection 1 of the kernel's section, so that the steady state falls
 import sys
 
 PD, RING = 6, 8
-STAGE, ROW = 16384, 256
 Q0, VADDR0, SB0, SC0, PA0, PB0, RING0, T0, KADDR0 = 120, 152, 160, 176, 192, 200, 208, 240, 248
+# set by configure(head_dim): k-steps of a score product (= P.V products of a half), head_dim blocks of 32, slots of a
+# step, scores whose vector work a slot carries, bytes of a tile row and of a stage, slots of the 4-tile body
+KST = NDB = NS = SPS = ROW = STAGE = BODY = 0
+NAME = ""
+
+
+def configure(head_dim):
+    global KST, NDB, NS, SPS, ROW, STAGE, BODY, NAME
+    KST, NDB = head_dim // 16, head_dim // 32
+    NS = 2 * KST
+    SPS = 16 // NS
+    ROW = 2 * head_dim
+    STAGE = 64 * ROW
+    BODY = 8 * NS
+    NAME = "P%d" % head_dim
 
 
 def vr(lo, n=1):
@@ -38,14 +53,14 @@ def vr(lo, n=1):
 
 
 def fetch(G):
-    """LDS operand request of slot G of the 128-slot body into its ring place."""
-    G &= 127
-    u, kind, s = (G >> 5) & 3, (G >> 4) & 1, G & 15
+    """LDS operand request of slot G of the 4-tile body into its ring place."""
+    G %= BODY
+    u, kind, s = G // (2 * NS), (G // NS) % 2, G % NS
     i, r = s >> 1, RING0 + 4 * (G % RING)
     if s % 2 == 0:  # K rows of half `kind` of tile u+1, k-step i
         off = ((u + 1) & 3) * STAGE + kind * 32 * ROW
         return ["ds_read_b128 %s, %s offset:%d" % (vr(r, 4), vr(KADDR0 + i), off)]
-    t, db = i >> 2, i & 3  # V^T of half `kind` of tile u, keys 16t..16t+15, head_dim block db
+    t, db = i // NDB, i % NDB  # V^T of half `kind` of tile u, keys 16t..16t+15, head_dim block db
     off = u * STAGE + kind * 32 * ROW + 16 * t * ROW
     return ["ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(r, 2), vr(VADDR0 + 2 * db), off),
             "ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(r + 2, 2), vr(VADDR0 + 2 * db + 1), off)]
@@ -59,7 +74,7 @@ def pending_after(G):
 def step(u, kind, elem, masked=False):
     mfma = "v_mfma_f32_32x32x16_%s" % elem
     cvt = "v_cvt_pk_%s_f32" % elem
-    G0 = 32 * u + 16 * kind
+    G0 = 2 * NS * u + NS * kind
     s_new, s_nxt = (SC0, SB0) if kind == 0 else (SB0, SC0)
     p_cur, p_nxt = (PA0, PB0) if kind == 0 else (PB0, PA0)
     F = [T0 + 4, T0 + 5]
@@ -71,8 +86,23 @@ def step(u, kind, elem, masked=False):
         return ["s_add_i32 m0, %%[kvs], %d" % (8 * (n >> 2) + (n & 3)), "v_cmp_le_i32 vcc, m0, %[rl]",
                 "v_cndmask_b32 %s, 0, %s, vcc" % (vr(T[n & 3]), vr(T[n & 3]))]
 
+    def vector_work(n):  # of score n: its exp2, the next score's scale/shift, the previous score's add, a pair's conversion
+        w = ["v_exp_f32 %s, %s" % (vr(T[n & 3]), vr(F[n & 1]))]
+        if n + 1 < 16:
+            w.append(fma(n + 1))
+        if masked:
+            w += hide(n)
+        if n == 2:  # the sum starts as (score 0) + (score 1): what 0 + x0 + x1 gives
+            w.append("v_add_f32 %%[ps], %s, %s" % (vr(T[0]), vr(T[1])))
+        elif n >= 3:
+            w.append("v_add_f32 %%[ps], %%[ps], %s" % vr(T[(n - 1) & 3]))
+        if n % 2 == 0 and n >= 2:
+            j = (n - 2) // 2  # scores n-2, n-1
+            w.append("%s %s, %s, %s" % (cvt, vr(p_nxt + j), vr(T[(n - 2) & 3]), vr(T[(n - 1) & 3])))
+        return w
+
     out.append(fma(0))
-    for n in range(16):
+    for n in range(NS):
         G = G0 + n
         r = RING0 + 4 * (G % RING)
         out.append("s_waitcnt lgkmcnt(%d)" % pending_after(G))
@@ -82,20 +112,10 @@ def step(u, kind, elem, masked=False):
             out.append("%s %s, %s, %s, %s" % (mfma, vr(s_new, 16), vr(r, 4), vr(Q0 + 4 * ks, 4), c))
         else:
             i = n // 2
-            out.append("%s %%[o%d], %s, %s, %%[o%d]" % (mfma, i & 3, vr(r, 4), vr(p_cur + 4 * (i >> 2), 4), i & 3))
+            out.append("%s %%[o%d], %s, %s, %%[o%d]" % (mfma, i % NDB, vr(r, 4), vr(p_cur + 4 * (i // NDB), 4), i % NDB))
         out += fetch(G + PD)  # directly behind the matrix instruction: measured 0.7% faster than behind the vector work
-        out.append("v_exp_f32 %s, %s" % (vr(T[n & 3]), vr(F[n & 1])))
-        if n + 1 < 16:
-            out.append(fma(n + 1))
-        if masked:
-            out += hide(n)
-        if n == 2:  # the sum starts as (score 0) + (score 1): what 0 + x0 + x1 gives
-            out.append("v_add_f32 %%[ps], %s, %s" % (vr(T[0]), vr(T[1])))
-        elif n >= 3:
-            out.append("v_add_f32 %%[ps], %%[ps], %s" % vr(T[(n - 1) & 3]))
-        if n % 2 == 0 and n >= 2:
-            j = (n - 2) // 2  # scores n-2, n-1
-            out.append("%s %s, %s, %s" % (cvt, vr(p_nxt + j), vr(T[(n - 2) & 3]), vr(T[(n - 1) & 3])))
+        for q in range(SPS * n, SPS * (n + 1)):
+            out += vector_work(q)
     if not masked:
         out.append("s_nop 0")
     out.append("v_add_f32 %%[ps], %%[ps], %s" % vr(T[15 & 3]))
@@ -117,20 +137,25 @@ def emit(name, lines):
 
 
 def main():
-    print("// Generated by gen_prefill128_steps.py; do not edit.  Instruction streams of the pipelined prefill kernel's")
-    print("// steady state: TT_P128_STEP_<elem>_U<tile of the unrolled body>_K<step of the tile> (with the causal variant out of")
-    print("// line), TT_P128_PSTEP_... the plain step alone.")
+    head_dim = 128
+    if len(sys.argv) > 1:
+        head_dim = int(sys.argv[1])
+    configure(head_dim)
+    lab = ".Ltt_%s" % NAME.lower()
+    print("// Generated by gen_prefill128_steps.py%s; do not edit.  Instruction streams of the pipelined prefill kernel's" % ("" if head_dim == 128 else " %d" % head_dim))
+    print("// steady state: TT_%s_STEP_<elem>_U<tile of the unrolled body>_K<step of the tile> (with the causal variant out of" % NAME)
+    print("// line), TT_%s_PSTEP_... the plain step alone." % NAME)
     print()
-    emit("TT_P128_PREFETCH", prefetch())
+    emit("TT_%s_PREFETCH" % NAME, prefetch())
     for elem in ("bf16", "f16"):
         for u in range(4):
             for kind in range(2):
                 # the variant with the causal predicate sits out of line (at the end of the kernel's section), so that the
                 # steady state runs through without a taken branch
-                both = (["s_cmp_eq_u32 %[mk], 0", "s_cbranch_scc0 .Ltt_p128_m%="] + step(u, kind, elem) + [".Ltt_p128_e%=:", ".subsection 1", ".Ltt_p128_m%=:"]
-                        + step(u, kind, elem, True) + ["s_branch .Ltt_p128_e%=", ".subsection 0"])
-                emit("TT_P128_STEP_%s_U%d_K%d" % (elem.upper(), u, kind), both)
-                emit("TT_P128_PSTEP_%s_U%d_K%d" % (elem.upper(), u, kind), step(u, kind, elem))  # calls without a causal mask
+                both = (["s_cmp_eq_u32 %[mk], 0", "s_cbranch_scc0 %s_m%%=" % lab] + step(u, kind, elem) + ["%s_e%%=:" % lab, ".subsection 1", "%s_m%%=:" % lab]
+                        + step(u, kind, elem, True) + ["s_branch %s_e%%=" % lab, ".subsection 0"])
+                emit("TT_%s_STEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), both)
+                emit("TT_%s_PSTEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), step(u, kind, elem))  # calls without a causal mask
 
 
 if __name__ == "__main__":

@@ -287,6 +287,7 @@ __device__ __forceinline__ int keys_of_batch(const KArgs& f, int b) {
 int launch_general(const KArgs& a, int dtype, hipStream_t stream);
 int launch_prefill(const KArgs& a, int dtype, hipStream_t stream);       // 128-row workgroups; head_dim 64 or 128
 int launch_prefill_d128(const KArgs& a, int dtype, hipStream_t stream);  // 256-row workgroups, pipelined; head_dim 128
+int launch_prefill_d64(const KArgs& a, int dtype, hipStream_t stream);   // the same at head_dim 64 (no attnMask, no pages)
 int launch_prefill_f32(const KArgs& a, hipStream_t stream);              // fp32 tensors on the fp32 matrix cores; head_dim 64 or 128
 int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream);
 // combines per-split records [pair][split][row][D + 2] (pair = batch * Hkv + kv head, row = l * G + g) into a.out

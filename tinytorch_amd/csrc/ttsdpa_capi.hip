@@ -123,6 +123,15 @@ bool pipelined_ok(const ttsdpa_params* p) {
   return p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22);
 }
 
+// The pipelined kernel at head_dim 64: no attnMask, no pages, and enough 256-row workgroups to fill the chip (smaller
+// calls stay on the 4-wavefront kernel, which has 128-row tiles and can divide the keys among workgroups).
+bool pipelined64_ok(const ttsdpa_params* p) {
+  if (p->D != 64 || p->L <= 128 || p->mask_kind != TTSDPA_MASK_NONE || p->block_table) return false;
+  if (!(p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22))) return false;
+  const long long tiles = (p->L + 255) / 256;
+  return (long long)p->B * p->Hq * (p->causal ? (tiles + 1) / 2 : tiles) >= 256;
+}
+
 // Few query rows per head against many keys on the 4-wavefront kernel: the G heads of a KV head share one row tile
 // (dense q / out make [B,Hq,L,D] a [B,Hkv,G*L,D] tensor), so K/V are streamed once per KV head instead of once per
 // query head and the tile is not mostly padding.
@@ -392,6 +401,7 @@ static int prefill_impl(const ttsdpa_params* p, void* workspace, size_t workspac
   // head_dim 128 with enough rows to fill 256-row workgroups takes the software-pipelined kernel (its tile loads
   // address 64 rows with 32-bit byte offsets)
   if (p->dtype != TTSDPA_F32 && pipelined_ok(p)) return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
+  if (p->dtype != TTSDPA_F32 && pipelined64_ok(p)) return launch_prefill_d64(a, p->dtype, (hipStream_t)stream);
   auto launch = [&](const KArgs& k) {
     return p->dtype == TTSDPA_F32 ? launch_prefill_f32(k, (hipStream_t)stream) : launch_prefill(k, p->dtype, (hipStream_t)stream);
   };
