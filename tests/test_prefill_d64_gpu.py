@@ -87,3 +87,50 @@ def test_large_score_range_head_dim_64_pipelined():
     rc, out = call("forward", *dev, causal=True)
     assert rc == 0
     assert sampled_rows_err(out, host, True, ROWS) <= 0.12
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("S", [1, 31, 33, 65, 130, 191])
+def test_head_dim_64_pipelined_few_keys(causal, S):
+    # fewer keys than the ring of tiles holds, down to one: ragged first tile, no steady state at all
+    B, Hq, Hkv, L, D = 8, 32, 8, 200, 64
+    host, dev = make_inputs(900 + S, B, Hq, Hkv, L, S, D, "bf16", 0.8)
+    assert route_of(*dev, causal=causal) == "prefill"
+    rc, out = call("forward", *dev, causal=causal)
+    assert rc == 0
+    rows = [(0, 0), (3, 9), (7, 31)]
+    assert sampled_rows_err(out, host, causal, rows) <= TOL["bf16"]
+
+
+def test_head_dim_64_pipelined_empty_cache_entries_give_zeros():
+    B, Hq, Hkv, L, S, D = 8, 32, 8, 200, 96, 64
+    host, dev = make_inputs(31337, B, Hq, Hkv, L, S, D, "bf16", 0.8)
+    lens = np.array([96, 0, 5, 0, 64, 65, 0, 96], np.int32)
+    out = torch.full(dev[0].shape, 7.0, dtype=dev[0].dtype, device="cuda")
+    rc, out = call("forward", *dev, causal=False, kv_lens=torch.from_numpy(lens).cuda(), out=out)
+    assert rc == 0
+    for b in (1, 3, 6):
+        assert torch.count_nonzero(out[b]).item() == 0
+    assert sampled_rows_err(out, host, False, [(0, 0), (2, 7), (4, 30), (5, 1), (7, 31)], kv_len=lens) <= TOL["bf16"]
+
+
+def test_head_dim_64_pipelined_strided_views_equal_contiguous_bitwise():
+    # q, k, v as views of one packed [B, L, 3, H, D] projection output: only the row stride differs
+    B, H, L, D = 4, 64, 300, 64
+    host, dev = make_inputs(2024, B, H, H, L, L, D, "f16", 0.8)
+    packed = torch.empty(B, L, 3, H, D, dtype=dev[0].dtype, device="cuda")
+    for i in range(3):
+        packed[:, :, i] = dev[i].permute(0, 2, 1, 3)
+    views = [packed[:, :, i].permute(0, 2, 1, 3) for i in range(3)]
+    assert not views[0].is_contiguous()
+    assert route_of(*views, causal=True) == "prefill"
+    rc, a = call("forward", *dev, causal=True)
+    assert rc == 0
+    rc, b = call("forward", *views, causal=True)
+    assert rc == 0
+    assert torch.equal(a, b)
+    # and into a strided output
+    outp = torch.zeros(B, L, H, D, dtype=dev[0].dtype, device="cuda")
+    rc, c = call("forward", *views, causal=True, out=outp.permute(0, 2, 1, 3))
+    assert rc == 0
+    assert torch.equal(a, outp.permute(0, 2, 1, 3))
