@@ -282,6 +282,34 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
   issue_tiles(0);
   u32x32 qv;  // the lane's Q operands, k-step ks in elements 4ks .. 4ks+3
+  // Q of a part into its registers, and everything sent for so far in place.  One statement: the compiler takes a statement's
+  // results as valid when it ends, so the wait has to be part of it (and, not knowing of the tile loads, the compiler
+  // would place waits of its own for plain loads that in effect wait for every tile).
+  auto load_q = [&](int part) __attribute__((always_inline)) {
+    int q0, ntiles_kv;
+    part_rows(part, q0, ntiles_kv);
+    const int qw0 = q0 + rowgroup * WM;
+    const int first = qw0 < a.L ? qw0 : a.L - 1;  // rows past the end re-read the last row (never stored)
+    int row = qw0 + lq;
+    row = row < a.L ? row : a.L - 1;
+    const char* qbase = (const char*)(qp + (long long)first * a.qs[2]);
+    const unsigned qoff = ((unsigned)(row - first) * (unsigned)a.qs[2] + 8u * lh) * 2u;  // the host checks that 32 rows fit 32 bits
+    asm volatile(
+        "s_nop 4\n\t"  // the base may have been written by a vector instruction (a restored scalar register): 5 wait states
+        "global_load_dwordx4 v[120:123], %1, %2\n\t"
+        "global_load_dwordx4 v[124:127], %1, %2 offset:32\n\t"
+        "global_load_dwordx4 v[128:131], %1, %2 offset:64\n\t"
+        "global_load_dwordx4 v[132:135], %1, %2 offset:96\n\t"
+        "global_load_dwordx4 v[136:139], %1, %2 offset:128\n\t"
+        "global_load_dwordx4 v[140:143], %1, %2 offset:160\n\t"
+        "global_load_dwordx4 v[144:147], %1, %2 offset:192\n\t"
+        "global_load_dwordx4 v[148:151], %1, %2 offset:224\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "={v[120:151]}"(qv)
+        : "v"(qoff), "s"(qbase)
+        : "memory");
+  };
+  load_q(0);
 
 
   for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
@@ -518,32 +546,9 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       for (int i = 0; i < 4; i++) pv[4 * t + i] = w[i];
     }
   };
-  // Q into its registers, and everything sent for so far in place.  One statement: the compiler takes a statement's
-  // results as valid when it ends, so the wait has to be part of it (and, not knowing of the tile loads, the compiler
-  // would place waits of its own for plain loads that in effect wait for every tile).
-  {
-    const int first = qw0 < a.L ? qw0 : a.L - 1;  // rows past the end re-read the last row (never stored)
-    int row = qw0 + lq;
-    row = row < a.L ? row : a.L - 1;
-    const char* qbase = (const char*)(qp + (long long)first * a.qs[2]);
-    const unsigned qoff = ((unsigned)(row - first) * (unsigned)a.qs[2] + 8u * lh) * 2u;  // the host checks that 32 rows fit 32 bits
-    asm volatile(
-        "s_nop 4\n\t"  // the base may have been written by a vector instruction (a restored scalar register): 5 wait states
-        "global_load_dwordx4 v[120:123], %1, %2\n\t"
-        "global_load_dwordx4 v[124:127], %1, %2 offset:32\n\t"
-        "global_load_dwordx4 v[128:131], %1, %2 offset:64\n\t"
-        "global_load_dwordx4 v[132:135], %1, %2 offset:96\n\t"
-        "global_load_dwordx4 v[136:139], %1, %2 offset:128\n\t"
-        "global_load_dwordx4 v[140:143], %1, %2 offset:160\n\t"
-        "global_load_dwordx4 v[144:147], %1, %2 offset:192\n\t"
-        "global_load_dwordx4 v[148:151], %1, %2 offset:224\n\t"
-        "s_waitcnt vmcnt(0)"
-        : "={v[120:151]}"(qv)
-        : "v"(qoff), "s"(qbase)
-        : "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-  }
+  // every wavefront's waits for the part's first tiles (in load_q) are behind it: the tiles are visible to all
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
   {  // P(0) and the scores of half 1
     qk_half(sC, half_base(0));
     if (1 < my_halves) qk_half(sB, half_base(1));
@@ -557,7 +562,12 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }
   // Every wavefront has read K(0): iteration 0 may overwrite its stage.  K(1), V(0), K(2), V(1) must be visible
   // before iteration 0; K(3) and V(2) (4 loads) are waited for at its end.
-  dma_wait_and_sync(0);
+  if (CAUSAL && part == 1) {  // all of this part's loads so far were waited for in load_q; what is in flight are part 0's output stores
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  } else {
+    dma_wait_and_sync(0);
+  }
 
   auto tile_dma = [&](int j) __attribute__((always_inline)) {
     int keep = 0;
@@ -651,7 +661,10 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     dma_wait_and_sync(keep);
   }
 
-  if (CAUSAL && part == 0 && two_parts) issue_tiles(1);
+  if (CAUSAL && part == 0 && two_parts) {
+    issue_tiles(1);
+    load_q(1);
+  }
 
   // ---- normalise, transpose through LDS, store whole rows -----------------------------------------------------------------
   // A lane holds 4 consecutive head_dim elements per register group of its query row: stored directly, every store
