@@ -652,6 +652,9 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
 #pragma unroll
       for (int rg = 0; rg < 4; rg++)
         *(typename TR::vec4*)(tbuf + rr * ROW_BYTES + (((4 * db + rg) ^ (rr & 7)) << 4) + 8 * lho) = y[db][rg];
+    // the reads below fetch what other lanes of the wavefront wrote: keep the compiler from relating them to this lane's
+    // own accesses.  The LDS runs a wavefront's instructions in order; nothing else is needed.
+    asm volatile("" ::: "memory");
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int row = 8 * i + (ln >> 3);
