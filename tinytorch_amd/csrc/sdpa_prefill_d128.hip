@@ -704,7 +704,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
             *(typename TR::vec4*)(tbuf + rr * ROW_BYTES + (((4 * db + rg) ^ rr) << 4) + 8 * lho) = y[db][rg];
       }
       // the reads below fetch what OTHER lanes of the wavefront wrote: without this the compiler may take a lane that
-      // wrote nothing in this round to read what it read in the last one (seen: the second round's reads issued only
+      // wrote nothing in this pass to read what it read in the pass before (seen: the second pass's reads issued only
       // for the writing lanes).  The LDS runs a wavefront's instructions in order; nothing else is needed.
       asm volatile("" ::: "memory");
 #pragma unroll
