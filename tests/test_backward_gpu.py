@@ -280,6 +280,72 @@ def test_backward_split_query_stream(dtype, D, mode):
         check(name, host, dev, dtype, causal=(mode == "causal"), route="prefill")
 
 
+@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64), ("f16", 128), ("bf16", 64)])
+@pytest.mark.parametrize("mode", ["causal", "full", "br-kvlen", "mask", "hiddenrow"])
+def test_backward_split_key_ranges(dtype, D, mode):
+    """16-bit matrix-core pairs with few query blocks and many keys: the dq kernel deals the key range of every 128-row
+    query block out to several workgroups (here eight: 8 query blocks, 2100 keys) and a merge kernel brings their fp32
+    partial sums to the common maximum.  The scratch the library asks for holds the partial records."""
+    B, Hq, Hkv, L, S = 1, 4, 2, 200, 2100
+    host, dev = make_inputs(4900 + D, B, Hq, Hkv, L, S, D, dtype)
+    q, k, v = dev
+    go = upstream(9, q.shape, dtype)[1]
+    bp = build_backward_params(q, k, v, torch.empty_like(q), go, torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+                               mode == "causal")
+    assert _capi.lib().ttsdpa_backward_workspace_bytes(ctypes.byref(bp)) >= B * Hq * L * 8 + 4 * B * Hq * L * (D + 2) * 4
+    name = "ksplit-%s-%s-%d" % (mode, dtype, D)
+    if mode == "br-kvlen":
+        # one query chunk at the end of 1500 valid keys of 2100; the oracle sees the alignment and the count as a Bool mask
+        n = 1500
+        kv = torch.tensor([n], dtype=torch.int32, device="cuda")
+        m = np.zeros((B, 1, L, S), dtype=bool)
+        m[0, 0] = np.arange(S)[None, :] <= np.arange(L)[:, None] + (n - L)
+        m[0, 0, :, n:] = False
+        check(name, host, dev, dtype, causal=True, kv_lens=kv, align="bottom-right", oracle_mask=m, route="prefill")
+    elif mode == "mask":
+        m = np.random.default_rng(8).random((Hq, L, S)) < 0.5
+        m[..., 7] = True
+        check(name, host, dev, dtype, mask_h=m, mask_d=torch.from_numpy(m).cuda(), route="prefill")
+    elif mode == "hiddenrow":
+        # rows whose keys are all hidden in some splits (keys 0..599 only) and one hidden in every split: dq = 0 there
+        m = np.random.default_rng(9).random((L, S)) < 0.5
+        m[:, 7] = True
+        m[10:20, 600:] = False
+        m[5, :] = False
+        md = torch.from_numpy(m).cuda()
+        go_h, go = upstream(9, q.shape, dtype)
+        rc, out = call("forward", q, k, v, mask=md)
+        assert rc == 0
+        out = torch.nan_to_num(out)
+        rc, (dq, dk, dv) = backward_call(q, k, v, out, go, mask=md)
+        assert rc == 0 and torch.all(dq[:, :, 5] == 0)
+        keep = np.ones(L, bool)
+        keep[5] = False
+        eq, ek, ev = oracle.sdpa_backward_f32(host[0][:, :, keep], host[1], host[2], go_h[:, :, keep], mask=m[keep])
+        assert grad_err(dq[:, :, torch.from_numpy(keep).cuda()], eq) <= TOL[dtype]
+        assert grad_err(dk, ek) <= TOL[dtype] and grad_err(dv, ev) <= TOL[dtype]
+    else:
+        check(name, host, dev, dtype, causal=(mode == "causal"), route="prefill")
+
+
+def test_backward_split_key_ranges_with_empty_pieces_and_entries():
+    """More splits than some query blocks have tiles (causal: the first block sees 128 keys, i.e. four 32-key tiles, dealt
+    out to eight workgroups), and a batch entry without keys (dq = 0 from the merge kernel, dk = dv = 0)."""
+    B, Hq, Hkv, L, S, D = 2, 1, 1, 4200, 4200, 128
+    dtype = "bf16"
+    host, dev = make_inputs(5151, B, Hq, Hkv, L, S, D, dtype)
+    q, k, v = dev
+    go_h, go = upstream(3, q.shape, dtype)
+    kv = torch.tensor([S, 0], dtype=torch.int32, device="cuda")
+    rc, out = call("forward", q, k, v, causal=True, kv_lens=kv)
+    assert rc == 0
+    rc, (dq, dk, dv) = backward_call(q, k, v, out, go, True, None, None, kv)
+    assert rc == 0
+    assert torch.count_nonzero(dq[1]).item() == 0 and torch.count_nonzero(dk[1]).item() == 0 and torch.count_nonzero(dv[1]).item() == 0
+    eq, ek, ev = oracle.sdpa_backward_f32(host[0][:1], host[1][:1], host[2][:1], go_h[:1], causal=True, nthreads=8)
+    assert grad_err(dq[:1], eq) <= TOL[dtype] and grad_err(dk[:1], ek) <= TOL[dtype] and grad_err(dv[:1], ev) <= TOL[dtype]
+
+
 def test_backward_strided_views_and_scale():
     """q/k/v as slices of one packed projection output, gradients into slices of one packed buffer."""
     B, H, N, D = 2, 4, 40, 64

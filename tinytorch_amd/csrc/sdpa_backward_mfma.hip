@@ -22,7 +22,8 @@
 // Seven matrix products in all, against five in the textbook count (the scores are computed in both kernels).
 // When a call has too few key blocks to fill and balance the chip, the query stream of a key block is dealt out to 2-4
 // workgroups of kernel 2, which leave fp32 partial sums in scratch, and backward_dkv_sum_kernel (sdpa_common.h) adds
-// them in a fixed order.
+// them in a fixed order.  Likewise kernel 1: with fewer than 512 query blocks the key range of a block is dealt out to
+// 2-8 workgroups, whose unnormalised fp32 sums and (maximum, sum of exponentials) backward_dq_merge_kernel combines.
 
 #include "sdpa_common.h"
 
@@ -122,6 +123,29 @@ __device__ __forceinline__ vec8 regs_to_operand(const f32x16& acc, int t) {
   return __builtin_convertvector(x, vec8);
 }
 
+// A lane's share of a query row's unnormalised dq sums (accumulator layout as above) and the row's (maximum in log2
+// units, sum of exponentials) as this split's partial record; split 0 also leaves delta for the dk/dv kernel.
+template <int D>
+__device__ __forceinline__ void store_dq_partial(const BwdArgs& a, int piece, long long row_id, int lh, const f32x16 (&dqacc)[D / 32],
+                                                 float mc, float l_tot, float delta) {
+  const long long rows = (long long)a.f.B * a.f.Hq * a.f.L;
+  float* dst = a.dq_partial + (piece * rows + row_id) * D;
+#pragma unroll
+  for (int db = 0; db < D / 32; db++)
+#pragma unroll
+    for (int rg = 0; rg < 4; rg++) {
+      f32x4 x;
+#pragma unroll
+      for (int i = 0; i < 4; i++) x[i] = dqacc[db][4 * rg + i];
+      *(f32x4*)(dst + 32 * db + 8 * rg + 4 * lh) = x;
+    }
+  if (lh == 0) {
+    float* ml = a.dq_partial + a.dq_splits * rows * D;
+    *(float2*)(ml + 2 * (piece * rows + row_id)) = make_float2(mc, l_tot);
+    if (piece == 0) a.stats[2 * row_id + 1] = delta;
+  }
+}
+
 // ---- kernel 1: dq, lse, delta ----------------------------------------------------------------------------------------
 // BN: keys per streamed tile.  64 for head_dim 64; 32 for head_dim 128, which keeps a wavefront under 256 registers:
 // two wavefronts per SIMD (one's vector work overlaps the other's matrix work), accumulators in ordinary registers.
@@ -147,8 +171,12 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
   const int lq = lane & 31, lh = lane >> 5;
 
   const int ntile = (f.L + BM - 1) / BM;
-  int pair, in;
-  map_workgroup(blockIdx.x, f.B * f.Hq, ntile, &pair, &in);
+  int pair, in, piece;  // piece: this workgroup's share of the row block's key range (dq_splits > 1)
+  {
+    int n;
+    split_of_workgroup(blockIdx.x, a.dq_splits, f.B * f.Hq, &n, &piece);
+    map_workgroup(n, f.B * f.Hq, ntile, &pair, &in);
+  }
   const int h = pair % f.Hq, b = pair / f.Hq;
   const int hk = h / f.G;
   const int rt = CAUSAL ? ntile - 1 - in : in;  // longest rows first
@@ -190,6 +218,7 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
 
   const int S = keys_of_batch(f, b);
   if (S == 0) {  // no keys (an empty cache entry): the output did not depend on q
+    if (a.dq_splits > 1) return;  // the merge kernel writes the zeros
     const int qi = qw0 + lq;
     if (qi < f.L) {
       T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
@@ -207,6 +236,8 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
     const int lastkv = last < S - 1 ? last : S - 1;
     ntiles_kv = lastkv / BN + 1;
   }
+  // this workgroup's tiles: all of them, or piece `piece` of dq_splits nearly equal ones (possibly none)
+  const int t0 = (int)((long long)ntiles_kv * piece / a.dq_splits), t1 = (int)((long long)ntiles_kv * (piece + 1) / a.dq_splits);
 
   // ---- global -> register -> LDS staging of one K/V tile (thread t moves 16-byte chunks t, t+256, ...) ----------------------
   u32x4 kst[NLD], vst[NLD];
@@ -240,19 +271,19 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
   const int r_lane = lq * RP + 8 * lh;
   const int t_lane = (4 * lh + ((lane & 15) >> 2)) * TP + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  if (ntiles_kv > 0) {
-    load_tile(0);
+  if (t0 < t1) {
+    load_tile(t0 * BN);
     store_tile(0);
-    if (1 < ntiles_kv) load_tile(BN);
+    if (t0 + 1 < t1) load_tile((t0 + 1) * BN);
   }
   __syncthreads();
 
-  for (int jt = 0; jt < ntiles_kv; jt++) {
+  for (int jt = t0; jt < t1; jt++) {
     const int kv0 = jt * BN;
-    const int cur = jt & 1;
-    if (jt + 1 < ntiles_kv) {
+    const int cur = (jt - t0) & 1;
+    if (jt + 1 < t1) {
       store_tile(cur ^ 1);
-      if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BN);
+      if (jt + 2 < t1) load_tile(kv0 + 2 * BN);
     }
     if (wave_live && (!CAUSAL || kv0 <= qw0 + 31 + coff)) {
       const T* Kr = smem + cur * DqTile<D>::STAGE;
@@ -340,6 +371,10 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const int qi = qw0 + lq;
+  if (a.dq_splits > 1) {
+    if (qi < f.L) store_dq_partial<D>(a, piece, ((long long)b * f.Hq + h) * f.L + qi, lh, dqacc, m_use * c, l_tot, delta);
+    return;
+  }
   if (qi < f.L) {
     const long long row_id = ((long long)b * f.Hq + h) * f.L + qi;
     // log2 of the row's sum of exponentials, the unit the second kernel's exp2 wants
@@ -853,8 +888,12 @@ __global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
   const int lq = lane & 31, lh = lane >> 5;
 
   const int ntile = (f.L + BM - 1) / BM;
-  int pair, in;
-  map_workgroup(blockIdx.x, f.B * f.Hq, ntile, &pair, &in);
+  int pair, in, piece;  // piece: this workgroup's share of the row block's key range (dq_splits > 1)
+  {
+    int n;
+    split_of_workgroup(blockIdx.x, a.dq_splits, f.B * f.Hq, &n, &piece);
+    map_workgroup(n, f.B * f.Hq, ntile, &pair, &in);
+  }
   const int h = pair % f.Hq, b = pair / f.Hq;
   const int hk = h / f.G;
   const int rt = CAUSAL ? ntile - 1 - in : in;  // longest rows first
@@ -893,6 +932,7 @@ __global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
 
   const int S = keys_of_batch(f, b);
   if (S == 0) {  // no keys (an empty cache entry): the output did not depend on q
+    if (a.dq_splits > 1) return;  // the merge kernel writes the zeros
     const int qi = qw0 + lq;
     if (qi < f.L) {
       T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
@@ -910,6 +950,8 @@ __global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
     const int lastkv = last < S - 1 ? last : S - 1;
     ntiles_kv = lastkv / BN + 1;
   }
+  // this workgroup's tiles: all of them, or piece `piece` of dq_splits nearly equal ones (possibly none)
+  const int t0 = (int)((long long)ntiles_kv * piece / a.dq_splits), t1 = (int)((long long)ntiles_kv * (piece + 1) / a.dq_splits);
 
   auto dma16 = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
@@ -944,17 +986,17 @@ __global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
     }
   }
 
-  dma_tile(0, 0);
-  if (1 < ntiles_kv) dma_tile(1, 1);
+  if (t0 < t1) dma_tile(t0, 0);
+  if (t0 + 1 < t1) dma_tile(t0 + 1, 1);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 
   int cur = 0;
-  for (int jt = 0; jt < ntiles_kv; jt++) {
+  for (int jt = t0; jt < t1; jt++) {
     const int kv0 = jt * BN;
-    const int nxt2 = cur == 0 ? 2 : cur - 1;  // (jt + 2) % 3: last read in iteration jt-1, which a barrier ended
-    const bool more = jt + 2 < ntiles_kv;
+    const int nxt2 = cur == 0 ? 2 : cur - 1;  // stage of tile jt + 2: last read in iteration jt-1, which a barrier ended
+    const bool more = jt + 2 < t1;
     if (more) dma_tile(jt + 2, nxt2);
     if (wave_live && (!CAUSAL || kv0 <= qw0 + 31 + coff)) {
       const char* kt = smem + cur * STAGE_BYTES;
@@ -1022,6 +1064,10 @@ __global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const int qi = qw0 + lq;
+  if (a.dq_splits > 1) {
+    if (qi < f.L) store_dq_partial<D>(a, piece, ((long long)b * f.Hq + h) * f.L + qi, lh, dqacc, m_use * c, l_tot, delta);
+    return;
+  }
   if (qi < f.L) {
     const long long row_id = ((long long)b * f.Hq + h) * f.L + qi;
     if (lh == 0) *(float2*)(a.stats + 2 * row_id) = make_float2(m_use * c + __log2f(l_tot), delta);
@@ -1056,7 +1102,7 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
     e = grant_dynamic_lds((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED>, Lds::KV_BYTES, state2, done2);
   }
   if (e != hipSuccess) return (int)e;
-  const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
+  const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM) * a.dq_splits;
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM) * a.dkv_splits;
   if (DMA) {
     hipLaunchKernelGGL((backward_dq128_kernel<TR, CAUSAL>), dim3((unsigned)g1), dim3(256), dq128::LDS_BYTES, stream, a);
@@ -1065,6 +1111,10 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   }
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
+  if (a.dq_splits > 1) {
+    const int rc = launch_backward_dq_merge<typename TR::elem>(a, stream);
+    if (rc != 0) return rc;
+  }
   if (DMA) {
     hipLaunchKernelGGL((backward_dkv128_kernel<TR, CAUSAL>), dim3((unsigned)g2), dim3(512), dkv128::LDS_BYTES, stream, a);
   } else {

@@ -180,6 +180,11 @@ struct BwdArgs {
   // workgroups, which leave partial dk / dv in `partial` ([split][dk | dv][B][Hkv][S][D] floats) for a third kernel to add.
   float* partial;
   int dkv_splits;
+  // 16-bit matrix-core pairs only: with dq_splits > 1 the key range of every 128-row query block is dealt out to that many
+  // workgroups of the dq kernel, which leave their unnormalised fp32 sums in `dq_partial` ([split][B][Hq][L][D] floats,
+  // then [split][B][Hq][L] pairs (maximum in log2 units, sum of exponentials)) for backward_dq_merge_kernel.
+  float* dq_partial;
+  int dq_splits;
 };
 
 // Workgroups that share a key block in the matrix-core dk/dv kernels (1: none, the kernel writes dk / dv itself).
@@ -198,6 +203,23 @@ inline int backward_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal
   const long long enough = causal ? 1024 : 256 * per_cu;
   int n = 1;
   while (n < 4 && wgs * n < enough && tiles >= 16 * n) n *= 2;
+  return n;
+}
+
+// Workgroups that share a 128-row query block in the 16-bit matrix-core dq kernels (1: none, the kernel writes dq itself).
+// Two of its workgroups fit a CU (512 at a time on the chip).  A launch of fewer is split: that gives every slot a
+// workgroup, and under a causal mask, where their lengths vary 1 : (number of row blocks) and they start longest first,
+// a second round to end evenly
+// (bf16 head_dim 128, one batch entry: 8 heads 4096 x 4096 causal +26 %, 32 heads 512 x 8192 +46 %, 8 heads 2048 x 2048
+// without a mask +22 %; 512 causal workgroups split in two measured 5 % slower: the partial records cost more than the
+// uneven end).  A split must still get a few hundred keys.
+inline int backward_dq_splits(int B, int Hq, int L, int S, bool causal) {
+  const long long wgs = (long long)B * Hq * ((L + 127) / 128);
+  const long long tiles = (S + 31) / 32;  // the longest key range, in 32-key tiles
+  if (wgs >= 512) return 1;
+  const long long enough = causal ? 1024 : 512;
+  int n = 1;
+  while (n < 8 && wgs * n < enough && tiles >= 16 * n) n *= 2;
   return n;
 }
 
@@ -242,6 +264,56 @@ template <typename T>
 int launch_backward_dkv_sum(const BwdArgs& a, hipStream_t stream) {
   const long long nvec = (long long)a.f.B * a.f.Hkv * a.f.S * (a.f.D / 4);
   hipLaunchKernelGGL(backward_dkv_sum_kernel<T>, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, stream, a, nvec);
+  return (int)hipGetLastError();
+}
+// dq of a call whose key ranges were split: the splits' sums brought to the common maximum, added in a fixed order (split
+// 0 first) and normalised; the row statistic for the dk/dv kernel.  One thread per four elements of a row.
+template <typename T>
+__global__ __launch_bounds__(256) void backward_dq_merge_kernel(BwdArgs a, long long nvec) {
+  typedef T vec4t __attribute__((ext_vector_type(4)));
+  const KArgs& f = a.f;
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  const int dvec = f.D / 4;
+  const int d = 4 * (int)(i % dvec);
+  const long long row_id = i / dvec;  // (b * Hq + h) * L + qi
+  const int qi = (int)(row_id % f.L);
+  const long long bh = row_id / f.L;
+  const int h = (int)(bh % f.Hq), b = (int)(bh / f.Hq);
+  const long long rows = (long long)f.B * f.Hq * f.L;
+  const float* ml = a.dq_partial + (long long)a.dq_splits * rows * f.D;
+  vec4t* out = (vec4t*)((T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2] + d);
+  f32x4 x = {0.f, 0.f, 0.f, 0.f};
+  int S = f.S;
+  if (f.kv_len) {
+    const int len = f.kv_len[b];
+    S = len < 0 ? 0 : (len < S ? len : S);
+  }
+  if (S == 0) {  // no keys: the dq kernel's workgroups returned at once
+    *out = __builtin_convertvector(x, vec4t);
+    return;
+  }
+  float m = -INFINITY;
+  for (int s = 0; s < a.dq_splits; s++) m = fmaxf(m, ml[2 * (s * rows + row_id)]);
+  float l = 0.f;
+  for (int s = 0; s < a.dq_splits; s++) {
+    const float2 st = *(const float2*)(ml + 2 * (s * rows + row_id));
+    const float w = fast_exp2(st.x - m);
+    l += st.y * w;
+    x += *(const f32x4*)(a.dq_partial + (s * rows + row_id) * f.D + d) * w;
+  }
+  // a row whose keys are all hidden: dq = 0, and a statistic that gives it weight 0 in the dk/dv kernel
+  const bool seen = l > 0.f;
+  const float w = seen ? f.scale / l : 0.f;
+#pragma unroll
+  for (int e = 0; e < 4; e++) x[e] = seen ? x[e] * w : 0.f;
+  *out = __builtin_convertvector(x, vec4t);
+  if (d == 0) a.stats[2 * row_id] = seen ? m + __log2f(l) : 1e30f;
+}
+template <typename T>
+int launch_backward_dq_merge(const BwdArgs& a, hipStream_t stream) {
+  const long long nvec = (long long)a.f.B * a.f.Hq * a.f.L * (a.f.D / 4);
+  hipLaunchKernelGGL(backward_dq_merge_kernel<T>, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, stream, a, nvec);
   return (int)hipGetLastError();
 }
 int launch_backward_general(const BwdArgs& a, int dtype, hipStream_t stream);

@@ -231,7 +231,7 @@ int validate_backward(const ttsdpa_backward_params* p, BwdArgs* a) {
   }
   if ((p->dout_stride[2] < f->D || p->dq_stride[2] < f->D) && f->L > 1) return TTSDPA_ERR_STRIDE;
   if ((p->dk_stride[2] < f->D || p->dv_stride[2] < f->D) && f->S > 1) return TTSDPA_ERR_STRIDE;
-  a->dout = p->dout, a->dq = p->dq, a->dk = p->dk, a->dv = p->dv, a->stats = nullptr, a->partial = nullptr, a->dkv_splits = 1;
+  a->dout = p->dout, a->dq = p->dq, a->dk = p->dk, a->dv = p->dv, a->stats = nullptr, a->partial = nullptr, a->dkv_splits = 1, a->dq_partial = nullptr, a->dq_splits = 1;
   return TTSDPA_OK;
 }
 
@@ -282,9 +282,23 @@ int dkv_splits_of(const ttsdpa_backward_params* p) {
   const int per_cu = f->D == 64 && f->mask_kind == TTSDPA_MASK_NONE ? 2 : 1;
   return backward_dkv_splits(f->B, f->Hkv, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE, groups, per_cu);
 }
+// ... then (16-bit matrix-core pairs whose dq kernel splits its key ranges) the partial dq records, 256-byte aligned.
+int dq_splits_of(const ttsdpa_backward_params* p) {
+  const ttsdpa_params* f = &p->fwd;
+  if (pick_backward_route(p) != TTSDPA_ROUTE_PREFILL || f->dtype == TTSDPA_F32) return 1;
+  return backward_dq_splits(f->B, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE);
+}
 size_t backward_partial_offset(const ttsdpa_backward_params* p) { return (backward_stats_bytes(p) + 255) & ~(size_t)255; }
-size_t backward_scratch_bytes(const ttsdpa_backward_params* p) {
+size_t backward_dq_partial_offset(const ttsdpa_backward_params* p) {
   const int n = dkv_splits_of(p);
+  if (n == 1) return backward_partial_offset(p);
+  const size_t end = backward_partial_offset(p) + (size_t)n * 2 * p->fwd.B * p->fwd.Hkv * p->fwd.S * p->fwd.D * sizeof(float);
+  return (end + 255) & ~(size_t)255;
+}
+size_t backward_scratch_bytes(const ttsdpa_backward_params* p) {
+  const int n = dkv_splits_of(p), nq = dq_splits_of(p);
+  if (nq > 1)
+    return backward_dq_partial_offset(p) + (size_t)nq * p->fwd.B * p->fwd.Hq * p->fwd.L * (p->fwd.D + 2) * sizeof(float);
   if (n == 1) return backward_stats_bytes(p);
   return backward_partial_offset(p) + (size_t)n * 2 * p->fwd.B * p->fwd.Hkv * p->fwd.S * p->fwd.D * sizeof(float);
 }
@@ -497,8 +511,10 @@ int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t wor
   a.stats = (float*)workspace;
   a.dkv_splits = dkv_splits_of(p);
   a.partial = a.dkv_splits > 1 ? (float*)((char*)workspace + backward_partial_offset(p)) : nullptr;
+  a.dq_splits = dq_splits_of(p);
+  a.dq_partial = a.dq_splits > 1 ? (float*)((char*)workspace + backward_dq_partial_offset(p)) : nullptr;
   if (route == TTSDPA_ROUTE_PREFILL) {
-    const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + 127) / 128), g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + 127) / 128);
+    const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + 127) / 128) * a.dq_splits, g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + 127) / 128);
     if (check_grid(g1) != TTSDPA_OK || check_grid(g2) != TTSDPA_OK) return TTSDPA_ERR_SHAPE;
     if (p->fwd.dtype == TTSDPA_F32) return launch_backward_f32(a, (hipStream_t)stream);
     return launch_backward_mfma(a, p->fwd.dtype, (hipStream_t)stream);
