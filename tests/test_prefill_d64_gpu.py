@@ -1,6 +1,6 @@
 """The pipelined prefill kernel at head_dim 64 (csrc/sdpa_prefill_d64.hip) against the oracle: it takes calls without an
 attnMask or pages that fill the chip with 256-row workgroups, so its cases are larger than the other parity tests'
-(B * Hq * row tiles >= 256).  Smaller head_dim-64 calls keep running on the 4-wavefront kernel and are covered in
+(B * Hq * row tiles >= 128).  Smaller head_dim-64 calls keep running on the 4-wavefront kernel and are covered in
 test_parity_gpu.py; both kernels must agree with the oracle on the same inputs."""
 import numpy as np
 import pytest
@@ -67,7 +67,7 @@ def test_head_dim_64_pipelined_bottom_right_and_key_counts(dtype):
 
 def test_head_dim_64_pipelined_equals_the_4_wavefront_kernel_within_rounding():
     # the same call through both kernels: a batch that fills the chip, and the same heads one batch entry at a time
-    # (which stays under the 256-workgroup bar and runs on the 4-wavefront kernel)
+    # (which stays under the 128-workgroup bar and runs on the 4-wavefront kernel)
     B, Hq, Hkv, L, S, D = 4, 64, 16, 512, 512, 64
     host, dev = make_inputs(4242, B, Hq, Hkv, L, S, D, "bf16", 0.8)
     rc, big = call("forward", *dev, causal=True)

@@ -123,13 +123,14 @@ bool pipelined_ok(const ttsdpa_params* p) {
   return p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22);
 }
 
-// The pipelined kernel at head_dim 64: no attnMask, no pages, and enough 256-row workgroups to fill the chip (smaller
-// calls stay on the 4-wavefront kernel, which has 128-row tiles and can divide the keys among workgroups).
+// The pipelined kernel at head_dim 64: no attnMask, no pages, and 256-row workgroups for at least half of the chip's CUs
+// (smaller calls stay on the 4-wavefront kernel, which has 128-row tiles and can divide the keys among workgroups; from
+// 128 workgroups on the pipelined kernel measured up to 28 % faster, at 64 up to 18 % slower).
 bool pipelined64_ok(const ttsdpa_params* p) {
   if (p->D != 64 || p->L <= 128 || p->mask_kind != TTSDPA_MASK_NONE || p->block_table) return false;
   if (!(p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22))) return false;
   const long long tiles = (p->L + 255) / 256;
-  return (long long)p->B * p->Hq * (p->causal ? (tiles + 1) / 2 : tiles) >= 256;
+  return (long long)p->B * p->Hq * (p->causal ? (tiles + 1) / 2 : tiles) >= 128;
 }
 
 // Few query rows per head against many keys on the 4-wavefront kernel: the G heads of a KV head share one row tile
