@@ -39,10 +39,13 @@ ROWS = [(0, 0), (0, 5), (1, 17), (1, 63), (3, 31)]
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("causal,L,S", [(True, 500, 500), (True, 769, 769), (False, 320, 411), (False, 257, 64)])
-def test_head_dim_64_pipelined_against_oracle(dtype, causal, L, S):
-    B, Hq, Hkv, D = 4, 64, 16, 64
-    host, dev = make_inputs(640 + L, B, Hq, Hkv, L, S, D, dtype, 0.8)
+def test_head_dim_64_pipelined_against_oracle(dtype, D, causal, L, S):
+    # (head_dim 128 rides along: its pipelined kernel with this many workgroups takes the causal row tiles in mirror
+    # pairs, which the smaller shapes of the other parity tests do not)
+    B, Hq, Hkv = 4, 64, 16
+    host, dev = make_inputs(640 + L + D, B, Hq, Hkv, L, S, D, dtype, 0.8)
     assert route_of(*dev, causal=causal) == "prefill"
     rc, out = call("forward", *dev, causal=causal)
     assert rc == 0
@@ -134,3 +137,18 @@ def test_head_dim_64_pipelined_strided_views_equal_contiguous_bitwise():
     rc, c = call("forward", *views, causal=True, out=outp.permute(0, 2, 1, 3))
     assert rc == 0
     assert torch.equal(a, outp.permute(0, 2, 1, 3))
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("B,L,S,align", [(1, 900, 900, "top-left"), (2, 600, 1000, "bottom-right"), (1, 4200, 4200, "top-left")])
+def test_pipelined_single_row_tiles(D, B, L, S, align):
+    # fewer mirror pairs than CUs (or a last round far from full): one causal row tile per workgroup, longest first
+    Hq, Hkv = 64, 16
+    if L > 4000:
+        Hq, Hkv = 40, 8   # 40 heads x 17 tiles: 360 pairs, 1.4 rounds of the chip
+    host, dev = make_inputs(8100 + L + D, B, Hq, Hkv, L, S, D, "bf16", 0.8)
+    assert route_of(*dev, causal=True, align=align) == "prefill"
+    rc, out = call("forward", *dev, causal=True, align=align)
+    assert rc == 0
+    rows = [(0, 0), (0, 5), (B - 1, 17), (B - 1, Hq - 1)] if L < 4000 else [(0, 3), (0, Hq - 1)]
+    assert sampled_rows_err(out, host, True, rows, align=align) <= TOL["bf16"]

@@ -33,6 +33,9 @@ struct KArgs {
   int kv_splits, kv_chunk;
   float* ws;
   int mask_vec4;  // keys are contiguous in the mask and groups of 4 keys starting at a multiple of 4 are naturally aligned
+  // Pipelined prefill kernels under a causal mask: 0 = a workgroup takes a row tile and its mirror (equal work for all),
+  // 1 = one row tile per workgroup, longest first (launches whose pairs would leave CUs without a workgroup).
+  int single_tiles;
 };
 
 // Offset of the causal diagonal in key coordinates for a batch entry with S keys.

@@ -62,7 +62,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   // Under a causal mask a workgroup takes row tile t and then its mirror ntile-1-t: every workgroup sees the same
   // number of KV tiles, so the launch has no long tail behind the heavy tiles.
   const int ntile = (a.L + BM - 1) / BM;
-  const int nslot = CAUSAL ? (ntile + 1) / 2 : ntile;
+  const bool paired = CAUSAL && !a.single_tiles;  // else one row tile per workgroup, longest first
+  const int nslot = paired ? (ntile + 1) / 2 : ntile;
   const int inner = a.G * nslot;
   const int npair = a.B * a.Hkv;
   int pair, in;
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
 
   // Neighbouring workgroups take their two tiles in opposite order, so that the load / store bursts between the
   // parts of one half of the workgroups fall into the steady loops of the other half.
-  const bool long_first = ((blockIdx.x >> 3) & 1) == 0;
+  const bool long_first = !paired || ((blockIdx.x >> 3) & 1) == 0;
   // Wavefronts w and w+4 share a SIMD.  Under a causal mask the row group g of a tile has g+1 halves of work on the
   // diagonal, so the second four wavefronts take the groups in reverse: every SIMD then carries groups g and 7-g.
   const int rowgroup = (CAUSAL && wave >= 4) ? 11 - wave : wave;
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
 #pragma unroll
     for (int i = 0; i < 8; i++) zero[i] = (T)0.f;
     for (int part = 0; part < (CAUSAL ? 2 : 1); part++) {
-      if (part == 1 && slot_rt >= ntile - 1 - slot_rt) break;
+      if (part == 1 && (!paired || slot_rt >= ntile - 1 - slot_rt)) break;
       const int rt = (CAUSAL && part == 0) ? ntile - 1 - slot_rt : slot_rt;
       for (int i = 0; i < 4; i++) {
         const int qi = rt * BM + rowgroup * WM + 8 * i + (lane >> 3);
@@ -131,7 +132,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
       ntiles_kv = lastkv / BN + 1;
     }
   };
-  const bool two_parts = CAUSAL && slot_rt < ntile - 1 - slot_rt;  // odd count: the middle tile has no mirror
+  const bool two_parts = paired && slot_rt < ntile - 1 - slot_rt;  // odd count: the middle tile has no mirror
 
   // ---- global -> LDS: wavefront w moves rows 8w .. 8w+7 of a tile with one instruction (8 rows, 1 KiB) -----------
   // lane l fills slot (row l/8, chunk slot l%8) and therefore fetches chunk (l%8) ^ f(row)
@@ -678,9 +679,22 @@ int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
 
 }  // namespace
 
-int launch_prefill_d64(const KArgs& a, int dtype, hipStream_t stream) {
+int launch_prefill_d64(const KArgs& args, int dtype, hipStream_t stream) {
+  KArgs a = args;
   const int ntile = (a.L + BM - 1) / BM;
   long long nwg = (long long)a.B * a.Hq * (a.causal ? (ntile + 1) / 2 : ntile);
+  // Mirror pairs are equal work, so a launch of them ends evenly only when the pairs fill whole rounds of the chip's 256
+  // CUs.  Fewer pairs than CUs, or long sequences whose last round is far from full: one row tile per workgroup instead,
+  // longest first (more CUs get one, and the launch ends with short tiles).  Measured at head_dim 128, bf16: 128 pairs of
+  // 2048 rows +19 %, 320 pairs of 4096 rows +25 %, 896 pairs of 16384 rows +4 %; but 512 pairs of 2048 rows -15 % and
+  // of 4096 rows -0.7 % (a workgroup's start costs more than the second part of a pair does).
+  if (a.causal && ntile > 1) {
+    const long long rounds = (nwg + 255) / 256;
+    if (nwg < 256 || (ntile >= 16 && nwg * 10 < rounds * 256 * 9)) {
+      a.single_tiles = 1;
+      nwg = (long long)a.B * a.Hq * ntile;
+    }
+  }
   // the kernel's XCD-aware numbering addresses workgroups in groups of 8 (classes of XCDs): round up, the extras return
   {
     const int npair = a.B * a.Hkv;

@@ -64,6 +64,7 @@ int validate(const ttsdpa_params* p, KArgs* a) {
   }
   if (p->mask_kind == TTSDPA_MASK_ADD && !ptr_aligned(p->mask, esz)) return TTSDPA_ERR_STRIDE;
   a->mask_vec4 = mask_vec4_ok(p) ? 1 : 0;
+  a->single_tiles = 0;
   a->pack_L = 0, a->kv_splits = 1, a->kv_chunk = 0, a->ws = nullptr;
   if (p->kv_len && !ptr_aligned(p->kv_len, 4)) return TTSDPA_ERR_STRIDE;
   a->kv_len = p->kv_len;
