@@ -684,13 +684,14 @@ int launch_prefill_d64(const KArgs& args, int dtype, hipStream_t stream) {
   const int ntile = (a.L + BM - 1) / BM;
   long long nwg = (long long)a.B * a.Hq * (a.causal ? (ntile + 1) / 2 : ntile);
   // Mirror pairs are equal work, so a launch of them ends evenly only when the pairs fill whole rounds of the chip's 256
-  // CUs.  Fewer pairs than CUs, or long sequences whose last round is far from full: one row tile per workgroup instead,
-  // longest first (more CUs get one, and the launch ends with short tiles).  Measured at head_dim 128, bf16: 128 pairs of
-  // 2048 rows +19 %, 320 pairs of 4096 rows +25 %, 896 pairs of 16384 rows +4 %; but 512 pairs of 2048 rows -15 % and
-  // of 4096 rows -0.7 % (a workgroup's start costs more than the second part of a pair does).
+  // CUs.  Fewer pairs than CUs, or a last round under 80 % full (90 % for sequences of 16 row tiles and more): one row
+  // tile per workgroup instead, longest first (more CUs get one, and the launch ends with short tiles).  Measured at
+  // head_dim 128, bf16: 128 pairs of 2048 rows +19 %, 320 pairs of 4096 rows +25 %, of 2048 rows +17 %, 384 of 2048 rows
+  // +4 %, 896 pairs of 16384 rows +4 %; but 640 pairs of 2048 rows -4 %, 512 of 2048 rows -15 % and of 4096 rows -0.7 %
+  // (a workgroup's start costs more than the second part of a pair does).
   if (a.causal && ntile > 1) {
     const long long rounds = (nwg + 255) / 256;
-    if (nwg < 256 || (ntile >= 16 && nwg * 10 < rounds * 256 * 9)) {
+    if (nwg < 256 || nwg * 10 < rounds * 256 * 8 || (ntile >= 16 && nwg * 10 < rounds * 256 * 9)) {
       a.single_tiles = 1;
       nwg = (long long)a.B * a.Hq * ntile;
     }
