@@ -280,10 +280,10 @@ def test_backward_split_query_stream(dtype, D, mode):
         check(name, host, dev, dtype, causal=(mode == "causal"), route="prefill")
 
 
-@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64), ("f16", 128), ("bf16", 64)])
+@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64), ("f16", 128), ("bf16", 64), ("f32", 128), ("f32", 64)])
 @pytest.mark.parametrize("mode", ["causal", "full", "br-kvlen", "mask", "hiddenrow"])
 def test_backward_split_key_ranges(dtype, D, mode):
-    """16-bit matrix-core pairs with few query blocks and many keys: the dq kernel deals the key range of every 128-row
+    """Matrix-core pairs with few query blocks and many keys: the dq kernel deals the key range of every 128-row
     query block out to several workgroups (here eight: 8 query blocks, 2100 keys) and a merge kernel brings their fp32
     partial sums to the common maximum.  The scratch the library asks for holds the partial records."""
     B, Hq, Hkv, L, S = 1, 4, 2, 200, 2100

@@ -95,8 +95,12 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
   const int lq = lane & 31, lh = lane >> 5;
 
   const int ntile = (f.L + BM - 1) / BM;
-  int pair, in;
-  map_workgroup(blockIdx.x, f.B * f.Hq, ntile, &pair, &in);
+  int pair, in, piece;  // piece: this workgroup's share of the row block's key range (dq_splits > 1)
+  {
+    int n;
+    split_of_workgroup(blockIdx.x, a.dq_splits, f.B * f.Hq, &n, &piece);
+    map_workgroup(n, f.B * f.Hq, ntile, &pair, &in);
+  }
   const int h = pair % f.Hq, b = pair / f.Hq;
   const int hk = h / f.G;
   const int rt = CAUSAL ? ntile - 1 - in : in;  // longest rows first
@@ -134,6 +138,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
 
   const int S = keys_of_batch(f, b);
   if (S == 0) {  // no keys (an empty cache entry): the output did not depend on q
+    if (a.dq_splits > 1) return;  // the merge kernel writes the zeros
     const int qi = qw0 + lq;
     if (qi < f.L) {
       float* dqp = (float*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
@@ -148,6 +153,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
     const int lastkv = last < S - 1 ? last : S - 1;
     ntiles_kv = lastkv / BT + 1;
   }
+  // this workgroup's tiles: all of them, or piece `piece` of dq_splits nearly equal ones (possibly none)
+  const int t0 = (int)((long long)ntiles_kv * piece / a.dq_splits), t1 = (int)((long long)ntiles_kv * (piece + 1) / a.dq_splits);
 
   // ---- global -> register -> LDS staging of one K/V tile (thread t moves 16-byte chunks t, t+256, ...) ----------------------
   f32x4 kst[NLD], vst[NLD];
@@ -181,17 +188,19 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
   const int s_lane = lq * PITCH + lh * (D / 2);  // score products: row l%32, this lane's half of head_dim
   const int g_lane = 4 * lh * PITCH + lq;        // gradient product: + (8*(t/4) + t%4) * PITCH + 32*db
 
-  load_tile(0);
-  store_tile(0);
-  if (1 < ntiles_kv) load_tile(BT);
+  if (t0 < t1) {
+    load_tile(t0 * BT);
+    store_tile(0);
+    if (t0 + 1 < t1) load_tile((t0 + 1) * BT);
+  }
   __syncthreads();
 
-  for (int jt = 0; jt < ntiles_kv; jt++) {
+  for (int jt = t0; jt < t1; jt++) {
     const int kv0 = jt * BT;
-    const int cur = jt & 1;
-    if (jt + 1 < ntiles_kv) {
+    const int cur = (jt - t0) & 1;
+    if (jt + 1 < t1) {
       store_tile(cur ^ 1);  // stage cur^1 was last read before the barrier that ended the previous iteration
-      if (jt + 2 < ntiles_kv) load_tile(kv0 + 2 * BT);
+      if (jt + 2 < t1) load_tile(kv0 + 2 * BT);
     }
     if (wave_live && (!CAUSAL || kv0 <= qw0 + 31 + coff)) {
       const float* Ks = smem + cur * Lds::STAGE;
@@ -250,6 +259,10 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const int qi = qw0 + lq;
+  if (a.dq_splits > 1) {
+    if (qi < f.L) store_dq_partial<D>(a, piece, ((long long)b * f.Hq + h) * f.L + qi, lh, dqacc, m_use * c, l_tot, delta);
+    return;
+  }
   if (qi < f.L) {
     const long long row_id = ((long long)b * f.Hq + h) * f.L + qi;
     // log2 of the row's sum of exponentials, the unit the second kernel's exp2 wants
@@ -472,11 +485,15 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   if (e != hipSuccess) return (int)e;
   e = grant_dynamic_lds((const void*)backward_dkv_f32_kernel<D, CAUSAL, MASKED>, BwdF32Lds<D>::BYTES, state2, done2);
   if (e != hipSuccess) return (int)e;
-  const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM);
+  const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM) * a.dq_splits;
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM) * a.dkv_splits;
   hipLaunchKernelGGL((backward_dq_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g1), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
+  if (a.dq_splits > 1) {
+    const int rc = launch_backward_dq_merge<float>(a, stream);
+    if (rc != 0) return rc;
+  }
   hipLaunchKernelGGL((backward_dkv_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g2), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess || a.dkv_splits == 1) return (int)e;

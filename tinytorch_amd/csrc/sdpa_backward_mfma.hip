@@ -123,29 +123,6 @@ __device__ __forceinline__ vec8 regs_to_operand(const f32x16& acc, int t) {
   return __builtin_convertvector(x, vec8);
 }
 
-// A lane's share of a query row's unnormalised dq sums (accumulator layout as above) and the row's (maximum in log2
-// units, sum of exponentials) as this split's partial record; split 0 also leaves delta for the dk/dv kernel.
-template <int D>
-__device__ __forceinline__ void store_dq_partial(const BwdArgs& a, int piece, long long row_id, int lh, const f32x16 (&dqacc)[D / 32],
-                                                 float mc, float l_tot, float delta) {
-  const long long rows = (long long)a.f.B * a.f.Hq * a.f.L;
-  float* dst = a.dq_partial + (piece * rows + row_id) * D;
-#pragma unroll
-  for (int db = 0; db < D / 32; db++)
-#pragma unroll
-    for (int rg = 0; rg < 4; rg++) {
-      f32x4 x;
-#pragma unroll
-      for (int i = 0; i < 4; i++) x[i] = dqacc[db][4 * rg + i];
-      *(f32x4*)(dst + 32 * db + 8 * rg + 4 * lh) = x;
-    }
-  if (lh == 0) {
-    float* ml = a.dq_partial + a.dq_splits * rows * D;
-    *(float2*)(ml + 2 * (piece * rows + row_id)) = make_float2(mc, l_tot);
-    if (piece == 0) a.stats[2 * row_id + 1] = delta;
-  }
-}
-
 // ---- kernel 1: dq, lse, delta ----------------------------------------------------------------------------------------
 // BN: keys per streamed tile.  64 for head_dim 64; 32 for head_dim 128, which keeps a wavefront under 256 registers:
 // two wavefronts per SIMD (one's vector work overlaps the other's matrix work), accumulators in ordinary registers.

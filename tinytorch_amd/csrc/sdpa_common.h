@@ -183,7 +183,7 @@ struct BwdArgs {
   // workgroups, which leave partial dk / dv in `partial` ([split][dk | dv][B][Hkv][S][D] floats) for a third kernel to add.
   float* partial;
   int dkv_splits;
-  // 16-bit matrix-core pairs only: with dq_splits > 1 the key range of every 128-row query block is dealt out to that many
+  // matrix-core pairs only: with dq_splits > 1 the key range of every 128-row query block is dealt out to that many
   // workgroups of the dq kernel, which leave their unnormalised fp32 sums in `dq_partial` ([split][B][Hq][L][D] floats,
   // then [split][B][Hq][L] pairs (maximum in log2 units, sum of exponentials)) for backward_dq_merge_kernel.
   float* dq_partial;
@@ -209,18 +209,19 @@ inline int backward_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal
   return n;
 }
 
-// Workgroups that share a 128-row query block in the 16-bit matrix-core dq kernels (1: none, the kernel writes dq itself).
+// Workgroups that share a 128-row query block in the matrix-core dq kernels (1: none, the kernel writes dq itself).
 // Two of its workgroups fit a CU (512 at a time on the chip).  A launch of fewer is split: that gives every slot a
 // workgroup, and under a causal mask, where their lengths vary 1 : (number of row blocks) and they start longest first,
 // a second round to end evenly
 // (bf16 head_dim 128, one batch entry: 8 heads 4096 x 4096 causal +26 %, 32 heads 512 x 8192 +46 %, 8 heads 2048 x 2048
 // without a mask +22 %; 512 causal workgroups split in two measured 5 % slower: the partial records cost more than the
 // uneven end).  A split must still get a few hundred keys.
-inline int backward_dq_splits(int B, int Hq, int L, int S, bool causal) {
+// `slots`: workgroups of the kernel the chip holds at a time (512; 256 for the fp32 kernel at head_dim 128).
+inline int backward_dq_splits(int B, int Hq, int L, int S, bool causal, int slots) {
   const long long wgs = (long long)B * Hq * ((L + 127) / 128);
   const long long tiles = (S + 31) / 32;  // the longest key range, in 32-key tiles
-  if (wgs >= 512) return 1;
-  const long long enough = causal ? 1024 : 512;
+  if (wgs >= slots) return 1;
+  const long long enough = causal ? 2 * slots : slots;
   int n = 1;
   while (n < 8 && wgs * n < enough && tiles >= 16 * n) n *= 2;
   return n;
@@ -269,6 +270,30 @@ int launch_backward_dkv_sum(const BwdArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL(backward_dkv_sum_kernel<T>, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, stream, a, nvec);
   return (int)hipGetLastError();
 }
+// A lane's share of a query row's unnormalised dq sums (accumulator layout of the 32 x 32 matrix instructions: registers 4rg .. 4rg+3 of block db are
+// elements 32db + 8rg + 4lh .. +3) and the row's (maximum in log2
+// units, sum of exponentials) as this split's partial record; split 0 also leaves delta for the dk/dv kernel.
+template <int D>
+__device__ __forceinline__ void store_dq_partial(const BwdArgs& a, int piece, long long row_id, int lh, const f32x16 (&dqacc)[D / 32],
+                                                 float mc, float l_tot, float delta) {
+  const long long rows = (long long)a.f.B * a.f.Hq * a.f.L;
+  float* dst = a.dq_partial + (piece * rows + row_id) * D;
+#pragma unroll
+  for (int db = 0; db < D / 32; db++)
+#pragma unroll
+    for (int rg = 0; rg < 4; rg++) {
+      f32x4 x;
+#pragma unroll
+      for (int i = 0; i < 4; i++) x[i] = dqacc[db][4 * rg + i];
+      *(f32x4*)(dst + 32 * db + 8 * rg + 4 * lh) = x;
+    }
+  if (lh == 0) {
+    float* ml = a.dq_partial + a.dq_splits * rows * D;
+    *(float2*)(ml + 2 * (piece * rows + row_id)) = make_float2(mc, l_tot);
+    if (piece == 0) a.stats[2 * row_id + 1] = delta;
+  }
+}
+
 // dq of a call whose key ranges were split: the splits' sums brought to the common maximum, added in a fixed order (split
 // 0 first) and normalised; the row statistic for the dk/dv kernel.  One thread per four elements of a row.
 template <typename T>

@@ -284,11 +284,12 @@ int dkv_splits_of(const ttsdpa_backward_params* p) {
   const int per_cu = f->D == 64 && f->mask_kind == TTSDPA_MASK_NONE ? 2 : 1;
   return backward_dkv_splits(f->B, f->Hkv, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE, groups, per_cu);
 }
-// ... then (16-bit matrix-core pairs whose dq kernel splits its key ranges) the partial dq records, 256-byte aligned.
+// ... then (matrix-core pairs whose dq kernel splits its key ranges) the partial dq records, 256-byte aligned.
 int dq_splits_of(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
-  if (pick_backward_route(p) != TTSDPA_ROUTE_PREFILL || f->dtype == TTSDPA_F32) return 1;
-  return backward_dq_splits(f->B, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE);
+  if (pick_backward_route(p) != TTSDPA_ROUTE_PREFILL) return 1;
+  const int slots = f->dtype == TTSDPA_F32 && f->D == 128 ? 256 : 512;
+  return backward_dq_splits(f->B, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE, slots);
 }
 size_t backward_partial_offset(const ttsdpa_backward_params* p) { return (backward_stats_bytes(p) + 255) & ~(size_t)255; }
 size_t backward_dq_partial_offset(const ttsdpa_backward_params* p) {
