@@ -114,8 +114,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     const long long item = (long long)slot * (8 / gq) + sub;  // work item of the class
     const long long items = (long long)(npair / gq) * inner;
     if (item >= items) return;  // the grid is rounded up to a multiple of 8
-    pair = cls + gq * (int)(item / inner);
-    in = (int)(item % inner);
+    if (a.single_tiles) {  // longest tiles first across all the pairs of the class
+      const int ppc = npair / gq;
+      pair = cls + gq * (int)(item % ppc);
+      in = (int)(item / ppc);
+    } else {
+      pair = cls + gq * (int)(item / inner);
+      in = (int)(item % inner);
+    }
   }
   const int b = pair / a.Hkv, hk = pair % a.Hkv;
   const int g = in % a.G;
@@ -742,14 +748,14 @@ int launch_prefill_d128(const KArgs& args, int dtype, hipStream_t stream) {
   const int ntile = (a.L + BM - 1) / BM;
   long long nwg = (long long)a.B * a.Hq * (a.causal ? (ntile + 1) / 2 : ntile);
   // Mirror pairs are equal work, so a launch of them ends evenly only when the pairs fill whole rounds of the chip's 256
-  // CUs.  Fewer pairs than CUs, or a last round under 80 % full (90 % for sequences of 16 row tiles and more): one row
-  // tile per workgroup instead, longest first (more CUs get one, and the launch ends with short tiles).  Measured at
-  // head_dim 128, bf16: 128 pairs of 2048 rows +19 %, 320 pairs of 4096 rows +25 %, of 2048 rows +17 %, 384 of 2048 rows
-  // +4 %, 896 pairs of 16384 rows +4 %; but 640 pairs of 2048 rows -4 %, 512 of 2048 rows -15 % and of 4096 rows -0.7 %
-  // (a workgroup's start costs more than the second part of a pair does).
+  // CUs.  Fewer pairs than CUs, or a last round under 90 % full: one row tile per workgroup instead, longest first across
+  // all the (batch, kv head) pairs of an XCD (more CUs get one, and the launch ends with short tiles).  Measured at
+  // head_dim 128, bf16, against pairs: 128 pairs of 2048 rows +19 %, 224 of 1024 rows +28 %, 320 of 4096 rows +25 %,
+  // of 2048 rows +17 %, 640 of 2048 rows +4.5 %, 896 of 2048 rows +4 %, of 16384 rows +4 %; with full rounds -2.5 %
+  // to +0.5 % (512 pairs of 1024 / 2048 / 4096 rows, 768 of 4096 rows).
   if (a.causal && ntile > 1) {
     const long long rounds = (nwg + 255) / 256;
-    if (nwg < 256 || nwg * 10 < rounds * 256 * 8 || (ntile >= 16 && nwg * 10 < rounds * 256 * 9)) {
+    if (nwg < 256 || nwg * 10 < rounds * 256 * 9) {
       a.single_tiles = 1;
       nwg = (long long)a.B * a.Hq * ntile;
     }
