@@ -1,7 +1,7 @@
 """The pipelined prefill kernel at head_dim 64 (csrc/sdpa_prefill_d64.hip) against the oracle: it takes calls without an
-attnMask or pages that fill the chip with 256-row workgroups, so its cases are larger than the other parity tests'
-(B * Hq * row tiles >= 128).  Smaller head_dim-64 calls keep running on the 4-wavefront kernel and are covered in
-test_parity_gpu.py; both kernels must agree with the oracle on the same inputs."""
+attnMask or pages of 512 query rows and more, or shorter ones that fill half of the chip's CUs with 256-row workgroups, so
+its cases are larger than the other parity tests'.  Smaller head_dim-64 calls keep running on the 4-wavefront kernel and
+are covered in test_parity_gpu.py; both kernels must agree with the oracle on the same inputs."""
 import numpy as np
 import pytest
 import torch
@@ -69,18 +69,20 @@ def test_head_dim_64_pipelined_bottom_right_and_key_counts(dtype):
 
 
 def test_head_dim_64_pipelined_equals_the_4_wavefront_kernel_within_rounding():
-    # the same call through both kernels: a batch that fills the chip, and the same heads one batch entry at a time
-    # (which stays under the 128-workgroup bar and runs on the 4-wavefront kernel)
+    # the same call through both kernels: causal on the pipelined kernel, and the same triangle as a Bool attnMask, which
+    # the pipelined kernel does not take (one batch entry: the other kernel reads the mask from memory)
     B, Hq, Hkv, L, S, D = 4, 64, 16, 512, 512, 64
     host, dev = make_inputs(4242, B, Hq, Hkv, L, S, D, "bf16", 0.8)
     rc, big = call("forward", *dev, causal=True)
     assert rc == 0
-    rc, one = call("forward", dev[0][:1].contiguous(), dev[1][:1].contiguous(), dev[2][:1].contiguous(), causal=True)
+    tril = torch.ones(L, S, dtype=torch.bool, device="cuda").tril()
+    rc, one = call("forward", dev[0][:1].contiguous(), dev[1][:1].contiguous(), dev[2][:1].contiguous(), mask=tril)
     assert rc == 0
     d = (big[:1].float() - one.float()).abs().max().item()
-    assert d <= 2e-2
+    assert 0 < d <= 2e-2   # two kernels: close, not identical
     # causal row 0 is v[0] exactly on both
     assert torch.equal(big[:, :, 0, :], dev[2][:, :, 0, :].repeat_interleave(Hq // Hkv, dim=1))
+    assert torch.equal(one[:, :, 0, :], dev[2][:1, :, 0, :].repeat_interleave(Hq // Hkv, dim=1))
 
 
 def test_large_score_range_head_dim_64_pipelined():

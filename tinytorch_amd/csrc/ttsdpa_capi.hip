@@ -124,14 +124,17 @@ bool pipelined_ok(const ttsdpa_params* p) {
   return p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22);
 }
 
-// The pipelined kernel at head_dim 64: no attnMask, no pages, and 256-row workgroups for at least half of the chip's CUs
-// (smaller calls stay on the 4-wavefront kernel, which has 128-row tiles and can divide the keys among workgroups; from
-// 128 workgroups on the pipelined kernel measured up to 28 % faster, at 64 up to 18 % slower).
+// The pipelined kernel at head_dim 64: no attnMask, no pages.  Against the 4-wavefront kernel (128-row tiles, keys
+// divided among workgroups) it measured level or up to 30 % faster from 512 query rows on, except under a causal mask
+// with fewer row tiles than CUs and more than 4096 keys (4 heads x 8192: 12 % slower — the launch then ends with its
+// longest row tile, which the other kernel splits); shorter calls take it when they fill half of the chip's CUs.
 bool pipelined64_ok(const ttsdpa_params* p) {
   if (p->D != 64 || p->L <= 128 || p->mask_kind != TTSDPA_MASK_NONE || p->block_table) return false;
   if (!(p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22))) return false;
   const long long tiles = (p->L + 255) / 256;
-  return (long long)p->B * p->Hq * (p->causal ? (tiles + 1) / 2 : tiles) >= 128;
+  if ((long long)p->B * p->Hq * (p->causal ? (tiles + 1) / 2 : tiles) >= 128) return true;
+  if (p->L < 512) return false;
+  return !(p->causal && p->S > 4096 && (long long)p->B * p->Hq * tiles < 256);
 }
 
 // Few query rows per head against many keys on the 4-wavefront kernel: the G heads of a KV head share one row tile
