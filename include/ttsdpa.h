@@ -135,7 +135,8 @@ void ttsdpa_params_init(ttsdpa_params* p, int dtype, int B, int Hq, int Hkv, int
 int ttsdpa_plan(const ttsdpa_params* p, int* route);
 
 /* Bytes of device scratch ttsdpa_forward / ttsdpa_decode use for *p (0 for calls that need none): the split-KV
- * partials of the decode route, and of short-L calls on the prefill route whose keys are divided among workgroups.
+ * partials of the decode route, and of calls on the prefill route whose keys are divided among workgroups (few query
+ * rows, or few 256-row tiles of head_dim 128 against many keys).
  * The decode route refuses to run with less (TTSDPA_ERR_WORKSPACE); the prefill route then runs unsplit.
  * The reference's precedent for op-owned device scratch is src/Operation/OpNNLayerCuda.cuh:415. */
 size_t ttsdpa_workspace_bytes(const ttsdpa_params* p);
