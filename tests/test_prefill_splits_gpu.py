@@ -1,7 +1,7 @@
 """Key splits of the pipelined head_dim-128 prefill kernel: calls with at most a quarter as many 256-row tiles as the chip
 has CUs (a chunk of rows against a long cache, a few heads) divide the keys of a row tile among workgroups, and the decode path's merge kernel combines their
 records.  ttsdpa_forward with its workspace takes that form; ttsdpa_prefill (no workspace) runs the same call unsplit:
-both against the oracle, and against each other."""
+both against the oracle, and against each other.  The records are combined by the kernel file's own merge kernel."""
 import ctypes
 
 import numpy as np
@@ -25,6 +25,7 @@ def workspace_bytes(q, k, v, **kw):
 CASES = [
     # B, Hq, Hkv, L, S, causal, align, dtype
     (1, 2, 2, 8192, 8192, True, "top-left", "bf16"),      # two heads of one long sequence
+    (2, 4, 1, 4096, 4096, True, "top-left", "bf16"),      # one KV head's share of config 3 (128 row tiles, causal)
     (2, 4, 1, 2048, 8192, True, "bottom-right", "bf16"),  # a 2048-row chunk of one KV head's share of a model
     (1, 8, 8, 1024, 16384, False, "top-left", "bf16"),
     (1, 8, 2, 700, 5000, True, "bottom-right", "f16"),    # a ragged chunk at the end of a ragged cache

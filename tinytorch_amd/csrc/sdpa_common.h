@@ -391,8 +391,7 @@ int launch_prefill_d64(const KArgs& a, int dtype, hipStream_t stream);   // the 
 int launch_prefill_f32(const KArgs& a, hipStream_t stream);              // fp32 tensors on the fp32 matrix cores; head_dim 64 or 128
 int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream);
 // combines per-split records [pair][split][row][D + 2] (pair = batch * Hkv + kv head, row = l * G + g) into a.out
-// chunk > 0: records of the pipelined prefill kernels' splits (`chunk` keys each; splits beyond a row's keys left none)
-int launch_merge(const KArgs& a, int dtype, int splits, const float* ws, hipStream_t stream, int chunk = 0);
+int launch_merge(const KArgs& a, int dtype, int splits, const float* ws, hipStream_t stream);
 int launch_zero(const KArgs& a, int dtype, hipStream_t stream);
 struct KvAppendArgs {
   void* kc;

@@ -291,31 +291,14 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int
 // then thread d accumulates head_dim element d over the splits with independent, coalesced loads.
 constexpr int kMaxSplits = 64;
 template <typename T, int DD>
-__global__ __launch_bounds__(DD) void merge_kernel(KArgs a, int splits, const float* __restrict__ ws, int chunk) {
+__global__ __launch_bounds__(DD) void merge_kernel(KArgs a, int splits, const float* __restrict__ ws) {
   __shared__ float weight[kMaxSplits];
   __shared__ float total;
-  const int nsplit_all = splits;  // records per (pair, row) in ws
   const int rows = a.L * a.G;
   const int pair = blockIdx.x / rows, x = blockIdx.x % rows;  // pair = b * Hkv + hk
   const int hk = pair % a.Hkv, b = pair / a.Hkv;
-  // chunk > 0 (splits of the pipelined prefill kernels, `chunk` keys each): a split that starts beyond the last key a
-  // row tile sees wrote no record; a row takes the splits up to its own last key (the others weigh nothing for it)
-  if (chunk > 0) {
-    int S = a.S;
-    if (a.kv_len) {
-      const int len = a.kv_len[b];
-      S = len < 0 ? 0 : (len < S ? len : S);
-    }
-    int last = S - 1;
-    if (a.causal) {
-      const int v = x / a.G + causal_offset(a, S);
-      last = v < last ? v : last;
-    }
-    const int n = last < 0 ? 0 : last / chunk + 1;
-    splits = n < splits ? n : splits;
-  }
   const float c = a.scale * kLog2e;
-  const float* rec0 = ws + ((long long)pair * nsplit_all * rows + x) * (DD + 2);
+  const float* rec0 = ws + ((long long)pair * splits * rows + x) * (DD + 2);
   const long long step = (long long)rows * (DD + 2);
   const int t = threadIdx.x;
   if (t < 64) {
@@ -360,7 +343,7 @@ int launch_decode_t(const KArgs& a, const DecodePlan& pl, float* ws, hipStream_t
 #undef TT_DECODE
   int rc = (int)hipGetLastError();
   if (rc != 0 || pl.splits == 1) return rc;
-  hipLaunchKernelGGL((merge_kernel<T, DD>), dim3((unsigned)((long long)a.B * a.Hkv * pl.rows)), dim3(DD), 0, stream, a, pl.splits, ws, 0);
+  hipLaunchKernelGGL((merge_kernel<T, DD>), dim3((unsigned)((long long)a.B * a.Hkv * pl.rows)), dim3(DD), 0, stream, a, pl.splits, ws);
   return (int)hipGetLastError();
 }
 
@@ -388,17 +371,17 @@ DecodePlan plan_decode(const KArgs& a) {
   return p;
 }
 
-int launch_merge(const KArgs& a, int dtype, int splits, const float* ws, hipStream_t stream, int chunk) {
+int launch_merge(const KArgs& a, int dtype, int splits, const float* ws, hipStream_t stream) {
   const dim3 grid((unsigned)((long long)a.B * a.Hkv * a.L * a.G));
   if (dtype == 0) {
-    if (a.D == 64) hipLaunchKernelGGL((merge_kernel<float, 64>), grid, dim3(64), 0, stream, a, splits, ws, chunk);
-    else hipLaunchKernelGGL((merge_kernel<float, 128>), grid, dim3(128), 0, stream, a, splits, ws, chunk);
+    if (a.D == 64) hipLaunchKernelGGL((merge_kernel<float, 64>), grid, dim3(64), 0, stream, a, splits, ws);
+    else hipLaunchKernelGGL((merge_kernel<float, 128>), grid, dim3(128), 0, stream, a, splits, ws);
   } else if (a.D == 64) {
-    if (dtype == 1) hipLaunchKernelGGL((merge_kernel<_Float16, 64>), grid, dim3(64), 0, stream, a, splits, ws, chunk);
-    else hipLaunchKernelGGL((merge_kernel<__bf16, 64>), grid, dim3(64), 0, stream, a, splits, ws, chunk);
+    if (dtype == 1) hipLaunchKernelGGL((merge_kernel<_Float16, 64>), grid, dim3(64), 0, stream, a, splits, ws);
+    else hipLaunchKernelGGL((merge_kernel<__bf16, 64>), grid, dim3(64), 0, stream, a, splits, ws);
   } else {
-    if (dtype == 1) hipLaunchKernelGGL((merge_kernel<_Float16, 128>), grid, dim3(128), 0, stream, a, splits, ws, chunk);
-    else hipLaunchKernelGGL((merge_kernel<__bf16, 128>), grid, dim3(128), 0, stream, a, splits, ws, chunk);
+    if (dtype == 1) hipLaunchKernelGGL((merge_kernel<_Float16, 128>), grid, dim3(128), 0, stream, a, splits, ws);
+    else hipLaunchKernelGGL((merge_kernel<__bf16, 128>), grid, dim3(128), 0, stream, a, splits, ws);
   }
   return (int)hipGetLastError();
 }

@@ -183,16 +183,18 @@ SplitPlan plan_prefill_splits(const ttsdpa_params* p, const KArgs& a /* after pa
 // Key splits for the pipelined head_dim-128 kernel: a call with a quarter as many 256-row tiles as the chip has CUs, or
 // fewer (a chunk of one sequence's rows against a long cache, a few heads of a tensor-parallel share), leaves most CUs
 // without work.  Its row tiles then share their keys among workgroups of `chunk` keys (a multiple of 256: four key
-// tiles, so the kernel's stages keep their constants), enough for two workgroups per CU, and the decode path's merge
-// kernel combines the records.  The records cost: with 128 row tiles the split measured 3 % faster to 20 % slower,
-// with 64 (32 heads x 512 rows on 8192 keys) 50 % faster.
+// tiles, so the kernel's stages keep their constants), enough for two workgroups per CU, and the
+// kernel's merge kernel combines the records.  The records cost: with 65-128 row tiles the split pays only under a
+// causal mask on 4096 keys or more (4 heads x 8192 rows +32 %, one KV head's share of 2 x 4096 rows +7 %; without a mask
+// -9 %, 2048 keys -18 %); with 64 and fewer it measured 1.1x to 5x (32 heads x 512 rows on 8192 keys 1.5x).
 SplitPlan plan_pipelined_splits(const ttsdpa_params* p) {
   SplitPlan s{1, 0, 0};
   if (p->dtype == TTSDPA_F32 || !pipelined_ok(p) || p->mask_kind != TTSDPA_MASK_NONE || p->block_table) return s;
   const long long units = (long long)p->B * p->Hq * ((p->L + 255) / 256);
   // keys a row can see: under a top-left aligned causal mask no more than there are rows
   const long long keys = effective_causal(p) == TTSDPA_CAUSAL_TOP_LEFT && p->L < p->S ? p->L : p->S;
-  if (units > 64 || keys < 2048) return s;
+  if (units > 128 || keys < 2048) return s;
+  if (units > 64 && !(p->causal && keys >= 4096)) return s;
   long long want = (512 + units - 1) / units;
   const long long most = keys / 512;  // at least 8 key tiles per split
   if (want > most) want = most;
@@ -454,11 +456,7 @@ static int prefill_impl(const ttsdpa_params* p, void* workspace, size_t workspac
     if (sp.splits > 1 && workspace && workspace_bytes >= sp.ws_bytes && ptr_aligned(workspace, 16)) {
       a.kv_splits = sp.splits, a.kv_chunk = sp.chunk, a.ws = (float*)workspace;
       if ((rc = check_grid((long long)a.B * a.Hq * ((a.L + 255) / 256 + 8) * sp.splits)) != TTSDPA_OK) return rc;
-      rc = launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
-      if (rc != 0) return rc;
-      KArgs m = a;  // the merge kernel's rows: every query head a "kv head" of its own
-      m.Hkv = a.Hq, m.G = 1;
-      return launch_merge(m, p->dtype, sp.splits, a.ws, (hipStream_t)stream, sp.chunk);
+      return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);  // the kernel and the merge of its records
     }
     a.kv_splits = 1, a.kv_chunk = 0, a.ws = nullptr;
     return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
