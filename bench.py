@@ -53,9 +53,11 @@ WORKLOADS = {
     "config5": (1, 28, 4, 16384, 16384, 128, "bf16", True, 1.0, "mfma"),
     "config3_f32": (2, 32, 8, 4096, 4096, 128, "f32", True, 1.0, "mfma"),  # config 3's shape in the reference's default dtype
     "config3_d64": (2, 32, 8, 4096, 4096, 64, "bf16", True, 1.0, "mfma"),   # config 3's shape at head_dim 64
+    # one GPU's share of config 3 when its 8 KV heads are dealt out to 8 GPUs (no exchange between them): 128 row tiles
+    "config3_share8": (2, 4, 1, 4096, 4096, 128, "bf16", True, 1.0, "mfma"),
 }
 SEEDS = {"config1": 0x5EED0001, "config2": 0x5EED0002, "config3": 0x5EED0003, "config4": 0x5EED0004, "config5": 0x5EED0005,
-         "config3_f32": 0x5EED0003, "config3_d64": 0x5EED0006}
+         "config3_f32": 0x5EED0003, "config3_d64": 0x5EED0006, "config3_share8": 0x5EED0007}
 DESCR = {
     "config1": "fp32 causal SDPA B1 H4 S128 D64",
     "config2": "fp16 causal MHA prefill B4 H32 S2048 D128",
@@ -64,6 +66,7 @@ DESCR = {
     "config5": "bf16 causal GQA prefill B1 28q/4kv S16384 D128",
     "config3_f32": "fp32 causal GQA prefill B2 32q/8kv S4096 D128",
     "config3_d64": "bf16 causal GQA prefill B2 32q/8kv S4096 D64",
+    "config3_share8": "bf16 causal GQA prefill B2 4q/1kv S4096 D128 (one KV head of config 3: an 8-GPU head-sharded share)",
 }
 
 
@@ -547,7 +550,7 @@ def main():
         # the baseline's other configurations (config 1: launch-sized, its time is the figure) and head_dim 64
         line["other_configs"] = []
         for name, corner, budget in (("config1", None, 2.0), ("config2", None, 4.0), ("config5", 4096, 4.0),
-                                     ("config3_d64", 2048, 3.0)):
+                                     ("config3_d64", 2048, 3.0), ("config3_share8", 2048, 2.0)):
             torch.cuda.empty_cache()
             res, tensors = run_gpu(name, max(1, min(args.steps, 50)), min(args.warmup, 20))
             if not args.no_cpu:
