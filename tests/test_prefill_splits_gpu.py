@@ -1,4 +1,4 @@
-"""Key splits of the pipelined head_dim-128 prefill kernel: calls with at most a quarter as many 256-row tiles as the chip
+"""Key splits of the pipelined prefill kernels (head_dim 128 and 64): calls with at most a quarter as many 256-row tiles as the chip
 has CUs (a chunk of rows against a long cache, a few heads) divide the keys of a row tile among workgroups, and the decode path's merge kernel combines their
 records.  ttsdpa_forward with its workspace takes that form; ttsdpa_prefill (no workspace) runs the same call unsplit:
 both against the oracle, and against each other.  The records are combined by the kernel file's own merge kernel."""
@@ -34,12 +34,13 @@ CASES = [
 ]
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B%dH%dk%dL%dS%d-c%d-%s-%s" % c)
-def test_split_keys_against_oracle_and_unsplit(case):
+def test_split_keys_against_oracle_and_unsplit(case, D):
     B, Hq, Hkv, L, S, causal, align, dtype = case
-    host, dev = make_inputs(9000 + L + S, B, Hq, Hkv, L, S, 128, dtype, 0.8)
+    host, dev = make_inputs(9000 + L + S + D, B, Hq, Hkv, L, S, D, dtype, 0.8)
     assert route_of(*dev, causal=causal, align=align) == "prefill"
-    assert workspace_bytes(*dev, causal=causal, align=align) >= 2 * B * Hq * L * 130 * 4   # at least two records per row
+    assert workspace_bytes(*dev, causal=causal, align=align) >= 2 * B * Hq * L * (D + 2) * 4   # at least two records per row
     rc, split = call("forward", *dev, causal=causal, align=align)
     assert rc == 0
     rc, whole = call("prefill", *dev, causal=causal, align=align)

@@ -392,6 +392,61 @@ int launch_prefill_f32(const KArgs& a, hipStream_t stream);              // fp32
 int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream);
 // combines per-split records [pair][split][row][D + 2] (pair = batch * Hkv + kv head, row = l * G + g) into a.out
 int launch_merge(const KArgs& a, int dtype, int splits, const float* ws, hipStream_t stream);
+
+// The records of a split launch of a pipelined prefill kernel -> out.  One thread per four elements of a row (eight rows per workgroup): the row's
+// splits up to its last visible key (a split wholly beyond the keys of a row tile wrote nothing), brought to their
+// common maximum, added in split order, normalised.  Rows of a batch entry without keys: zeros.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void prefill_split_merge_kernel(KArgs a, long long nvec) {
+  typedef T vec4t __attribute__((ext_vector_type(4)));
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  const int d = 4 * (int)(i % (D / 4));
+  const long long row_id = i / (D / 4);  // (b * Hq + h) * L + qi
+  const int qi = (int)(row_id % a.L);
+  const long long bh = row_id / a.L;
+  const int h = (int)(bh % a.Hq), b = (int)(bh / a.Hq);
+  int S = a.S;
+  if (a.kv_len) {
+    const int len = a.kv_len[b];
+    S = len < 0 ? 0 : (len < S ? len : S);
+  }
+  int last = S - 1;
+  if (a.causal) {
+    const int v = qi + causal_offset(a, S);
+    last = v < last ? v : last;
+  }
+  int n = last < 0 ? 0 : last / a.kv_chunk + 1;
+  n = n < a.kv_splits ? n : a.kv_splits;
+  const float c = a.scale * kLog2e;
+  const long long step = (long long)a.L * (D + 2);
+  const float* rec = a.ws + (bh * a.kv_splits * a.L + qi) * (D + 2);
+  float m = -1e30f;
+  for (int s = 0; s < n; s++) m = fmaxf(m, rec[s * step + D]);
+  float l = 0.f;
+  f32x4 x = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < n; s++) {
+    const float w = fast_exp2((rec[s * step + D] - m) * c);
+    l = fmaf(w, rec[s * step + D + 1], l);
+    const float2 lo = *(const float2*)(rec + s * step + d), hi = *(const float2*)(rec + s * step + d + 2);
+    x[0] = fmaf(w, lo.x, x[0]), x[1] = fmaf(w, lo.y, x[1]), x[2] = fmaf(w, hi.x, x[2]), x[3] = fmaf(w, hi.y, x[3]);
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int e = 0; e < 4; e++) x[e] *= inv;
+  *(vec4t*)((T*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2] + d) = __builtin_convertvector(x, vec4t);
+}
+
+template <int D>
+int launch_prefill_split_merge(const KArgs& a, int dtype, hipStream_t stream) {
+  const long long nvec = (long long)a.B * a.Hq * a.L * (D / 4);
+  const dim3 grid((unsigned)((nvec + 255) / 256));
+  if (dtype == 1) hipLaunchKernelGGL((prefill_split_merge_kernel<_Float16, D>), grid, dim3(256), 0, stream, a, nvec);
+  else hipLaunchKernelGGL((prefill_split_merge_kernel<__bf16, D>), grid, dim3(256), 0, stream, a, nvec);
+  return (int)hipGetLastError();
+}
+
+
 int launch_zero(const KArgs& a, int dtype, hipStream_t stream);
 struct KvAppendArgs {
   void* kc;

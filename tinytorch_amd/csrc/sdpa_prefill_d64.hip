@@ -44,7 +44,10 @@ typedef __attribute__((address_space(1))) const void gbl_void;
 
 __device__ __forceinline__ int swz(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
 
-template <typename TR, bool CAUSAL>
+// SPLIT (launches with very few row tiles): a workgroup takes key tiles kt0 .. kt0 + kv_chunk/64 - 1 of its row tile (kt0 a
+// multiple of 4, so the stages keep their constants) and leaves (unnormalised accumulator, maximum, sum) records in a.ws
+// for prefill_split_merge_kernel; row tiles are single (no mirror pairs).
+template <typename TR, bool CAUSAL, bool SPLIT>
 __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   constexpr bool PAGED = false;  // paged caches stay on the 4-wavefront kernel
   typedef typename TR::elem T;
@@ -62,7 +65,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   // Under a causal mask a workgroup takes row tile t and then its mirror ntile-1-t: every workgroup sees the same
   // number of KV tiles, so the launch has no long tail behind the heavy tiles.
   const int ntile = (a.L + BM - 1) / BM;
-  const bool paired = CAUSAL && !a.single_tiles;  // else one row tile per workgroup, longest first
+  const bool paired = CAUSAL && !SPLIT && !a.single_tiles;  // else one row tile per workgroup, longest first
+  const bool by_length = CAUSAL && !paired;  // work items ordered by row tile across the pairs of a class
   const int nslot = paired ? (ntile + 1) / 2 : ntile;
   const int inner = a.G * nslot;
   const int npair = a.B * a.Hkv;
@@ -72,14 +76,15 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
     // g = gcd(pairs, 8) the XCDs form g classes of 8/g, class x % g serves the pairs congruent to it and deals the
     // work items (heads x row tiles) of those pairs out to its XCDs in turn.  A multiple of 8 pairs puts every pair on
     // one XCD; 4 pairs (config 5) give each pair two XCDs instead of all eight streaming all four.
-    const int n = blockIdx.x;
+    int n = blockIdx.x;
+    if (SPLIT) n = (int)(blockIdx.x / (8u * a.kv_splits)) * 8 + (blockIdx.x & 7);  // the splits of a work item follow each other on its XCD
     const int gq = (npair & 7) == 0 ? 8 : ((npair & 3) == 0 ? 4 : ((npair & 1) == 0 ? 2 : 1));
     const int xcd = n & 7, slot = n >> 3;
     const int cls = xcd % gq, sub = xcd / gq;
     const long long item = (long long)slot * (8 / gq) + sub;  // work item of the class
     const long long items = (long long)(npair / gq) * inner;
     if (item >= items) return;  // the grid is rounded up to a multiple of 8
-    if (a.single_tiles) {  // longest tiles first across all the pairs of the class
+    if (by_length) {  // longest tiles first across all the pairs of the class
       const int ppc = npair / gq;
       pair = cls + gq * (int)(item % ppc);
       in = (int)(item / ppc);
@@ -92,6 +97,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   const int g = in % a.G;
   const int slot_rt = in / a.G;
   const int h = hk * a.G + g;
+  const int split = SPLIT ? (int)(blockIdx.x % (8u * a.kv_splits)) >> 3 : 0;
+  const int kt0 = SPLIT ? split * (a.kv_chunk / BN) : 0;  // first key tile of this workgroup
 
   const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
   const int* table = PAGED ? a.block_table + (long long)b * a.bt_stride : nullptr;
@@ -111,6 +118,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   const int rowgroup = (CAUSAL && wave >= 4) ? 11 - wave : wave;
 
   if (S == 0) {  // no keys for this batch entry: zeros, the reference's empty contraction (kept out of the main loop)
+    if (SPLIT) return;  // the merge kernel writes them
     T* obase = (T*)a.out + b * a.os[0] + h * a.os[1];
     vec8 zero;
 #pragma unroll
@@ -137,7 +145,16 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
       int lastkv = last < S - 1 ? last : S - 1;
       ntiles_kv = lastkv / BN + 1;
     }
+    if (SPLIT) {  // this workgroup's tiles end with its split (none at all: ntiles_kv <= kt0)
+      const int end = kt0 + a.kv_chunk / BN;
+      ntiles_kv = end < ntiles_kv ? end : ntiles_kv;
+    }
   };
+  if (SPLIT) {  // a split beyond the row tile's keys has nothing to do; the merge kernel knows which those are
+    int q0, ntiles_kv;
+    part_rows(0, q0, ntiles_kv);
+    if (ntiles_kv <= kt0) return;
+  }
   const bool two_parts = paired && slot_rt < ntile - 1 - slot_rt;  // odd count: the middle tile has no mirror
 
   // ---- global -> LDS: wavefront w moves rows 8w .. 8w+7 of a tile with one instruction (8 rows, 1 KiB) -----------
@@ -240,13 +257,13 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
     int q0, ntiles_kv;
     part_rows(part, q0, ntiles_kv);
     kpage[0] = -1, vpage[0] = -1;
-    dma_k(0, 0);
-    if (1 < ntiles_kv) dma_k(1, 1);
-    dma_v(0, 0);
-    if (2 < ntiles_kv) dma_k(2, 2);
-    if (1 < ntiles_kv) dma_v(1, 1);
-    if (3 < ntiles_kv) dma_k(3, 3);
-    if (2 < ntiles_kv) dma_v(2, 2);
+    dma_k(kt0, 0);
+    if (kt0 + 1 < ntiles_kv) dma_k(kt0 + 1, 1);
+    dma_v(kt0, 0);
+    if (kt0 + 2 < ntiles_kv) dma_k(kt0 + 2, 2);
+    if (kt0 + 1 < ntiles_kv) dma_v(kt0 + 1, 1);
+    if (kt0 + 3 < ntiles_kv) dma_k(kt0 + 3, 3);
+    if (kt0 + 2 < ntiles_kv) dma_v(kt0 + 2, 2);
   };
   issue_tiles(0);
   u32x16 qv;  // the lane's Q operands, k-step ks in elements 4ks .. 4ks+3
@@ -514,10 +531,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   {  // P(0) and the scores of half 1
+    const int kb = BN * kt0;  // the workgroup's first key (kt0 is a multiple of 4: its tile sits in stage 0)
     qk_half(sC, half_base(0));
-    if (1 < my_halves) qk_half(sB, half_base(1));
-    if ((CAUSAL && 31 > qc0) || 32 > S) mask_half(sC, 0);
-    if (!CAUSAL && a.mask_kind != 0) user_mask_half(sC, 0);
+    if (2 * kt0 + 1 < my_halves) qk_half(sB, half_base(1));
+    if ((CAUSAL && kb + 31 > qc0) || kb + 32 > S) mask_half(sC, kb);
+    if (!CAUSAL && a.mask_kind != 0) user_mask_half(sC, kb);
     // first half of a row: the maximum is formed directly (what the lazy rule arrives at after exponentials against
     // -1e30, with nothing to rescale yet); a fully hidden half keeps -1e30 and gives zeros
     m_use = fmaxf(m_use, row_max(sC));
@@ -548,8 +566,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   };
   // The fast form's requests: whole tiles through two running pointers (the general form multiplies the tile number
   // out and carries the ragged and paged cases); U = j % 4 makes the stages constants.
-  const char* kfast = (const char*)(kp + (long long)(4 * BN) * a.ks[2]);
-  const char* vfast = (const char*)(vp + (long long)(3 * BN) * a.vs[2]);
+  const char* kfast = (const char*)(kp + (long long)((kt0 + 4) * BN) * a.ks[2]);
+  const char* vfast = (const char*)(vp + (long long)((kt0 + 3) * BN) * a.vs[2]);
   const long long kfast_step = (long long)BN * a.ks[2] * 2, vfast_step = (long long)BN * a.vs[2] * 2;
   auto tile_dma_fast = [&](int j, int U) __attribute__((always_inline)) {
     int keep = 0;
@@ -566,8 +584,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
     vfast += vfast_step;
     return keep;
   };
-  int j = 0;
-  if (nfast_all >= 1) {
+  int j = kt0;
+  if (nfast_all >= kt0 + 1) {
     auto settle_fast = [&](f32x16& s, u32x8& pv, int masked_kv0) __attribute__((always_inline)) {
       vec8 p[2];
       p_load(pv, p);
@@ -627,6 +645,26 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
     load_q(1);
   }
 
+  if constexpr (SPLIT) {  // a partial result: unnormalised accumulator, the maximum it is relative to, the sum
+    const float l_part = l_run + __shfl_xor(l_run, 32);
+    int ln;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+    const int qi = qw0 + (ln & 31);
+    if (qi < a.L) {
+      float* rec = a.ws + (((long long)(b * a.Hq + h) * a.kv_splits + split) * a.L + qi) * (D + 2);  // 8-byte aligned
+#pragma unroll
+      for (int db = 0; db < 2; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          float* dst = rec + 32 * db + 8 * rg + 4 * (ln >> 5);
+          *(float2*)dst = make_float2(oacc[db][4 * rg], oacc[db][4 * rg + 1]);
+          *(float2*)(dst + 2) = make_float2(oacc[db][4 * rg + 2], oacc[db][4 * rg + 3]);
+        }
+      if ((ln >> 5) == 0) rec[D] = m_use, rec[D + 1] = l_part;
+    }
+    return;
+  }
+
   // ---- normalise, transpose through LDS, store whole rows -----------------------------------------------------------------
   // A lane holds 4 consecutive head_dim elements per register group of its query row: stored directly, every store
   // instruction would touch 32 rows with 16 bytes each.  Instead each wavefront stages its 32 rows in its 4 KiB of the
@@ -673,14 +711,19 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   }  // part
 }
 
-template <typename TR, bool CAUSAL>
-int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
+template <typename TR, bool CAUSAL, bool SPLIT>
+int launch_v(const KArgs& a, dim3 grid, hipStream_t stream) {
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)prefill64_kernel<TR, CAUSAL>, LDS_BYTES, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill64_kernel<TR, CAUSAL, SPLIT>, LDS_BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
-  hipLaunchKernelGGL((prefill64_kernel<TR, CAUSAL>), grid, dim3(NW * 64), LDS_BYTES, stream, a);
+  hipLaunchKernelGGL((prefill64_kernel<TR, CAUSAL, SPLIT>), grid, dim3(NW * 64), LDS_BYTES, stream, a);
   return (int)hipGetLastError();
+}
+
+template <typename TR, bool CAUSAL>
+int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
+  return a.kv_splits > 1 ? launch_v<TR, CAUSAL, true>(a, grid, stream) : launch_v<TR, CAUSAL, false>(a, grid, stream);
 }
 
 }  // namespace
@@ -695,7 +738,10 @@ int launch_prefill_d64(const KArgs& args, int dtype, hipStream_t stream) {
   // head_dim 128, bf16, against pairs: 128 pairs of 2048 rows +19 %, 224 of 1024 rows +28 %, 320 of 4096 rows +25 %,
   // of 2048 rows +17 %, 640 of 2048 rows +4.5 %, 896 of 2048 rows +4 %, of 16384 rows +4 %; with full rounds -2.5 %
   // to +0.5 % (512 pairs of 1024 / 2048 / 4096 rows, 768 of 4096 rows).
-  if (a.causal && ntile > 1) {
+  if (a.kv_splits > 1) {  // split keys: single row tiles whether causal or not
+    a.single_tiles = 1;
+    nwg = (long long)a.B * a.Hq * ntile;
+  } else if (a.causal && ntile > 1) {
     const long long rounds = (nwg + 255) / 256;
     if (nwg < 256 || nwg * 10 < rounds * 256 * 9) {
       a.single_tiles = 1;
@@ -710,9 +756,13 @@ int launch_prefill_d64(const KArgs& args, int dtype, hipStream_t stream) {
     const long long slots = (per_class + 8 / gq - 1) / (8 / gq);  // per XCD of the class
     nwg = slots * 8;
   }
+  if (a.kv_splits > 1) nwg *= a.kv_splits;
   dim3 grid((unsigned)nwg);
-  if (dtype == 1) return a.causal ? launch_k<F16, true>(a, grid, stream) : launch_k<F16, false>(a, grid, stream);
-  return a.causal ? launch_k<BF16, true>(a, grid, stream) : launch_k<BF16, false>(a, grid, stream);
+  int rc;
+  if (dtype == 1) rc = a.causal ? launch_k<F16, true>(a, grid, stream) : launch_k<F16, false>(a, grid, stream);
+  else rc = a.causal ? launch_k<BF16, true>(a, grid, stream) : launch_k<BF16, false>(a, grid, stream);
+  if (rc != 0 || a.kv_splits <= 1) return rc;
+  return launch_prefill_split_merge<D>(a, dtype, stream);
 }
 
 }  // namespace ttsdpa

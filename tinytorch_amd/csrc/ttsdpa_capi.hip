@@ -124,17 +124,26 @@ bool pipelined_ok(const ttsdpa_params* p) {
   return p->D == 128 && p->L > 128 && p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22);
 }
 
+// Shapes whose row tiles the pipelined kernels divide among workgroups by keys (plan_pipelined_splits): `units` 256-row
+// tiles in all, `keys` = what a row can see (under a top-left aligned causal mask no more than there are rows).
+bool split_shape(const ttsdpa_params* p, long long* units, long long* keys) {
+  *units = (long long)p->B * p->Hq * ((p->L + 255) / 256);
+  *keys = effective_causal(p) == TTSDPA_CAUSAL_TOP_LEFT && p->L < p->S ? p->L : p->S;
+  if (p->mask_kind != TTSDPA_MASK_NONE || p->block_table || *units > 128 || *keys < 2048) return false;
+  return *units <= 64 || (p->causal && *keys >= 4096);
+}
+
 // The pipelined kernel at head_dim 64: no attnMask, no pages.  Against the 4-wavefront kernel (128-row tiles, keys
-// divided among workgroups) it measured level or up to 30 % faster from 512 query rows on, except under a causal mask
-// with fewer row tiles than CUs and more than 4096 keys (4 heads x 8192: 12 % slower — the launch then ends with its
-// longest row tile, which the other kernel splits); shorter calls take it when they fill half of the chip's CUs.
+// divided among workgroups when the heads are not grouped) it measured level or up to 30 % faster from 512 query rows
+// on; shorter calls take it when they fill half of the chip's CUs, or when their keys are split (16 heads x 256 rows on
+// 32768 keys: 0.56 ms on the 4-wavefront kernel, which cannot split grouped heads).
 bool pipelined64_ok(const ttsdpa_params* p) {
   if (p->D != 64 || p->L <= 128 || p->mask_kind != TTSDPA_MASK_NONE || p->block_table) return false;
   if (!(p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22))) return false;
   const long long tiles = (p->L + 255) / 256;
   if ((long long)p->B * p->Hq * (p->causal ? (tiles + 1) / 2 : tiles) >= 128) return true;
-  if (p->L < 512) return false;
-  return !(p->causal && p->S > 4096 && (long long)p->B * p->Hq * tiles < 256);
+  long long units, keys;
+  return p->L >= 512 || split_shape(p, &units, &keys);
 }
 
 // Few query rows per head against many keys on the 4-wavefront kernel: the G heads of a KV head share one row tile
@@ -180,7 +189,7 @@ SplitPlan plan_prefill_splits(const ttsdpa_params* p, const KArgs& a /* after pa
 }
 
 
-// Key splits for the pipelined head_dim-128 kernel: a call with a quarter as many 256-row tiles as the chip has CUs, or
+// Key splits for the pipelined kernels (head_dim 128 and 64): a call with a quarter as many 256-row tiles as the chip has CUs, or
 // fewer (a chunk of one sequence's rows against a long cache, a few heads of a tensor-parallel share), leaves most CUs
 // without work.  Its row tiles then share their keys among workgroups of `chunk` keys (a multiple of 256: four key
 // tiles, so the kernel's stages keep their constants), enough for two workgroups per CU, and the
@@ -189,12 +198,8 @@ SplitPlan plan_prefill_splits(const ttsdpa_params* p, const KArgs& a /* after pa
 // -9 %, 2048 keys -18 %); with 64 and fewer it measured 1.1x to 5x (32 heads x 512 rows on 8192 keys 1.5x).
 SplitPlan plan_pipelined_splits(const ttsdpa_params* p) {
   SplitPlan s{1, 0, 0};
-  if (p->dtype == TTSDPA_F32 || !pipelined_ok(p) || p->mask_kind != TTSDPA_MASK_NONE || p->block_table) return s;
-  const long long units = (long long)p->B * p->Hq * ((p->L + 255) / 256);
-  // keys a row can see: under a top-left aligned causal mask no more than there are rows
-  const long long keys = effective_causal(p) == TTSDPA_CAUSAL_TOP_LEFT && p->L < p->S ? p->L : p->S;
-  if (units > 128 || keys < 2048) return s;
-  if (units > 64 && !(p->causal && keys >= 4096)) return s;
+  long long units, keys;
+  if (p->dtype == TTSDPA_F32 || !(pipelined_ok(p) || pipelined64_ok(p)) || !split_shape(p, &units, &keys)) return s;
   long long want = (512 + units - 1) / units;
   const long long most = keys / 512;  // at least 8 key tiles per split
   if (want > most) want = most;
@@ -461,7 +466,14 @@ static int prefill_impl(const ttsdpa_params* p, void* workspace, size_t workspac
     a.kv_splits = 1, a.kv_chunk = 0, a.ws = nullptr;
     return launch_prefill_d128(a, p->dtype, (hipStream_t)stream);
   }
-  if (p->dtype != TTSDPA_F32 && pipelined64_ok(p)) return launch_prefill_d64(a, p->dtype, (hipStream_t)stream);
+  if (p->dtype != TTSDPA_F32 && pipelined64_ok(p)) {
+    const SplitPlan sp = plan_pipelined_splits(p);
+    if (sp.splits > 1 && workspace && workspace_bytes >= sp.ws_bytes && ptr_aligned(workspace, 16))
+      a.kv_splits = sp.splits, a.kv_chunk = sp.chunk, a.ws = (float*)workspace;
+    else
+      a.kv_splits = 1, a.kv_chunk = 0, a.ws = nullptr;
+    return launch_prefill_d64(a, p->dtype, (hipStream_t)stream);  // with splits: the kernel and the merge of its records
+  }
   auto launch = [&](const KArgs& k) {
     return p->dtype == TTSDPA_F32 ? launch_prefill_f32(k, (hipStream_t)stream) : launch_prefill(k, p->dtype, (hipStream_t)stream);
   };
