@@ -6,7 +6,8 @@
 A step is one call of the hot path (ttsdpa_forward through the C ABI) over one batch of synthetic input already
 resident in HBM.  The headline workload is "config3" (bf16 causal GQA prefill, B2 32q/8kv S4096 D128: the shape the
 prefill throughput target is quoted on); the decode workload "config4" (bf16, B64 32q/8kv KV 8192) is measured in the
-same run and reported under "secondary", config 3's shape in fp32 (the reference's default dtype,
+same run and reported under "secondary" and, in short, as "roofline"."decode" of the headline (the metric is prefill
+TFLOP/s + decode GB/s: both halves sit in the one object), config 3's shape in fp32 (the reference's default dtype,
 on the fp32 MFMA kernel, against the 157.3 TFLOP/s fp32 peak) under "fp32", and the row-wise neighbour ops (rmsNorm,
 fusedAddRmsNorm, siluMul, softmax; HBM-bound) under "fused_ops" and the linear layer (QKV projection of the same
 token batch; MFMA-bound) under "linear", and the attention backward (dq, dk, dv at config 3's shape; MFMA-bound) under
@@ -21,6 +22,10 @@ Inputs are drawn by tinytorch_amd.synth (counter-based normal generator, seed 0x
 per tensor), rounded to the workload's element type.
 The other configurations of the baseline (1, 2, 5) and config 3's shape at head_dim 64 are measured the same way and
 reported under "other_configs".
+
+"roofline"."zero_operands" is the headline launch repeated on all-zero Q, K, V: the same instruction stream without operand
+toggling, i.e. what the kernel's schedule reaches when the chip's power management leaves the clock alone (the prefill
+kernel is power-bound on N(0,1) data).  "roofline"."summary" lists the fraction of every other line of the run.
 
 Algorithmic work per launch (what "achieved" divides by the measured launch time):
   prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)
@@ -42,7 +47,24 @@ PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}  # MI355X dense MFMA
 PEAK_HBM_GBS = 8000.0
 SETTLE_SECONDS = 0.4   # untimed launches after the warm-up, until the core clock has settled under the kernel
 TRAFFIC_SOURCE = ("profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of the same "
-                  "command, scaled by a 1 GiB copy; not measured in this run")
+                  "command, scaled by a 1 GiB copy; not measured in this run")  # said once per line, under "traffic_source"
+PROBE_LIB = os.path.join(ROOT, "bench_probes", "libttbench_probes.so")
+_probe_lib = None
+
+
+def probe_lib():
+    """The measurement probes (bench_probes/probes.hip): a shared object of their own, not part of the product library."""
+    global _probe_lib
+    if _probe_lib is None:
+        import torch  # noqa: F401  (one HIP runtime per process: torch's)
+        if not os.path.exists(PROBE_LIB):
+            raise ImportError("bench.py: %s is missing; build it with `make -C bench_probes`" % PROBE_LIB)
+        L = ctypes.CDLL(PROBE_LIB)
+        L.ttbench_probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
+                                    ctypes.POINTER(ctypes.c_double)]
+        L.ttbench_probe.restype = ctypes.c_int
+        _probe_lib = L
+    return _probe_lib
 
 WORKLOADS = {
     # name: (B, Hq, Hkv, L, S, D, dtype, causal, input multiplier, bound)
@@ -139,12 +161,14 @@ def synth_qkv(name):
     return q, k, v
 
 
-def run_gpu(name, steps, warmup):
+def run_gpu(name, steps, warmup, zero_inputs=False):
     import torch
     from tinytorch_amd import _capi, build_params
 
     B, Hq, Hkv, L, S, D, dtype, causal, mul, bound = WORKLOADS[name]
     q, k, v = synth_qkv(name)
+    if zero_inputs:  # the same launch without operand toggling
+        q.zero_(), k.zero_(), v.zero_()
     out = torch.empty_like(q)
     p = build_params(q, k, v, out, causal)
     lib = _capi.lib()
@@ -174,7 +198,6 @@ def run_gpu(name, steps, warmup):
         "value": round(value, 3), "unit": unit, "ms_per_step": round(wall_ms, 5),
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
                      "frac": round(achieved / peak, 4), "traffic": measured_traffic(name),
-                     "traffic_source": TRAFFIC_SOURCE if measured_traffic(name) is not None else None,
                      "kernel_ms": round(dev_ms, 5), "kernel_ms_mean": round(t["mean_ms"], 5),
                      "kernel_ms_min": round(t["min_ms"], 5), "timing": "median of %d launches, one HIP event pair each" % steps,
                      "settle_launches": t["settle_launches"], "algorithmic_flops": flops, "algorithmic_bytes": abytes},
@@ -183,23 +206,23 @@ def run_gpu(name, steps, warmup):
 
 
 def run_probes():
-    """What this GPU sustains on the two bounding resources, measured with the library's probe kernels (ttsdpa_probe):
-    a register-only MFMA loop and a streaming read of 1 GiB, plain and nontemporal.  HIP events on the launch stream."""
+    """What this GPU sustains on the two bounding resources, measured with the probe kernels of bench_probes/ (a shared
+    object of their own): a register-only MFMA loop on constant and on random operands, and a streaming read of 1 GiB,
+    plain and nontemporal.  HIP events on the launch stream."""
     import torch
-    from tinytorch_amd import _capi
 
-    lib = _capi.lib()
+    lib = probe_lib()
     stream = torch.cuda.current_stream()
     buf = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
     out = {}
-    for key, kind, iters, reps, unit in (("mfma_loop", 0, 20000, 300, 1e12), ("read_plain", 1, 1, 300, 1e9),
-                                         ("read_nontemporal", 2, 1, 300, 1e9)):
+    for key, kind, iters, reps, unit in (("mfma_loop", 0, 20000, 300, 1e12), ("mfma_loop_random", 3, 20000, 300, 1e12),
+                                         ("read_plain", 1, 1, 300, 1e9), ("read_nontemporal", 2, 1, 300, 1e9)):
         work = ctypes.c_double(0.0)
 
         def go():
-            rc = lib.ttsdpa_probe(kind, buf.data_ptr(), buf.numel(), iters, stream.cuda_stream, ctypes.byref(work))
+            rc = lib.ttbench_probe(kind, buf.data_ptr(), buf.numel(), iters, stream.cuda_stream, ctypes.byref(work))
             if rc != 0:
-                raise RuntimeError("ttsdpa_probe: %s" % _capi.status_string(rc))
+                raise RuntimeError("ttbench_probe: status %d" % rc)
         for _ in range(reps):
             go()
         torch.cuda.synchronize()
@@ -213,9 +236,10 @@ def run_probes():
         out[key] = round(work.value / (ms * 1e-3) / unit, 1)
     del buf
     torch.cuda.empty_cache()
-    return {"mfma_loop_tflops": out["mfma_loop"], "read_plain_gbs": out["read_plain"],
-            "read_nontemporal_gbs": out["read_nontemporal"],
-            "note": "sustained by ttsdpa_probe kernels in this run: bf16 32x32x16 MFMA loop, 1 GiB streaming reads"}
+    return {"mfma_loop_tflops": out["mfma_loop"], "mfma_loop_random_operands_tflops": out["mfma_loop_random"],
+            "read_plain_gbs": out["read_plain"], "read_nontemporal_gbs": out["read_nontemporal"],
+            "note": "sustained by the bench_probes kernels in this run: register-only bf16 32x32x16 MFMA loop on constant and on "
+                    "random operands (the chip lowers its clock under the latter), 1 GiB streaming reads"}
 
 
 FUSED_WORKLOADS = {
@@ -275,8 +299,7 @@ def run_fused(name, steps, warmup, cpu=True):
                 "kernel_ms_mean": round(t["mean_ms"], 5), "settle_launches": t["settle_launches"],
                 "roofline": {"bound": "hbm", "achieved": round(abytes / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                              "unit": "GB/s", "frac": round(abytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                             "traffic": measured_traffic(name), "traffic_source": TRAFFIC_SOURCE,
-                             "algorithmic_bytes": abytes}}
+                             "traffic": measured_traffic(name), "algorithmic_bytes": abytes}}
     if cpu:
         import oracle
         kind = "reference" if oracle.have_ref() else "port"
@@ -342,7 +365,7 @@ def run_linear(steps, warmup, cpu=True):
            "kernel_ms_mean": round(t["mean_ms"], 5), "settle_launches": t["settle_launches"],
            "roofline": {"bound": "mfma", "achieved": round(flops / (ms * 1e-3) / 1e12, 1), "peak": PEAK_TFLOPS["bf16"],
                         "unit": "TFLOP/s", "frac": round(flops / (ms * 1e-3) / 1e12 / PEAK_TFLOPS["bf16"], 4),
-                        "traffic": measured_traffic("linear"), "traffic_source": TRAFFIC_SOURCE, "algorithmic_flops": flops,
+                        "traffic": measured_traffic("linear"), "algorithmic_flops": flops,
                         "algorithmic_bytes": 2 * (M * K + N * K + M * N + N)}}
     if cpu:
         import oracle
@@ -409,7 +432,7 @@ def run_backward(steps, warmup, cpu=True, dtype="bf16"):
            "settle_launches": t["settle_launches"], "value": round(tf, 1), "unit": "TFLOP/s",
            "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_TFLOPS[dtype], "unit": "TFLOP/s",
                         "frac": round(tf / PEAK_TFLOPS[dtype], 4),
-                        "traffic": measured_traffic("backward" if dtype == "bf16" else "backward_f32"), "traffic_source": TRAFFIC_SOURCE,
+                        "traffic": measured_traffic("backward" if dtype == "bf16" else "backward_f32"),
                         "algorithmic_flops": flops, "kernels": kernels + " per step"}}
     if cpu:
         import oracle
@@ -484,6 +507,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-probes", action="store_true", help="skip the hardware ceiling probes")
+    ap.add_argument("--no-zero", action="store_true", help="skip the repeat of the headline launch on all-zero operands")
     ap.add_argument("--settle", type=float, default=None,
                     help="seconds of untimed launches after the warm-up (default %.1f; 0 for counter runs that only need a few dispatches)" % SETTLE_SECONDS)
     ap.add_argument("--no-other", action="store_true", help="skip the baseline's other configurations (1, 2, 5) and head_dim 64")
@@ -527,6 +551,18 @@ def main():
     cpu = None if args.no_cpu else run_cpu_baseline(args.workload, tensors, args.cpu_seconds)
     del tensors
     torch.cuda.empty_cache()
+    main_res["roofline"]["traffic_source"] = TRAFFIC_SOURCE  # for every "traffic" figure of this line
+    if not args.no_zero and WORKLOADS[args.workload][9] == "mfma":
+        # the same launch on all-zero operands: the instruction stream without operand toggling (the kernel is power-bound
+        # on N(0,1) data: the chip lowers its clock under it)
+        z, tensors = run_gpu(args.workload, args.steps, args.warmup, zero_inputs=True)
+        del tensors
+        torch.cuda.empty_cache()
+        main_res["roofline"]["zero_operands"] = {
+            "kernel_ms": z["roofline"]["kernel_ms"], "achieved": z["roofline"]["achieved"], "frac": z["roofline"]["frac"],
+            "note": "the same launch with Q = K = V = 0: identical instruction stream, no operand toggling; not a result, "
+                    "the clock the power management grants is the difference"}
+    summary = {}
     line = {
         "metric": "attn prefill TFLOP/s + decode KV GB/s on 1 MI355X (% of roofline)",
         "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps,
@@ -542,10 +578,18 @@ def main():
         sec["cpu_baseline"] = None if args.no_cpu else run_cpu_baseline(args.secondary, tensors, args.cpu_seconds)
         del tensors
         line["secondary"] = sec
+        if args.secondary == "config4":  # the metric's second half, inside the object that is kept whole
+            r = sec["roofline"]
+            line["roofline"]["decode"] = {
+                "workload": "config4: " + sec["description"], "bound": r["bound"], "achieved": r["achieved"], "peak": r["peak"],
+                "unit": r["unit"], "frac": r["frac"], "kernel_ms": r["kernel_ms"], "traffic": r["traffic"],
+                "algorithmic_bytes": r["algorithmic_bytes"], "settle_launches": r["settle_launches"],
+                "cpu_baseline": sec["cpu_baseline"]}
         if args.workload == "config3":  # the same shape in fp32, against the fp32 MFMA peak (no CPU leg: same arithmetic as config 3's)
             f32, tensors = run_gpu("config3_f32", max(1, min(args.steps, 100)), min(args.warmup, 20))
             del tensors
             line["fp32"] = f32
+            summary["config3_f32"] = f32["roofline"]["frac"]
     if not args.no_other and args.workload == "config3":
         # the baseline's other configurations (config 1: launch-sized, its time is the figure) and head_dim 64
         line["other_configs"] = []
@@ -557,6 +601,7 @@ def main():
                 res["cpu_baseline"] = run_cpu_baseline(name, tensors, budget, corner)
             del tensors
             line["other_configs"].append(res)
+            summary[name] = res["roofline"]["kernel_ms"] if name == "config1" else res["roofline"]["frac"]
     if not args.no_fused:
         torch.cuda.empty_cache()
         line["fused_ops"] = [run_fused(n, max(1, min(args.steps, 100)), min(args.warmup, 20), cpu=not args.no_cpu)
@@ -566,6 +611,13 @@ def main():
         torch.cuda.empty_cache()
         line["backward"] = run_backward(max(1, min(args.steps, 50)), min(args.warmup, 20), cpu=not args.no_cpu)
         line["backward"]["fp32"] = run_backward(max(1, min(args.steps, 10)), min(args.warmup, 3), cpu=False, dtype="f32")
+        for r in line["fused_ops"]:
+            summary[r["workload"].split()[0]] = r["roofline"]["frac"]
+        summary["linear"] = line["linear"]["roofline"]["frac"]
+        summary["backward_bf16"] = line["backward"]["roofline"]["frac"]
+        summary["backward_f32"] = line["backward"]["fp32"]["roofline"]["frac"]
+    if summary:  # fraction of its own roofline for every other line of this run (config1: launch-sized, its kernel ms)
+        line["roofline"]["summary"] = summary
     print(json.dumps(line), flush=True)
 
 

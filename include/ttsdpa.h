@@ -240,16 +240,6 @@ typedef struct ttsdpa_kv_append_params {
 void ttsdpa_kv_append_params_init(ttsdpa_kv_append_params* p, int dtype, int B, int Hkv, int Smax, int Lnew, int D);
 int ttsdpa_kv_append(const ttsdpa_kv_append_params* p, void* stream);
 
-/*
- * Measurement probes (no counterpart in the reference; for benchmarks, not for the attention path): enqueue one kernel
- * that exercises a single resource, so a caller can time what this GPU sustains next to the attention kernels.
- *   kind 0: register-only loop of `iters` pairs of v_mfma_f32_32x32x16_bf16 per wavefront, 2048 wavefronts;
- *   kind 1: streaming read of `buffer` (16-byte loads);  kind 2: the same with nontemporal loads.
- * `buffer` is device memory of `bytes` bytes (16-byte aligned; >= 64 MiB is sensible for the reads, 64 bytes suffice
- * for kind 0).  *work receives the flop (kind 0) or the bytes read (kinds 1, 2) of the enqueued launch.
- */
-int ttsdpa_probe(int kind, void* buffer, size_t bytes, int iters, void* stream, double* work);
-
 #ifdef __cplusplus
 }
 #endif

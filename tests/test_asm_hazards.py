@@ -42,3 +42,25 @@ def test_the_checker_sees_the_hazard(tmp_path):
     tool = os.path.join(CSRC, "check_asm_hazards.py")
     assert subprocess.run([sys.executable, tool, str(bad)], capture_output=True).returncode == 1
     assert subprocess.run([sys.executable, tool, str(good)], capture_output=True).returncode == 0
+
+
+def test_the_checker_passes_nothing_asm_issued_that_it_cannot_classify(tmp_path):
+    tool = os.path.join(CSRC, "check_asm_hazards.py")
+    run = lambda name, text: (tmp_path / name).write_text(text) and subprocess.run(
+        [sys.executable, tool, str(tmp_path / name)], capture_output=True, text=True)
+    asm = lambda body: "\ts_add_u32 s4, s4, 1\n\t;;#ASMSTART\n%s\t;;#ASMEND\n" % body
+    # a statement with its own five wait states in front of the load: proven whatever ran before it
+    assert run("ok.s", ".LBB0_1:\n" + asm("\ts_mov_b32 m0, s9\n\ts_nop 3\n\tglobal_load_lds_dwordx4 v1, s[2:3]\n")).returncode == 0
+    # the same load at the head of a statement behind a label: nothing is known about the path that led here
+    r = run("label.s", ".LBB0_1:\n" + asm("\tglobal_load_dwordx4 v[0:3], v4, s[2:3]\n"))
+    assert r.returncode == 1 and "provably" in r.stdout
+    # a scalar compare result written by a vector instruction three instructions before the statement's load
+    r = run("cmp.s", "\tv_cmp_lt_i32_e64 s[2:3], v0, v1\n\ts_nop 0\n" + asm("\ts_nop 0\n\tbuffer_load_dword v1, v2, s[0:3], 0 offen\n"))
+    assert r.returncode == 1
+    # no scalar base: nothing to prove
+    assert run("off.s", ".LBB0_1:\n" + asm("\tglobal_load_dwordx4 v[0:3], v[4:5], off\n")).returncode == 0
+    # scalar-memory instructions and unknown mnemonics in a statement are findings, not passes
+    r = run("smem.s", asm("\ts_load_dwordx2 s[2:3], s[0:1], 0x0\n"))
+    assert r.returncode == 1 and "unclassified" in r.stdout
+    r = run("unknown.s", asm("\timage_load v[0:3], v4, s[0:7] dmask:0xf\n"))
+    assert r.returncode == 1 and "cannot classify" in r.stdout

@@ -178,14 +178,12 @@ def test_kv_len_routes_and_append_validation():
     assert L.ttsdpa_kv_append(ctypes.byref(kp), None) == 0
 
 
-def test_probe_argument_checks():
+def test_product_library_holds_no_bench_probes():
+    # the measurement probes are bench tooling with a shared object of their own (bench_probes/)
     L = _capi.lib()
-    w = ctypes.c_double(0.0)
-    assert L.ttsdpa_probe(0, None, 64, 10, None, ctypes.byref(w)) == _capi.ERR_NULL
-    assert L.ttsdpa_probe(0, FAKE, 64, 10, None, None) == _capi.ERR_NULL
-    assert L.ttsdpa_probe(7, FAKE, 64, 10, None, ctypes.byref(w)) == _capi.ERR_UNSUPPORTED
-    assert L.ttsdpa_probe(1, FAKE + 4, 1 << 26, 1, None, ctypes.byref(w)) == _capi.ERR_UNSUPPORTED  # not 16-byte aligned
-    assert L.ttsdpa_probe(1, FAKE, 1024, 1, None, ctypes.byref(w)) == _capi.ERR_SHAPE                 # buffer too small
+    assert not hasattr(L, "ttsdpa_probe") and not hasattr(L, "ttbench_probe")
+    with open(os.path.join(ROOT, "include", "ttsdpa.h")) as f:
+        assert "probe" not in f.read()
 
 
 def test_kernel_domains_and_workspace():

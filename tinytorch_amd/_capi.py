@@ -21,7 +21,7 @@ STATIC_SCRATCH_BYTES = 2 << 20
 EXPORTS = [
     "ttsdpa_abi_version", "ttsdpa_status_string", "ttsdpa_params_init", "ttsdpa_plan", "ttsdpa_workspace_bytes",
     "ttsdpa_forward", "ttsdpa_prefill", "ttsdpa_decode", "ttsdpa_decode_static", "ttsdpa_general",
-    "ttsdpa_kv_append_params_init", "ttsdpa_kv_append", "ttsdpa_probe",
+    "ttsdpa_kv_append_params_init", "ttsdpa_kv_append",
     "ttsdpa_backward_params_init", "ttsdpa_backward_plan", "ttsdpa_backward_workspace_bytes", "ttsdpa_backward",
     # include/ttfused.h
     "ttfused_rms_norm", "ttfused_add_rms_norm", "ttfused_silu_mul", "ttfused_softmax", "ttfused_softmax_backward",
@@ -145,9 +145,6 @@ def lib():
         L.ttsdpa_backward_workspace_bytes.restype = ctypes.c_size_t
         L.ttsdpa_backward.argtypes = [BP, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         L.ttsdpa_backward.restype = ctypes.c_int
-        L.ttsdpa_probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
-                                   ctypes.POINTER(ctypes.c_double)]
-        L.ttsdpa_probe.restype = ctypes.c_int
         vp, i64 = ctypes.c_void_p, ctypes.c_int64
         L.ttfused_rms_norm.argtypes = [ctypes.c_int, vp, vp, vp, i64, i64, ctypes.c_float, vp]
         L.ttfused_rms_norm.restype = ctypes.c_int

@@ -460,8 +460,6 @@ struct KvAppendArgs {
   long long kcs[3], vcs[3], kns[3], vns[3];
 };
 int launch_kv_append(const KvAppendArgs& a, hipStream_t stream);
-// measurement probes: kind 0 matrix-pipe loop, 1 streaming read, 2 nontemporal streaming read; *work = flop or bytes
-int launch_probe(int kind, void* buffer, size_t bytes, int iters, hipStream_t stream, double* work);
 
 // Decode tiling, shared by the workspace-size query and the launcher.
 struct DecodePlan {

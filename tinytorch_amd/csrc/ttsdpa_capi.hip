@@ -624,11 +624,4 @@ int ttsdpa_kv_append(const ttsdpa_kv_append_params* p, void* stream) {
   return launch_kv_append(a, (hipStream_t)stream);
 }
 
-int ttsdpa_probe(int kind, void* buffer, size_t bytes, int iters, void* stream, double* work) {
-  if (!buffer || !work) return TTSDPA_ERR_NULL;
-  if (kind < 0 || kind > 2 || iters < 1 || !ptr_aligned(buffer, 16)) return TTSDPA_ERR_UNSUPPORTED;
-  const int rc = launch_probe(kind, buffer, bytes, iters, (hipStream_t)stream, work);
-  return rc < 0 ? TTSDPA_ERR_SHAPE : rc;
-}
-
 }  // extern "C"
