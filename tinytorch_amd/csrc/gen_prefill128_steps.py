@@ -26,11 +26,18 @@ Every string holds the step twice: as above, and with the causal predicate appli
 key is visible iff kvs + 8*(n/4) + n%4 <= rl: two more instructions per score, a compare through m0 and vcc and a
 select).  The second form serves the one or two tiles of a wavefront's row group that touch the diagonal; it sits out
 of line, in subsection 1 of the kernel's section, so that the steady state falls through without a taken branch.
+
+Calls with a Bool attnMask (head_dim 128) have a third form of the plain step, TT_P128_MSTEP_...: a score's probability is
+kept iff its mask byte is set (a compare on one byte of a register through SDWA and a select: two more instructions per
+score).  A lane's 16 mask bytes of a 32-key half are four dwords (keys 8g + 4*(lane/32) .. +3 of the lane's query row, g = 0..3) in
+    v[104:119]  mask ring: 4 halves x 4 dwords, half H in place H % 4
+loaded one tile ahead by TT_P128_MLOAD_E / _O (tiles with even / odd index in the unrolled body; operands: the lane's byte offset
+and the scalar address of the tile's first mask byte) and TT_P128_MLOAD_FIRST (halves 1 and 2 of a workgroup's first tile).
 """
 import sys
 
 PD, RING = 6, 8
-Q0, VADDR0, SB0, SC0, PA0, PB0, RING0, T0, KADDR0 = 120, 152, 160, 176, 192, 200, 208, 240, 248
+MASK0, Q0, VADDR0, SB0, SC0, PA0, PB0, RING0, T0, KADDR0 = 104, 120, 152, 160, 176, 192, 200, 208, 240, 248
 # set by configure(head_dim): k-steps of a score product (= P.V products of a half), head_dim blocks of 32, slots of a
 # step, scores whose vector work a slot carries, bytes of a tile row and of a stage, slots of the 4-tile body
 KST = NDB = NS = SPS = ROW = STAGE = BODY = 0
@@ -71,7 +78,7 @@ def pending_after(G):
     return sum(len(fetch(g)) for g in range(G + 1, G + PD))
 
 
-def step(u, kind, elem, masked=False):
+def step(u, kind, elem, masked=False, bmask=False):
     mfma = "v_mfma_f32_32x32x16_%s" % elem
     cvt = "v_cvt_pk_%s_f32" % elem
     G0 = 2 * NS * u + NS * kind
@@ -92,6 +99,10 @@ def step(u, kind, elem, masked=False):
             w.append(fma(n + 1))
         if masked:
             w += hide(n)
+        if bmask:  # keep the probability iff the score's mask byte is set: byte n%4 of dword n/4 of the half's place in the ring
+            place = (2 * u + kind + 1) & 3  # the step takes the exponentials of half 2j + kind + 1, j = u (mod 4)
+            w += ["v_cmp_ne_u32_sdwa vcc, %s, %%[zero] src0_sel:BYTE_%d src1_sel:DWORD" % (vr(MASK0 + 4 * place + (n >> 2)), n & 3),
+                  "v_cndmask_b32 %s, 0, %s, vcc" % (vr(T[n & 3]), vr(T[n & 3]))]
         if n == 2:  # the sum starts as (score 0) + (score 1): what 0 + x0 + x1 gives
             w.append("v_add_f32 %%[ps], %s, %s" % (vr(T[0]), vr(T[1])))
         elif n >= 3:
@@ -130,6 +141,16 @@ def prefetch():
     return out
 
 
+def mask_loads(halves, base):
+    """Loads of the mask dwords of `halves` (index relative to the tile whose first mask byte the scalar operand points at, plus
+    `base` bytes) into their ring places; s_nop 4: the scalar address may have been restored by a vector instruction."""
+    out = ["s_nop 4"]
+    for rel, place in halves:
+        for g in range(4):
+            out.append("global_load_dword %s, %%[moff], %%[mtile] offset:%d" % (vr(MASK0 + 4 * place + g), base + 32 * rel + 8 * g))
+    return out
+
+
 def emit(name, lines):
     print("#define %s \\" % name)
     print(" \\\n".join('  "%s\\n\\t"' % l for l in lines))
@@ -156,6 +177,14 @@ def main():
                         + step(u, kind, elem, True) + ["s_branch %s_e%%=" % lab, ".subsection 0"])
                 emit("TT_%s_STEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), both)
                 emit("TT_%s_PSTEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), step(u, kind, elem))  # calls without a causal mask
+                if head_dim == 128:
+                    emit("TT_%s_MSTEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), step(u, kind, elem, bmask=True))  # Bool attnMask
+    if head_dim == 128:
+        # tile j (first mask byte at the scalar operand) sends for halves 2j+3 and 2j+4: places (2u+3)%4 and (2u+4)%4, u = j%4
+        emit("TT_%s_MLOAD_E" % NAME, mask_loads([(3, 3), (4, 0)], 0))
+        emit("TT_%s_MLOAD_O" % NAME, mask_loads([(3, 1), (4, 2)], 0))
+        # before the first tile (an index that is a multiple of 4): halves 1 and 2 of that tile, then everything in place
+        emit("TT_%s_MLOAD_FIRST" % NAME, mask_loads([(1, 1), (2, 2)], 0) + ["s_waitcnt vmcnt(0)"])
 
 
 if __name__ == "__main__":

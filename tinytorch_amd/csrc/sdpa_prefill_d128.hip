@@ -44,8 +44,11 @@
 // applied to each probability (selected by a scalar flag), so that only a row group's last one or two steps take the
 // general form.  The eight row groups of a workgroup reach the diagonal in eight different tiles, and with the
 // general form on every one of them each of the workgroup's last five tiles waited for one wavefront in that form.
-// Under a causal mask a workgroup takes a row tile and its mirror (equal work for every workgroup), and neighbouring
-// workgroups take the two in opposite order so their load/store bursts do not coincide.
+// Under a causal mask a workgroup takes a row tile and its mirror (equal work for every workgroup), the long one first.
+// A Bool attnMask whose keys can be read four at a time (variant MASKB; the reference's masked fill, src/Function/FuncNNLayer.h:249-255)
+// stays in the pipelined form as well: a lane's 16 mask bytes of a half are four dwords, loaded one tile ahead into a ring of
+// 16 registers, and the step's streams keep a probability iff its byte is set (a byte compare through SDWA and a select per
+// score).  Other masks (additive, other layouts) take the general form of a step.
 // Grouped-query attention: kv head = query head / (Hq/Hkv), resolved in the kernel; the workgroup order puts the
 // query heads and row tiles that share a KV head on the same XCD so its L2 holds that K/V once.
 
@@ -69,6 +72,7 @@ constexpr int LDS_BYTES = (KSTAGES + VSTAGES) * STAGE_BYTES + OUT_BYTES;
 constexpr float kSumLimit = 1024.f;  // a lane's 16 probabilities of a half may sum to this much before the maximum is raised
 
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x32 __attribute__((ext_vector_type(32)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -83,8 +87,11 @@ __device__ __forceinline__ int swz(int row) { return ((row & 3) << 2) | ((row >>
 // SPLIT (launches with fewer row tiles than the chip needs): a workgroup takes key tiles kt0 .. kt0 + kv_chunk/64 - 1 of
 // its row tile (kt0 a multiple of 4, so the stages keep their constants) and leaves (unnormalised accumulator, maximum,
 // sum) records in a.ws for the merge kernel of the decode path; row tiles are single (no mirror pairs).
-template <typename TR, bool CAUSAL, bool PAGED, bool SPLIT>
+// MASKB (calls without a causal mask, pages or splits): a.mask is a Bool mask with unit key stride, dword-aligned rows and
+// row offsets below 2^32; the steady state applies it in the streams.
+template <typename TR, bool CAUSAL, bool PAGED, bool SPLIT, bool MASKB = false>
 __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
+  static_assert(!MASKB || (!CAUSAL && !PAGED && !SPLIT), "the Bool-mask streams exist for the plain variant only");
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
 
@@ -145,9 +152,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     S = len < 0 ? 0 : (len < S ? len : S);
   }
 
-  // Neighbouring workgroups take their two tiles in opposite order, so that the load / store bursts between the
-  // parts of one half of the workgroups fall into the steady loops of the other half.
-  const bool long_first = !paired || ((blockIdx.x >> 3) & 1) == 0;
+  // Every workgroup takes its long tile first: the workgroups of a head that run together then walk its keys from the
+  // first one on in step, and an XCD's L2 serves all but the first of them.  (With neighbouring workgroups in opposite
+  // order a head's K/V came from memory about three times where one KV head serves one query head: B4 32 heads of 2048
+  // rows, fp16: 468 -> 275 MB read per launch, same time; grouped heads were and are read once.)
+  const bool long_first = true;
   // Wavefronts w and w+4 share a SIMD.  Under a causal mask the row group g of a tile has g+1 halves of work on the
   // diagonal, so the second four wavefronts take the groups in reverse: every SIMD then carries groups g and 7-g.
   const int rowgroup = (CAUSAL && wave >= 4) ? 11 - wave : wave;
@@ -305,6 +314,25 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     if (kt0 + 2 < ntiles_kv) dma_v(kt0 + 2, 2);
   };
   issue_tiles(0);
+  // ---- Bool attnMask in the streams (MASKB): a lane's mask bytes, four keys per dword -------------------------------------
+  // half H of the workgroup's keys sits in places 4(H%4) .. +3 of the ring: dword g = keys 32H + 8g + 4(lane/32) .. +3 of the
+  // lane's query row.  A tile sends for the halves its successor takes (two statements by the tile's parity in the
+  // unrolled body, TT_P128_MLOAD_E / _O), ahead of its K/V loads: the wait at the tile's end covers them.
+  u32x16 mring;
+  unsigned moff = 0;              // the lane's byte offset in the mask: its query row and its four keys of a group
+  const char* mbase = nullptr;    // first mask byte of this (batch, head); uniform
+  if constexpr (MASKB) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) mring[i] = 0u;
+    int q0, ntiles_kv;
+    part_rows(0, q0, ntiles_kv);
+    int qi = q0 + rowgroup * WM + lq;
+    qi = qi < a.L ? qi : a.L - 1;
+    moff = (unsigned)qi * (unsigned)a.ms[2] + 4u * lh;  // the host checks that the last row's offset fits 32 bits
+    mbase = (const char*)a.mask + b * a.ms[0] + h * a.ms[1];
+    if (S >= 160)  // (shorter rows have no tile in the fast form)
+      asm volatile(TT_P128_MLOAD_FIRST : "+{v[104:119]}"(mring) : [moff] "v"(moff), [mtile] "s"(mbase) : "memory");
+  }
   u32x32 qv;  // the lane's Q operands, k-step ks in elements 4ks .. 4ks+3
   // Q of a part into its registers, and everything sent for so far in place.  One statement: the compiler takes a statement's
   // results as valid when it ends, so the wait has to be part of it (and, not knowing of the tile loads, the compiler
@@ -373,7 +401,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     t = f < t ? f : t;
     nfast_all = t > nfast ? t : nfast;
   }
-  if (a.mask_kind != 0) nfast = 0, nfast_all = 0;  // an attnMask is applied in the general form of a step
+  if (MASKB ? S < 160 : a.mask_kind != 0) nfast = 0, nfast_all = 0;  // other attnMasks are applied in the general form of a step
   // The fast form requests its tiles without the ragged-tile case: iteration j sends for K(j+4) and V(j+3), which have to
   // be whole tiles.
   if (!PAGED && (S % BN) != 0) {
@@ -467,8 +495,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   // then the true row maximum is formed, sum and accumulator are rescaled and the half is redone.  Every
   // probability that reaches the matrix pipe is therefore at most kSumLimit.
   const int rl = CAUSAL ? qc0 + lq - 4 * lh : 0;  // the causal predicate's lane operand: key k of a score is visible iff k - 4*(lane/32) <= rl
-  auto settle_half = [&](f32x16& s, vec8 (&pb)[2], float psum, int masked_kv0 = -1) __attribute__((always_inline)) {
+  auto settle_half = [&](f32x16& s, vec8 (&pb)[2], float psum, int masked_kv0 = -1, int mask_place = -1) __attribute__((always_inline)) {
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(psum <= kSumLimit)) != 0, 0)) {
+      // after a step that applied a Bool attnMask in the stream: scores whose mask byte is clear must not enter the maximum
+      if (MASKB && mask_place >= 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          if (((mring[4 * mask_place + (r >> 2)] >> (8 * (r & 3))) & 0xffu) == 0u) s[r] = -INFINITY;
+      }
       // after a step whose exponentials took the causal predicate in the stream, the scores themselves are masked only
       // here (hidden scores, or what a stage held beyond the workgroup's last tile, must not enter the maximum)
       if (CAUSAL && masked_kv0 >= 0) {
@@ -547,6 +581,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
                  "+{v[208:239]}"(ring)                                                                                 \
                : [c] "v"(c), [mc] "v"(mc), "{v[120:151]}"(qv), "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr)            \
                : "v240", "v241", "v242", "v243", "v244", "v245", "memory")
+// the plain step with a Bool attnMask applied to each probability (mask ring v[104:119], a zero in a scalar register)
+#define TT_P128_RUN_MSTEP(TXT)                                                                                         \
+  asm volatile(TXT                                                                                                     \
+               : [o0] "+v"(oacc[0]), [o1] "+v"(oacc[1]), [o2] "+v"(oacc[2]), [o3] "+v"(oacc[3]), [ps] "=&v"(psum_step),  \
+                 "+{v[160:175]}"(sB), "+{v[176:191]}"(sC), "+{v[192:199]}"(pAv), "+{v[200:207]}"(pBv),                   \
+                 "+{v[208:239]}"(ring), "+{v[104:119]}"(mring)                                                          \
+               : [c] "v"(c), [mc] "v"(mc), [zero] "s"(0), "{v[120:151]}"(qv), "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr) \
+               : "v240", "v241", "v242", "v243", "v244", "v245", "vcc", "memory")
   constexpr bool kIsBf16 = sizeof(typename TR::elem) == 2 && __is_same(typename TR::elem, __bf16);
 
   f32x16 sB, sC;
@@ -632,12 +674,15 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   };
   int j = kt0;
   if (nfast_all >= kt0 + 1) {
-    auto settle_fast = [&](f32x16& s, u32x8& pv, int masked_kv0) __attribute__((always_inline)) {
+    auto settle_fast = [&](f32x16& s, u32x8& pv, int masked_kv0, int mask_place) __attribute__((always_inline)) {
       vec8 p[2];
       p_load(pv, p);
-      settle_half(s, p, psum_step, masked_kv0);
+      settle_half(s, p, psum_step, masked_kv0, mask_place);
       p_store(pv, p);
     };
+    // MASKB: tile j sends for the mask bytes of halves 2j+3 and 2j+4 (the tile after it takes them); the last tiles'
+    // requests are moved back into the row (nobody takes what they bring)
+    const int mlast = S - 160;
     p_store(pAv, pA);
     p_store(pBv, pB);
     asm volatile(TT_P128_PREFETCH : "+{v[208:239]}"(ring) : "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr) : "memory");
@@ -645,6 +690,13 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #define TT_P128_TILE(U)                                                                                  \
     if (__builtin_expect(j >= nfast_all, 0)) break;                                                       \
     {                                                                                                    \
+      if constexpr (MASKB) {                                                                             \
+        const int mk0 = 64 * j < mlast ? 64 * j : mlast;                                                 \
+        if constexpr ((U & 1) == 0)                                                                      \
+          asm volatile(TT_P128_MLOAD_E : "+{v[104:119]}"(mring) : [moff] "v"(moff), [mtile] "s"(mbase + mk0) : "memory"); \
+        else                                                                                             \
+          asm volatile(TT_P128_MLOAD_O : "+{v[104:119]}"(mring) : [moff] "v"(moff), [mtile] "s"(mbase + mk0) : "memory"); \
+      }                                                                                                  \
       const int keep = PAGED ? tile_dma(j) : tile_dma_fast(j, U);                                        \
       /* mk = 1: the tile's exponentials take the causal predicate; kvs = first key of the half whose exponentials   \
          the step takes; kvm = kvs on such a tile, else -1.  As scalar instructions: the compiler's own form of     \
@@ -655,15 +707,19 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
             : "=&s"(mk), "=&s"(kvm0), "=&s"(kvm1) : "s"(j), "s"(nfast), "s"(kvs), "s"(kvs + 32) : "scc"); \
       if constexpr (kIsBf16 && CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_BF16_U##U##_K0);                    \
       else if constexpr (CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_F16_U##U##_K0);                           \
+      else if constexpr (MASKB && kIsBf16) TT_P128_RUN_MSTEP(TT_P128_MSTEP_BF16_U##U##_K0);              \
+      else if constexpr (MASKB) TT_P128_RUN_MSTEP(TT_P128_MSTEP_F16_U##U##_K0);                          \
       else if constexpr (kIsBf16) TT_P128_RUN_PSTEP(TT_P128_PSTEP_BF16_U##U##_K0);                       \
       else TT_P128_RUN_PSTEP(TT_P128_PSTEP_F16_U##U##_K0);                                               \
-      settle_fast(sB, pBv, kvm0);                                                                        \
+      settle_fast(sB, pBv, kvm0, MASKB ? (2 * U + 1) & 3 : -1);                                          \
       kvs += 32;                                                                                         \
       if constexpr (kIsBf16 && CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_BF16_U##U##_K1);                    \
       else if constexpr (CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_F16_U##U##_K1);                           \
+      else if constexpr (MASKB && kIsBf16) TT_P128_RUN_MSTEP(TT_P128_MSTEP_BF16_U##U##_K1);              \
+      else if constexpr (MASKB) TT_P128_RUN_MSTEP(TT_P128_MSTEP_F16_U##U##_K1);                          \
       else if constexpr (kIsBf16) TT_P128_RUN_PSTEP(TT_P128_PSTEP_BF16_U##U##_K1);                       \
       else TT_P128_RUN_PSTEP(TT_P128_PSTEP_F16_U##U##_K1);                                               \
-      settle_fast(sC, pAv, kvm1);                                                                        \
+      settle_fast(sC, pAv, kvm1, MASKB ? (2 * U + 2) & 3 : -1);                                          \
       dma_wait_and_sync(keep);                                                                           \
       j++;                                                                                               \
     }
@@ -764,19 +820,27 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
   }  // part
 }
 
-template <typename TR, bool CAUSAL, bool PAGED, bool SPLIT>
+template <typename TR, bool CAUSAL, bool PAGED, bool SPLIT, bool MASKB = false>
 int launch_v(const KArgs& a, dim3 grid, hipStream_t stream) {
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)prefill128_kernel<TR, CAUSAL, PAGED, SPLIT>, LDS_BYTES, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill128_kernel<TR, CAUSAL, PAGED, SPLIT, MASKB>, LDS_BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
-  hipLaunchKernelGGL((prefill128_kernel<TR, CAUSAL, PAGED, SPLIT>), grid, dim3(NW * 64), LDS_BYTES, stream, a);
+  hipLaunchKernelGGL((prefill128_kernel<TR, CAUSAL, PAGED, SPLIT, MASKB>), grid, dim3(NW * 64), LDS_BYTES, stream, a);
   return (int)hipGetLastError();
+}
+
+// A Bool attnMask the streams can apply: four keys per aligned dword, row offsets of a (batch, head) within 32 bits.
+bool bool_mask_in_streams(const KArgs& a) {
+  return !a.causal && a.mask_kind == 1 && a.mask_vec4 && (a.S % 4) == 0 && !a.kv_len && !a.block_table && a.kv_splits <= 1 &&
+         (long long)(a.L - 1) * a.ms[2] + 8 < (1ll << 32);
 }
 
 template <typename TR, bool CAUSAL>
 int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
   if (a.kv_splits > 1) return launch_v<TR, CAUSAL, false, true>(a, grid, stream);  // (the host never splits a paged call)
+  if constexpr (!CAUSAL)
+    if (bool_mask_in_streams(a)) return launch_v<TR, false, false, false, true>(a, grid, stream);
   return a.block_table ? launch_v<TR, CAUSAL, true, false>(a, grid, stream) : launch_v<TR, CAUSAL, false, false>(a, grid, stream);
 }
 

@@ -110,9 +110,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
     S = len < 0 ? 0 : (len < S ? len : S);
   }
 
-  // Neighbouring workgroups take their two tiles in opposite order, so that the load / store bursts between the
-  // parts of one half of the workgroups fall into the steady loops of the other half.
-  const bool long_first = !paired || ((blockIdx.x >> 3) & 1) == 0;
+  // Every workgroup takes its long tile first: the workgroups of a head that run together then walk its keys from the
+  // first one on in step, and an XCD's L2 serves all but the first of them.  (With neighbouring workgroups in opposite
+  // order a head's K/V came from memory about three times where one KV head serves one query head: B4 32 heads of 2048
+  // rows, fp16: 468 -> 275 MB read per launch, same time; grouped heads were and are read once.)
+  const bool long_first = true;
   // Wavefronts w and w+4 share a SIMD.  Under a causal mask the row group g of a tile has g+1 halves of work on the
   // diagonal, so the second four wavefronts take the groups in reverse: every SIMD then carries groups g and 7-g.
   const int rowgroup = (CAUSAL && wave >= 4) ? 11 - wave : wave;
