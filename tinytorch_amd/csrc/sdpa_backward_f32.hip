@@ -348,6 +348,8 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
   if (CAUSAL) it0 = (k0 - coff > 0 ? k0 - coff : 0) / BT;
   const int nt = ntq > it0 ? ntq - it0 : 0;
   const int total = f.G * nt;
+  const bool walk_up = dkv_walks_up(a, CAUSAL);  // every second round of an XCD's workgroups (sdpa_common.h)
+  auto tile_of = [&](int idx) __attribute__((always_inline)) { return walk_up ? it0 + idx / f.G : ntq - 1 - idx / f.G; };
 
   f32x4 qst[NLD], gst[NLD];
   float2 sst = make_float2(0.f, 0.f);
@@ -360,7 +362,7 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
   }
   auto load_tile = [&](int idx) {
     const int h = hk * f.G + idx % f.G;
-    const int i0 = (ntq - 1 - idx / f.G) * BT;
+    const int i0 = tile_of(idx) * BT;
     const float* qp = (const float*)f.q + b * f.qs[0] + h * f.qs[1];
     const float* gp = (const float*)a.dout + b * a.dos[0] + h * a.dos[1];
 #pragma unroll
@@ -403,7 +405,7 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
       store_tile(cur ^ 1);
       if (idx + 2 * nsplit < total) load_tile(idx + 2 * nsplit);
     }
-    const int i0 = (ntq - 1 - idx / f.G) * BT;
+    const int i0 = tile_of(idx) * BT;
     const int h_of_tile = hk * f.G + idx % f.G;
     if (wave_live && (!CAUSAL || kw0 <= i0 + BT - 1 + coff)) {
       const float* Qs = smem + cur * Lds::STAGE;
@@ -478,7 +480,8 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
 }
 
 template <int D, bool CAUSAL, bool MASKED>
-int launch_k(const BwdArgs& a, hipStream_t stream) {
+int launch_k(const BwdArgs& args, hipStream_t stream) {
+  BwdArgs a = args;
   static hipError_t state1[kMaxDevices], state2[kMaxDevices];
   static bool done1[kMaxDevices], done2[kMaxDevices];
   hipError_t e = grant_dynamic_lds((const void*)backward_dq_f32_kernel<D, CAUSAL, MASKED>, BwdF32Lds<D>::BYTES, state1, done1);
@@ -487,6 +490,8 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM) * a.dq_splits;
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM) * a.dkv_splits;
+  static int round_cache[kMaxDevices];
+  a.dkv_round = CAUSAL ? dkv_round_of((const void*)backward_dkv_f32_kernel<D, CAUSAL, MASKED>, 256, BwdF32Lds<D>::BYTES, round_cache) : 0;
   hipLaunchKernelGGL((backward_dq_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g1), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;

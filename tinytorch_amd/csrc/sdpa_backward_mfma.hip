@@ -437,6 +437,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   if (CAUSAL) it0 = (k0 - coff > 0 ? k0 - coff : 0) / BQ;
   const int nt = ntq > it0 ? ntq - it0 : 0;
   const int total = f.G * nt;
+  const bool walk_up = dkv_walks_up(a, CAUSAL);  // every second round of an XCD's workgroups (sdpa_common.h)
+  auto tile_of = [&](int idx) __attribute__((always_inline)) { return walk_up ? it0 + idx / f.G : ntq - 1 - idx / f.G; };
 
   u32x4 qst[NLD], gst[NLD];
   float2 sst = make_float2(0.f, 0.f);
@@ -449,7 +451,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   }
   auto load_tile = [&](int idx) {
     const int h = hk * f.G + idx % f.G;
-    const int i0 = (ntq - 1 - idx / f.G) * BQ;
+    const int i0 = tile_of(idx) * BQ;
     const T* qp = (const T*)f.q + b * f.qs[0] + h * f.qs[1];
     const T* gp = (const T*)a.dout + b * a.dos[0] + h * a.dos[1];
 #pragma unroll
@@ -494,7 +496,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
       store_tile(cur ^ 1);
       if (idx + 2 * nsplit < total) load_tile(idx + 2 * nsplit);
     }
-    const int i0 = (ntq - 1 - idx / f.G) * BQ;
+    const int i0 = tile_of(idx) * BQ;
     const int h_of_tile = hk * f.G + idx % f.G;
     if (wave_live && (!CAUSAL || kw0 <= i0 + BQ - 1 + coff)) {
       const T* Qr = smem + cur * Lds::KV_STAGE;
@@ -676,6 +678,8 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
   const int nt = ntq > it0 ? ntq - it0 : 0;
   const int total = split < f.G * nt ? (f.G * nt - split + nsplit - 1) / nsplit : 0;
   const int niter = (total + 1) / 2;  // iterations of either group (the second may have one entry less)
+  const bool walk_up = dkv_walks_up(a, CAUSAL);  // every second round of an XCD's workgroups (sdpa_common.h)
+  auto tile_of = [&](int entry) __attribute__((always_inline)) { return walk_up ? it0 + entry / f.G : ntq - 1 - entry / f.G; };
 
   // wavefront gw of a group brings rows 8gw .. 8gw+7 of the Q tile and of the dout tile (two loads each) into the
   // group's ring; its first wavefront the statistics as well
@@ -683,7 +687,7 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
   auto dma_tile = [&](int idx, int stage) __attribute__((always_inline)) {
     const int entry = split + nsplit * idx;
     const int h = hk * f.G + entry % f.G;
-    const int i0 = (ntq - 1 - entry / f.G) * BQ;
+    const int i0 = tile_of(entry) * BQ;
     const char* qb = (const char*)((const T*)f.q + b * f.qs[0] + h * f.qs[1] + (long long)i0 * f.qs[2]);
     const char* gb = (const char*)((const T*)a.dout + b * a.dos[0] + h * a.dos[1] + (long long)i0 * a.dos[2]);
     const unsigned at = ring_addr + stage * STAGE_BYTES;
@@ -736,7 +740,7 @@ __global__ __launch_bounds__(512, 1) void backward_dkv128_kernel(BwdArgs a) {
     const bool more = idx + 4 < total;
     if (more) dma_tile(idx + 4, nxt2);
     if (idx < total) {
-      const int i0 = (ntq - 1 - (split + nsplit * idx) / f.G) * BQ;
+      const int i0 = tile_of(split + nsplit * idx) * BQ;
       const char* qt = ring + cur * STAGE_BYTES;
       const char* gt = qt + TILE_BYTES;
       const float* st = (const float*)(qt + 2 * TILE_BYTES);
@@ -1063,7 +1067,8 @@ __global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
 }
 
 template <typename TR, int D, bool CAUSAL, bool MASKED>
-int launch_k(const BwdArgs& a, hipStream_t stream) {
+int launch_k(const BwdArgs& args, hipStream_t stream) {
+  BwdArgs a = args;
   typedef BwdLds<D> Lds;
   // with an attnMask, head_dim 128 takes the register-staged dk/dv kernel: the mask's 16 values per tile do not fit the
   // 256 registers of the direct-to-LDS one
@@ -1081,6 +1086,10 @@ int launch_k(const BwdArgs& a, hipStream_t stream) {
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM) * a.dq_splits;
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM) * a.dkv_splits;
+  static int round_cache[kMaxDevices];
+  a.dkv_round = !CAUSAL ? 0
+                : DMA   ? dkv_round_of((const void*)backward_dkv128_kernel<TR, CAUSAL>, 512, dkv128::LDS_BYTES, round_cache)
+                        : dkv_round_of((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED>, 256, Lds::KV_BYTES, round_cache);
   if (DMA) {
     hipLaunchKernelGGL((backward_dq128_kernel<TR, CAUSAL>), dim3((unsigned)g1), dim3(256), dq128::LDS_BYTES, stream, a);
   } else {

@@ -69,6 +69,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 // launch on a device (the device is the current one of the calling thread) and remembered; safe from several host
 // threads (the worst case is granting twice).
 constexpr int kMaxDevices = 64;
+constexpr int kCusPerXcd = 32;  // MI355X: 256 compute units in 8 XCDs, each XCD with an L2 of its own
 inline hipError_t grant_dynamic_lds(const void* kernel, int bytes, hipError_t (&state)[kMaxDevices], bool (&done)[kMaxDevices]) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -188,6 +189,9 @@ struct BwdArgs {
   // then [split][B][Hq][L] pairs (maximum in log2 units, sum of exponentials)) for backward_dq_merge_kernel.
   float* dq_partial;
   int dq_splits;
+  // dk/dv kernels under a causal mask: workgroups of an XCD that run together (CUs per XCD x workgroups per CU), or 0.
+  // The workgroups of every second such round walk their query tiles upwards (dkv_walks_up).
+  int dkv_round;
 };
 
 // Workgroups that share a key block in the matrix-core dk/dv kernels (1: none, the kernel writes dk / dv itself).
@@ -371,6 +375,29 @@ __device__ __forceinline__ void map_workgroup(int n, int npair, int nblk, int* p
 template <bool PIN>
 __device__ __forceinline__ void pin_accumulator(f32x16& acc) {
   if constexpr (PIN) asm volatile("" : "+a"(acc));
+}
+
+// Direction in which a dk/dv workgroup walks the query tiles it0 .. ntq-1 that see its key block.  The workgroups of an XCD
+// start longest first (map_workgroup), `dkv_round` of them at a time.  Those of the first round start together at the last
+// tile and walk down in step (the tile one fetches is in the XCD's L2 for the others); the workgroup of key block kb ends
+// after ntq - it0(kb) tiles, and the CU it frees takes the longest block left, which has as many tiles as the first had
+// few.  Walking UP from its first tile, that workgroup is at the same tile at the same time as every other one of the
+// second round (all arrive at the last tile together); walking down, each would be alone with its position and fetch
+// its tiles from memory itself.  The third round starts together again: rounds alternate.  (bf16 head_dim 128, B2 32q/8kv
+// 4096 x 4096: 458 -> 240 MB read per launch of the dk/dv kernel.)
+__device__ __forceinline__ bool dkv_walks_up(const BwdArgs& a, bool causal) {
+  return causal && a.dkv_round > 0 && ((a.f.B * a.f.Hkv) & 7) == 0 && (((int)(blockIdx.x >> 3) / a.dkv_round) & 1) != 0;
+}
+
+// Workgroups of `kernel` that fit one CU, times the CUs of an XCD: the dkv_round of a launch (looked up once per device).
+inline int dkv_round_of(const void* kernel, int threads, int lds_bytes, int (&cache)[kMaxDevices]) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  if (cache[dev] == 0) {
+    int n = 0;
+    cache[dev] = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, threads, (size_t)lds_bytes) == hipSuccess && n > 0 ? n * kCusPerXcd : -1;
+  }
+  return cache[dev] > 0 ? cache[dev] : 0;
 }
 
 // Keys of batch entry b: all S of them, or the filled prefix of a cache / the unpadded length (kv_len).

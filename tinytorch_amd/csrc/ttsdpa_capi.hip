@@ -270,7 +270,7 @@ int validate_backward(const ttsdpa_backward_params* p, BwdArgs* a) {
   }
   if ((p->dout_stride[2] < f->D || p->dq_stride[2] < f->D) && f->L > 1) return TTSDPA_ERR_STRIDE;
   if ((p->dk_stride[2] < f->D || p->dv_stride[2] < f->D) && f->S > 1) return TTSDPA_ERR_STRIDE;
-  a->dout = p->dout, a->dq = p->dq, a->dk = p->dk, a->dv = p->dv, a->stats = nullptr, a->partial = nullptr, a->dkv_splits = 1, a->dq_partial = nullptr, a->dq_splits = 1;
+  a->dout = p->dout, a->dq = p->dq, a->dk = p->dk, a->dv = p->dv, a->stats = nullptr, a->partial = nullptr, a->dkv_splits = 1, a->dq_partial = nullptr, a->dq_splits = 1, a->dkv_round = 0;
   return TTSDPA_OK;
 }
 
