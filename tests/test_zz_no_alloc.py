@@ -47,3 +47,48 @@ def test_static_scratch_decode_matches_decode_twice_in_a_row():
     # and a call that needs no scratch at all (enough (batch, head) pairs to run unsplit), fp16, head_dim 64
     host, a, b, n3 = _both(64, 8, 8, 1, 512, 64, "f16", 33)
     assert n3 == 0 and torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_static_scratch_decode_allocates_nothing_and_replays_in_a_graph():
+    """The property the entry point exists for.  After a warm call (the library looks up its buffer's address once per
+    device) further calls leave the device's free memory unchanged, and a call recorded into a HIP graph — where an
+    allocation would fail the capture — replays to what ttsdpa_decode gives with caller scratch, replay after replay,
+    with eager work and synchronisations between the replays."""
+    B, Hq, Hkv, S, D = 1, 8, 2, 16384, 128   # many splits: the partial records are in use
+    host, dev = make_inputs(41, B, Hq, Hkv, 1, S, D, "bf16")
+    lib = _capi.lib()
+    out_ws, out_static = torch.empty_like(dev[0]), torch.empty_like(dev[0])
+    p_ws, p_static = build_params(*dev, out_ws, False), build_params(*dev, out_static, False)
+    nbytes = lib.ttsdpa_workspace_bytes(ctypes.byref(p_ws))
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    assert nbytes > 0 and lib.ttsdpa_decode(ctypes.byref(p_ws), ws.data_ptr(), nbytes, stream) == 0
+    assert lib.ttsdpa_decode_static(ctypes.byref(p_static), stream) == 0   # warm call
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(8):
+        assert lib.ttsdpa_decode_static(ctypes.byref(p_static), stream) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, "device memory changed across ttsdpa_decode_static calls: %d -> %d" % (free0, free1)
+    assert torch.equal(out_ws.view(torch.int16), out_static.view(torch.int16))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = lib.ttsdpa_decode_static(ctypes.byref(p_static), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _capi.status_string(rc)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        qh, qb = oracle.round_to(oracle.randn(50 + rep, 0, (B, Hq, 1, D)), "bf16")
+        dev[0].copy_(torch.from_numpy(qb.view(np.int16)).cuda().view(torch.bfloat16))   # new queries in the recorded buffer
+        out_static.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        assert lib.ttsdpa_decode(ctypes.byref(p_ws), ws.data_ptr(), nbytes, stream) == 0   # eager, caller scratch
+        torch.cuda.synchronize()
+        assert torch.equal(out_ws.view(torch.int16), out_static.view(torch.int16)), "replay %d" % rep
+        err = float(np.abs(to_host_f32(out_static) - oracle.sdpa_f32(qh, host[1], host[2])).max())
+        assert err <= TOL["bf16"]
