@@ -608,6 +608,17 @@ static void test_matmul_batched_reference_vectors() {
         }
     EXPECT_TRUE(vectorNear(got, ref, 2e-2f * std::sqrt(static_cast<float>(D))));
   }
+  // a 1-D second operand against a batched first operand: the reference's reshape of the [2, 3, 1] result to {3} does not
+  // fit; refused loudly here (and by the Python mirror), a 1-D first operand keeps its row ([..., 1, n])
+  {
+    AssertHandler old = setAssertHandler(countingAssertHandler);
+    const int before = g_asserts;
+    Tensor none = op::matmul(ar({2, 3, 4}), ar({4}), false, false, Tensor{});
+    EXPECT_TRUE(g_asserts > before && !none.defined());
+    setAssertHandler(old);
+    Tensor row = op::matmul(ar({4}), ar({2, 4, 2}), false, false, Tensor{});
+    EXPECT_TRUE(row.defined() && row.shape() == std::vector<int64_t>({2, 1, 2}));
+  }
 }
 
 int main() {

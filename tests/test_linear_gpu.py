@@ -224,6 +224,9 @@ def test_matmul_batch_rules_reference_vectors():
     ((2, 1, 64, 130), (1, 4, 64, 40), True, False, True),         # both operands broadcast, transposed first operand
     ((5, 33, 128), (128, 48), False, False, True),                 # a batch against one matrix
     ((2, 2, 1, 256, 256), (2, 1, 3, 256, 256), False, True, False),  # two broadcast axes, tile-sized entries
+    ((16, 8, 64, 32), (16, 8, 48, 32), False, True, True),         # 128 small entries: one grid on the vector-ALU kernel
+    ((4, 8, 96, 160), (4, 8, 160, 64), False, False, False),       # probabilities x values: one grid, operands read in place
+    ((6, 1, 70, 64), (6, 5, 36, 64), False, True, False),           # a shared by five entries each: no uniform stride, entry by entry
 ])
 def test_matmul_batched_against_oracle(dtype, case):
     import tinytorch_amd

@@ -32,6 +32,9 @@ struct LinArgs {
   long long M, N, K, ldx, ldw, ldo;
   // general kernel only: x is stored [K, M] (x(m,k) = x[k*ldx + m]) / w is stored [K, N] (w(n,k) = w[k*ldw + n])
   int xt = 0, wt = 0;
+  // batch entries of one launch (linear_mfma_kernel: blockIdx.y, linear_general_kernel: blockIdx.z): entry e reads
+  // x + e*bsx, w + e*bsw and writes out + e*bso (elements; 0 = the operand is shared by all entries)
+  long long bsx = 0, bsw = 0, bso = 0;
 };
 
 typedef __attribute__((address_space(3))) void lds_void_t;
@@ -111,8 +114,8 @@ __global__ __launch_bounds__(WN * WM * 64, 1) void linear_mfma_kernel(LinArgs a)
     const long long r = row < lim ? row : lim;
     return (unsigned)((r * ld + G::KPC * chunk) * ESZ);
   };
-  const char* xbase = (const char*)((const T*)a.x + m0 * a.ldx);
-  const char* wbase = (const char*)((const T*)a.w + n0 * a.ldw);
+  const char* xbase = (const char*)((const T*)a.x + (long long)blockIdx.y * a.bsx + m0 * a.ldx);
+  const char* wbase = (const char*)((const T*)a.w + (long long)blockIdx.y * a.bsw + n0 * a.ldw);
   const unsigned smem_addr = (unsigned)(unsigned long)(lds_void_t*)smem;
   // issued as asm so that the compiler does not treat it as an LDS store it must order every later LDS read behind
   // (the lane's full address goes in a register pair: a scalar base operand is not always kept in scalar registers by
@@ -215,7 +218,7 @@ __global__ __launch_bounds__(WN * WM * 64, 1) void linear_mfma_kernel(LinArgs a)
   for (int j = 0; j < MJ; j++) {
     const long long m = m0 + (TM / WM) * wm + 32 * j + lq;
     if (m >= a.M) continue;
-    T* orow = (T*)a.out + m * a.ldo;
+    T* orow = (T*)a.out + (long long)blockIdx.y * a.bso + m * a.ldo;
 #pragma unroll
     for (int i = 0; i < NI; i++)
 #pragma unroll
@@ -546,8 +549,8 @@ __global__ __launch_bounds__(256) void linear_general_kernel(LinArgs a) {
   const int tid = threadIdx.x;
   const int tx = tid & 15, ty = tid >> 4;
   const long long m0 = (long long)blockIdx.y * 64, n0 = (long long)blockIdx.x * 64;
-  const T* x = (const T*)a.x;
-  const T* w = (const T*)a.w;
+  const T* x = (const T*)a.x + (long long)blockIdx.z * a.bsx;
+  const T* w = (const T*)a.w + (long long)blockIdx.z * a.bsw;
   float acc[4][4];
 #pragma unroll
   for (int j = 0; j < 4; j++) {
@@ -587,7 +590,7 @@ __global__ __launch_bounds__(256) void linear_general_kernel(LinArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const long long n = n0 + 4 * tx + j;
-      if (n < a.N) store_from_float((T*)a.out + m * a.ldo + n, acc[i][j]);
+      if (n < a.N) store_from_float((T*)a.out + (long long)blockIdx.z * a.bso + m * a.ldo + n, acc[i][j]);
     }
   }
 }
@@ -672,7 +675,7 @@ int check(int dtype, const void* x, const void* w, const void* out, long long M,
 }
 
 template <typename TR, int TM, int TN, int WN, int WM>
-int launch_mfma_tile(const LinArgs& a, hipStream_t stream) {
+int launch_mfma_tile(const LinArgs& a, hipStream_t stream, unsigned entries = 1) {
   constexpr int lds = 2 * (TM + TN) * ROWB;
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
@@ -682,7 +685,7 @@ int launch_mfma_tile(const LinArgs& a, hipStream_t stream) {
   const long long nsuper = ((tiles_m + 3) / 4) * ((tiles_n + 7) / 8);
   const long long nwg = (nsuper + 7) / 8 * 8 * 32;
   if (nwg > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
-  hipLaunchKernelGGL((linear_mfma_kernel<TR, TM, TN, WN, WM>), dim3((unsigned)nwg), dim3(WN * WM * 64), lds, stream, a);
+  hipLaunchKernelGGL((linear_mfma_kernel<TR, TM, TN, WN, WM>), dim3((unsigned)nwg, entries), dim3(WN * WM * 64), lds, stream, a);
   return (int)hipGetLastError();
 }
 
@@ -716,8 +719,8 @@ int launch_mfma(const LinArgs& a, hipStream_t stream) {
 }
 
 template <typename T>
-int launch_general_linear(const LinArgs& a, hipStream_t stream) {
-  dim3 grid((unsigned)((a.N + 63) / 64), (unsigned)((a.M + 63) / 64));
+int launch_general_linear(const LinArgs& a, hipStream_t stream, unsigned entries = 1) {
+  dim3 grid((unsigned)((a.N + 63) / 64), (unsigned)((a.M + 63) / 64), entries);
   hipLaunchKernelGGL((linear_general_kernel<T>), grid, dim3(256), 0, stream, a);
   return (int)hipGetLastError();
 }
@@ -834,6 +837,53 @@ int ttlinear_matmul_batched(int dtype, const void* a, const void* b, const void*
   }
   if (out_batch_stride < 0) return TTSDPA_ERR_STRIDE;
   const size_t esz = dtype == TTSDPA_F32 ? 4 : 2;
+  auto offsets = [&](long long i, long long* ao, long long* bo) {
+    // offsets of entry i: the reference's index walk from the innermost batch dimension outwards
+    long long rest = i;
+    *ao = 0, *bo = 0;
+    for (int d = nbatch_dims - 1; d >= 0; d--) {
+      const long long idx = rest % batch_shape[d];
+      rest /= batch_shape[d];
+      *ao += idx * a_batch_stride[d];
+      *bo += idx * b_batch_stride[d];
+    }
+  };
+  // One grid for all entries (the reference's strided-batched product, src/Operation/OpLinalg.cpp:113-150) when the
+  // entries' offsets are a multiple of the entry index in both operands (no broadcast pattern that breaks the stride)
+  // and an entry is small enough that a launch each would be launch-bound; x . w^T on the tiled matrix-core kernel when
+  // the layout allows, every other flag pair on the vector-ALU kernel, which reads the operands in place.
+  if (entries > 1 && entries <= 65535 && M > 0 && N > 0 && K > 0 && a && b && out && (double)M * N * K <= (double)(1 << 27)) {
+    long long sa = 0, sb = 0;
+    offsets(1, &sa, &sb);
+    bool uniform = true;
+    for (long long i = 2; i < entries && uniform; i++) {
+      long long ao, bo;
+      offsets(i, &ao, &bo);
+      uniform = ao == i * sa && bo == i * sb;
+    }
+    if (uniform && lda >= (trans_a ? M : K) && ldb >= (trans_b ? K : N) && ldo >= N && aligned(a, esz) && aligned(b, esz) &&
+        aligned(out, esz) && (!bias || aligned(bias, esz)) && (M + 63) / 64 <= 65535) {
+      hipStream_t s = (hipStream_t)stream;
+      LinArgs g{a, b, bias, out, M, N, K, lda, ldb, ldo, trans_a ? 1 : 0, trans_b ? 0 : 1};
+      g.bsx = sa, g.bsw = sb, g.bso = out_batch_stride;
+      int route = TTLINEAR_ROUTE_NONE;
+      const long long kpc = 16 / (long long)esz;
+      if (!trans_a && trans_b && check(dtype, a, b, out, M, N, K, lda, ldb, ldo, &route) == TTSDPA_OK && route == TTLINEAR_ROUTE_MFMA &&
+          sa % kpc == 0 && sb % kpc == 0 && out_batch_stride % 4 == 0 && !(dtype != TTSDPA_F32 && M <= 64 && N >= 64)) {
+        g.xt = g.wt = 0;
+        switch (dtype) {
+          case TTSDPA_F32: return launch_mfma_tile<F32, 128, 128, 4, 2>(g, s, (unsigned)entries);
+          case TTSDPA_F16: return launch_mfma_tile<F16, 128, 128, 4, 2>(g, s, (unsigned)entries);
+          default: return launch_mfma_tile<BF16, 128, 128, 4, 2>(g, s, (unsigned)entries);
+        }
+      }
+      switch (dtype) {
+        case TTSDPA_F32: return launch_general_linear<float>(g, s, (unsigned)entries);
+        case TTSDPA_F16: return launch_general_linear<_Float16>(g, s, (unsigned)entries);
+        default: return launch_general_linear<__bf16>(g, s, (unsigned)entries);
+      }
+    }
+  }
   for (long long i = 0; i < entries; i++) {
     // offsets of entry i: the reference's index walk from the innermost batch dimension outwards
     long long ao = 0, bo = 0, rest = i;

@@ -89,6 +89,11 @@ Tensor matmulNdGpuImpl(const Tensor& a, const Tensor& b, bool transA, bool trans
       runB *= db;
     }
   }
+  // A 1-D second operand against a first operand with batch dimensions: the reference reshapes the [..., m, 1] result to
+  // {m} (src/Operation/OpLinalg.cpp:196-200, :232-238), which its element count does not fit.  No result shape is defined:
+  // refused, as the Python mirror does.
+  ASSERT(!(appendB && nd > 0) && "matmul error: a 1-D second operand against a batched first operand has no result shape");
+  if (appendB && nd > 0) return {};
   std::vector<int64_t> shape = batch;
   shape.push_back(m);
   shape.push_back(n);
