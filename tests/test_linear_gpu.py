@@ -137,6 +137,11 @@ MATMUL_CASES = [
     (33, 47, 65, True, False, "bf16", True),
     (5, 3, 2, True, True, "f32", False),
     (64, 64, 64, False, True, "bf16", True),        # the linear layer's own form
+    (296, 264, 192, False, False, "bf16", True),    # contraction-major b read in place, ragged 128-tiles
+    (264, 200, 320, True, False, "f16", True),      # both operands contraction-major, ragged
+    (136, 72, 64, True, True, "bf16", False),       # contraction-major a, row-major b
+    (4088, 4088, 128, True, False, "bf16", False),  # 256 ragged 256 x 256 tiles, both operands contraction-major
+    (4088, 4088, 64, False, False, "f16", True),    # the same tiles, row-major a
 ]
 
 
@@ -165,6 +170,31 @@ def test_matmul_transpose_flags_against_oracle(case):
     torch.cuda.synchronize()
     assert rc == 0
     assert float(np.abs(to_host_f32(out).astype(np.float64) - exp).max()) <= tol
+
+
+def test_matmul_in_place_operands_with_leading_dimensions():
+    """Operands that are views of larger buffers (leading dimension beyond the row): the matrix-core kernel that reads
+    contraction-major operands in place takes their strides; against torch's fp32 product of the same values."""
+    L = _capi.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device="cuda").manual_seed(7)
+    M, N, K = 392, 328, 256
+    for ta, tb in ((True, False), (False, False), (True, True)):
+        abuf = torch.randn((K, M + 40) if ta else (M, K + 24), device="cuda", generator=g).bfloat16()
+        bbuf = torch.randn((N, K + 8) if tb else (K, N + 16), device="cuda", generator=g).bfloat16()
+        a = abuf[:, 8:8 + M] if ta else abuf[:, 16:16 + K]
+        b = bbuf[:, :K] if tb else bbuf[:, 8:8 + N]
+        obuf = torch.zeros(M, N + 12, device="cuda", dtype=torch.bfloat16)
+        out = obuf[:, 4:4 + N]
+        rc = L.ttlinear_matmul(_capi.BF16, a.data_ptr(), b.data_ptr(), None, out.data_ptr(), M, N, K, int(ta), int(tb),
+                               a.stride(0), b.stride(0), out.stride(0), None, 0, st)
+        torch.cuda.synchronize()
+        assert rc == 0
+        ref = (a.float().t() if ta else a.float()) @ (b.float().t() if tb else b.float())
+        err = float((out.float() - ref).abs().max())
+        say("in-place operands transA=%d transB=%d: max-abs-err %.3e" % (ta, tb, err))
+        assert err <= 2e-2 * np.sqrt(K)
+        assert float(obuf[:, :4].abs().max()) == 0 and float(obuf[:, 4 + N:].abs().max()) == 0   # nothing beyond the view
 
 
 def test_linear_backward_against_torch_autograd():

@@ -234,6 +234,217 @@ __global__ __launch_bounds__(WN * WM * 64, 1) void linear_mfma_kernel(LinArgs a)
   }
 }
 
+// ---- 16-bit tensors with an operand stored contraction-major (op::matmul's other transpose flags) -------------------------
+// out[m][n] = sum_k x(m,k) w(n,k) + bias[n] with x(m,k) = XT ? x[k*ldx + m] : x[m*ldx + k] and w(n,k) = WT ? w[k*ldw + n] :
+// w[n*ldw + k]: the operands of op::matmul(a, b, transA, transB) as they lie in memory (reference
+// src/Operation/OpLinalg.cpp:107-150 hands its flags to the GEMM; no transposed copy is made here either).
+// Same tiles, workgroup order, stages and pipeline as linear_mfma_kernel.  What differs is the tile of a contraction-major
+// operand and how fragments are read:
+//  * such a tile is 64 k-rows of its 128 or 256 columns, kept as sub-tiles of 128 columns (64 rows x 256 bytes, the
+//    layout of the attention kernels' V tile: 16-byte chunk c of row r at slot c ^ f(r), f(r) = (r%4)*4 + (r/4)%4), and a
+//    fragment of it comes through the LDS transpose load: two ds_read_b64_tr_b16 give a lane the k values
+//    {4h..4h+3} and {8+4h..8+4h+3} of a 16-k step for its row (h = lane/32);
+//  * the contraction index has to be permuted identically on both sides, so a row-major operand's fragment is read in
+//    the same order, as two 8-byte pieces (chunks 2ks and 2ks+1 of the k-step, bytes 8h..8h+7 of each).
+namespace lint {
+__device__ __forceinline__ int swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+}  // namespace lint
+
+template <typename TR, int TM, int TN, bool XT, bool WT>
+__global__ __launch_bounds__(512, 1) void linear_mfma_t_kernel(LinArgs a) {
+  static_assert(XT || WT, "both operands row-major: linear_mfma_kernel");
+  constexpr int WN = 4, WM = 2, NW = 8;
+  constexpr int XTILE = TM * ROWB, STAGE = (TM + TN) * ROWB;  // bytes: 64 k of 2 bytes per row or column, either layout
+  constexpr int XI = TM / NW / 8, WI = TN / NW / 8;           // load instructions per wavefront and tile, either layout
+  constexpr int NI = TN / WN / 32, MJ = TM / WM / 32;
+  constexpr int BK = 64, SUB = 64 * 256;                      // k per tile; bytes of a 128-column sub-tile
+  typedef typename TR::elem T;
+  typedef typename TR::vec8 vec8;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, lh = lane >> 5;
+
+  // workgroup -> tile: 4 x 8 tile blocks per XCD, as in linear_mfma_kernel
+  const int tiles_m = (int)((a.M + TM - 1) / TM), tiles_n = (int)((a.N + TN - 1) / TN);
+  const int super_n = (tiles_n + 7) / 8;
+  const int nsuper = ((tiles_m + 3) / 4) * super_n;
+  const int slot = blockIdx.x >> 3;
+  const int super = (slot >> 5) * 8 + (blockIdx.x & 7);
+  if (super >= nsuper) return;
+  const int tm = (super / super_n) * 4 + ((slot & 31) >> 3);
+  const int tn = (super % super_n) * 8 + (slot & 7);
+  if (tm >= tiles_m || tn >= tiles_n) return;
+  const long long m0 = (long long)tm * TM, n0 = (long long)tn * TN;
+
+  // ---- global -> LDS -------------------------------------------------------------------------------------------------------
+  // row-major operand: wavefront w moves rows (T/8)w .. of the tile, 8 rows (1 KB) per instruction, lane l fills (row l/8,
+  // chunk slot l%8) with chunk (l%8) ^ ((row/2) % 8); rows past the end re-read the last row.
+  // contraction-major operand: wavefront w moves k-rows 8w .. 8w+7 of every 128-column sub-tile, 4 rows (1 KB) per
+  // instruction, lane l fills (row l/16, chunk slot l%16) with chunk (l%16) ^ f(row); columns past the end re-read the
+  // last 8 valid ones (their products land in outputs that are not stored).
+  const long long mlim = a.M - 1 - m0, nlim = a.N - 1 - n0;
+  auto rm_off = [&](int row, long long lim, long long ld) __attribute__((always_inline)) {
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    const long long r = row < lim ? row : lim;
+    return (unsigned)((r * ld + 8 * chunk) * 2);
+  };
+  auto km_off = [&](int row, int sub, long long cols_left, long long ld) __attribute__((always_inline)) {  // cols_left: valid columns from the tile's first
+    const int chunk = (lane & 15) ^ lint::swz(row);
+    long long col = 128 * sub + 8 * chunk;
+    col = col + 8 <= cols_left ? col : cols_left - 8;
+    return (unsigned)(((long long)row * ld + col) * 2);
+  };
+  const T* xb = (const T*)a.x + (long long)blockIdx.y * a.bsx;
+  const T* wb = (const T*)a.w + (long long)blockIdx.y * a.bsw;
+  const char* xbase = (const char*)(XT ? xb + m0 : xb + m0 * a.ldx);
+  const char* wbase = (const char*)(WT ? wb + n0 : wb + n0 * a.ldw);
+  const unsigned smem_addr = (unsigned)(unsigned long)(lds_void_t*)smem;
+  auto dma_issue = [&](const char* sbase, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
+    const char* p = sbase + voff;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(p), "s"(lds_addr) : "memory", "m0");
+  };
+  auto dma_operand = [&](bool km, const char* base, long long ld, long long lim, int T_, int NINSTR, long long t, unsigned dst) __attribute__((always_inline)) {
+    if (km) {
+      const char* src = base + t * BK * ld * 2;  // 64 k-rows further
+#pragma unroll
+      for (int i = 0; i < NINSTR; i++) {
+        const int sub = i >> 1, row = 8 * wave + 4 * (i & 1) + (lane >> 4);
+        dma_issue(src, km_off(row, sub, lim + 1, ld), dst + sub * SUB + (8 * wave + 4 * (i & 1)) * 256);
+      }
+    } else {
+      const char* src = base + t * ROWB;
+#pragma unroll
+      for (int i = 0; i < NINSTR; i++) {
+        const int row = (T_ / NW) * wave + 8 * i + (lane >> 3);
+        dma_issue(src, rm_off(row, lim, ld), dst + ((T_ / NW) * wave + 8 * i) * ROWB);
+      }
+    }
+  };
+  auto dma_tile = [&](int t, int stage) __attribute__((always_inline)) {
+    const unsigned dst = smem_addr + stage * STAGE;
+    dma_operand(XT, xbase, a.ldx, mlim, TM, XI, t, dst);
+    dma_operand(WT, wbase, a.ldw, nlim, TN, WI, t, dst + XTILE);
+  };
+
+  // ---- fragments ---------------------------------------------------------------------------------------------------------------
+  const int wn = wave % WN, wm = wave / WN;
+  // row-major: (block, ks, piece p): row 32*block + lq, bytes 8lh .. 8lh+7 of chunk 2ks + p
+  const unsigned rm_base = (unsigned)(lq * ROWB + 8 * lh + 16 * ((lq >> 1) & 7));
+  // contraction-major: piece ld of k-step ks for the 32 columns 32*db .. of a sub-tile (see sdpa_prefill_d128.hip, V operand)
+  unsigned km_base[2];
+  {
+    const int s = lane & 15, dhalf = (lane >> 4) & 1;
+#pragma unroll
+    for (int ld = 0; ld < 2; ld++) {
+      const int row = 8 * ld + 4 * lh + (s >> 2);
+      const int chunk = 2 * dhalf + ((s & 3) >> 1);
+      km_base[ld] = (unsigned)(row * 256 + 16 * (chunk ^ lint::swz(row)) + 8 * (s & 1));
+    }
+  }
+  // fragment of the 32 rows / columns starting at `first` of an operand's tile at `region`, k-step ks
+  auto frag_of = [&](bool km, const char* region, int first, int ks) __attribute__((always_inline)) {
+    if (km) {
+      const char* sub = region + (first >> 7) * SUB + 16 * ks * 256;
+      const unsigned db = (unsigned)((first & 127) >> 5);
+      const lint::s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lint::lds_s16x4*)(sub + (km_base[0] ^ (64u * db))));
+      const lint::s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lint::lds_s16x4*)(sub + (km_base[1] ^ (64u * db))));
+      return __builtin_bit_cast(vec8, (lint::s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    } else {
+      const char* rows = region + first * ROWB;
+      const lint::s16x4 lo = *(const lint::s16x4*)(rows + (rm_base ^ (unsigned)(32 * ks)));
+      const lint::s16x4 hi = *(const lint::s16x4*)(rows + (rm_base ^ (unsigned)(32 * ks + 16)));
+      return __builtin_bit_cast(vec8, (lint::s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+  };
+
+  f32x16 acc[NI][MJ];
+#pragma unroll
+  for (int i = 0; i < NI; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const long long n = n0 + (TN / WN) * wn + 32 * i + 8 * (r >> 2) + 4 * lh + (r & 3);
+      const float b = (a.bias && n < a.N) ? (float)((const T*)a.bias)[n] : 0.f;
+#pragma unroll
+      for (int j = 0; j < MJ; j++) acc[i][j][r] = b;
+    }
+
+  vec8 fw[2][NI], fx[2][MJ];
+  auto load_frag = [&](int buf, const char* st, int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NI; i++) fw[buf][i] = frag_of(WT, st + XTILE, (TN / WN) * wn + 32 * i, ks);
+#pragma unroll
+    for (int j = 0; j < MJ; j++) fx[buf][j] = frag_of(XT, st, (TM / WM) * wm + 32 * j, ks);
+  };
+  auto mma = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NI; i++)
+#pragma unroll
+      for (int j = 0; j < MJ; j++) acc[i][j] = TR::mfma32(fw[buf][i], fx[buf][j], acc[i][j]);
+  };
+
+  // the pipeline of linear_mfma_kernel: fragments double-buffered in registers, one barrier per tile before its last k-step
+  const int ntk = (int)(a.K / BK);
+  if (ntk > 0) {
+    dma_tile(0, 0);
+    if (ntk > 1) {
+      dma_tile(1, 1);
+      if constexpr (XI + WI == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      static_assert(XI + WI == 8 || XI + WI == 4, "add the matching wait");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    load_frag(0, smem, 0);
+  }
+  for (int t = 0; t < ntk; t++) {
+    const char* st = smem + (t & 1) * STAGE;
+    load_frag(1, st, 1);
+    mma(0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frag(0, st, 2);
+    mma(1);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frag(1, st, 3);
+    mma(0);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (t + 2 < ntk) dma_tile(t + 2, t & 1);
+    if (t + 1 < ntk) load_frag(0, smem + ((t + 1) & 1) * STAGE, 0);
+    mma(1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // store: register group rg of acc[i][j] is out[m = .. + 32j + lq][n = .. + 32i + 8rg + 4lh .. +3]
+#pragma unroll
+  for (int j = 0; j < MJ; j++) {
+    const long long m = m0 + (TM / WM) * wm + 32 * j + lq;
+    if (m >= a.M) continue;
+    T* orow = (T*)a.out + (long long)blockIdx.y * a.bso + m * a.ldo;
+#pragma unroll
+    for (int i = 0; i < NI; i++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        const long long n = n0 + (TN / WN) * wn + 32 * i + 8 * rg + 4 * lh;
+        if (n < a.N) {  // N is a multiple of 4 on this route
+          f32x4 v;
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * rg + e];
+          *(typename TR::vec4*)(orow + n) = __builtin_convertvector(v, typename TR::vec4);
+        }
+      }
+  }
+}
+
 // ---- 16-bit tensors, 256 x 256 tiles: four wavefronts with 128 x 128 each and the tile's arithmetic as one hand-ordered stream
 // Same tiles, LDS layout and direct loads as linear_mfma_kernel<TR, 256, 256>; what differs is who owns what, the matrix
 // instruction and who orders the instructions.  The clock of these kernels is power-managed, so what a tile costs is
@@ -689,6 +900,34 @@ int launch_mfma_tile(const LinArgs& a, hipStream_t stream, unsigned entries = 1)
   return (int)hipGetLastError();
 }
 
+template <typename TR, int T_, bool XT, bool WT>
+int launch_mfma_t_tile(const LinArgs& a, hipStream_t stream) {
+  constexpr int lds = 2 * (T_ + T_) * ROWB;
+  static hipError_t state[kMaxDevices];
+  static bool done[kMaxDevices];
+  const hipError_t granted = grant_dynamic_lds((const void*)linear_mfma_t_kernel<TR, T_, T_, XT, WT>, lds, state, done);
+  if (granted != hipSuccess) return (int)granted;
+  const long long tiles_m = (a.M + T_ - 1) / T_, tiles_n = (a.N + T_ - 1) / T_;
+  const long long nsuper = ((tiles_m + 3) / 4) * ((tiles_n + 7) / 8);
+  const long long nwg = (nsuper + 7) / 8 * 8 * 32;
+  if (nwg > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
+  hipLaunchKernelGGL((linear_mfma_t_kernel<TR, T_, T_, XT, WT>), dim3((unsigned)nwg), dim3(512), lds, stream, a);
+  return (int)hipGetLastError();
+}
+
+// 16-bit operands read as they lie in memory (a.xt / a.wt: stored contraction-major)
+template <typename TR>
+int launch_mfma_t(const LinArgs& a, hipStream_t stream) {
+  // 256 x 256 tiles once they fill the chip, unless their last round over the 256 CUs would be under 85 % full: then four
+  // times as many 128 x 128 tiles (weight gradient of the QKV projection, 384 large tiles: 878 -> 936 TFLOP/s; its input
+  // gradient, 512 large tiles, runs 1063 against 795 on the small ones)
+  const long long n256 = ((a.M + 255) / 256) * ((a.N + 255) / 256);
+  const bool big = n256 >= 256 && n256 * 100 >= (n256 + 255) / 256 * 256 * 85;
+  if (a.xt && a.wt) return big ? launch_mfma_t_tile<TR, 256, true, true>(a, stream) : launch_mfma_t_tile<TR, 128, true, true>(a, stream);
+  if (a.xt) return big ? launch_mfma_t_tile<TR, 256, true, false>(a, stream) : launch_mfma_t_tile<TR, 128, true, false>(a, stream);
+  return big ? launch_mfma_t_tile<TR, 256, false, true>(a, stream) : launch_mfma_t_tile<TR, 128, false, true>(a, stream);
+}
+
 template <typename TR>
 int launch_linear256(const LinArgs& a, hipStream_t stream) {
   constexpr int lds = 2 * (256 + 256) * ROWB;
@@ -787,6 +1026,19 @@ int ttlinear_matmul(int dtype, const void* a, const void* b, const void* bias, v
   if (!aligned(a, esz) || !aligned(b, esz) || !aligned(out, esz) || (bias && !aligned(bias, esz))) return TTSDPA_ERR_STRIDE;
   if ((M + 63) / 64 > 65535 || (N + 63) / 64 > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
+
+  // 16-bit tensors: the matrix-core kernel that reads contraction-major operands in place (no copies, no scratch)
+  if (dtype != TTSDPA_F32 && K > 0 && K % 64 == 0 && N % 4 == 0 && ldo % 4 == 0 && aligned(out, 8)) {
+    auto in_place = [](const void* p, bool contraction_major, int64_t rows, int64_t ld) {
+      if (!aligned(p, 16) || ld % 8 != 0) return false;
+      // a tile's rows are addressed with 32-bit byte offsets: 64 k-rows of a contraction-major operand, 256 rows otherwise
+      return contraction_major ? (rows % 8 == 0 && ld < (1 << 24)) : ld < (1 << 21);
+    };
+    if (in_place(a, trans_a, M, lda) && in_place(b, !trans_b, N, ldb)) {
+      LinArgs g{a, b, bias, out, M, N, K, lda, ldb, ldo, trans_a ? 1 : 0, trans_b ? 0 : 1};
+      return dtype == TTSDPA_F16 ? launch_mfma_t<F16>(g, s) : launch_mfma_t<BF16>(g, s);
+    }
+  }
 
   // MFMA route: dense row-major copies of the operands that are stored contraction-major, then the x . w^T kernel
   const size_t need = ttlinear_matmul_workspace_bytes(dtype, M, N, K, trans_a, trans_b);
