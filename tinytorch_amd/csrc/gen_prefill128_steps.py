@@ -30,14 +30,18 @@ of line, in subsection 1 of the kernel's section, so that the steady state falls
 Calls with a Bool attnMask (head_dim 128) have a third form of the plain step, TT_P128_MSTEP_...: a score's probability is
 kept iff its mask byte is set (a compare on one byte of a register through SDWA and a select: two more instructions per
 score).  A lane's 16 mask bytes of a 32-key half are four dwords (keys 8g + 4*(lane/32) .. +3 of the lane's query row, g = 0..3) in
-    v[104:119]  mask ring: 4 halves x 4 dwords, half H in place H % 4
-loaded one tile ahead by TT_P128_MLOAD_E / _O (tiles with even / odd index in the unrolled body; operands: the lane's byte offset
-and the scalar address of the tile's first mask byte) and TT_P128_MLOAD_FIRST (halves 1 and 2 of a workgroup's first tile).
+    v[112:119]  mask registers: 2 halves x 4 dwords, half H in place H % 2
+The mask bytes of a tile (a wavefront's 32 rows x 64 keys: 2 KiB) come into LDS by direct loads two tiles ahead
+(TT_P128_MDMA: 2 loads of 16 whole 64-byte row segments each, 16 bytes per lane, so a tile costs 32 line requests where
+loads of every lane's own dwords cost 256) into a ring of two tiles per wavefront: rows 16i .. 16i+15 in KiB i of the
+tile, the 16-byte chunk c of a row segment at 256 c + 16 (row % 16).  A step starts by reading the lane's four dwords of
+the half after next with two ds_read2_b32 (dwords h and h + 2 of chunks 2H and 2H + 1, h = lane/32, H the half of the tile;
+operand mlds: the lane's row in the ring + 4h; TT_P128_MREAD_FIRST: the half the workgroup's first step takes).
 """
 import sys
 
 PD, RING = 6, 8
-MASK0, Q0, VADDR0, SB0, SC0, PA0, PB0, RING0, T0, KADDR0 = 104, 120, 152, 160, 176, 192, 200, 208, 240, 248
+MASK0, Q0, VADDR0, SB0, SC0, PA0, PB0, RING0, T0, KADDR0 = 112, 120, 152, 160, 176, 192, 200, 208, 240, 248
 # set by configure(head_dim): k-steps of a score product (= P.V products of a half), head_dim blocks of 32, slots of a
 # step, scores whose vector work a slot carries, bytes of a tile row and of a stage, slots of the 4-tile body
 KST = NDB = NS = SPS = ROW = STAGE = BODY = 0
@@ -99,8 +103,8 @@ def step(u, kind, elem, masked=False, bmask=False):
             w.append(fma(n + 1))
         if masked:
             w += hide(n)
-        if bmask:  # keep the probability iff the score's mask byte is set: byte n%4 of dword n/4 of the half's place in the ring
-            place = (2 * u + kind + 1) & 3  # the step takes the exponentials of half 2j + kind + 1, j = u (mod 4)
+        if bmask:  # keep the probability iff the score's mask byte is set: byte n%4 of dword n/4 of the half's place
+            place = (kind + 1) & 1  # the step takes the exponentials of half 2j + kind + 1
             w += ["v_cmp_ne_u32_sdwa vcc, %s, %%[zero] src0_sel:BYTE_%d src1_sel:DWORD" % (vr(MASK0 + 4 * place + (n >> 2)), n & 3),
                   "v_cndmask_b32 %s, 0, %s, vcc" % (vr(T[n & 3]), vr(T[n & 3]))]
         if n == 2:  # the sum starts as (score 0) + (score 1): what 0 + x0 + x1 gives
@@ -113,10 +117,14 @@ def step(u, kind, elem, masked=False, bmask=False):
         return w
 
     out.append(fma(0))
+    extra = 0
+    if bmask:  # the mask dwords of half 2j + kind + 2 (tile j+1, its half `kind`) from the wavefront's ring in LDS
+        out += mask_reads((u + 1) & 1, kind, kind & 1)
+        extra = 2  # requests behind those of the step's first operands
     for n in range(NS):
         G = G0 + n
         r = RING0 + 4 * (G % RING)
-        out.append("s_waitcnt lgkmcnt(%d)" % pending_after(G))
+        out.append("s_waitcnt lgkmcnt(%d)" % (pending_after(G) + (extra if n < PD else 0)))
         if n % 2 == 0:
             ks = n // 2
             c = "0" if n == 0 else vr(s_new, 16)
@@ -141,13 +149,21 @@ def prefetch():
     return out
 
 
-def mask_loads(halves, base):
-    """Loads of the mask dwords of `halves` (index relative to the tile whose first mask byte the scalar operand points at, plus
-    `base` bytes) into their ring places; s_nop 4: the scalar address may have been restored by a vector instruction."""
+def mask_reads(region, half, place):
+    """The four mask dwords of half `half` of the tile in ring place `region` into register place `place`."""
+    if region:  # the second ring place lies beyond the 8-bit dword offsets of ds_read2_b32: its own address operand
+        return ["ds_read2_b32 %s, %%[mlds1] offset0:%d offset1:%d" % (vr(MASK0 + 4 * place + 2 * c, 2), 128 * half + 64 * c, 128 * half + 64 * c + 2) for c in range(2)]
+    return ["ds_read2_b32 %s, %%[mlds] offset0:%d offset1:%d" % (vr(MASK0 + 4 * place + 2 * c, 2), 128 * half + 64 * c, 128 * half + 64 * c + 2) for c in range(2)]
+
+
+def mask_dma():
+    """A tile's mask bytes into the wavefront's ring in LDS: load i brings the 64-byte segments of rows 16i .. 16i+15
+    (operands o0, o1: the lane's byte offset for each — its row, rows past the end moved back, and 16-byte chunk; mtile:
+    scalar address of the tile's first key in the mask; dst: LDS address of the ring place).  s_nop 4: the scalar address may
+    have been restored by a vector instruction."""
     out = ["s_nop 4"]
-    for rel, place in halves:
-        for g in range(4):
-            out.append("global_load_dword %s, %%[moff], %%[mtile] offset:%d" % (vr(MASK0 + 4 * place + g), base + 32 * rel + 8 * g))
+    for i in range(2):
+        out += ["s_add_u32 m0, %%[dst], %d" % (1024 * i), "s_nop 0", "global_load_lds_dwordx4 %%[o%d], %%[mtile]" % i]
     return out
 
 
@@ -180,11 +196,10 @@ def main():
                 if head_dim == 128:
                     emit("TT_%s_MSTEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), step(u, kind, elem, bmask=True))  # Bool attnMask
     if head_dim == 128:
-        # tile j (first mask byte at the scalar operand) sends for halves 2j+3 and 2j+4: places (2u+3)%4 and (2u+4)%4, u = j%4
-        emit("TT_%s_MLOAD_E" % NAME, mask_loads([(3, 3), (4, 0)], 0))
-        emit("TT_%s_MLOAD_O" % NAME, mask_loads([(3, 1), (4, 2)], 0))
-        # before the first tile (an index that is a multiple of 4): halves 1 and 2 of that tile, then everything in place
-        emit("TT_%s_MLOAD_FIRST" % NAME, mask_loads([(1, 1), (2, 2)], 0) + ["s_waitcnt vmcnt(0)"])
+        emit("TT_%s_MDMA" % NAME, mask_dma())
+        # before the first step of a workgroup (tile index a multiple of 4: ring place 0): the half it takes, half 1 of that tile
+        # (waited for at once: the first tile's own loads go to the same ring place)
+        emit("TT_%s_MREAD_FIRST" % NAME, mask_reads(0, 1, 1) + ["s_waitcnt lgkmcnt(0)"])
 
 
 if __name__ == "__main__":

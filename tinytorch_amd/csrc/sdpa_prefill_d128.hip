@@ -46,9 +46,11 @@
 // general form on every one of them each of the workgroup's last five tiles waited for one wavefront in that form.
 // Under a causal mask a workgroup takes a row tile and its mirror (equal work for every workgroup), the long one first.
 // A Bool attnMask whose keys can be read four at a time (variant MASKB; the reference's masked fill, src/Function/FuncNNLayer.h:249-255)
-// stays in the pipelined form as well: a lane's 16 mask bytes of a half are four dwords, loaded one tile ahead into a ring of
-// 16 registers, and the step's streams keep a probability iff its byte is set (a byte compare through SDWA and a select per
-// score).  Other masks (additive, other layouts) take the general form of a step.
+// stays in the pipelined form as well.  A wavefront's mask bytes of a tile (32 rows x 64 keys) come into LDS by direct loads two
+// tiles ahead, as whole 64-byte row segments (a ring of two tiles per wavefront in the area the output later leaves through,
+// idle during the loop); a step reads the lane's four dwords of the half after next from there, and its streams keep a
+// probability iff its byte is set (a byte compare through SDWA and a select per score).  Other masks (additive: a ring of 32
+// registers would be needed beside the 200 the pipelined form pins; other layouts) take the general form of a step.
 // Grouped-query attention: kv head = query head / (Hq/Hkv), resolved in the kernel; the workgroup order puts the
 // query heads and row tiles that share a KV head on the same XCD so its L2 holds that K/V once.
 
@@ -314,24 +316,49 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
     if (kt0 + 2 < ntiles_kv) dma_v(kt0 + 2, 2);
   };
   issue_tiles(0);
-  // ---- Bool attnMask in the streams (MASKB): a lane's mask bytes, four keys per dword -------------------------------------
-  // half H of the workgroup's keys sits in places 4(H%4) .. +3 of the ring: dword g = keys 32H + 8g + 4(lane/32) .. +3 of the
-  // lane's query row.  A tile sends for the halves its successor takes (two statements by the tile's parity in the
-  // unrolled body, TT_P128_MLOAD_E / _O), ahead of its K/V loads: the wait at the tile's end covers them.
-  u32x16 mring;
-  unsigned moff = 0;              // the lane's byte offset in the mask: its query row and its four keys of a group
+  // ---- Bool attnMask in the streams (MASKB) -------------------------------------------------------------------------------
+  // Ring in LDS: two tiles of 2 KiB per wavefront behind the K/V stages.  Load i of a tile (two per tile) brings the 64-byte
+  // segments of rows 16i .. 16i+15 of the wavefront, 16 bytes per lane: lane l the chunk l/16 of row 16i + l%16, which lands at
+  // 1024 i + 16 l, i.e. chunk c of row q at 1024 (q/16) + 256 c + 16 (q%16).  A lane (row q, h = lane/32) needs dwords g = 0..3 of
+  // a 32-key half: keys 8g + 4h .. +3, i.e. dwords h and h + 2 of chunks 2H and 2H + 1 of its row (H: the half of the tile).
+  // Registers: half H of the workgroup's keys in places 4(H%2) .. +3.
+  // Tile j sends for the mask bytes of tile j+2 ahead of its K/V loads (the wait at the tile's end covers them), and its two
+  // steps read halves 2j+2 and 2j+3 (tile j+1) into registers for the steps after them.
+  u32x8 mring;
+  unsigned mrow_off[2];           // the lane's byte offset in a (batch, head)'s mask for the two loads of a tile
+  unsigned mlds = 0;              // LDS address of the lane's row in the wavefront's ring, plus 4 * (lane/32)
   const char* mbase = nullptr;    // first mask byte of this (batch, head); uniform
+  unsigned mring_addr = 0;        // LDS address of the wavefront's ring
   if constexpr (MASKB) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) mring[i] = 0u;
+    for (int i = 0; i < 8; i++) mring[i] = 0u;
     int q0, ntiles_kv;
     part_rows(0, q0, ntiles_kv);
-    int qi = q0 + rowgroup * WM + lq;
-    qi = qi < a.L ? qi : a.L - 1;
-    moff = (unsigned)qi * (unsigned)a.ms[2] + 4u * lh;  // the host checks that the last row's offset fits 32 bits
+    const int qw = q0 + rowgroup * WM;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      int row = qw + 16 * i + (lane & 15);
+      row = row < a.L ? row : a.L - 1;  // rows past the end re-read the last one
+      mrow_off[i] = (unsigned)row * (unsigned)a.ms[2] + 16u * (lane >> 4);  // the host checks that the last row's offset fits 32 bits
+    }
     mbase = (const char*)a.mask + b * a.ms[0] + h * a.ms[1];
-    if (S >= 160)  // (shorter rows have no tile in the fast form)
-      asm volatile(TT_P128_MLOAD_FIRST : "+{v[104:119]}"(mring) : [moff] "v"(moff), [mtile] "s"(mbase) : "memory");
+    mring_addr = smem_addr + (KSTAGES + VSTAGES) * STAGE_BYTES + wave * 4096;
+    mlds = mring_addr + 1024 * (lq >> 4) + 16 * (lq & 15) + 4 * lh;
+  }
+  // a tile's mask bytes into ring place `place`; tiles beyond the row's last whole one are moved back into it (nobody takes them)
+  auto mask_dma = [&](int tile, int place) __attribute__((always_inline)) {
+    const int k0 = 64 * tile < S - 64 ? 64 * tile : S - 64;
+    asm volatile(TT_P128_MDMA
+                 :
+                 : [o0] "v"(mrow_off[0]), [o1] "v"(mrow_off[1]), [mtile] "s"(mbase + k0),
+                   [dst] "s"(mring_addr + 2048 * place)
+                 : "memory", "m0", "scc");
+  };
+  if constexpr (MASKB) {
+    if (S >= 160) {  // (shorter rows have no tile in the fast form)
+      mask_dma(kt0, 0);
+      mask_dma(kt0 + 1, 1);
+    }
   }
   u32x32 qv;  // the lane's Q operands, k-step ks in elements 4ks .. 4ks+3
   // Q of a part into its registers, and everything sent for so far in place.  One statement: the compiler takes a statement's
@@ -581,13 +608,13 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
                  "+{v[208:239]}"(ring)                                                                                 \
                : [c] "v"(c), [mc] "v"(mc), "{v[120:151]}"(qv), "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr)            \
                : "v240", "v241", "v242", "v243", "v244", "v245", "memory")
-// the plain step with a Bool attnMask applied to each probability (mask ring v[104:119], a zero in a scalar register)
+// the plain step with a Bool attnMask applied to each probability (mask registers v[112:119], a zero in a scalar register)
 #define TT_P128_RUN_MSTEP(TXT)                                                                                         \
   asm volatile(TXT                                                                                                     \
                : [o0] "+v"(oacc[0]), [o1] "+v"(oacc[1]), [o2] "+v"(oacc[2]), [o3] "+v"(oacc[3]), [ps] "=&v"(psum_step),  \
                  "+{v[160:175]}"(sB), "+{v[176:191]}"(sC), "+{v[192:199]}"(pAv), "+{v[200:207]}"(pBv),                   \
-                 "+{v[208:239]}"(ring), "+{v[104:119]}"(mring)                                                          \
-               : [c] "v"(c), [mc] "v"(mc), [zero] "s"(0), "{v[120:151]}"(qv), "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr) \
+                 "+{v[208:239]}"(ring), "+{v[112:119]}"(mring)                                                          \
+               : [c] "v"(c), [mc] "v"(mc), [zero] "s"(0), [mlds] "v"(mlds), [mlds1] "v"(mlds + 2048), "{v[120:151]}"(qv), "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr) \
                : "v240", "v241", "v242", "v243", "v244", "v245", "vcc", "memory")
   constexpr bool kIsBf16 = sizeof(typename TR::elem) == 2 && __is_same(typename TR::elem, __bf16);
 
@@ -680,9 +707,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       settle_half(s, p, psum_step, masked_kv0, mask_place);
       p_store(pv, p);
     };
-    // MASKB: tile j sends for the mask bytes of halves 2j+3 and 2j+4 (the tile after it takes them); the last tiles'
-    // requests are moved back into the row (nobody takes what they bring)
-    const int mlast = S - 160;
+    if constexpr (MASKB)  // the mask bytes of the half the first step takes (the steps read those of the halves after it)
+      asm volatile(TT_P128_MREAD_FIRST : "+{v[112:119]}"(mring) : [mlds] "v"(mlds), [mlds1] "v"(mlds + 2048) : "memory");
     p_store(pAv, pA);
     p_store(pBv, pB);
     asm volatile(TT_P128_PREFETCH : "+{v[208:239]}"(ring) : "{v[152:159]}"(v_addr), "{v[248:255]}"(k_addr) : "memory");
@@ -690,13 +716,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
 #define TT_P128_TILE(U)                                                                                  \
     if (__builtin_expect(j >= nfast_all, 0)) break;                                                       \
     {                                                                                                    \
-      if constexpr (MASKB) {                                                                             \
-        const int mk0 = 64 * j < mlast ? 64 * j : mlast;                                                 \
-        if constexpr ((U & 1) == 0)                                                                      \
-          asm volatile(TT_P128_MLOAD_E : "+{v[104:119]}"(mring) : [moff] "v"(moff), [mtile] "s"(mbase + mk0) : "memory"); \
-        else                                                                                             \
-          asm volatile(TT_P128_MLOAD_O : "+{v[104:119]}"(mring) : [moff] "v"(moff), [mtile] "s"(mbase + mk0) : "memory"); \
-      }                                                                                                  \
+      if constexpr (MASKB) mask_dma(j + 2, U & 1);                                                       \
       const int keep = PAGED ? tile_dma(j) : tile_dma_fast(j, U);                                        \
       /* mk = 1: the tile's exponentials take the causal predicate; kvs = first key of the half whose exponentials   \
          the step takes; kvm = kvs on such a tile, else -1.  As scalar instructions: the compiler's own form of     \
@@ -711,7 +731,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       else if constexpr (MASKB) TT_P128_RUN_MSTEP(TT_P128_MSTEP_F16_U##U##_K0);                          \
       else if constexpr (kIsBf16) TT_P128_RUN_PSTEP(TT_P128_PSTEP_BF16_U##U##_K0);                       \
       else TT_P128_RUN_PSTEP(TT_P128_PSTEP_F16_U##U##_K0);                                               \
-      settle_fast(sB, pBv, kvm0, MASKB ? (2 * U + 1) & 3 : -1);                                          \
+      settle_fast(sB, pBv, kvm0, MASKB ? 1 : -1);                                                        \
       kvs += 32;                                                                                         \
       if constexpr (kIsBf16 && CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_BF16_U##U##_K1);                    \
       else if constexpr (CAUSAL) TT_P128_RUN_STEP(TT_P128_STEP_F16_U##U##_K1);                           \
@@ -719,7 +739,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill128_kernel(KArgs a) {
       else if constexpr (MASKB) TT_P128_RUN_MSTEP(TT_P128_MSTEP_F16_U##U##_K1);                          \
       else if constexpr (kIsBf16) TT_P128_RUN_PSTEP(TT_P128_PSTEP_BF16_U##U##_K1);                       \
       else TT_P128_RUN_PSTEP(TT_P128_PSTEP_F16_U##U##_K1);                                               \
-      settle_fast(sC, pAv, kvm1, MASKB ? (2 * U + 2) & 3 : -1);                                          \
+      settle_fast(sC, pAv, kvm1, MASKB ? 0 : -1);                                                        \
       dma_wait_and_sync(keep);                                                                           \
       j++;                                                                                               \
     }
