@@ -77,9 +77,12 @@ WORKLOADS = {
     "config3_d64": (2, 32, 8, 4096, 4096, 64, "bf16", True, 1.0, "mfma"),   # config 3's shape at head_dim 64
     # one GPU's share of config 3 when its 8 KV heads are dealt out to 8 GPUs (no exchange between them): 128 row tiles
     "config3_share8": (2, 4, 1, 4096, 4096, 128, "bf16", True, 1.0, "mfma"),
+    # config 3's shape with a Bool attnMask [L, S] instead of the causal flag (the reference's masked fill; every product is executed)
+    "config3_boolmask": (2, 32, 8, 4096, 4096, 128, "bf16", False, 1.0, "mfma"),
 }
+MASKED = {"config3_boolmask"}  # workloads that pass an attnMask: [L, S] Bool, about 70 % of the entries set, the first key always
 SEEDS = {"config1": 0x5EED0001, "config2": 0x5EED0002, "config3": 0x5EED0003, "config4": 0x5EED0004, "config5": 0x5EED0005,
-         "config3_f32": 0x5EED0003, "config3_d64": 0x5EED0006, "config3_share8": 0x5EED0007}
+         "config3_f32": 0x5EED0003, "config3_d64": 0x5EED0006, "config3_share8": 0x5EED0007, "config3_boolmask": 0x5EED0008}
 DESCR = {
     "config1": "fp32 causal SDPA B1 H4 S128 D64",
     "config2": "fp16 causal MHA prefill B4 H32 S2048 D128",
@@ -89,6 +92,7 @@ DESCR = {
     "config3_f32": "fp32 causal GQA prefill B2 32q/8kv S4096 D128",
     "config3_d64": "bf16 causal GQA prefill B2 32q/8kv S4096 D64",
     "config3_share8": "bf16 causal GQA prefill B2 4q/1kv S4096 D128 (one KV head of config 3: an 8-GPU head-sharded share)",
+    "config3_boolmask": "bf16 GQA prefill B2 32q/8kv S4096 D128 with a Bool attnMask [L,S] (not causal)",
 }
 
 
@@ -161,6 +165,18 @@ def synth_qkv(name):
     return q, k, v
 
 
+def synth_mask(name):
+    """The workload's attnMask on the device (None unless it has one): uniform numbers from the same generator, set where
+    below 0.7 of the unit normal's range; key 0 visible to every row."""
+    if name not in MASKED:
+        return None
+    from tinytorch_amd import synth
+    B, Hq, Hkv, L, S, D, dtype, causal, mul, bound = WORKLOADS[name]
+    m = synth.randn(SEEDS[name], 7, (L, S)) < 0.5244  # P(N(0,1) < 0.5244) = 0.70
+    m[:, 0] = True
+    return m
+
+
 def run_gpu(name, steps, warmup, zero_inputs=False):
     import torch
     from tinytorch_amd import _capi, build_params
@@ -170,7 +186,8 @@ def run_gpu(name, steps, warmup, zero_inputs=False):
     if zero_inputs:  # the same launch without operand toggling
         q.zero_(), k.zero_(), v.zero_()
     out = torch.empty_like(q)
-    p = build_params(q, k, v, out, causal)
+    mask = synth_mask(name)
+    p = build_params(q, k, v, out, causal, mask)
     lib = _capi.lib()
     rc, route = _capi.plan(p)
     assert rc == 0, _capi.status_string(rc)
@@ -202,7 +219,7 @@ def run_gpu(name, steps, warmup, zero_inputs=False):
                      "kernel_ms_min": round(t["min_ms"], 5), "timing": "median of %d launches, one HIP event pair each" % steps,
                      "settle_launches": t["settle_launches"], "algorithmic_flops": flops, "algorithmic_bytes": abytes},
     }
-    return res, (q, k, v, out)
+    return res, (q, k, v, out, mask)
 
 
 def run_probes():
@@ -460,7 +477,8 @@ def run_cpu_baseline(name, tensors, budget_s=20.0, corner=None):
     import oracle
 
     B, Hq, Hkv, L, S, D, dtype, causal, mul, bound = WORKLOADS[name]
-    q, k, v, out = tensors
+    q, k, v, out, mask = tensors
+    mask_h = None if mask is None else mask.cpu().numpy().astype(np.uint8)
     kind = "reference" if oracle.have_ref() else "port"
     fn = oracle.ref_sdpa_f32 if kind == "reference" else (lambda *a, **kw: oracle.sdpa_f32(*a, nthreads=1, **kw))
     G = Hq // Hkv
@@ -475,7 +493,7 @@ def run_cpu_baseline(name, tensors, budget_s=20.0, corner=None):
         ks = k[b:b + 1, h // G:h // G + 1, :S].float().cpu().numpy()
         vs = v[b:b + 1, h // G:h // G + 1, :S].float().cpu().numpy()
         t0 = time.perf_counter()
-        ref = fn(qs, ks, vs, causal=causal)
+        ref = fn(qs, ks, vs, causal=causal) if mask_h is None else fn(qs, ks, vs, causal=causal, mask=mask_h)
         dt = time.perf_counter() - t0
         err = float(np.abs(ref - out[b:b + 1, h:h + 1, :L].float().cpu().numpy()).max())
         worst = max(worst, err)
@@ -508,6 +526,8 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-probes", action="store_true", help="skip the hardware ceiling probes")
     ap.add_argument("--no-zero", action="store_true", help="skip the repeat of the headline launch on all-zero operands")
+    ap.add_argument("--zero-inputs", action="store_true",
+                    help="run the workload on all-zero Q, K, V only (for profiling the same instruction stream without operand toggling)")
     ap.add_argument("--settle", type=float, default=None,
                     help="seconds of untimed launches after the warm-up (default %.1f; 0 for counter runs that only need a few dispatches)" % SETTLE_SECONDS)
     ap.add_argument("--no-other", action="store_true", help="skip the baseline's other configurations (1, 2, 5) and head_dim 64")
@@ -546,13 +566,13 @@ def main():
         print(json.dumps(run_backward(args.steps, args.warmup, cpu=not args.no_cpu and args.backward_dtype == "bf16",
                                       dtype=args.backward_dtype)), flush=True)
         return
-    main_res, tensors = run_gpu(args.workload, args.steps, args.warmup)
+    main_res, tensors = run_gpu(args.workload, args.steps, args.warmup, zero_inputs=args.zero_inputs)
     ceilings = None if args.no_probes else run_probes()
     cpu = None if args.no_cpu else run_cpu_baseline(args.workload, tensors, args.cpu_seconds)
     del tensors
     torch.cuda.empty_cache()
     main_res["roofline"]["traffic_source"] = TRAFFIC_SOURCE  # for every "traffic" figure of this line
-    if not args.no_zero and WORKLOADS[args.workload][9] == "mfma":
+    if not args.no_zero and not args.zero_inputs and WORKLOADS[args.workload][9] == "mfma":
         # the same launch on all-zero operands: the instruction stream without operand toggling (the kernel is power-bound
         # on N(0,1) data: the chip lowers its clock under it)
         z, tensors = run_gpu(args.workload, args.steps, args.warmup, zero_inputs=True)
@@ -594,7 +614,7 @@ def main():
         # the baseline's other configurations (config 1: launch-sized, its time is the figure) and head_dim 64
         line["other_configs"] = []
         for name, corner, budget in (("config1", None, 2.0), ("config2", None, 4.0), ("config5", 4096, 4.0),
-                                     ("config3_d64", 2048, 3.0), ("config3_share8", 2048, 2.0)):
+                                     ("config3_d64", 2048, 3.0), ("config3_share8", 2048, 2.0), ("config3_boolmask", None, 3.0)):
             torch.cuda.empty_cache()
             res, tensors = run_gpu(name, max(1, min(args.steps, 50)), min(args.warmup, 20))
             if not args.no_cpu:
