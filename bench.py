@@ -25,7 +25,8 @@ reported under "other_configs".
 
 "roofline"."zero_operands" is the headline launch repeated on all-zero Q, K, V: the same instruction stream without operand
 toggling, i.e. what the kernel's schedule reaches when the chip's power management leaves the clock alone (the prefill
-kernel is power-bound on N(0,1) data).  "roofline"."summary" lists the fraction of every other line of the run.
+kernel is power-bound on N(0,1) data).  "roofline"."summary" lists the fraction of every other line of the run, and the
+line's last key, "in_short", repeats the headline, decode and summary figures in a few hundred characters.
 
 Algorithmic work per launch (what "achieved" divides by the measured launch time):
   prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)
@@ -638,6 +639,17 @@ def main():
         summary["backward_f32"] = line["backward"]["fp32"]["roofline"]["frac"]
     if summary:  # fraction of its own roofline for every other line of this run (config1: launch-sized, its kernel ms)
         line["roofline"]["summary"] = summary
+    # the figures the metric is quoted on once more as the line's last key: a record that keeps only the end of a
+    # long line still holds them
+    r = line["roofline"]
+    line["in_short"] = {"prefill_%s" % args.workload: {"frac": r["frac"], "kernel_ms": r["kernel_ms"], "achieved": r["achieved"], "unit": r["unit"]}}
+    if "zero_operands" in r:
+        line["in_short"]["prefill_%s_zero_operands_frac" % args.workload] = r["zero_operands"]["frac"]
+    if "decode" in r:
+        d = r["decode"]
+        line["in_short"]["decode_config4"] = {"frac": d["frac"], "kernel_ms": d["kernel_ms"], "achieved": d["achieved"], "unit": d["unit"]}
+    if summary:
+        line["in_short"]["frac_of_other_lines"] = summary
     print(json.dumps(line), flush=True)
 
 
