@@ -67,7 +67,11 @@ def test_struct_layout_matches_header():
     ((_capi.BF16, 1, 8, 8, 300, 300, 64), _capi.ROUTE_PREFILL),
     ((_capi.BF16, 1, 8, 8, 300, 300, 96), _capi.ROUTE_PREFILL),
     ((_capi.F16, 1, 8, 8, 300, 300, 256), _capi.ROUTE_PREFILL),
-    ((_capi.BF16, 1, 8, 8, 300, 300, 80), _capi.ROUTE_GENERAL),      # not one of the MFMA head sizes
+    ((_capi.BF16, 1, 8, 8, 300, 300, 80), _capi.ROUTE_PREFILL),      # a multiple of 8: the head_dim-96 kernel with zero columns
+    ((_capi.F16, 1, 8, 8, 300, 300, 8), _capi.ROUTE_PREFILL),
+    ((_capi.F16, 1, 8, 8, 300, 300, 248), _capi.ROUTE_PREFILL),
+    ((_capi.BF16, 1, 8, 8, 300, 300, 84), _capi.ROUTE_GENERAL),      # rows that are not whole 16-byte chunks
+    ((_capi.BF16, 1, 8, 8, 300, 300, 20), _capi.ROUTE_GENERAL),
     ((_capi.BF16, 1, 64, 2, 1, 4096, 128), _capi.ROUTE_PREFILL),     # 32 rows per KV head: too many for decode
     ((_capi.BF16, 1, 8, 8, 0, 16, 128), _capi.ROUTE_NONE),
     ((_capi.BF16, 0, 8, 8, 4, 16, 128), _capi.ROUTE_NONE),
@@ -86,7 +90,8 @@ def test_routes_depend_on_flags():
     assert _capi.plan(params(*base, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_PREFILL
     assert _capi.plan(params(_capi.BF16, 2, 8, 2, 64, 512, 128, mask_kind=_capi.MASK_ADD, mask=FAKE))[1] == _capi.ROUTE_PREFILL
     assert _capi.plan(params(_capi.BF16, 2, 8, 2, 512, 512, 64, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_PREFILL
-    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 512, 512, 80, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 512, 512, 80, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.BF16, 2, 8, 2, 512, 512, 84, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
     assert _capi.plan(params(*base, scale=-1.0))[1] == _capi.ROUTE_GENERAL
     p = params(*base)
     p.k_stride[2] = 132  # rows not 16-byte aligned
@@ -154,7 +159,8 @@ def test_kv_len_routes_and_append_validation():
     assert _capi.plan(params(*base, causal=1, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
     assert _capi.plan(params(_capi.BF16, 2, 32, 8, 4096, 4096, 64, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
     assert _capi.plan(params(_capi.BF16, 2, 32, 8, 100, 4096, 128, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
-    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 100, 4096, 80, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 100, 4096, 80, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.BF16, 2, 32, 8, 100, 4096, 84, kv_len=FAKE))[1] == _capi.ROUTE_GENERAL
     assert _capi.plan(params(_capi.BF16, 8, 32, 8, 1, 4096, 128, kv_len=FAKE))[1] == _capi.ROUTE_DECODE
     assert _capi.plan(params(_capi.BF16, 8, 32, 8, 1, 4096, 128, kv_len=FAKE + 2))[0] == _capi.ERR_STRIDE
     L = _capi.lib()

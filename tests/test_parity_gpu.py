@@ -450,6 +450,71 @@ def test_other_head_sizes_on_the_mfma_route(D, dtype, causal):
     assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("D", [8, 24, 40, 56, 72, 80, 112, 120, 136, 160, 192, 200, 248])
+@pytest.mark.parametrize("dtype,causal", [("bf16", True), ("f16", False)])
+def test_head_sizes_between_the_mfma_kernels(D, dtype, causal):
+    # any multiple of 8 up to 256 runs on the matrix-core kernel of the next size up (the reference takes any head size)
+    B, Hq, Hkv, L, S = 2, 6, 2, 200, 200 if causal else 330
+    say("padded head_dim", (D, dtype, causal))
+    host, dev = make_inputs(195 + D, B, Hq, Hkv, L, S, D, dtype, 0.7)
+    assert route_of(*dev, causal=causal) == "prefill"
+    exp = oracle.sdpa_f32(*host, causal=causal)
+    rc, out = call("forward", *dev, causal=causal)
+    assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("D", [40, 80, 200])
+def test_head_sizes_between_the_mfma_kernels_read_and_write_their_columns_only(D):
+    # q, k, v and out are views of wider rows whose other columns hold NaN (inputs) or a sentinel (output)
+    B, Hq, Hkv, L, S, W = 1, 4, 2, 150, 260, 256
+    say("padded head_dim in wider rows", D)
+    host, dev = make_inputs(411 + D, B, Hq, Hkv, L, S, D, "bf16", 0.7)
+    wide = []
+    for t in dev:
+        w = torch.full(t.shape[:-1] + (W,), float("nan"), dtype=t.dtype, device="cuda")
+        w[..., :D] = t
+        wide.append(w[..., :D])
+    exp = oracle.sdpa_f32(*host, causal=True)
+    from tinytorch_amd import sdpAttention
+    assert route_of(*wide, causal=True) == "prefill"
+    y = sdpAttention(*wide, isCausal=True)
+    assert max_abs_err(y, exp) <= TOL["bf16"]
+    outw = torch.full((B, Hq, L, W), 7.0, dtype=torch.bfloat16, device="cuda")
+    rc, _ = call("forward", *wide, causal=True, out=outw[..., :D])
+    assert rc == 0 and max_abs_err(outw[..., :D], exp) <= TOL["bf16"] and bool((outw[..., D:] == 7.0).all())
+
+
+@pytest.mark.parametrize("D,kind", [(80, "bool"), (48, "add"), (160, "bool")])
+def test_head_sizes_between_the_mfma_kernels_with_masks_key_counts_and_grouped_heads(D, kind):
+    B, Hq, Hkv, L, S = 2, 8, 2, 140, 264
+    say("padded head_dim, mask", (D, kind))
+    host, dev = make_inputs(511 + D, B, Hq, Hkv, L, S, D, "f16", 0.7)
+    rng = np.random.RandomState(D)
+    if kind == "bool":
+        m = (rng.rand(L, S) > 0.4).astype(np.uint8)
+        m[:, 1] = 1
+        md = torch.from_numpy(m).cuda().bool()
+    else:
+        m = rng.randn(Hq, L, S).astype(np.float32)
+        md = torch.from_numpy(m).cuda().half()
+        m = md.float().cpu().numpy()
+    assert route_of(*dev, mask=md) == "prefill"
+    rc, out = call("forward", *dev, mask=md)
+    assert rc == 0 and max_abs_err(out, oracle.sdpa_f32(*host, mask=m)) <= TOL["f16"]
+    # per-batch key counts, bottom-right causal, few rows per head (the grouped heads of a KV head are packed into one)
+    from tinytorch_amd import sdpAttention
+    lens = np.array([S, 77], np.int32)
+    ld = torch.from_numpy(lens).cuda()
+    Lq = 5
+    q = dev[0][:, :, :Lq].contiguous()
+    y = sdpAttention(q, dev[1], dev[2], isCausal=True, kvLens=ld, causalAlign="bottom-right")
+    for b in range(B):
+        n = int(lens[b])
+        mask = np.tril(np.ones((Lq, n), np.uint8), n - Lq)
+        e = oracle.sdpa_f32(host[0][b:b + 1, :, :Lq], host[1][b:b + 1, :, :n], host[2][b:b + 1, :, :n], mask=mask)
+        assert max_abs_err(y[b:b + 1], e) <= TOL["f16"]
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
 def test_per_batch_key_counts_on_the_mfma_route(causal, dtype):

@@ -63,7 +63,10 @@ __device__ __forceinline__ vec8 v_operand(const void* lane_base, int byte_off_lo
 }
 
 // MASKED: an attnMask is applied (a variant of its own: the mask addressing costs registers the other variants keep).
-template <typename TR, int D, bool CAUSAL, bool MASKED>
+// PAD: the tensors' head_dim a.D is a multiple of 8 below D.  The 16-byte chunks of a row beyond a.D are taken as zeros
+// (Q and K: they add nothing to a score; V: columns of the output that are not stored), everything else is the
+// kernel for head_dim D.  The reference takes any head size (src/Function/FuncNNLayer.h:231-236).
+template <typename TR, int D, bool CAUSAL, bool MASKED, bool PAD>
 __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
@@ -119,7 +122,14 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
     row = row < a.L ? row : a.L - 1;
     const T* qr = qp + row * a.qs[2] + 8 * lh;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) qreg[ks] = *(const vec8*)(qr + 16 * ks);
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      if (!PAD || 16 * ks + 8 * lh < a.D) {
+        qreg[ks] = *(const vec8*)(qr + 16 * ks);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) qreg[ks][i] = (T)0.f;
+      }
+    }
   }
 
   f32x16 oacc[DBLK];
@@ -144,7 +154,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
       typename TR::vec4 zero;
 #pragma unroll
       for (int i = 0; i < 4; i++) zero[i] = (T)0.f;
-      for (int d = 4 * lh; d < D; d += 8) *(typename TR::vec4*)(op + d) = zero;
+      for (int d = 4 * lh; d < (PAD ? a.D : D); d += 8) *(typename TR::vec4*)(op + d) = zero;
     }
     return;
   }
@@ -170,14 +180,18 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
   // thread t moves chunks t, t+256, ...: chunk c is row c / (D/8), 16-byte column c % (D/8)
   u32x4 kst[NLD], vst[NLD];
   unsigned koff[NLD], voff[NLD];  // byte offsets of this thread's chunks inside a full tile
-  int lrow[NLD], lcol[NLD];
+  int lrow[NLD], lcol[NLD], gcol[NLD];
+  bool cval[NLD];                 // PAD: the chunk lies inside the tensors' rows; the others are loaded from the row's
+                                  // first chunk instead (the loads stay unconditional) and reach LDS as zeros
 #pragma unroll
   for (int i = 0; i < NLD; i++) {
     int cidx = tid + 256 * i;
     lrow[i] = cidx / (D / 8);
     lcol[i] = cidx % (D / 8);
-    koff[i] = (unsigned)(lrow[i] * a.ks[2] + 8 * lcol[i]) * 2u;
-    voff[i] = (unsigned)(lrow[i] * a.vs[2] + 8 * lcol[i]) * 2u;
+    cval[i] = !PAD || 8 * lcol[i] < a.D;
+    gcol[i] = cval[i] ? lcol[i] : 0;
+    koff[i] = (unsigned)(lrow[i] * a.ks[2] + 8 * gcol[i]) * 2u;
+    voff[i] = (unsigned)(lrow[i] * a.vs[2] + 8 * gcol[i]) * 2u;
   }
   auto load_tile = [&](int kv0) {
     const T* ktile = kp + kv_tile_offset(a, table, kv0, a.ks[2], a.ks[0]);
@@ -195,8 +209,8 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
       for (int i = 0; i < NLD; i++) {
         int row = lrow[i];
         row = kv0 + row < S ? row : S - 1 - kv0;
-        kst[i] = *(const u32x4*)(ktile + row * a.ks[2] + 8 * lcol[i]);
-        vst[i] = *(const u32x4*)(vtile + row * a.vs[2] + 8 * lcol[i]);
+        kst[i] = *(const u32x4*)(ktile + row * a.ks[2] + 8 * gcol[i]);
+        vst[i] = *(const u32x4*)(vtile + row * a.vs[2] + 8 * gcol[i]);
       }
     }
   };
@@ -205,8 +219,9 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
     T* Vs = Ks + BN * K_PITCH;
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
-      *(u32x4*)(Ks + lrow[i] * K_PITCH + 8 * lcol[i]) = kst[i];
-      *(u32x4*)(Vs + lrow[i] * V_PITCH + 8 * lcol[i]) = vst[i];
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+      *(u32x4*)(Ks + lrow[i] * K_PITCH + 8 * lcol[i]) = cval[i] ? kst[i] : zero;
+      *(u32x4*)(Vs + lrow[i] * V_PITCH + 8 * lcol[i]) = cval[i] ? vst[i] : zero;
     }
   };
 
@@ -358,27 +373,29 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void prefill_kernel(KArgs a
 #pragma unroll
         for (int i = 0; i < 4; i++) x[i] = oacc[db][4 * rg + i] * inv;
         typename TR::vec4 y = __builtin_convertvector(x, typename TR::vec4);
-        *(typename TR::vec4*)(op + 32 * db + 8 * rg + 4 * lh) = y;
+        if (!PAD || 32 * db + 8 * rg + 4 * lh < a.D) *(typename TR::vec4*)(op + 32 * db + 8 * rg + 4 * lh) = y;
       }
   }
 }
 
-template <typename TR, int D, bool CAUSAL, bool MASKED>
+template <typename TR, int D, bool CAUSAL, bool MASKED, bool PAD>
 int launch_prefill_k(const KArgs& a, dim3 grid, hipStream_t stream) {
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)prefill_kernel<TR, D, CAUSAL, MASKED>, PrefillLds<D>::BYTES, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill_kernel<TR, D, CAUSAL, MASKED, PAD>, PrefillLds<D>::BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
-  hipLaunchKernelGGL((prefill_kernel<TR, D, CAUSAL, MASKED>), grid, dim3(256), PrefillLds<D>::BYTES, stream, a);
+  hipLaunchKernelGGL((prefill_kernel<TR, D, CAUSAL, MASKED, PAD>), grid, dim3(256), PrefillLds<D>::BYTES, stream, a);
   return (int)hipGetLastError();
 }
 
-template <typename TR, int D>
+template <typename TR, int D, bool PAD>
 int launch_prefill_t(const KArgs& a, hipStream_t stream) {
+  // the callers keep to this (the records of a split are laid out for D, rows are read in 16-byte chunks)
+  if (PAD && (a.kv_splits > 1 || a.D % 8 != 0 || a.D >= D || a.D < 8)) return (int)hipErrorInvalidValue;
   long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM) * (a.kv_splits > 1 ? a.kv_splits : 1);
   dim3 grid((unsigned)nwg);
-  if (a.mask_kind != 0) return launch_prefill_k<TR, D, false, true>(a, grid, stream);  // exclusive with causal (validated)
-  return a.causal ? launch_prefill_k<TR, D, true, false>(a, grid, stream) : launch_prefill_k<TR, D, false, false>(a, grid, stream);
+  if (a.mask_kind != 0) return launch_prefill_k<TR, D, false, true, PAD>(a, grid, stream);  // exclusive with causal (validated)
+  return a.causal ? launch_prefill_k<TR, D, true, false, PAD>(a, grid, stream) : launch_prefill_k<TR, D, false, false, PAD>(a, grid, stream);
 }
 
 }  // namespace
@@ -386,12 +403,21 @@ int launch_prefill_t(const KArgs& a, hipStream_t stream) {
 template <typename TR>
 int launch_prefill_d(const KArgs& a, hipStream_t stream) {
   switch (a.D) {
-    case 32: return launch_prefill_t<TR, 32>(a, stream);
-    case 64: return launch_prefill_t<TR, 64>(a, stream);
-    case 96: return launch_prefill_t<TR, 96>(a, stream);
-    case 128: return launch_prefill_t<TR, 128>(a, stream);
-    default: return launch_prefill_t<TR, 256>(a, stream);
+    case 32: return launch_prefill_t<TR, 32, false>(a, stream);
+    case 64: return launch_prefill_t<TR, 64, false>(a, stream);
+    case 96: return launch_prefill_t<TR, 96, false>(a, stream);
+    case 128: return launch_prefill_t<TR, 128, false>(a, stream);
+    case 192: return launch_prefill_t<TR, 192, false>(a, stream);
+    case 256: return launch_prefill_t<TR, 256, false>(a, stream);
+    default: break;
   }
+  // any other multiple of 8 up to 256: the kernel of the next size up, the missing columns as zeros
+  if (a.D < 32) return launch_prefill_t<TR, 32, true>(a, stream);
+  if (a.D < 64) return launch_prefill_t<TR, 64, true>(a, stream);
+  if (a.D < 96) return launch_prefill_t<TR, 96, true>(a, stream);
+  if (a.D < 128) return launch_prefill_t<TR, 128, true>(a, stream);
+  if (a.D < 192) return launch_prefill_t<TR, 192, true>(a, stream);
+  return launch_prefill_t<TR, 256, true>(a, stream);
 }
 
 int launch_prefill(const KArgs& a, int dtype, hipStream_t stream) {

@@ -217,7 +217,8 @@ SplitPlan plan_pipelined_splits(const ttsdpa_params* p) {
 bool prefill_ok(const ttsdpa_params* p) {
   if (f32_prefill_ok(p)) return true;
   // the pipelined head_dim-128 kernel takes any attnMask; the 4-wavefront kernel those it can read four keys at a time
-  const bool mfma_head_dim = p->D == 32 || p->D == 64 || p->D == 96 || p->D == 128 || p->D == 256;
+  // head sizes between the 4-wavefront kernel's (32, 64, 96, 128, 192, 256) run on the next one up with zero columns
+  const bool mfma_head_dim = p->D >= 8 && p->D <= 256 && p->D % 8 == 0;
   if (p->block_table && p->page_size < kPrefillMinPage) return false;
   // the 16-bit kernels address the rows of a K / V tile with 32-bit byte offsets (the fp32 kernel returned above does not)
   const bool tile_offsets_ok = p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24);
