@@ -69,17 +69,22 @@ def test_head_dim_64_pipelined_bottom_right_and_key_counts(dtype):
 
 
 def test_head_dim_64_pipelined_equals_the_4_wavefront_kernel_within_rounding():
-    # the same call through both kernels: causal on the pipelined kernel, and the same triangle as a Bool attnMask, which
-    # the pipelined kernel does not take (one batch entry: the other kernel reads the mask from memory)
+    # the same call through both kernels: causal on the pipelined kernel, and the same triangle as an additive attnMask
+    # (0 / -inf), which the pipelined kernel does not take (one batch entry: the other kernel reads the mask from memory)
     B, Hq, Hkv, L, S, D = 4, 64, 16, 512, 512, 64
     host, dev = make_inputs(4242, B, Hq, Hkv, L, S, D, "bf16", 0.8)
     rc, big = call("forward", *dev, causal=True)
     assert rc == 0
     tril = torch.ones(L, S, dtype=torch.bool, device="cuda").tril()
-    rc, one = call("forward", dev[0][:1].contiguous(), dev[1][:1].contiguous(), dev[2][:1].contiguous(), mask=tril)
+    first = (dev[0][:1].contiguous(), dev[1][:1].contiguous(), dev[2][:1].contiguous())
+    bias = torch.zeros(L, S, dtype=torch.bfloat16, device="cuda").masked_fill(~tril, float("-inf"))
+    rc, one = call("forward", *first, mask=bias)
     assert rc == 0
     d = (big[:1].float() - one.float()).abs().max().item()
     assert 0 < d <= 2e-2   # two kernels: close, not identical
+    # the triangle as a Bool attnMask runs in the pipelined kernel's streams like the causal flag
+    rc, two = call("forward", *first, mask=tril)
+    assert rc == 0 and (big[:1].float() - two.float()).abs().max().item() <= 2e-2
     # causal row 0 is v[0] exactly on both
     assert torch.equal(big[:, :, 0, :], dev[2][:, :, 0, :].repeat_interleave(Hq // Hkv, dim=1))
     assert torch.equal(one[:, :, 0, :], dev[2][:1, :, 0, :].repeat_interleave(Hq // Hkv, dim=1))

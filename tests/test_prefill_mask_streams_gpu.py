@@ -1,6 +1,6 @@
-"""Bool attnMasks applied inside the pipelined head_dim-128 kernel's instruction streams (a lane's mask bytes loaded one
-tile ahead into a register ring, a byte compare and a select per probability): against the oracle, which restates the
-reference's masked fill and broadcasting add (reference src/Function/FuncNNLayer.h:249-260)."""
+"""Bool attnMasks applied inside the pipelined kernels' instruction streams (head_dim 128 and 64: a wavefront's mask bytes
+of a tile brought into LDS two tiles ahead, a byte compare and a select per probability): against the oracle, which
+restates the reference's masked fill and broadcasting add (reference src/Function/FuncNNLayer.h:249-260)."""
 import numpy as np
 import pytest
 import torch
@@ -29,11 +29,16 @@ def bool_mask(seed, shape, keep=0.6):
     (1, 4, 4, 600, 164, (4, 600, 164), "bf16"),           # the shortest rows that still have a tile in that form
     (1, 2, 2, 384, 156, (384, 156), "f16"),               # below it: every step in the general form
     (1, 3, 1, 1024, 4096, (1024, 4096), "bf16"),          # grouped heads, long rows
+    # (the head_dim-64 pipelined kernel takes calls of 512 rows and more)
+    (2, 4, 2, 700, 1024, (2, 4, 700, 1024), "f16"),       # a mask per (batch, head), ragged last row tile
+    (2, 4, 1, 513, 1000, (2, 1, 1, 1000), "bf16"),        # key padding; keys not a multiple of the 64-key tile
+    (1, 2, 2, 640, 156, (640, 156), "f16"),               # every step in the general form
 ], ids=lambda c: "B%dH%dk%dL%dS%d-m%s-%s" % (c[0], c[1], c[2], c[3], c[4], "x".join(map(str, c[5])), c[6]))
-def test_bool_mask_in_streams_against_oracle(case):
+@pytest.mark.parametrize("D", [128, 64])
+def test_bool_mask_in_streams_against_oracle(case, D):
     B, Hq, Hkv, L, S, mshape, dtype = case
-    say("bool mask in streams", case)
-    host, dev = make_inputs(700 + L + S, B, Hq, Hkv, L, S, 128, dtype)
+    say("bool mask in streams", case, D)
+    host, dev = make_inputs(700 + L + S + D, B, Hq, Hkv, L, S, D, dtype)
     m = bool_mask(L + S, mshape)
     md = torch.from_numpy(m).cuda().bool()
     assert route_of(*dev, mask=md) == "prefill"
@@ -45,12 +50,14 @@ def test_bool_mask_in_streams_against_oracle(case):
     assert err <= TOL[dtype]
 
 
-def test_hidden_scores_do_not_enter_the_maximum():
+@pytest.mark.parametrize("D", [128, 64])
+def test_hidden_scores_do_not_enter_the_maximum(D):
     """Large scores behind cleared mask bytes: the maximum the exponentials are taken against is raised from visible
     scores only (a hidden score of 300 would flush every visible probability to zero), also where it is raised inside
     the pipelined form."""
-    B, Hq, Hkv, L, S, D = 1, 2, 2, 512, 1024, 128
-    host, dev = make_inputs(733, B, Hq, Hkv, L, S, D, "bf16", 0.5)
+    B, Hq, Hkv, L, S = 1, 2, 2, 512, 1024
+    say("hidden large scores", D)
+    host, dev = make_inputs(733, B, Hq, Hkv, L, S, D, "bf16", 0.5 if D == 128 else 0.7)
     q, k, v = host
     k = k.copy()
     rng = np.random.RandomState(5)
@@ -73,8 +80,10 @@ def test_hidden_scores_do_not_enter_the_maximum():
     assert rc == 0 and np.abs(to_host_f32(out) - to_host_f32(out2)).max() <= 2e-2
 
 
-def test_fully_hidden_rows_and_views():
-    B, Hq, Hkv, L, S, D = 2, 4, 2, 520, 640, 128
+@pytest.mark.parametrize("D", [128, 64])
+def test_fully_hidden_rows_and_views(D):
+    B, Hq, Hkv, L, S = 2, 4, 2, 520, 640
+    say("fully hidden rows, mask views", D)
     host, dev = make_inputs(741, B, Hq, Hkv, L, S, D, "bf16")
     m = bool_mask(3, (B, 1, L, S))
     m[0, 0, 17] = 0             # rows without a visible key: NaN in the reference (0 * inf)

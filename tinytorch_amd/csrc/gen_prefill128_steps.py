@@ -27,7 +27,7 @@ key is visible iff kvs + 8*(n/4) + n%4 <= rl: two more instructions per score, a
 select).  The second form serves the one or two tiles of a wavefront's row group that touch the diagonal; it sits out
 of line, in subsection 1 of the kernel's section, so that the steady state falls through without a taken branch.
 
-Calls with a Bool attnMask (head_dim 128) have a third form of the plain step, TT_P128_MSTEP_...: a score's probability is
+Calls with a Bool attnMask have a third form of the plain step, TT_P128_MSTEP_... (TT_P64_MSTEP_...): a score's probability is
 kept iff its mask byte is set (a compare on one byte of a register through SDWA and a select: two more instructions per
 score).  A lane's 16 mask bytes of a 32-key half are four dwords (keys 8g + 4*(lane/32) .. +3 of the lane's query row, g = 0..3) in
     v[112:119]  mask registers: 2 halves x 4 dwords, half H in place H % 2
@@ -193,13 +193,11 @@ def main():
                         + step(u, kind, elem, True) + ["s_branch %s_e%%=" % lab, ".subsection 0"])
                 emit("TT_%s_STEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), both)
                 emit("TT_%s_PSTEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), step(u, kind, elem))  # calls without a causal mask
-                if head_dim == 128:
-                    emit("TT_%s_MSTEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), step(u, kind, elem, bmask=True))  # Bool attnMask
-    if head_dim == 128:
-        emit("TT_%s_MDMA" % NAME, mask_dma())
-        # before the first step of a workgroup (tile index a multiple of 4: ring place 0): the half it takes, half 1 of that tile
-        # (waited for at once: the first tile's own loads go to the same ring place)
-        emit("TT_%s_MREAD_FIRST" % NAME, mask_reads(0, 1, 1) + ["s_waitcnt lgkmcnt(0)"])
+                emit("TT_%s_MSTEP_%s_U%d_K%d" % (NAME, elem.upper(), u, kind), step(u, kind, elem, bmask=True))  # Bool attnMask
+    emit("TT_%s_MDMA" % NAME, mask_dma())
+    # before the first step of a workgroup (tile index a multiple of 4: ring place 0): the half it takes, half 1 of that tile
+    # (waited for at once: the first tile's own loads go to the same ring place)
+    emit("TT_%s_MREAD_FIRST" % NAME, mask_reads(0, 1, 1) + ["s_waitcnt lgkmcnt(0)"])
 
 
 if __name__ == "__main__":

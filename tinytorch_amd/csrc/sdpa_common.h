@@ -400,6 +400,13 @@ inline int dkv_round_of(const void* kernel, int threads, int lds_bytes, int (&ca
   return cache[dev] > 0 ? cache[dev] : 0;
 }
 
+// A Bool attnMask the pipelined prefill kernels' streams can apply: four keys per aligned dword, row offsets of a
+// (batch, head) within 32 bits, no causal flag, per-batch key counts, pages or key splits beside it.
+inline bool bool_mask_streams_ok(const KArgs& a) {
+  return !a.causal && a.mask_kind == 1 && a.mask_vec4 && (a.S % 4) == 0 && !a.kv_len && !a.block_table && a.kv_splits <= 1 &&
+         (long long)(a.L - 1) * a.ms[2] + 8 < (1ll << 32);
+}
+
 // Keys of batch entry b: all S of them, or the filled prefix of a cache / the unpadded length (kv_len).
 __device__ __forceinline__ int keys_of_batch(const KArgs& f, int b) {
   int S = f.S;

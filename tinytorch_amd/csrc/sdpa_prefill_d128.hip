@@ -850,17 +850,11 @@ int launch_v(const KArgs& a, dim3 grid, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
-// A Bool attnMask the streams can apply: four keys per aligned dword, row offsets of a (batch, head) within 32 bits.
-bool bool_mask_in_streams(const KArgs& a) {
-  return !a.causal && a.mask_kind == 1 && a.mask_vec4 && (a.S % 4) == 0 && !a.kv_len && !a.block_table && a.kv_splits <= 1 &&
-         (long long)(a.L - 1) * a.ms[2] + 8 < (1ll << 32);
-}
-
 template <typename TR, bool CAUSAL>
 int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
   if (a.kv_splits > 1) return launch_v<TR, CAUSAL, false, true>(a, grid, stream);  // (the host never splits a paged call)
   if constexpr (!CAUSAL)
-    if (bool_mask_in_streams(a)) return launch_v<TR, false, false, false, true>(a, grid, stream);
+    if (bool_mask_streams_ok(a)) return launch_v<TR, false, false, false, true>(a, grid, stream);
   return a.block_table ? launch_v<TR, CAUSAL, true, false>(a, grid, stream) : launch_v<TR, CAUSAL, false, false>(a, grid, stream);
 }
 

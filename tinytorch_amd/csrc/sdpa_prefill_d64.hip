@@ -12,7 +12,10 @@
 //   * a wavefront brings its 8 rows of a tile with one load instruction (1 KiB), so the waits count one load per tile
 //     and stream;
 //   * the 32 rows of a wavefront leave through LDS in one round (4 KiB of staging each).
-// Calls with an attnMask or a paged cache stay on the 4-wavefront kernel (sdpa_prefill.hip).
+// A Bool attnMask whose keys can be read four at a time is applied in the streams as in that file (variant MASKB: the
+// wavefront's mask bytes of a tile come into a ring in LDS two tiles ahead, a step reads the lane's dwords of the half
+// after next and keeps a probability iff its byte is set).  Calls with another attnMask or a paged cache stay on the
+// 4-wavefront kernel (sdpa_prefill.hip).
 
 #include "sdpa_common.h"
 #include "prefill64_steps.inc"  // hand-ordered instruction streams of the steady state (gen_prefill128_steps.py 64)
@@ -47,8 +50,11 @@ __device__ __forceinline__ int swz(int row) { return (((row >> 1) & 1) << 2) | (
 // SPLIT (launches with very few row tiles): a workgroup takes key tiles kt0 .. kt0 + kv_chunk/64 - 1 of its row tile (kt0 a
 // multiple of 4, so the stages keep their constants) and leaves (unnormalised accumulator, maximum, sum) records in a.ws
 // for prefill_split_merge_kernel; row tiles are single (no mirror pairs).
-template <typename TR, bool CAUSAL, bool SPLIT>
+// MASKB (calls without a causal mask or splits): a.mask is a Bool mask with unit key stride, dword-aligned rows and row
+// offsets below 2^32; the steady state applies it in the streams.
+template <typename TR, bool CAUSAL, bool SPLIT, bool MASKB = false>
 __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
+  static_assert(!MASKB || (!CAUSAL && !SPLIT), "the Bool-mask streams exist for the plain variant only");
   constexpr bool PAGED = false;  // paged caches stay on the 4-wavefront kernel
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
@@ -268,6 +274,49 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
     if (kt0 + 2 < ntiles_kv) dma_v(kt0 + 2, 2);
   };
   issue_tiles(0);
+  // ---- Bool attnMask in the streams (MASKB): the scheme of sdpa_prefill_d128.hip ------------------------------------------
+  // Ring in LDS: two tiles of 2 KiB per wavefront in the output staging area (idle during the loop).  Load i of a tile
+  // (two per tile) brings the 64-byte segments of rows 16i .. 16i+15 of the wavefront, 16 bytes per lane: chunk c of row q
+  // lands at 1024 (q/16) + 256 c + 16 (q%16).  A lane (row q, h = lane/32) needs dwords h and h + 2 of chunks 2H and 2H + 1
+  // of its row for half H of a tile; registers: half H of the workgroup's keys in places 4(H%2) .. +3.  Tile j sends for
+  // the mask bytes of tile j+2 ahead of its K/V loads (the wait at the tile's end covers them), and its two steps read
+  // halves 2j+2 and 2j+3 into registers for the steps after them.
+  u32x8 mring;
+  unsigned mrow_off[2];           // the lane's byte offset in a (batch, head)'s mask for the two loads of a tile
+  unsigned mlds = 0;              // LDS address of the lane's row in the wavefront's ring, plus 4 * (lane/32)
+  const char* mbase = nullptr;    // first mask byte of this (batch, head); uniform
+  unsigned mring_addr = 0;        // LDS address of the wavefront's ring
+  if constexpr (MASKB) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) mring[i] = 0u;
+    int q0, ntiles_kv;
+    part_rows(0, q0, ntiles_kv);
+    const int qw = q0 + rowgroup * WM;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      int row = qw + 16 * i + (lane & 15);
+      row = row < a.L ? row : a.L - 1;  // rows past the end re-read the last one
+      mrow_off[i] = (unsigned)row * (unsigned)a.ms[2] + 16u * (lane >> 4);  // the host checks that the last row's offset fits 32 bits
+    }
+    mbase = (const char*)a.mask + b * a.ms[0] + h * a.ms[1];
+    mring_addr = smem_addr + (KSTAGES + VSTAGES) * STAGE_BYTES + wave * 4096;
+    mlds = mring_addr + 1024 * (lq >> 4) + 16 * (lq & 15) + 4 * lh;
+  }
+  // a tile's mask bytes into ring place `place`; tiles beyond the row's last whole one are moved back into it (nobody takes them)
+  auto mask_dma = [&](int tile, int place) __attribute__((always_inline)) {
+    const int k0 = 64 * tile < S - 64 ? 64 * tile : S - 64;
+    asm volatile(TT_P64_MDMA
+                 :
+                 : [o0] "v"(mrow_off[0]), [o1] "v"(mrow_off[1]), [mtile] "s"(mbase + k0),
+                   [dst] "s"(mring_addr + 2048 * place)
+                 : "memory", "m0", "scc");
+  };
+  if constexpr (MASKB) {
+    if (S >= 160) {  // (shorter rows have no tile in the fast form)
+      mask_dma(kt0, 0);
+      mask_dma(kt0 + 1, 1);
+    }
+  }
   u32x16 qv;  // the lane's Q operands, k-step ks in elements 4ks .. 4ks+3
   // Q of a part into its registers, and everything sent for so far in place.  One statement: the compiler takes a statement's
   // results as valid when it ends, so the wait has to be part of it (and, not knowing of the tile loads, the compiler
@@ -332,7 +381,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
     t = f < t ? f : t;
     nfast_all = t > nfast ? t : nfast;
   }
-  if (a.mask_kind != 0) nfast = 0, nfast_all = 0;  // an attnMask is applied in the general form of a step
+  if (MASKB ? S < 160 : a.mask_kind != 0) nfast = 0, nfast_all = 0;  // other attnMasks are applied in the general form of a step
   // The fast form requests its tiles without the ragged-tile case: iteration j sends for K(j+4) and V(j+3), which have to
   // be whole tiles.
   if (!PAGED && (S % BN) != 0) {
@@ -426,8 +475,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   // then the true row maximum is formed, sum and accumulator are rescaled and the half is redone.  Every
   // probability that reaches the matrix pipe is therefore at most kSumLimit.
   const int rl = CAUSAL ? qc0 + lq - 4 * lh : 0;  // the causal predicate's lane operand: key k of a score is visible iff k - 4*(lane/32) <= rl
-  auto settle_half = [&](f32x16& s, vec8 (&pb)[2], float psum, int masked_kv0 = -1) __attribute__((always_inline)) {
+  auto settle_half = [&](f32x16& s, vec8 (&pb)[2], float psum, int masked_kv0 = -1, int mask_place = -1) __attribute__((always_inline)) {
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(psum <= kSumLimit)) != 0, 0)) {
+      // after a step that applied a Bool attnMask in the stream: scores whose mask byte is clear must not enter the maximum
+      if (MASKB && mask_place >= 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          if (((mring[4 * mask_place + (r >> 2)] >> (8 * (r & 3))) & 0xffu) == 0u) s[r] = -INFINITY;
+      }
       // after a step whose exponentials took the causal predicate in the stream, the scores themselves are masked only
       // here (hidden scores, or what a stage held beyond the workgroup's last tile, must not enter the maximum)
       if (CAUSAL && masked_kv0 >= 0) {
@@ -506,6 +561,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
                  "+{v[208:239]}"(ring)                                                                                 \
                : [c] "v"(c), [mc] "v"(mc), "{v[120:135]}"(qv), "{v[152:155]}"(v_addr), "{v[248:251]}"(k_addr)            \
                : "v240", "v241", "v242", "v243", "v244", "v245", "memory")
+// the plain step with a Bool attnMask applied to each probability (mask registers v[112:119], a zero in a scalar register)
+#define TT_P64_RUN_MSTEP(TXT)                                                                                         \
+  asm volatile(TXT                                                                                                     \
+               : [o0] "+v"(oacc[0]), [o1] "+v"(oacc[1]), [ps] "=&v"(psum_step),                                          \
+                 "+{v[160:175]}"(sB), "+{v[176:191]}"(sC), "+{v[192:199]}"(pAv), "+{v[200:207]}"(pBv),                   \
+                 "+{v[208:239]}"(ring), "+{v[112:119]}"(mring)                                                          \
+               : [c] "v"(c), [mc] "v"(mc), [zero] "s"(0), [mlds] "v"(mlds), [mlds1] "v"(mlds + 2048), "{v[120:135]}"(qv), "{v[152:155]}"(v_addr), "{v[248:251]}"(k_addr) \
+               : "v240", "v241", "v242", "v243", "v244", "v245", "vcc", "memory")
   constexpr bool kIsBf16 = sizeof(typename TR::elem) == 2 && __is_same(typename TR::elem, __bf16);
 
   f32x16 sB, sC;
@@ -588,12 +651,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   };
   int j = kt0;
   if (nfast_all >= kt0 + 1) {
-    auto settle_fast = [&](f32x16& s, u32x8& pv, int masked_kv0) __attribute__((always_inline)) {
+    auto settle_fast = [&](f32x16& s, u32x8& pv, int masked_kv0, int mask_place) __attribute__((always_inline)) {
       vec8 p[2];
       p_load(pv, p);
-      settle_half(s, p, psum_step, masked_kv0);
+      settle_half(s, p, psum_step, masked_kv0, mask_place);
       p_store(pv, p);
     };
+    if constexpr (MASKB)  // the mask bytes of the half the first step takes (the steps read those of the halves after it)
+      asm volatile(TT_P64_MREAD_FIRST : "+{v[112:119]}"(mring) : [mlds] "v"(mlds), [mlds1] "v"(mlds + 2048) : "memory");
     p_store(pAv, pA);
     p_store(pBv, pB);
     asm volatile(TT_P64_PREFETCH : "+{v[208:239]}"(ring) : "{v[152:155]}"(v_addr), "{v[248:251]}"(k_addr) : "memory");
@@ -601,6 +666,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
 #define TT_P64_TILE(U)                                                                                  \
     if (__builtin_expect(j >= nfast_all, 0)) break;                                                       \
     {                                                                                                    \
+      if constexpr (MASKB) mask_dma(j + 2, U & 1);                                                       \
       const int keep = PAGED ? tile_dma(j) : tile_dma_fast(j, U);                                        \
       /* mk = 1: the tile's exponentials take the causal predicate; kvs = first key of the half whose exponentials   \
          the step takes; kvm = kvs on such a tile, else -1.  As scalar instructions: the compiler's own form of     \
@@ -611,15 +677,19 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
             : "=&s"(mk), "=&s"(kvm0), "=&s"(kvm1) : "s"(j), "s"(nfast), "s"(kvs), "s"(kvs + 32) : "scc"); \
       if constexpr (kIsBf16 && CAUSAL) TT_P64_RUN_STEP(TT_P64_STEP_BF16_U##U##_K0);                    \
       else if constexpr (CAUSAL) TT_P64_RUN_STEP(TT_P64_STEP_F16_U##U##_K0);                           \
+      else if constexpr (MASKB && kIsBf16) TT_P64_RUN_MSTEP(TT_P64_MSTEP_BF16_U##U##_K0);              \
+      else if constexpr (MASKB) TT_P64_RUN_MSTEP(TT_P64_MSTEP_F16_U##U##_K0);                          \
       else if constexpr (kIsBf16) TT_P64_RUN_PSTEP(TT_P64_PSTEP_BF16_U##U##_K0);                       \
       else TT_P64_RUN_PSTEP(TT_P64_PSTEP_F16_U##U##_K0);                                               \
-      settle_fast(sB, pBv, kvm0);                                                                        \
+      settle_fast(sB, pBv, kvm0, MASKB ? 1 : -1);                                                                      \
       kvs += 32;                                                                                         \
       if constexpr (kIsBf16 && CAUSAL) TT_P64_RUN_STEP(TT_P64_STEP_BF16_U##U##_K1);                    \
       else if constexpr (CAUSAL) TT_P64_RUN_STEP(TT_P64_STEP_F16_U##U##_K1);                           \
+      else if constexpr (MASKB && kIsBf16) TT_P64_RUN_MSTEP(TT_P64_MSTEP_BF16_U##U##_K1);              \
+      else if constexpr (MASKB) TT_P64_RUN_MSTEP(TT_P64_MSTEP_F16_U##U##_K1);                          \
       else if constexpr (kIsBf16) TT_P64_RUN_PSTEP(TT_P64_PSTEP_BF16_U##U##_K1);                       \
       else TT_P64_RUN_PSTEP(TT_P64_PSTEP_F16_U##U##_K1);                                               \
-      settle_fast(sC, pAv, kvm1);                                                                        \
+      settle_fast(sC, pAv, kvm1, MASKB ? 0 : -1);                                                                      \
       dma_wait_and_sync(keep);                                                                           \
       j++;                                                                                               \
     }
@@ -713,18 +783,23 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill64_kernel(KArgs a) {
   }  // part
 }
 
-template <typename TR, bool CAUSAL, bool SPLIT>
+template <typename TR, bool CAUSAL, bool SPLIT, bool MASKB = false>
 int launch_v(const KArgs& a, dim3 grid, hipStream_t stream) {
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)prefill64_kernel<TR, CAUSAL, SPLIT>, LDS_BYTES, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill64_kernel<TR, CAUSAL, SPLIT, MASKB>, LDS_BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
-  hipLaunchKernelGGL((prefill64_kernel<TR, CAUSAL, SPLIT>), grid, dim3(NW * 64), LDS_BYTES, stream, a);
+  hipLaunchKernelGGL((prefill64_kernel<TR, CAUSAL, SPLIT, MASKB>), grid, dim3(NW * 64), LDS_BYTES, stream, a);
   return (int)hipGetLastError();
 }
 
 template <typename TR, bool CAUSAL>
 int launch_k(const KArgs& a, dim3 grid, hipStream_t stream) {
+  if constexpr (!CAUSAL)
+    if (a.mask_kind != 0) {  // the host sends only Bool masks the streams can apply (bool_mask_streams_ok)
+      if (!bool_mask_streams_ok(a)) return (int)hipErrorInvalidValue;
+      return launch_v<TR, false, false, true>(a, grid, stream);
+    }
   return a.kv_splits > 1 ? launch_v<TR, CAUSAL, true>(a, grid, stream) : launch_v<TR, CAUSAL, false>(a, grid, stream);
 }
 

@@ -133,12 +133,19 @@ bool split_shape(const ttsdpa_params* p, long long* units, long long* keys) {
   return *units <= 64 || (p->causal && *keys >= 4096);
 }
 
-// The pipelined kernel at head_dim 64: no attnMask, no pages.  Against the 4-wavefront kernel (128-row tiles, keys
+// A Bool attnMask the pipelined kernels apply inside their instruction streams (bool_mask_streams_ok on the kernels' side).
+bool bool_mask_streams_param_ok(const ttsdpa_params* p) {
+  return p->mask_kind == TTSDPA_MASK_BOOL && !p->causal && mask_vec4_ok(p) && p->S % 4 == 0 && !p->kv_len && !p->block_table &&
+         (long long)(p->L - 1) * p->mask_stride[2] + 8 < (1ll << 32);
+}
+
+// The pipelined kernel at head_dim 64: no pages, and of attnMasks only Bool masks its streams can apply.  Against the 4-wavefront kernel (128-row tiles, keys
 // divided among workgroups when the heads are not grouped) it measured level or up to 30 % faster from 512 query rows
 // on; shorter calls take it when they fill half of the chip's CUs, or when their keys are split (16 heads x 256 rows on
 // 32768 keys: 0.56 ms on the 4-wavefront kernel, which cannot split grouped heads).
 bool pipelined64_ok(const ttsdpa_params* p) {
-  if (p->D != 64 || p->L <= 128 || p->mask_kind != TTSDPA_MASK_NONE || p->block_table) return false;
+  if (p->D != 64 || p->L <= 128 || p->block_table) return false;
+  if (p->mask_kind != TTSDPA_MASK_NONE && !bool_mask_streams_param_ok(p)) return false;
   if (!(p->k_stride[2] < (1 << 24) && p->v_stride[2] < (1 << 24) && p->q_stride[2] < (1 << 22))) return false;
   const long long tiles = (p->L + 255) / 256;
   if ((long long)p->B * p->Hq * (p->causal ? (tiles + 1) / 2 : tiles) >= 128) return true;
