@@ -58,7 +58,9 @@ def test_struct_layout_matches_header():
 @pytest.mark.parametrize("args,route", [
     ((_capi.F32, 1, 4, 4, 128, 128, 64), _capi.ROUTE_PREFILL),       # config 1: fp32 MFMA kernel
     ((_capi.F32, 2, 8, 2, 300, 300, 128), _capi.ROUTE_PREFILL),
-    ((_capi.F32, 2, 8, 2, 300, 300, 96), _capi.ROUTE_GENERAL),       # fp32 MFMA kernel: head_dim 64 and 128 only
+    ((_capi.F32, 2, 8, 2, 300, 300, 96), _capi.ROUTE_PREFILL),       # fp32 MFMA kernel: multiples of 4 up to 128 (zero columns up to 64 / 128)
+    ((_capi.F32, 2, 8, 2, 300, 300, 90), _capi.ROUTE_GENERAL),
+    ((_capi.F32, 2, 8, 2, 300, 300, 132), _capi.ROUTE_GENERAL),
     ((_capi.F16, 4, 32, 32, 2048, 2048, 128), _capi.ROUTE_PREFILL),  # config 2
     ((_capi.BF16, 2, 32, 8, 4096, 4096, 128), _capi.ROUTE_PREFILL),  # config 3
     ((_capi.BF16, 64, 32, 8, 1, 8192, 128), _capi.ROUTE_DECODE),     # config 4
@@ -104,7 +106,8 @@ def test_routes_depend_on_flags():
     assert _capi.plan(params(*f32, causal=1))[1] == _capi.ROUTE_PREFILL
     assert _capi.plan(params(*f32, mask_kind=_capi.MASK_ADD, mask=FAKE))[1] == _capi.ROUTE_PREFILL
     assert _capi.plan(params(*f32, kv_len=FAKE))[1] == _capi.ROUTE_PREFILL
-    assert _capi.plan(params(_capi.F32, 2, 8, 2, 512, 512, 96, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
+    assert _capi.plan(params(_capi.F32, 2, 8, 2, 512, 512, 96, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_PREFILL
+    assert _capi.plan(params(_capi.F32, 2, 8, 2, 512, 512, 98, mask_kind=_capi.MASK_BOOL, mask=FAKE))[1] == _capi.ROUTE_GENERAL
     p = params(*f32)
     p.v_stride[2] = 130
     assert _capi.plan(p)[1] == _capi.ROUTE_GENERAL
@@ -194,7 +197,7 @@ def test_product_library_holds_no_bench_probes():
 
 def test_kernel_domains_and_workspace():
     L = _capi.lib()
-    fp32 = params(_capi.F32, 1, 4, 4, 128, 128, 96)  # the fp32 MFMA kernel covers head_dim 64 and 128
+    fp32 = params(_capi.F32, 1, 4, 4, 128, 128, 90)  # the fp32 MFMA kernel covers the multiples of 4 up to 128
     assert L.ttsdpa_prefill(ctypes.byref(fp32), None) == _capi.ERR_UNSUPPORTED
     assert L.ttsdpa_decode(ctypes.byref(fp32), None, 0, None) == _capi.ERR_UNSUPPORTED
     # config 4 has 512 (batch, kv head) pairs: enough workgroups without splitting the cache, hence no scratch

@@ -34,7 +34,8 @@ CASES = [
     (1, 2, 1, 130, 200, 256, "bf16", "prefill"),    # head_dim 256
     (1, 4, 2, 150, 400, 128, "f32", "prefill"),     # fp32 MFMA kernel
     (2, 2, 2, 77, 99, 64, "f32", "prefill"),
-    (1, 2, 2, 70, 131, 96, "f32", "general"),       # vector-ALU kernel
+    (1, 2, 2, 70, 131, 96, "f32", "prefill"),       # a head size between the fp32 templates
+    (1, 2, 2, 70, 131, 90, "f32", "general"),       # vector-ALU kernel
     (1, 2, 1, 40, 90, 80, "bf16", "prefill"),       # a head size between the templates: the head_dim-96 kernel
     (1, 2, 1, 40, 90, 84, "bf16", "general"),       # rows that are not whole 16-byte chunks
     (2, 8, 2, 4, 2048, 128, "bf16", "prefill"),     # 16 rows per KV head: 4 new tokens, packed heads on the MFMA kernel

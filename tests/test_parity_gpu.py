@@ -238,7 +238,7 @@ def test_general_against_oracle(case):
     assert rc == 0
     assert max_abs_err(out, exp) <= TOL[dtype]
     if dtype == "f32":
-        assert route_of(*dev, causal=causal) == ("prefill" if D in (64, 128) else "general")
+        assert route_of(*dev, causal=causal) == ("prefill" if D % 4 == 0 and D <= 128 else "general")
 
 
 def test_general_masks_large():
@@ -461,6 +461,33 @@ def test_head_sizes_between_the_mfma_kernels(D, dtype, causal):
     exp = oracle.sdpa_f32(*host, causal=causal)
     rc, out = call("forward", *dev, causal=causal)
     assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("D", [4, 20, 36, 60, 68, 96, 100, 124])
+@pytest.mark.parametrize("causal", [True, False])
+def test_fp32_head_sizes_between_the_mfma_kernels(D, causal):
+    # fp32 tensors: any multiple of 4 up to 128 runs on the fp32 matrix-core kernel for 64 or 128 (zero columns)
+    B, Hq, Hkv, L, S = 2, 4, 2, 150, 150 if causal else 233
+    say("padded head_dim, fp32", (D, causal))
+    host, dev = make_inputs(295 + D, B, Hq, Hkv, L, S, D, "f32", 0.7)
+    assert route_of(*dev, causal=causal) == "prefill"
+    exp = oracle.sdpa_f32(*host, causal=causal)
+    rc, out = call("forward", *dev, causal=causal)
+    assert rc == 0 and max_abs_err(out, exp) <= TOL["f32"]
+    if D == 100:  # views of wider rows: other columns hold NaN (inputs) or a sentinel (output)
+        wide = []
+        for t in dev:
+            w = torch.full(t.shape[:-1] + (128,), float("nan"), dtype=t.dtype, device="cuda")
+            w[..., :D] = t
+            wide.append(w[..., :D])
+        outw = torch.full((B, Hq, L, 128), 7.0, dtype=torch.float32, device="cuda")
+        rc, _ = call("forward", *wide, causal=causal, out=outw[..., :D])
+        assert rc == 0 and max_abs_err(outw[..., :D], exp) <= TOL["f32"] and bool((outw[..., D:] == 7.0).all())
+        m = (np.random.RandomState(D).rand(L, S) > 0.4).astype(np.uint8)
+        m[:, 0] = 1
+        if not causal and S % 4 == 0:
+            rc, out = call("forward", *dev, mask=torch.from_numpy(m).cuda().bool())
+            assert rc == 0 and max_abs_err(out, oracle.sdpa_f32(*host, mask=m)) <= TOL["f32"]
 
 
 @pytest.mark.parametrize("D", [40, 80, 200])

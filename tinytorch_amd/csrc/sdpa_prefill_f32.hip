@@ -37,7 +37,10 @@ struct F32Lds {
 };
 
 // MASKED: an attnMask is applied (a variant of its own: the mask addressing costs registers the other variants keep).
-template <int D, bool CAUSAL, bool MASKED>
+// PAD: the tensors' head_dim a.D is a multiple of 4 below D; the 16-byte chunks of a row beyond it are taken as zeros (Q
+// and K: nothing added to a score; V: output columns that are not stored).  The reference takes any head size
+// (src/Function/FuncNNLayer.h:231-236).
+template <int D, bool CAUSAL, bool MASKED, bool PAD>
 __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
   typedef F32Lds<D> Lds;
   constexpr int K_PITCH = Lds::K_PITCH, V_PITCH = Lds::V_PITCH;
@@ -92,7 +95,8 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
     const float* qr = qp + row * a.qs[2] + lh * (D / 2);
 #pragma unroll
     for (int i = 0; i < KSTEPS / 4; i++) {
-      f32x4 t = *(const f32x4*)(qr + 4 * i);
+      f32x4 t = {0.f, 0.f, 0.f, 0.f};
+      if (!PAD || lh * (D / 2) + 4 * i < a.D) t = *(const f32x4*)(qr + 4 * i);
 #pragma unroll
       for (int e = 0; e < 4; e++) qreg[4 * i + e] = t[e];
     }
@@ -118,7 +122,7 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
     const int qi = qw0 + lq;
     if (qi < a.L) {
       float* op = (float*)a.out + b * a.os[0] + h * a.os[1] + qi * a.os[2];
-      for (int d = 4 * lh; d < D; d += 8) *(f32x4*)(op + d) = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int d = 4 * lh; d < (PAD ? a.D : D); d += 8) *(f32x4*)(op + d) = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
     return;
   }
@@ -143,12 +147,16 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
 
   // ---- global -> register -> LDS staging: thread t moves 16-byte chunks t, t+256, ... of a tile ----------------------
   f32x4 kst[NLD], vst[NLD];
-  int lrow[NLD], lcol[NLD];
+  int lrow[NLD], lcol[NLD], gcol[NLD];
+  bool cval[NLD];  // PAD: the chunk lies inside the tensors' rows; the others are loaded from the row's first chunk instead
+                   // (the loads stay unconditional) and reach LDS as zeros
 #pragma unroll
   for (int i = 0; i < NLD; i++) {
     int cidx = tid + 256 * i;
     lrow[i] = cidx / (D / 4);
     lcol[i] = cidx % (D / 4);
+    cval[i] = !PAD || 4 * lcol[i] < a.D;
+    gcol[i] = cval[i] ? lcol[i] : 0;
   }
   auto load_tile = [&](int kv0) {
     const float* ktile = kp + kv_tile_offset(a, table, kv0, a.ks[2], a.ks[0]);
@@ -157,8 +165,8 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
     for (int i = 0; i < NLD; i++) {
       int row = lrow[i];
       row = kv0 + row < S ? row : S - 1 - kv0;  // rows past the end re-read the last valid row (masked later)
-      kst[i] = *(const f32x4*)(ktile + row * a.ks[2] + 4 * lcol[i]);
-      vst[i] = *(const f32x4*)(vtile + row * a.vs[2] + 4 * lcol[i]);
+      kst[i] = *(const f32x4*)(ktile + row * a.ks[2] + 4 * gcol[i]);
+      vst[i] = *(const f32x4*)(vtile + row * a.vs[2] + 4 * gcol[i]);
     }
   };
   auto store_tile = [&](int stage) {
@@ -167,8 +175,8 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
 #pragma unroll
-      for (int e = 0; e < 4; e++) Ks[lrow[i] * K_PITCH + 4 * lcol[i] + e] = kst[i][e];  // rows are not 16-byte aligned
-      *(f32x4*)(Vs + lrow[i] * V_PITCH + 4 * lcol[i]) = vst[i];
+      for (int e = 0; e < 4; e++) Ks[lrow[i] * K_PITCH + 4 * lcol[i] + e] = cval[i] ? kst[i][e] : 0.f;  // rows are not 16-byte aligned
+      *(f32x4*)(Vs + lrow[i] * V_PITCH + 4 * lcol[i]) = cval[i] ? vst[i] : (f32x4){0.f, 0.f, 0.f, 0.f};
     }
   };
 
@@ -290,19 +298,27 @@ __global__ __launch_bounds__(256, 2) void prefill_f32_kernel(KArgs a) {
         f32x4 x;
 #pragma unroll
         for (int i = 0; i < 4; i++) x[i] = oacc[db][4 * rg + i] * inv;
-        *(f32x4*)(op + 32 * db + 8 * rg + 4 * lh) = x;
+        if (!PAD || 32 * db + 8 * rg + 4 * lh < a.D) *(f32x4*)(op + 32 * db + 8 * rg + 4 * lh) = x;
       }
   }
 }
 
-template <int D, bool CAUSAL, bool MASKED>
+template <int D, bool CAUSAL, bool MASKED, bool PAD>
 int launch_f32_k(const KArgs& a, dim3 grid, hipStream_t stream) {
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)prefill_f32_kernel<D, CAUSAL, MASKED>, F32Lds<D>::BYTES, state, done);
+  const hipError_t granted = grant_dynamic_lds((const void*)prefill_f32_kernel<D, CAUSAL, MASKED, PAD>, F32Lds<D>::BYTES, state, done);
   if (granted != hipSuccess) return (int)granted;
-  hipLaunchKernelGGL((prefill_f32_kernel<D, CAUSAL, MASKED>), grid, dim3(256), F32Lds<D>::BYTES, stream, a);
+  hipLaunchKernelGGL((prefill_f32_kernel<D, CAUSAL, MASKED, PAD>), grid, dim3(256), F32Lds<D>::BYTES, stream, a);
   return (int)hipGetLastError();
+}
+
+template <int D, bool PAD>
+int launch_f32_d(const KArgs& a, dim3 grid, hipStream_t stream) {
+  // the callers keep to this (the records of a split are laid out for D, rows are read in 16-byte chunks)
+  if (PAD && (a.kv_splits > 1 || a.D % 4 != 0 || a.D >= D || a.D < 4)) return (int)hipErrorInvalidValue;
+  if (a.mask_kind != 0) return launch_f32_k<D, false, true, PAD>(a, grid, stream);  // exclusive with causal (validated by the caller, as the reference asserts)
+  return a.causal ? launch_f32_k<D, true, false, PAD>(a, grid, stream) : launch_f32_k<D, false, false, PAD>(a, grid, stream);
 }
 
 }  // namespace
@@ -310,11 +326,10 @@ int launch_f32_k(const KArgs& a, dim3 grid, hipStream_t stream) {
 int launch_prefill_f32(const KArgs& a, hipStream_t stream) {
   long long nwg = (long long)a.B * a.Hq * ((a.L + BM - 1) / BM) * (a.kv_splits > 1 ? a.kv_splits : 1);
   dim3 grid((unsigned)nwg);
-  if (a.mask_kind != 0)  // exclusive with causal (validated by the caller, as the reference asserts)
-    return a.D == 128 ? launch_f32_k<128, false, true>(a, grid, stream) : launch_f32_k<64, false, true>(a, grid, stream);
-  if (a.D == 128)
-    return a.causal ? launch_f32_k<128, true, false>(a, grid, stream) : launch_f32_k<128, false, false>(a, grid, stream);
-  return a.causal ? launch_f32_k<64, true, false>(a, grid, stream) : launch_f32_k<64, false, false>(a, grid, stream);
+  if (a.D == 128) return launch_f32_d<128, false>(a, grid, stream);
+  if (a.D == 64) return launch_f32_d<64, false>(a, grid, stream);
+  // any other multiple of 4 up to 128: the kernel of the next size up, the missing columns as zeros
+  return a.D < 64 ? launch_f32_d<64, true>(a, grid, stream) : launch_f32_d<128, true>(a, grid, stream);
 }
 
 }  // namespace ttsdpa

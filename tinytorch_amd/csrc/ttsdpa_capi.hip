@@ -111,7 +111,7 @@ bool simple_mask_ok(const ttsdpa_params* p) {
 // fp32 tensors the fp32 MFMA kernel can read and write with 16-byte accesses.
 bool f32_prefill_ok(const ttsdpa_params* p) {
   if (p->dtype != TTSDPA_F32 || (p->block_table && p->page_size < kPrefillMinPage) || !simple_mask_ok(p)) return false;
-  if (p->D != 128 && p->D != 64) return false;
+  if (p->D < 4 || p->D > 128 || p->D % 4 != 0) return false;  // 64 and 128; other multiples of 4 on the next one up with zero columns
   if (!(p->scale > 0.f) || !isfinite(p->scale) || p->S < 1 || p->L < 1) return false;
   if (!dense_last_ok(p->q_stride, 4) || !dense_last_ok(p->k_stride, 4) || !dense_last_ok(p->v_stride, 4) ||
       !dense_last_ok(p->o_stride, 4))
