@@ -102,6 +102,65 @@ def test_backward_mfma_against_oracle(case):
         check("mfma-%s" % (case,), host, dev, dtype, causal=causal, route="prefill")
 
 
+PADDED_CASES = [
+    # head sizes between the matrix-core kernels' (64, 128): the register-staged pair of the next one up, zero columns
+    (2, 4, 2, 150, 150, 80, "bf16", True),
+    (1, 4, 4, 200, 333, 40, "f16", False),
+    (2, 6, 2, 130, 70, 96, "bf16", True),
+    (1, 8, 2, 64, 500, 112, "f16", "br"),
+    (2, 2, 1, 96, 96, 8, "bf16", True),
+    (1, 2, 2, 1, 129, 120, "bf16", False),
+    (1, 4, 1, 300, 17, 24, "f16", "br"),
+    (2, 4, 2, 260, 260, 72, "bf16", "mask"),
+    (2, 4, 2, 160, 300, 104, "f16", "kvlen"),
+]
+
+
+@pytest.mark.parametrize("case", PADDED_CASES, ids=lambda c: "B%dH%dk%dL%dS%dD%d-%s-%s" % c)
+def test_backward_mfma_head_sizes_between_the_kernels(case):
+    B, Hq, Hkv, L, S, D, dtype, mode = case
+    print("backward, padded head_dim", case, flush=True)
+    host, dev = make_inputs(4700 + L + S + D, B, Hq, Hkv, L, S, D, dtype)
+    name = "padded-%s" % (case,)
+    if mode == "br":
+        m = np.arange(S)[None, :] <= np.arange(L)[:, None] + max(0, S - L)
+        check(name, host, dev, dtype, causal=True, align="bottom-right", oracle_mask=m, route="prefill")
+    elif mode == "mask":
+        m = np.random.default_rng(D).random((Hq, L, S)) < 0.7
+        m[..., 0] = True
+        check(name, host, dev, dtype, mask_h=m, mask_d=torch.from_numpy(m).cuda(), route="prefill")
+    elif mode == "kvlen":
+        lens = np.array([S, 77], np.int32)
+        kv = torch.from_numpy(lens).cuda()
+        m = (np.arange(S)[None, None, :] < lens[:, None, None]) & (np.arange(S)[None, None, :] <= np.arange(L)[None, :, None] + np.maximum(0, lens - L)[:, None, None])
+        check(name, host, dev, dtype, causal=True, kv_lens=kv, align="bottom-right", oracle_mask=m[:, None], route="prefill")
+    else:
+        check(name, host, dev, dtype, causal=mode, route="prefill")
+
+
+def test_backward_mfma_padded_head_size_touches_its_columns_only():
+    # q, k, v, out, dout are views of wider rows whose other columns hold NaN; the gradients are views whose other columns
+    # keep a sentinel
+    B, Hq, Hkv, L, S, D, W = 1, 4, 2, 140, 200, 80, 128
+    host, dev = make_inputs(4801, B, Hq, Hkv, L, S, D, "bf16")
+    go_h, go_b = oracle.round_to(oracle.randn(4801, 7, host[0].shape), "bf16")
+    go = to_device(go_h, go_b, "bf16")
+    out = sdpAttention(*dev, isCausal=True)
+
+    def widen(t, fill):
+        w = torch.full(t.shape[:-1] + (W,), fill, dtype=t.dtype, device="cuda")
+        w[..., :D] = t
+        return w
+
+    wide = [widen(t, float("nan"))[..., :D] for t in (*dev, out, go)]
+    gw = [torch.full(t.shape[:-1] + (W,), 7.0, dtype=t.dtype, device="cuda") for t in dev]
+    rc, grads = backward_call(wide[0], wide[1], wide[2], wide[3], wide[4], causal=True, grads=tuple(g[..., :D] for g in gw))
+    assert rc == 0
+    exp = oracle.sdpa_backward_f32(*host, go_h, causal=True)
+    for g, w, e in zip(grads, gw, exp):
+        assert grad_err(g, e) <= TOL["bf16"] and bool((w[..., D:] == 7.0).all())
+
+
 def test_backward_mfma_properties_at_size():
     """Config 3's shape (B2 32q/8kv 4096 x 4096 x 128 bf16, causal), where the oracle would take minutes: the gradients are
     linear in dout (doubling it doubles them exactly: every product has one factor from dout), the columns of dk sum to ~0

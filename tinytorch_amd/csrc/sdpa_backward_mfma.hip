@@ -70,7 +70,8 @@ __device__ __forceinline__ vec8 transposed_operand(const void* lane_base, int by
 // A lane's share of the dk / dv rows of key `key` (accumulator layout: registers 4rg .. 4rg+3 of block db are elements
 // 32db + 8rg + 4lh .. +3) goes to the gradient tensors, or — when the key block's query stream is split over several
 // workgroups — as fp32 to this split's partial sums, dense [split][dk | dv][B][Hkv][S][D].
-template <typename TR, int D>
+// PAD: the tensors' head_dim a.f.D is a multiple of 8 below D; only its columns are written (no splits then).
+template <typename TR, int D, bool PAD = false>
 __device__ __forceinline__ void store_key_grads(const BwdArgs& a, int split, int b, int hk, int key, int lh,
                                                 const f32x16 (&dkacc)[D / 32], const f32x16 (&dvacc)[D / 32], float scale) {
   typedef typename TR::elem T;
@@ -99,20 +100,21 @@ __device__ __forceinline__ void store_key_grads(const BwdArgs& a, int split, int
       f32x4 x, y;
 #pragma unroll
       for (int i = 0; i < 4; i++) x[i] = dkacc[db][4 * rg + i] * scale, y[i] = dvacc[db][4 * rg + i];
+      if (PAD && 32 * db + 8 * rg + 4 * lh >= a.f.D) continue;
       *(typename TR::vec4*)(dkp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
       *(typename TR::vec4*)(dvp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(y, typename TR::vec4);
     }
 }
 
 // dk and dv rows of a key no query row attends to (at or beyond the batch entry's key count): zeros.
-template <typename TR, int D>
+template <typename TR, int D, bool PAD = false>
 __device__ __forceinline__ void zero_key_rows(const BwdArgs& a, int split, int b, int hk, int key, int lh) {
   f32x16 zero[D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; i++)
 #pragma unroll
     for (int r = 0; r < 16; r++) zero[i][r] = 0.f;
-  store_key_grads<TR, D>(a, split, b, hk, key, lh, zero, zero, 0.f);
+  store_key_grads<TR, D, PAD>(a, split, b, hk, key, lh, zero, zero, 0.f);
 }
 
 template <typename vec8>
@@ -127,7 +129,11 @@ __device__ __forceinline__ vec8 regs_to_operand(const f32x16& acc, int t) {
 // BN: keys per streamed tile.  64 for head_dim 64; 32 for head_dim 128, which keeps a wavefront under 256 registers:
 // two wavefronts per SIMD (one's vector work overlaps the other's matrix work), accumulators in ordinary registers.
 // MASKED: an attnMask (exclusive with CAUSAL) whose keys can be read four at a time, as in the forward kernels.
-template <typename TR, int D, bool CAUSAL, bool MASKED>
+// PAD (both register-staged kernels): the tensors' head_dim f.D is a multiple of 8 below D.  The 16-byte chunks of a row
+// beyond it are taken as zeros (q, k: nothing added to a score; dout, v: nothing added to dP or delta; the gradients'
+// columns beyond f.D are not stored); everything else is the kernel for head_dim D.  No splits (their records are laid
+// out for D).
+template <typename TR, int D, bool CAUSAL, bool MASKED, bool PAD>
 __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
   constexpr int BN = DqTile<D>::BN;
   typedef typename TR::elem T;
@@ -175,6 +181,11 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
     float part = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
+      if (PAD && 16 * ks + 8 * lh >= f.D) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) qreg[ks][i] = (T)0.f, greg[ks][i] = (T)0.f;
+        continue;
+      }
       qreg[ks] = *(const vec8*)(qr + 16 * ks);
       greg[ks] = *(const vec8*)(gr + 16 * ks);
       const vec8 o = *(const vec8*)(orow + 16 * ks);
@@ -202,7 +213,7 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
       typename TR::vec4 zero;
 #pragma unroll
       for (int i = 0; i < 4; i++) zero[i] = (T)0.f;
-      for (int d = 4 * lh; d < D; d += 8) *(typename TR::vec4*)(dqp + d) = zero;
+      for (int d = 4 * lh; d < (PAD ? f.D : D); d += 8) *(typename TR::vec4*)(dqp + d) = zero;
     }
     return;
   }
@@ -218,20 +229,25 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
 
   // ---- global -> register -> LDS staging of one K/V tile (thread t moves 16-byte chunks t, t+256, ...) ----------------------
   u32x4 kst[NLD], vst[NLD];
-  int lrow[NLD], lcol[NLD];
+  int lrow[NLD], lcol[NLD], gcol[NLD];
+  bool cval[NLD];  // PAD: the chunk lies inside the tensors' rows; the others are loaded from the row's first chunk instead
+                   // (the loads stay unconditional) and reach LDS as zeros
 #pragma unroll
   for (int i = 0; i < NLD; i++) {
     const int cidx = tid + 256 * i;
     lrow[i] = cidx / (D / 8);
     lcol[i] = cidx % (D / 8);
+    cval[i] = !PAD || 8 * lcol[i] < f.D;
+    gcol[i] = cval[i] ? lcol[i] : 0;
   }
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
   auto load_tile = [&](int kv0) {
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
       int key = kv0 + lrow[i];
       key = key < S ? key : S - 1;  // rows past the end re-read the last valid row (hidden below)
-      kst[i] = *(const u32x4*)(kp + key * f.ks[2] + 8 * lcol[i]);
-      vst[i] = *(const u32x4*)(vp + key * f.vs[2] + 8 * lcol[i]);
+      kst[i] = *(const u32x4*)(kp + key * f.ks[2] + 8 * gcol[i]);
+      vst[i] = *(const u32x4*)(vp + key * f.vs[2] + 8 * gcol[i]);
     }
   };
   auto store_tile = [&](int stage) {
@@ -240,9 +256,9 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
     T* Kt = Vr + BN * RP;
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
-      *(u32x4*)(Kr + lrow[i] * RP + 8 * lcol[i]) = kst[i];
-      *(u32x4*)(Kt + lrow[i] * TP + 8 * lcol[i]) = kst[i];
-      *(u32x4*)(Vr + lrow[i] * RP + 8 * lcol[i]) = vst[i];
+      *(u32x4*)(Kr + lrow[i] * RP + 8 * lcol[i]) = cval[i] ? kst[i] : zero4;
+      *(u32x4*)(Kt + lrow[i] * TP + 8 * lcol[i]) = cval[i] ? kst[i] : zero4;
+      *(u32x4*)(Vr + lrow[i] * RP + 8 * lcol[i]) = cval[i] ? vst[i] : zero4;
     }
   };
   const int r_lane = lq * RP + 8 * lh;
@@ -367,13 +383,14 @@ __global__ __launch_bounds__(256, 2) void backward_dq_mfma_kernel(BwdArgs a) {
         f32x4 x;
 #pragma unroll
         for (int i = 0; i < 4; i++) x[i] = seen ? dqacc[db][4 * rg + i] * w : 0.f;
+        if (PAD && 32 * db + 8 * rg + 4 * lh >= f.D) continue;
         *(typename TR::vec4*)(dqp + 32 * db + 8 * rg + 4 * lh) = __builtin_convertvector(x, typename TR::vec4);
       }
   }
 }
 
 // ---- kernel 2: dk, dv ---------------------------------------------------------------------------------------------------
-template <typename TR, int D, bool CAUSAL, bool MASKED>
+template <typename TR, int D, bool CAUSAL, bool MASKED, bool PAD>
 __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kernel(BwdArgs a) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
@@ -402,7 +419,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
   const int k0 = kb * BM, kw0 = k0 + wave * 32;
   const int S = keys_of_batch(f, b);  // rows of dk / dv from here to f.S are written as zeros
   if (k0 >= S) {
-    zero_key_rows<TR, D>(a, split, b, hk, kw0 + lq, lh);
+    zero_key_rows<TR, D, PAD>(a, split, b, hk, kw0 + lq, lh);
     return;
   }
   const bool wave_live = kw0 < S;
@@ -417,6 +434,11 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
     const T* vr = (const T*)f.v + b * f.vs[0] + hk * f.vs[1] + row * f.vs[2] + 8 * lh;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
+      if (PAD && 16 * ks + 8 * lh >= f.D) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) kreg[ks][i] = (T)0.f, vreg[ks][i] = (T)0.f;
+        continue;
+      }
       kreg[ks] = *(const vec8*)(kr + 16 * ks);
       vreg[ks] = *(const vec8*)(vr + 16 * ks);
     }
@@ -442,13 +464,17 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
 
   u32x4 qst[NLD], gst[NLD];
   float2 sst = make_float2(0.f, 0.f);
-  int lrow[NLD], lcol[NLD];
+  int lrow[NLD], lcol[NLD], gcol[NLD];
+  bool cval[NLD];  // PAD: as in the dq kernel
 #pragma unroll
   for (int i = 0; i < NLD; i++) {
     const int cidx = tid + 256 * i;
     lrow[i] = cidx / (D / 8);
     lcol[i] = cidx % (D / 8);
+    cval[i] = !PAD || 8 * lcol[i] < f.D;
+    gcol[i] = cval[i] ? lcol[i] : 0;
   }
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
   auto load_tile = [&](int idx) {
     const int h = hk * f.G + idx % f.G;
     const int i0 = tile_of(idx) * BQ;
@@ -458,8 +484,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
     for (int i = 0; i < NLD; i++) {
       int row = i0 + lrow[i];
       row = row < f.L ? row : f.L - 1;  // rows past the end re-read the last valid row (their weight is forced to 0)
-      qst[i] = *(const u32x4*)(qp + row * f.qs[2] + 8 * lcol[i]);
-      gst[i] = *(const u32x4*)(gp + row * a.dos[2] + 8 * lcol[i]);
+      qst[i] = *(const u32x4*)(qp + row * f.qs[2] + 8 * gcol[i]);
+      gst[i] = *(const u32x4*)(gp + row * a.dos[2] + 8 * gcol[i]);
     }
     if (tid < BQ) {
       const int row = i0 + tid;
@@ -473,10 +499,10 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
     T* Gt = Qt + BQ * TP;
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
-      *(u32x4*)(Qr + lrow[i] * RP + 8 * lcol[i]) = qst[i];
-      *(u32x4*)(Qt + lrow[i] * TP + 8 * lcol[i]) = qst[i];
-      *(u32x4*)(Gr + lrow[i] * RP + 8 * lcol[i]) = gst[i];
-      *(u32x4*)(Gt + lrow[i] * TP + 8 * lcol[i]) = gst[i];
+      *(u32x4*)(Qr + lrow[i] * RP + 8 * lcol[i]) = cval[i] ? qst[i] : zero4;
+      *(u32x4*)(Qt + lrow[i] * TP + 8 * lcol[i]) = cval[i] ? qst[i] : zero4;
+      *(u32x4*)(Gr + lrow[i] * RP + 8 * lcol[i]) = cval[i] ? gst[i] : zero4;
+      *(u32x4*)(Gt + lrow[i] * TP + 8 * lcol[i]) = cval[i] ? gst[i] : zero4;
     }
     if (tid < BQ) *(float2*)(sstats + stage * Lds::KV_STATS + 2 * tid) = sst;
   };
@@ -570,7 +596,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dkv_mfma_kerne
     __syncthreads();
   }
 
-  store_key_grads<TR, D>(a, split, b, hk, kw0 + lq, lh, dkacc, dvacc, f.scale);
+  store_key_grads<TR, D, PAD>(a, split, b, hk, kw0 + lq, lh, dkacc, dvacc, f.scale);
 }
 
 // ---- kernel 2 for head_dim 128: the same products with the tiles brought in by direct global->LDS loads ----------------
@@ -1066,22 +1092,24 @@ __global__ __launch_bounds__(256, 2) void backward_dq128_kernel(BwdArgs a) {
   }
 }
 
-template <typename TR, int D, bool CAUSAL, bool MASKED>
+template <typename TR, int D, bool CAUSAL, bool MASKED, bool PAD>
 int launch_k(const BwdArgs& args, hipStream_t stream) {
   BwdArgs a = args;
+  // the callers keep to this (the records of a split are laid out for D, rows are read in 16-byte chunks)
+  if (PAD && (a.dkv_splits > 1 || a.dq_splits > 1 || a.f.D % 8 != 0 || a.f.D >= D || a.f.D < 8)) return (int)hipErrorInvalidValue;
   typedef BwdLds<D> Lds;
   // with an attnMask, head_dim 128 takes the register-staged dk/dv kernel: the mask's 16 values per tile do not fit the
   // 256 registers of the direct-to-LDS one
-  constexpr bool DMA = D == 128 && !MASKED;
+  constexpr bool DMA = D == 128 && !MASKED && !PAD;
   static hipError_t state1[kMaxDevices], state2[kMaxDevices];
   static bool done1[kMaxDevices], done2[kMaxDevices];
   hipError_t e = DMA ? grant_dynamic_lds((const void*)backward_dq128_kernel<TR, CAUSAL>, dq128::LDS_BYTES, state1, done1)
-                     : grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED>, DqTile<D>::BYTES, state1, done1);
+                     : grant_dynamic_lds((const void*)backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED, PAD>, DqTile<D>::BYTES, state1, done1);
   if (e != hipSuccess) return (int)e;
   if (DMA) {
     e = grant_dynamic_lds((const void*)backward_dkv128_kernel<TR, CAUSAL>, dkv128::LDS_BYTES, state2, done2);
   } else {
-    e = grant_dynamic_lds((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED>, Lds::KV_BYTES, state2, done2);
+    e = grant_dynamic_lds((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED, PAD>, Lds::KV_BYTES, state2, done2);
   }
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM) * a.dq_splits;
@@ -1089,11 +1117,11 @@ int launch_k(const BwdArgs& args, hipStream_t stream) {
   static int round_cache[kMaxDevices];
   a.dkv_round = !CAUSAL ? 0
                 : DMA   ? dkv_round_of((const void*)backward_dkv128_kernel<TR, CAUSAL>, 512, dkv128::LDS_BYTES, round_cache)
-                        : dkv_round_of((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED>, 256, Lds::KV_BYTES, round_cache);
+                        : dkv_round_of((const void*)backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED, PAD>, 256, Lds::KV_BYTES, round_cache);
   if (DMA) {
     hipLaunchKernelGGL((backward_dq128_kernel<TR, CAUSAL>), dim3((unsigned)g1), dim3(256), dq128::LDS_BYTES, stream, a);
   } else {
-    hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED>), dim3((unsigned)g1), dim3(256), DqTile<D>::BYTES, stream, a);
+    hipLaunchKernelGGL((backward_dq_mfma_kernel<TR, D, CAUSAL, MASKED, PAD>), dim3((unsigned)g1), dim3(256), DqTile<D>::BYTES, stream, a);
   }
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
@@ -1104,22 +1132,25 @@ int launch_k(const BwdArgs& args, hipStream_t stream) {
   if (DMA) {
     hipLaunchKernelGGL((backward_dkv128_kernel<TR, CAUSAL>), dim3((unsigned)g2), dim3(512), dkv128::LDS_BYTES, stream, a);
   } else {
-    hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
+    hipLaunchKernelGGL((backward_dkv_mfma_kernel<TR, D, CAUSAL, MASKED, PAD>), dim3((unsigned)g2), dim3(256), Lds::KV_BYTES, stream, a);
   }
   e = hipGetLastError();
   if (e != hipSuccess || a.dkv_splits == 1) return (int)e;
   return launch_backward_dkv_sum<typename TR::elem>(a, stream);
 }
 
-template <typename TR, int D>
+template <typename TR, int D, bool PAD>
 int launch_d(const BwdArgs& a, hipStream_t stream) {
-  if (a.f.mask_kind != 0) return launch_k<TR, D, false, true>(a, stream);  // exclusive with causal (validated)
-  return a.f.causal ? launch_k<TR, D, true, false>(a, stream) : launch_k<TR, D, false, false>(a, stream);
+  if (a.f.mask_kind != 0) return launch_k<TR, D, false, true, PAD>(a, stream);  // exclusive with causal (validated)
+  return a.f.causal ? launch_k<TR, D, true, false, PAD>(a, stream) : launch_k<TR, D, false, false, PAD>(a, stream);
 }
 
 template <typename TR>
 int launch_t(const BwdArgs& a, hipStream_t stream) {
-  return a.f.D == 64 ? launch_d<TR, 64>(a, stream) : launch_d<TR, 128>(a, stream);
+  if (a.f.D == 64) return launch_d<TR, 64, false>(a, stream);
+  if (a.f.D == 128) return launch_d<TR, 128, false>(a, stream);
+  // any other multiple of 8 up to 128: the register-staged kernels of the next size up, the missing columns as zeros
+  return a.f.D < 64 ? launch_d<TR, 64, true>(a, stream) : launch_d<TR, 128, true>(a, stream);
 }
 
 }  // namespace

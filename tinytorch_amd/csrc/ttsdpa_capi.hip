@@ -286,7 +286,8 @@ int validate_backward(const ttsdpa_backward_params* p, BwdArgs* a) {
 // 128, attnMasks the forward's 4-wavefront kernel takes (keys readable four at a time, no kv_len beside them).
 bool backward_mfma_ok(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
-  if (!fast_layout_ok(f, true) || !simple_mask_ok(f) || (f->D != 64 && f->D != 128) || f->L < 1 || f->S < 1) return false;
+  // head_dim 64 and 128; other multiples of 8 up to 128 on the register-staged kernels of the next one up (zero columns)
+  if (!fast_layout_ok(f, true) || !simple_mask_ok(f) || f->D < 8 || f->D > 128 || f->D % 8 != 0 || f->L < 1 || f->S < 1) return false;
   if (!dense_last_ok(p->dout_stride, 8) || !dense_last_ok(p->dq_stride, 8) || !dense_last_ok(p->dk_stride, 8) ||
       !dense_last_ok(p->dv_stride, 8))
     return false;
@@ -325,6 +326,7 @@ size_t backward_stats_bytes(const ttsdpa_backward_params* p) {
 int dkv_splits_of(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
   if (pick_backward_route(p) != TTSDPA_ROUTE_PREFILL) return 1;
+  if (f->D != 64 && f->D != 128) return 1;  // the zero-column variants do not split (their records are laid out for 64 / 128)
   const int groups = f->dtype != TTSDPA_F32 && f->D == 128 && f->mask_kind == TTSDPA_MASK_NONE ? 2 : 1;
   const int per_cu = f->D == 64 && f->mask_kind == TTSDPA_MASK_NONE ? 2 : 1;
   return backward_dkv_splits(f->B, f->Hkv, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE, groups, per_cu);
@@ -333,6 +335,7 @@ int dkv_splits_of(const ttsdpa_backward_params* p) {
 int dq_splits_of(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
   if (pick_backward_route(p) != TTSDPA_ROUTE_PREFILL) return 1;
+  if (f->D != 64 && f->D != 128) return 1;
   const int slots = f->dtype == TTSDPA_F32 && f->D == 128 ? 256 : 512;
   return backward_dq_splits(f->B, f->Hq, f->L, f->S, effective_causal(f) != TTSDPA_CAUSAL_NONE, slots);
 }
