@@ -113,6 +113,12 @@ PADDED_CASES = [
     (1, 4, 1, 300, 17, 24, "f16", "br"),
     (2, 4, 2, 260, 260, 72, "bf16", "mask"),
     (2, 4, 2, 160, 300, 104, "f16", "kvlen"),
+    # fp32: multiples of 4 up to 128 on the fp32 matrix-core pair
+    (2, 4, 2, 150, 150, 40, "f32", True),
+    (1, 4, 4, 100, 233, 100, "f32", False),
+    (1, 2, 1, 70, 300, 20, "f32", "br"),
+    (2, 4, 2, 130, 260, 96, "f32", "mask"),
+    (2, 2, 2, 90, 200, 4, "f32", "kvlen"),
 ]
 
 

@@ -336,9 +336,16 @@ def test_backward_params_layout_routes_and_validation():
     bp.dq_stride[2] = 64
     bp.fwd.k = FAKE + 4
     assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_GENERAL
-    L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.F32, 1, 4, 4, 32, 32, 96)
-    bp.fwd.q = bp.fwd.k = bp.fwd.v = bp.fwd.out = bp.dout = bp.dq = bp.dk = bp.dv = FAKE
-    assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_GENERAL
+    # other head sizes: multiples of 4 up to 128 on the same pair (zero columns up to 64 / 128), the rest on the vector ALUs
+    for D, route in ((96, _capi.ROUTE_PREFILL), (20, _capi.ROUTE_PREFILL), (90, _capi.ROUTE_GENERAL), (160, _capi.ROUTE_GENERAL)):
+        L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.F32, 1, 4, 4, 32, 32, D)
+        bp.fwd.q = bp.fwd.k = bp.fwd.v = bp.fwd.out = bp.dout = bp.dq = bp.dk = bp.dv = FAKE
+        assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == route, D
+    # 16-bit tensors: multiples of 8 up to 128
+    for D, route in ((80, _capi.ROUTE_PREFILL), (8, _capi.ROUTE_PREFILL), (84, _capi.ROUTE_GENERAL), (136, _capi.ROUTE_GENERAL)):
+        L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.BF16, 1, 4, 4, 32, 32, D)
+        bp.fwd.q = bp.fwd.k = bp.fwd.v = bp.fwd.out = bp.dout = bp.dq = bp.dk = bp.dv = FAKE
+        assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == route, D
     L.ttsdpa_backward_params_init(ctypes.byref(bp), _capi.F32, 0, 4, 4, 32, 32, 64)
     assert L.ttsdpa_backward_plan(ctypes.byref(bp), ctypes.byref(r)) == 0 and r.value == _capi.ROUTE_NONE
 

@@ -66,13 +66,15 @@ __device__ __forceinline__ f32x16 score_product(const float* xrow, const float (
   return s0;
 }
 
-// This lane's half (lh) of a row of D floats, 16 bytes at a time.
+// This lane's half (lh) of a row of D floats, 16 bytes at a time; the row holds `have` floats (a multiple of 4, at most
+// D), the rest reads as zeros.
 template <int D>
-__device__ __forceinline__ void load_half_row(const float* row, int lh, float (&reg)[D / 2]) {
+__device__ __forceinline__ void load_half_row(const float* row, int lh, float (&reg)[D / 2], int have) {
   const float* p = row + lh * (D / 2);
 #pragma unroll
   for (int i = 0; i < D / 8; i++) {
-    const f32x4 t = *(const f32x4*)(p + 4 * i);
+    f32x4 t = {0.f, 0.f, 0.f, 0.f};
+    if (lh * (D / 2) + 4 * i < have) t = *(const f32x4*)(p + 4 * i);
 #pragma unroll
     for (int e = 0; e < 4; e++) reg[4 * i + e] = t[e];
   }
@@ -80,11 +82,15 @@ __device__ __forceinline__ void load_half_row(const float* row, int lh, float (&
 
 // ---- kernel 1: dq, lse, delta -------------------------------------------------------------------------------------
 // MASKED: an attnMask (exclusive with CAUSAL) whose keys can be read four at a time, as in the forward kernel.
-template <int D, bool CAUSAL, bool MASKED>
+// PAD (both kernels): the tensors' head_dim f.D is a multiple of 4 below D.  The 16-byte chunks of a row beyond it are
+// taken as zeros (q, k: nothing added to a score; dout, v: nothing added to dP or delta; gradient columns beyond f.D are
+// not stored); everything else is the kernel for head_dim D.  No splits (their records are laid out for D).
+template <int D, bool CAUSAL, bool MASKED, bool PAD>
 __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(BwdArgs a) {
   typedef BwdF32Lds<D> Lds;
   constexpr int PITCH = Lds::PITCH, NLD = Lds::NLD, DBLK = D / 32;
   const KArgs& f = a.f;
+  const int have = PAD ? f.D : D;  // floats of a row
 
   extern __shared__ __attribute__((aligned(16))) float smem_bwd_f32[];
   float* smem = smem_bwd_f32;
@@ -116,12 +122,13 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
   {
     int row = qw0 + lq;
     row = row < f.L ? row : f.L - 1;
-    load_half_row<D>((const float*)f.q + b * f.qs[0] + h * f.qs[1] + row * f.qs[2], lh, qreg);
-    load_half_row<D>((const float*)a.dout + b * a.dos[0] + h * a.dos[1] + row * a.dos[2], lh, greg);
+    load_half_row<D>((const float*)f.q + b * f.qs[0] + h * f.qs[1] + row * f.qs[2], lh, qreg, have);
+    load_half_row<D>((const float*)a.dout + b * a.dos[0] + h * a.dos[1] + row * a.dos[2], lh, greg, have);
     const float* orow = (const float*)f.out + b * f.os[0] + h * f.os[1] + row * f.os[2] + lh * (D / 2);
     float part = 0.f;
 #pragma unroll
     for (int i = 0; i < D / 8; i++) {
+      if (PAD && lh * (D / 2) + 4 * i >= have) continue;
       const f32x4 o = *(const f32x4*)(orow + 4 * i);
 #pragma unroll
       for (int e = 0; e < 4; e++) part = fmaf(o[e], greg[4 * i + e], part);
@@ -142,7 +149,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
     const int qi = qw0 + lq;
     if (qi < f.L) {
       float* dqp = (float*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qi * a.dqs[2];
-      for (int d = 4 * lh; d < D; d += 8) *(f32x4*)(dqp + d) = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int d = 4 * lh; d < have; d += 8) *(f32x4*)(dqp + d) = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
     return;
   }
@@ -158,20 +165,24 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
 
   // ---- global -> register -> LDS staging of one K/V tile (thread t moves 16-byte chunks t, t+256, ...) ----------------------
   f32x4 kst[NLD], vst[NLD];
-  int lrow[NLD], lcol[NLD];
+  int lrow[NLD], lcol[NLD], gcol[NLD];
+  bool cval[NLD];  // PAD: the chunk lies inside the tensors' rows; the others are loaded from the row's first chunk instead
+                   // (the loads stay unconditional) and reach LDS as zeros
 #pragma unroll
   for (int i = 0; i < NLD; i++) {
     const int cidx = tid + 256 * i;
     lrow[i] = cidx / (D / 4);
     lcol[i] = cidx % (D / 4);
+    cval[i] = !PAD || 4 * lcol[i] < have;
+    gcol[i] = cval[i] ? lcol[i] : 0;
   }
   auto load_tile = [&](int kv0) {
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
       int key = kv0 + lrow[i];
       key = key < S ? key : S - 1;  // rows past the end re-read the last valid row (hidden below)
-      kst[i] = *(const f32x4*)(kp + key * f.ks[2] + 4 * lcol[i]);
-      vst[i] = *(const f32x4*)(vp + key * f.vs[2] + 4 * lcol[i]);
+      kst[i] = *(const f32x4*)(kp + key * f.ks[2] + 4 * gcol[i]);
+      vst[i] = *(const f32x4*)(vp + key * f.vs[2] + 4 * gcol[i]);
     }
   };
   auto store_tile = [&](int stage) {
@@ -181,8 +192,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
     for (int i = 0; i < NLD; i++)
 #pragma unroll
       for (int e = 0; e < 4; e++) {  // rows are not 16-byte aligned
-        Ks[lrow[i] * PITCH + 4 * lcol[i] + e] = kst[i][e];
-        Vs[lrow[i] * PITCH + 4 * lcol[i] + e] = vst[i][e];
+        Ks[lrow[i] * PITCH + 4 * lcol[i] + e] = cval[i] ? kst[i][e] : 0.f;
+        Vs[lrow[i] * PITCH + 4 * lcol[i] + e] = cval[i] ? vst[i][e] : 0.f;
       }
   };
   const int s_lane = lq * PITCH + lh * (D / 2);  // score products: row l%32, this lane's half of head_dim
@@ -278,6 +289,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
         f32x4 x;
 #pragma unroll
         for (int i = 0; i < 4; i++) x[i] = seen ? dqacc[db][4 * rg + i] * w : 0.f;
+        if (PAD && 32 * db + 8 * rg + 4 * lh >= have) continue;
         *(f32x4*)(dqp + 32 * db + 8 * rg + 4 * lh) = x;
       }
   }
@@ -286,11 +298,12 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void backward_dq_f32_kernel(
 // ---- kernel 2: dk, dv -----------------------------------------------------------------------------------------------
 // MASKED reads one mask value per score (a key is a lane column here, the mask's rows run across registers); with its
 // addressing the head_dim-64 variant no longer fits two wavefronts per SIMD either.
-template <int D, bool CAUSAL, bool MASKED>
+template <int D, bool CAUSAL, bool MASKED, bool PAD>
 __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_f32_kernel(BwdArgs a) {
   typedef BwdF32Lds<D> Lds;
   constexpr int PITCH = Lds::PITCH, NLD = Lds::NLD, DBLK = D / 32;
   const KArgs& f = a.f;
+  const int have = PAD ? f.D : D;  // floats of a row
 
   extern __shared__ __attribute__((aligned(16))) float smem_bwd_f32[];
   float* smem = smem_bwd_f32;
@@ -319,7 +332,7 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
   }
   if (k0 >= S) {  // keys no query row attends to (at or beyond the batch entry's key count): zeros
     if (key < f.S)
-      for (int d = 4 * lh; d < D; d += 8) {
+      for (int d = 4 * lh; d < have; d += 8) {
         *(f32x4*)(dkp + d) = (f32x4){0.f, 0.f, 0.f, 0.f};
         *(f32x4*)(dvp + d) = (f32x4){0.f, 0.f, 0.f, 0.f};
       }
@@ -332,8 +345,8 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
   float kreg[D / 2], vreg[D / 2];
   {
     const int row = key < S ? key : S - 1;
-    load_half_row<D>((const float*)f.k + b * f.ks[0] + hk * f.ks[1] + row * f.ks[2], lh, kreg);
-    load_half_row<D>((const float*)f.v + b * f.vs[0] + hk * f.vs[1] + row * f.vs[2], lh, vreg);
+    load_half_row<D>((const float*)f.k + b * f.ks[0] + hk * f.ks[1] + row * f.ks[2], lh, kreg, have);
+    load_half_row<D>((const float*)f.v + b * f.vs[0] + hk * f.vs[1] + row * f.vs[2], lh, vreg, have);
   }
   f32x16 dkacc[DBLK], dvacc[DBLK];
 #pragma unroll
@@ -353,12 +366,15 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
 
   f32x4 qst[NLD], gst[NLD];
   float2 sst = make_float2(0.f, 0.f);
-  int lrow[NLD], lcol[NLD];
+  int lrow[NLD], lcol[NLD], gcol[NLD];
+  bool cval[NLD];  // PAD: as in the dq kernel
 #pragma unroll
   for (int i = 0; i < NLD; i++) {
     const int cidx = tid + 256 * i;
     lrow[i] = cidx / (D / 4);
     lcol[i] = cidx % (D / 4);
+    cval[i] = !PAD || 4 * lcol[i] < have;
+    gcol[i] = cval[i] ? lcol[i] : 0;
   }
   auto load_tile = [&](int idx) {
     const int h = hk * f.G + idx % f.G;
@@ -369,8 +385,8 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
     for (int i = 0; i < NLD; i++) {
       int row = i0 + lrow[i];
       row = row < f.L ? row : f.L - 1;  // rows past the end re-read the last valid row (their weight is forced to 0)
-      qst[i] = *(const f32x4*)(qp + row * f.qs[2] + 4 * lcol[i]);
-      gst[i] = *(const f32x4*)(gp + row * a.dos[2] + 4 * lcol[i]);
+      qst[i] = *(const f32x4*)(qp + row * f.qs[2] + 4 * gcol[i]);
+      gst[i] = *(const f32x4*)(gp + row * a.dos[2] + 4 * gcol[i]);
     }
     if (tid < BT) {
       const int row = i0 + tid;
@@ -384,8 +400,8 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
     for (int i = 0; i < NLD; i++)
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        Qs[lrow[i] * PITCH + 4 * lcol[i] + e] = qst[i][e];
-        Gs[lrow[i] * PITCH + 4 * lcol[i] + e] = gst[i][e];
+        Qs[lrow[i] * PITCH + 4 * lcol[i] + e] = cval[i] ? qst[i][e] : 0.f;
+        Gs[lrow[i] * PITCH + 4 * lcol[i] + e] = cval[i] ? gst[i][e] : 0.f;
       }
     if (tid < BT) *(float2*)(Gs + Lds::TILE + 2 * tid) = sst;
   };
@@ -473,45 +489,54 @@ __global__ __launch_bounds__(256, (D > 64 || MASKED ? 1 : 2)) void backward_dkv_
         f32x4 x, y;
 #pragma unroll
         for (int i = 0; i < 4; i++) x[i] = dkacc[db][4 * rg + i] * f.scale, y[i] = dvacc[db][4 * rg + i];
+        if (PAD && 32 * db + 8 * rg + 4 * lh >= have) continue;
         *(f32x4*)(dkp + 32 * db + 8 * rg + 4 * lh) = x;
         *(f32x4*)(dvp + 32 * db + 8 * rg + 4 * lh) = y;
       }
   }
 }
 
-template <int D, bool CAUSAL, bool MASKED>
+template <int D, bool CAUSAL, bool MASKED, bool PAD>
 int launch_k(const BwdArgs& args, hipStream_t stream) {
   BwdArgs a = args;
+  // the callers keep to this (the records of a split are laid out for D, rows are read in 16-byte chunks)
+  if (PAD && (a.dkv_splits > 1 || a.dq_splits > 1 || a.f.D % 4 != 0 || a.f.D >= D || a.f.D < 4)) return (int)hipErrorInvalidValue;
   static hipError_t state1[kMaxDevices], state2[kMaxDevices];
   static bool done1[kMaxDevices], done2[kMaxDevices];
-  hipError_t e = grant_dynamic_lds((const void*)backward_dq_f32_kernel<D, CAUSAL, MASKED>, BwdF32Lds<D>::BYTES, state1, done1);
+  hipError_t e = grant_dynamic_lds((const void*)backward_dq_f32_kernel<D, CAUSAL, MASKED, PAD>, BwdF32Lds<D>::BYTES, state1, done1);
   if (e != hipSuccess) return (int)e;
-  e = grant_dynamic_lds((const void*)backward_dkv_f32_kernel<D, CAUSAL, MASKED>, BwdF32Lds<D>::BYTES, state2, done2);
+  e = grant_dynamic_lds((const void*)backward_dkv_f32_kernel<D, CAUSAL, MASKED, PAD>, BwdF32Lds<D>::BYTES, state2, done2);
   if (e != hipSuccess) return (int)e;
   const long long g1 = (long long)a.f.B * a.f.Hq * ((a.f.L + BM - 1) / BM) * a.dq_splits;
   const long long g2 = (long long)a.f.B * a.f.Hkv * ((a.f.S + BM - 1) / BM) * a.dkv_splits;
   static int round_cache[kMaxDevices];
-  a.dkv_round = CAUSAL ? dkv_round_of((const void*)backward_dkv_f32_kernel<D, CAUSAL, MASKED>, 256, BwdF32Lds<D>::BYTES, round_cache) : 0;
-  hipLaunchKernelGGL((backward_dq_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g1), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
+  a.dkv_round = CAUSAL ? dkv_round_of((const void*)backward_dkv_f32_kernel<D, CAUSAL, MASKED, PAD>, 256, BwdF32Lds<D>::BYTES, round_cache) : 0;
+  hipLaunchKernelGGL((backward_dq_f32_kernel<D, CAUSAL, MASKED, PAD>), dim3((unsigned)g1), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   if (a.dq_splits > 1) {
     const int rc = launch_backward_dq_merge<float>(a, stream);
     if (rc != 0) return rc;
   }
-  hipLaunchKernelGGL((backward_dkv_f32_kernel<D, CAUSAL, MASKED>), dim3((unsigned)g2), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
+  hipLaunchKernelGGL((backward_dkv_f32_kernel<D, CAUSAL, MASKED, PAD>), dim3((unsigned)g2), dim3(256), BwdF32Lds<D>::BYTES, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess || a.dkv_splits == 1) return (int)e;
   return launch_backward_dkv_sum<float>(a, stream);
 }
 
+template <int D, bool PAD>
+int launch_d(const BwdArgs& a, hipStream_t stream) {
+  if (a.f.mask_kind != 0) return launch_k<D, false, true, PAD>(a, stream);  // exclusive with causal (validated by the caller, as the reference asserts)
+  return a.f.causal ? launch_k<D, true, false, PAD>(a, stream) : launch_k<D, false, false, PAD>(a, stream);
+}
+
 }  // namespace
 
 int launch_backward_f32(const BwdArgs& a, hipStream_t stream) {
-  if (a.f.mask_kind != 0)  // exclusive with causal (validated by the caller, as the reference asserts)
-    return a.f.D == 128 ? launch_k<128, false, true>(a, stream) : launch_k<64, false, true>(a, stream);
-  if (a.f.D == 128) return a.f.causal ? launch_k<128, true, false>(a, stream) : launch_k<128, false, false>(a, stream);
-  return a.f.causal ? launch_k<64, true, false>(a, stream) : launch_k<64, false, false>(a, stream);
+  if (a.f.D == 128) return launch_d<128, false>(a, stream);
+  if (a.f.D == 64) return launch_d<64, false>(a, stream);
+  // any other multiple of 4 up to 128: the kernels of the next size up, the missing columns as zeros
+  return a.f.D < 64 ? launch_d<64, true>(a, stream) : launch_d<128, true>(a, stream);
 }
 
 }  // namespace ttsdpa

@@ -302,7 +302,7 @@ bool backward_mfma_ok(const ttsdpa_backward_params* p) {
 // the 16-bit pair.
 bool backward_f32_ok(const ttsdpa_backward_params* p) {
   const ttsdpa_params* f = &p->fwd;
-  if (f->dtype != TTSDPA_F32 || f->block_table || !simple_mask_ok(f) || (f->D != 64 && f->D != 128)) return false;
+  if (f->dtype != TTSDPA_F32 || f->block_table || !simple_mask_ok(f) || f->D < 4 || f->D > 128 || f->D % 4 != 0) return false;
   if (!(f->scale > 0.f) || !isfinite(f->scale) || f->L < 1 || f->S < 1) return false;  // the row maximum is taken on unscaled scores
   if (!dense_last_ok(f->q_stride, 4) || !dense_last_ok(f->k_stride, 4) || !dense_last_ok(f->v_stride, 4) ||
       !dense_last_ok(f->o_stride, 4) || !dense_last_ok(p->dout_stride, 4) || !dense_last_ok(p->dq_stride, 4) ||
