@@ -65,7 +65,7 @@ enum ttsdpa_route {
   TTSDPA_ROUTE_NONE = 0,    /* nothing to launch (an empty output) */
   TTSDPA_ROUTE_GENERAL = 1, /* any dtype / head_dim / mask / per-batch key counts; fp32 arithmetic on the vector ALUs */
   TTSDPA_ROUTE_PREFILL = 2, /* MFMA flash-attention forward: fp16/bf16 with any head_dim that is a multiple of 8 up to 256 (attnMasks readable four keys at a time; any attnMask at head_dim 128 with L > 128); fp32 with any head_dim that is a multiple of 4 up to 128 */
-  TTSDPA_ROUTE_DECODE = 3,  /* fp16/bf16, head_dim 128 or 64, few query rows against a long KV cache: split-KV streaming */
+  TTSDPA_ROUTE_DECODE = 3,  /* fp16/bf16, head_dim a multiple of 8 up to 128, few query rows against a long KV cache: split-KV streaming */
   TTSDPA_ROUTE_ZERO = 4     /* S == 0: the reference's empty contraction yields zeros */
 };
 

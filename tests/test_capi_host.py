@@ -66,6 +66,9 @@ def test_struct_layout_matches_header():
     ((_capi.BF16, 64, 32, 8, 1, 8192, 128), _capi.ROUTE_DECODE),     # config 4
     ((_capi.BF16, 1, 28, 4, 16384, 16384, 128), _capi.ROUTE_PREFILL),  # config 5
     ((_capi.BF16, 1, 28, 4, 1, 4096, 128), _capi.ROUTE_DECODE),      # 7 heads per KV head
+    ((_capi.BF16, 4, 32, 8, 1, 4096, 96), _capi.ROUTE_DECODE),       # a multiple of 8 below 128: the head_dim-128 kernel, zero columns
+    ((_capi.F16, 4, 32, 8, 1, 4096, 40), _capi.ROUTE_DECODE),
+    ((_capi.BF16, 4, 32, 8, 1, 4096, 100), _capi.ROUTE_GENERAL),     # rows that are not whole 16-byte chunks
     ((_capi.BF16, 1, 8, 8, 300, 300, 64), _capi.ROUTE_PREFILL),
     ((_capi.BF16, 1, 8, 8, 300, 300, 96), _capi.ROUTE_PREFILL),
     ((_capi.F16, 1, 8, 8, 300, 300, 256), _capi.ROUTE_PREFILL),

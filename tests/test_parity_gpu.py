@@ -188,6 +188,40 @@ def test_decode_against_oracle(case):
     assert err <= TOL[dtype]
 
 
+@pytest.mark.parametrize("D", [8, 40, 56, 72, 80, 96, 112, 120])
+@pytest.mark.parametrize("shape", [(4, 32, 8, 1, 2048, "bf16"), (2, 8, 2, 1, 33, "f16"), (1, 16, 1, 1, 513, "bf16"),
+                                   (2, 4, 1, 4, 640, "f16"), (1, 32, 8, 1, 9000, "bf16")],
+                         ids=lambda c: "B%dH%dk%dL%dS%d-%s" % c)
+def test_decode_head_sizes_between_the_kernels(D, shape):
+    # any multiple of 8 up to 128 on the streaming kernel for 64 or 128 (zero columns); views of wider rows whose other
+    # columns hold NaN (inputs) or a sentinel (output), so that nothing beyond head_dim is read into the result or written
+    B, Hq, Hkv, L, S, dtype = shape
+    say("decode, padded head_dim", D, shape)
+    host, dev = make_inputs(2300 + S + D, B, Hq, Hkv, L, S, D, dtype)
+    assert route_of(*dev) == "decode"
+    exp = oracle.sdpa_f32(*host, causal=False)
+    rc, out = call("forward", *dev)
+    assert rc == 0 and max_abs_err(out, exp) <= TOL[dtype]
+    wide = []
+    for t in dev:
+        w = torch.full(t.shape[:-1] + (128,), float("nan"), dtype=t.dtype, device="cuda")
+        w[..., :D] = t
+        wide.append(w[..., :D])
+    outw = torch.full((B, Hq, L, 128), 7.0, dtype=dev[0].dtype, device="cuda")
+    rc, _ = call("decode", *wide, out=outw[..., :D])
+    assert rc == 0 and torch.equal(outw[..., :D], out) and bool((outw[..., D:] == 7.0).all())
+    # per-batch key counts and the bottom-right causal rows of a multi-token step
+    if S >= 513:
+        lens = np.array([S - 5 * b for b in range(B)], np.int32)
+        rc, out = call("forward", *dev, causal=L > 1, align="bottom-right", kv_lens=torch.from_numpy(lens).cuda())
+        assert rc == 0
+        for b in range(B):
+            n = int(lens[b])
+            m = np.tril(np.ones((L, n), np.uint8), n - L)
+            e = oracle.sdpa_f32(host[0][b:b + 1], host[1][b:b + 1, :, :n], host[2][b:b + 1, :, :n], mask=m)
+            assert max_abs_err(out[b:b + 1], e) <= TOL[dtype]
+
+
 def test_decode_cache_view_and_key_permutation():
     B, Hq, Hkv, S, D = 4, 8, 2, 1500, 128
     host, dev = make_inputs(31, B, Hq, Hkv, 1, S, D, "bf16")

@@ -55,7 +55,10 @@ __device__ __forceinline__ void wave_lds_sync() {
 // R = registers of query rows per score lane: rows handled = up to 4*R.
 // PAGED: K/V are page pools addressed through a block table (a variant of its own, so that the contiguous kernel
 // carries none of the lookups).
-template <typename TR, int R, int DD, bool PAGED>
+// PAD: the tensors' head_dim a.D is a multiple of 8 below DD.  The 16-byte chunks of a row beyond it read as zeros (q, k)
+// or are left out of the output (v: the lanes of those chunks fetch the row's first chunk instead, so that the loads stay
+// unconditional); the split records keep the pitch DD + 2.
+template <typename TR, int R, int DD, bool PAGED, bool PAD>
 __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int chunk, float* __restrict__ ws) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
@@ -101,9 +104,10 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int
     const T* qr = (const T*)a.q + b * a.qs[0] + (hk * a.G + xg) * a.qs[1] + xl * a.qs[2] + 8 * lg;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      vec8 t = *(const vec8*)(qr + 32 * ks);
+      const bool there = used && (!PAD || 32 * ks + 8 * lg < a.D);
+      vec8 t = *(const vec8*)(there ? qr + 32 * ks : qr - 8 * lg);
 #pragma unroll
-      for (int i = 0; i < 8; i++) qa[ks][i] = used ? t[i] : (T)0.f;
+      for (int i = 0; i < 8; i++) qa[ks][i] = there ? t[i] : (T)0.f;
     }
   }
 
@@ -158,14 +162,22 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int
       key = (key < S ? key : S - 1) - key0;
       const T* kr = kpb + key * a.ks[2] + 8 * lg;
 #pragma unroll
-      for (int ks = 0; ks < KS; ks++) kreg[gi][ks] = __builtin_nontemporal_load((const u32x4*)(kr + 32 * ks));  // read once: keep it out of the caches
+      for (int ks = 0; ks < KS; ks++) {
+        if (!PAD) {
+          kreg[gi][ks] = __builtin_nontemporal_load((const u32x4*)(kr + 32 * ks));  // read once: keep it out of the caches
+        } else {
+          const bool there = 32 * ks + 8 * lg < a.D;
+          const u32x4 t = __builtin_nontemporal_load((const u32x4*)(there ? kr + 32 * ks : kr - 8 * lg));
+          kreg[gi][ks] = there ? t : u32x4{0u, 0u, 0u, 0u};
+        }
+      }
     }
     u32x4 vreg[KB / PH];
 #pragma unroll
     for (int i = 0; i < KB / PH; i++) {
       int key = k0 + PH * i + vph;
       key = (key < S ? key : S - 1) - key0;
-      vreg[i] = __builtin_nontemporal_load((const u32x4*)(vpb + key * a.vs[2] + 8 * vc));
+      vreg[i] = __builtin_nontemporal_load((const u32x4*)(vpb + key * a.vs[2] + (PAD && 8 * vc >= a.D ? 0 : 8 * vc)));
     }
 
     // ---- scores --------------------------------------------------------------------------------------------------------
@@ -274,7 +286,7 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(KArgs a, int splits, int
     if (splits == 1) {
       int xl = x / a.G, xg = x % a.G;
       T* op = (T*)a.out + b * a.os[0] + (hk * a.G + xg) * a.os[1] + xl * a.os[2];
-      store_from_float(op + d, lsum > 0.f ? o / lsum : 0.f);  // no keys at all: zeros, as the reference's empty contraction
+      if (!PAD || d < a.D) store_from_float(op + d, lsum > 0.f ? o / lsum : 0.f);  // no keys at all: zeros, as the reference's empty contraction
     } else {
       float* rec = ws + ((long long)blockIdx.x * rows + x) * (DD + 2);
       rec[d] = o;
@@ -321,19 +333,19 @@ __global__ __launch_bounds__(DD) void merge_kernel(KArgs a, int splits, const fl
   for (int s = 0; s < splits; s++) o = fmaf(weight[s], rec0[s * step + t], o);
   const int xl = x / a.G, xg = x % a.G;
   T* op = (T*)a.out + b * a.os[0] + (hk * a.G + xg) * a.os[1] + xl * a.os[2];
-  store_from_float(op + t, total > 0.f ? o / total : 0.f);
+  if (t < a.D) store_from_float(op + t, total > 0.f ? o / total : 0.f);  // (a.D < DD: the decode kernel's zero-column variant)
 }
 
-template <typename TR, int DD>
+template <typename TR, int DD, bool PAD>
 int launch_decode_t(const KArgs& a, const DecodePlan& pl, float* ws, hipStream_t stream) {
   typedef typename TR::elem T;
   dim3 grid((unsigned)((long long)a.B * a.Hkv * pl.splits)), block(256);
   int R = (pl.rows + 3) / 4;
 #define TT_DECODE(R_)                                                                                                      \
   if (a.block_table)                                                                                                       \
-    hipLaunchKernelGGL((decode_kernel<TR, R_, DD, true>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws);            \
+    hipLaunchKernelGGL((decode_kernel<TR, R_, DD, true, PAD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws);       \
   else                                                                                                                     \
-    hipLaunchKernelGGL((decode_kernel<TR, R_, DD, false>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws)
+    hipLaunchKernelGGL((decode_kernel<TR, R_, DD, false, PAD>), grid, block, 0, stream, a, pl.splits, pl.chunk, ws)
   switch (R) {
     case 1: TT_DECODE(1); break;
     case 2: TT_DECODE(2); break;
@@ -367,7 +379,7 @@ DecodePlan plan_decode(const KArgs& a) {
   if (splits < 1) splits = 1;
   p.splits = splits;
   p.chunk = chunk;
-  p.ws_bytes = splits > 1 ? (size_t)pairs * splits * p.rows * (a.D + 2) * sizeof(float) : 0;
+  p.ws_bytes = splits > 1 ? (size_t)pairs * splits * p.rows * ((a.D <= 64 ? 64 : 128) + 2) * sizeof(float) : 0;  // the kernel's head_dim: 64 or 128
   return p;
 }
 
@@ -389,10 +401,18 @@ int launch_merge(const KArgs& a, int dtype, int splits, const float* ws, hipStre
 int launch_decode(const KArgs& a, int dtype, void* workspace, hipStream_t stream) {
   DecodePlan pl = plan_decode(a);
   if (a.D == 64)
-    return dtype == 1 ? launch_decode_t<F16, 64>(a, pl, (float*)workspace, stream)
-                      : launch_decode_t<BF16, 64>(a, pl, (float*)workspace, stream);
-  return dtype == 1 ? launch_decode_t<F16, 128>(a, pl, (float*)workspace, stream)
-                    : launch_decode_t<BF16, 128>(a, pl, (float*)workspace, stream);
+    return dtype == 1 ? launch_decode_t<F16, 64, false>(a, pl, (float*)workspace, stream)
+                      : launch_decode_t<BF16, 64, false>(a, pl, (float*)workspace, stream);
+  if (a.D == 128)
+    return dtype == 1 ? launch_decode_t<F16, 128, false>(a, pl, (float*)workspace, stream)
+                      : launch_decode_t<BF16, 128, false>(a, pl, (float*)workspace, stream);
+  // any other multiple of 8 up to 128: the kernel of the next size up, the missing columns as zeros
+  if (a.D % 8 != 0 || a.D < 8 || a.D > 128) return (int)hipErrorInvalidValue;  // (the callers keep to this)
+  if (a.D < 64)
+    return dtype == 1 ? launch_decode_t<F16, 64, true>(a, pl, (float*)workspace, stream)
+                      : launch_decode_t<BF16, 64, true>(a, pl, (float*)workspace, stream);
+  return dtype == 1 ? launch_decode_t<F16, 128, true>(a, pl, (float*)workspace, stream)
+                    : launch_decode_t<BF16, 128, true>(a, pl, (float*)workspace, stream);
 }
 
 }  // namespace ttsdpa

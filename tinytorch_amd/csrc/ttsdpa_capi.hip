@@ -235,7 +235,8 @@ bool prefill_ok(const ttsdpa_params* p) {
 
 bool decode_ok(const ttsdpa_params* p) {
   // a top-left aligned causal mask leaves a few keys per row: not the streaming kernel's case
-  if (!fast_layout_ok(p, false, true) || (p->D != 128 && p->D != 64) || effective_causal(p) == TTSDPA_CAUSAL_TOP_LEFT ||
+  // head_dim 64 and 128; other multiples of 8 up to 128 on the next one up with zero columns
+  if (!fast_layout_ok(p, false, true) || p->D < 8 || p->D > 128 || p->D % 8 != 0 || effective_causal(p) == TTSDPA_CAUSAL_TOP_LEFT ||
       p->S < 1 || p->L < 1)
     return false;
   if (p->block_table && p->page_size < 32) return false;  // a 32-key block of a wavefront must lie in one page
@@ -250,7 +251,9 @@ int pick_route(const ttsdpa_params* p) {
     // 9-16 rows per KV head: the streaming kernel does P.V on the vector ALUs and measures 5.5 TB/s there; the
     // 4-wavefront MFMA kernel with packed heads and split keys 5.85 TB/s, when the call allows it
     const long long rows = (long long)p->L * (p->Hq / p->Hkv);
-    if (rows > 8 && prefill_ok(p) && !pipelined_ok(p) && (p->Hq == p->Hkv || pack_heads_ok(p))) return TTSDPA_ROUTE_PREFILL;
+    // (head_dim 64 / 128: the zero-column variants of that kernel do not split their keys)
+    if (rows > 8 && (p->D == 64 || p->D == 128) && prefill_ok(p) && !pipelined_ok(p) && (p->Hq == p->Hkv || pack_heads_ok(p)))
+      return TTSDPA_ROUTE_PREFILL;
     return TTSDPA_ROUTE_DECODE;
   }
   if (prefill_ok(p) && p->L >= 16) return TTSDPA_ROUTE_PREFILL;
