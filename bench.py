@@ -25,8 +25,10 @@ reported under "other_configs".
 
 "roofline"."zero_operands" is the headline launch repeated on all-zero Q, K, V: the same instruction stream without operand
 toggling, i.e. what the kernel's schedule reaches when the chip's power management leaves the clock alone (the prefill
-kernel is power-bound on N(0,1) data).  "roofline"."summary" lists the fraction of every other line of the run, and the
-line's last key, "in_short", repeats the headline, decode and summary figures in a few hundred characters.
+kernel is power-bound on N(0,1) data: "roofline"."power" and "zero_operands"."power" hold the socket power and the
+core clock the driver's sysfs files report while each of the two runs back to back, after its timed launches).
+"roofline"."summary" lists the fraction of every other line of the run, and the line's last key, "in_short", repeats
+the headline, decode and summary figures in a few hundred characters.
 
 Algorithmic work per launch (what "achieved" divides by the measured launch time):
   prefill, causal:  4 * B * Hq * D * S(S+1)/2 flop   (two GEMMs over the visible triangle)
@@ -152,6 +154,66 @@ def time_launches(step, stream, steps, warmup, settle_seconds=None):
             "settle_launches": settle}
 
 
+def power_under(step, seconds=2.0):
+    """Socket power and core clock while `step` is launched back to back for `seconds`, read from the driver's sysfs
+    files (hwmon power1_input in microwatts, the current entry of pp_dpm_sclk; None where they are missing).  Untimed: it
+    runs after the timed launches."""
+    import glob
+    import re
+    import threading
+    import torch
+
+    pfiles = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))
+    if not pfiles:
+        return None
+    pfile = pfiles[0]
+    dev = pfile.split("/hwmon/")[0]
+    samples, stop = [], threading.Event()
+
+    def read(path):
+        with open(path) as f:
+            return f.read()
+
+    def sampler():
+        while not stop.is_set():
+            try:
+                watts = int(read(pfile).strip()) / 1e6
+                mhz = None
+                for ln in read(os.path.join(dev, "pp_dpm_sclk")).splitlines():
+                    m = re.match(r"\s*\S+:\s*(\d+)\s*Mhz\s*\*", ln, re.I)
+                    if m:
+                        mhz = int(m.group(1))
+                samples.append((watts, mhz))
+            except Exception:
+                pass
+            time.sleep(0.05)
+
+    th = threading.Thread(target=sampler)
+    th.start()
+    t_end = time.perf_counter() + seconds
+    n = 0
+    while time.perf_counter() < t_end:
+        for _ in range(256):
+            step()
+        n += 256
+        torch.cuda.synchronize()
+    stop.set()
+    th.join()
+    samples = samples[len(samples) // 4:]  # the first ones see the ramp
+    if not samples:
+        return None
+    watts = sorted(w for w, _ in samples)
+    clocks = sorted(c for _, c in samples if c is not None)
+    cap = None
+    try:
+        cap = int(read(os.path.join(os.path.dirname(pfile), "power1_cap")).strip()) / 1e6
+    except Exception:
+        pass
+    return {"socket_power_w": round(watts[len(watts) // 2], 1), "power_cap_w": cap,
+            "gfx_clock_mhz": clocks[len(clocks) // 2] if clocks else None, "samples": len(samples), "launches": n,
+            "source": "sysfs hwmon power1_input and pp_dpm_sclk during back-to-back launches (medians)"}
+
+
 def synth_qkv(name):
     """The workload's Q, K, V on the device: N(0,1) * multiplier from the repository's generator, rounded to its dtype."""
     import torch
@@ -178,7 +240,7 @@ def synth_mask(name):
     return m
 
 
-def run_gpu(name, steps, warmup, zero_inputs=False):
+def run_gpu(name, steps, warmup, zero_inputs=False, power=False):
     import torch
     from tinytorch_amd import _capi, build_params
 
@@ -220,6 +282,8 @@ def run_gpu(name, steps, warmup, zero_inputs=False):
                      "kernel_ms_min": round(t["min_ms"], 5), "timing": "median of %d launches, one HIP event pair each" % steps,
                      "settle_launches": t["settle_launches"], "algorithmic_flops": flops, "algorithmic_bytes": abytes},
     }
+    if power:  # what the chip's power management does under this launch (after the timed region)
+        res["roofline"]["power"] = power_under(step)
     return res, (q, k, v, out, mask)
 
 
@@ -527,6 +591,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-probes", action="store_true", help="skip the hardware ceiling probes")
     ap.add_argument("--no-zero", action="store_true", help="skip the repeat of the headline launch on all-zero operands")
+    ap.add_argument("--no-power", action="store_true", help="skip the socket power / core clock samples of the headline launch")
     ap.add_argument("--zero-inputs", action="store_true",
                     help="run the workload on all-zero Q, K, V only (for profiling the same instruction stream without operand toggling)")
     ap.add_argument("--settle", type=float, default=None,
@@ -567,7 +632,7 @@ def main():
         print(json.dumps(run_backward(args.steps, args.warmup, cpu=not args.no_cpu and args.backward_dtype == "bf16",
                                       dtype=args.backward_dtype)), flush=True)
         return
-    main_res, tensors = run_gpu(args.workload, args.steps, args.warmup, zero_inputs=args.zero_inputs)
+    main_res, tensors = run_gpu(args.workload, args.steps, args.warmup, zero_inputs=args.zero_inputs, power=not args.no_power)
     ceilings = None if args.no_probes else run_probes()
     cpu = None if args.no_cpu else run_cpu_baseline(args.workload, tensors, args.cpu_seconds)
     del tensors
@@ -576,11 +641,12 @@ def main():
     if not args.no_zero and not args.zero_inputs and WORKLOADS[args.workload][9] == "mfma":
         # the same launch on all-zero operands: the instruction stream without operand toggling (the kernel is power-bound
         # on N(0,1) data: the chip lowers its clock under it)
-        z, tensors = run_gpu(args.workload, args.steps, args.warmup, zero_inputs=True)
+        z, tensors = run_gpu(args.workload, args.steps, args.warmup, zero_inputs=True, power=not args.no_power)
         del tensors
         torch.cuda.empty_cache()
         main_res["roofline"]["zero_operands"] = {
             "kernel_ms": z["roofline"]["kernel_ms"], "achieved": z["roofline"]["achieved"], "frac": z["roofline"]["frac"],
+            "power": z["roofline"].get("power"),
             "note": "the same launch with Q = K = V = 0: identical instruction stream, no operand toggling; not a result, "
                     "the clock the power management grants is the difference"}
     summary = {}
@@ -645,6 +711,11 @@ def main():
     line["in_short"] = {"prefill_%s" % args.workload: {"frac": r["frac"], "kernel_ms": r["kernel_ms"], "achieved": r["achieved"], "unit": r["unit"]}}
     if "zero_operands" in r:
         line["in_short"]["prefill_%s_zero_operands_frac" % args.workload] = r["zero_operands"]["frac"]
+    pw, zpw = r.get("power"), r.get("zero_operands", {}).get("power")
+    if pw and zpw:
+        line["in_short"]["socket_power_w_and_gfx_mhz"] = {
+            "n01_operands": [pw["socket_power_w"], pw["gfx_clock_mhz"]],
+            "zero_operands": [zpw["socket_power_w"], zpw["gfx_clock_mhz"]], "power_cap_w": pw["power_cap_w"]}
     if "decode" in r:
         d = r["decode"]
         line["in_short"]["decode_config4"] = {"frac": d["frac"], "kernel_ms": d["kernel_ms"], "achieved": d["achieved"], "unit": d["unit"]}
