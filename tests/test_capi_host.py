@@ -211,6 +211,10 @@ def test_kernel_domains_and_workspace():
     assert L.ttsdpa_decode(ctypes.byref(dec), None, 0, None) == _capi.ERR_WORKSPACE
     assert L.ttsdpa_decode(ctypes.byref(dec), FAKE, need - 1, None) == _capi.ERR_WORKSPACE
     assert L.ttsdpa_forward(ctypes.byref(dec), FAKE, need - 1, None) == _capi.ERR_WORKSPACE
+    # a head size between the decode kernel's: the records have the pitch of the kernel that runs (head_dim 128 here)
+    assert L.ttsdpa_workspace_bytes(ctypes.byref(params(_capi.BF16, 2, 32, 8, 1, 8192, 96))) == need
+    assert L.ttsdpa_workspace_bytes(ctypes.byref(params(_capi.BF16, 2, 32, 8, 1, 8192, 40))) == \
+        L.ttsdpa_workspace_bytes(ctypes.byref(params(_capi.BF16, 2, 32, 8, 1, 8192, 64)))
     short = params(_capi.BF16, 2, 8, 2, 1, 64, 128)
     assert L.ttsdpa_workspace_bytes(ctypes.byref(short)) == 0          # one split: no scratch
     assert L.ttsdpa_workspace_bytes(ctypes.byref(fp32)) == 0
