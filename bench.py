@@ -27,6 +27,7 @@ reported under "other_configs".
 toggling, i.e. what the kernel's schedule reaches when the chip's power management leaves the clock alone (the prefill
 kernel is power-bound on N(0,1) data: "roofline"."power" and "zero_operands"."power" hold the socket power and the
 core clock the driver's sysfs files report while each of the two runs back to back, after its timed launches).
+The linear and backward lines carry the same repeat as "roofline"."zero_operands_frac".
 "roofline"."summary" lists the fraction of every other line of the run, and the line's last key, "in_short", repeats
 the headline, decode and summary figures in a few hundred characters.
 
@@ -471,6 +472,10 @@ def run_linear(steps, warmup, cpu=True):
                                "kind": kind, "sample": "a [%d, %d] corner of the output, %d passes in %.1f s, one thread (fp32 on the bf16 values)"
                                % (rows, cols, reps, spent),
                                "max_abs_err_gpu_vs_cpu": float("%.3g" % float(np.abs(ref - got).max()))}
+    # the same launch on all-zero operands: what the kernel's schedule reaches without the power its data draws
+    x.zero_(), w.zero_(), b.zero_()
+    tz = time_launches(step, stream, steps, warmup)
+    res["roofline"]["zero_operands_frac"] = round(flops / (tz["median_ms"] * 1e-3) / 1e12 / PEAK_TFLOPS["bf16"], 4)
     return res
 
 
@@ -530,6 +535,11 @@ def run_backward(steps, warmup, cpu=True, dtype="bf16"):
                                "sample": "the first %d queries x %d keys of one KV head (its %d query heads), %.1f s, one thread, double accumulation"
                                % (n, n, Hq // Hkv, spent),
                                "max_abs_err_gpu_vs_cpu_dq": float("%.3g" % float(np.abs(rq - got).max()))}
+    if dtype == "bf16":  # the same launches on all-zero tensors (as for the forward: the share of the power limit)
+        for t_ in (q, k, v, go, out):
+            t_.zero_()
+        tz = time_launches(step, stream, steps, warmup)
+        res["roofline"]["zero_operands_frac"] = round(flops / (tz["median_ms"] * 1e-3) / 1e12 / PEAK_TFLOPS[dtype], 4)
     return res
 
 
@@ -701,7 +711,9 @@ def main():
         for r in line["fused_ops"]:
             summary[r["workload"].split()[0]] = r["roofline"]["frac"]
         summary["linear"] = line["linear"]["roofline"]["frac"]
+        summary["linear_zero_operands"] = line["linear"]["roofline"]["zero_operands_frac"]
         summary["backward_bf16"] = line["backward"]["roofline"]["frac"]
+        summary["backward_bf16_zero_operands"] = line["backward"]["roofline"]["zero_operands_frac"]
         summary["backward_f32"] = line["backward"]["fp32"]["roofline"]["frac"]
     if summary:  # fraction of its own roofline for every other line of this run (config1: launch-sized, its kernel ms)
         line["roofline"]["summary"] = summary
