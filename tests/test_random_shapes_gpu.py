@@ -11,12 +11,22 @@ from tinytorch_amd import sdpAttention
 pytestmark = pytest.mark.gpu
 
 
-def _cases():
-    rng = np.random.RandomState(20240607)
+def _head_dim(rng, dtype, other, limit):
+    """A head size: one of the kernels' own, or (other) any size their zero-column variants take, up to `limit`."""
+    if not other:
+        return None
+    step = 4 if dtype == "f32" else 8
+    top = min(limit, 128) if dtype == "f32" else limit
+    return int(rng.randint(1, top // step + 1)) * step
+
+
+def _cases(other=False):
+    rng = np.random.RandomState(20250115 if other else 20240607)
     out = []
-    for i in range(48):
+    for i in range(40 if other else 48):
         dtype = ["bf16", "f16", "f32"][rng.randint(3)]
         D = [128, 128, 128, 64, 32, 80][rng.randint(6)]
+        D = _head_dim(rng, dtype, other, 256) or D
         Hkv = int(rng.randint(1, 4))
         G = [1, 1, 2, 4, 7][rng.randint(5)]
         B = int(rng.randint(1, 4))
@@ -32,11 +42,11 @@ def _cases():
             L = int(rng.randint(1, 129))
             S = int(rng.randint(1, 400))
         extra = ["none", "none", "causal", "causal", "boolmask", "addmask", "kvlen"][rng.randint(7)]
-        out.append((i, dtype, B, Hkv * G, Hkv, L, S, D, extra))
+        out.append((i + (100 if other else 0), dtype, B, Hkv * G, Hkv, L, S, D, extra))
     return out
 
 
-@pytest.mark.parametrize("case", _cases(), ids=lambda c: "%d-%s-B%d-H%d/%d-L%d-S%d-D%d-%s" % c)
+@pytest.mark.parametrize("case", _cases() + _cases(other=True), ids=lambda c: "%d-%s-B%d-H%d/%d-L%d-S%d-D%d-%s" % c)
 def test_random_shape(case):
     i, dtype, B, Hq, Hkv, L, S, D, extra = case
     host, dev = make_inputs(3000 + i, B, Hq, Hkv, L, S, D, dtype)
@@ -67,12 +77,13 @@ def test_random_shape(case):
     assert max_abs_err(out, exp) <= TOL[dtype], route_of(*dev, causal=extra == "causal")
 
 
-def _backward_cases():
-    rng = np.random.RandomState(20240911)
+def _backward_cases(other=False):
+    rng = np.random.RandomState(20250116 if other else 20240911)
     out = []
-    for i in range(40):
+    for i in range(32 if other else 40):
         dtype = ["bf16", "f16", "f32"][rng.randint(3)]
         D = [128, 128, 64, 64, 32, 80][rng.randint(6)]
+        D = _head_dim(rng, dtype, other, 128) or D
         Hkv = int(rng.randint(1, 3))
         G = [1, 1, 2, 4, 3][rng.randint(5)]
         B = int(rng.randint(1, 3))
@@ -81,11 +92,11 @@ def _backward_cases():
         extra = ["none", "causal", "causal-br", "boolmask", "addmask", "kvlen", "boolmask4"][rng.randint(7)]
         if extra == "boolmask4":
             S = (S + 3) // 4 * 4   # keys readable four at a time: the MFMA pair's masks
-        out.append((i, dtype, B, Hkv * G, Hkv, L, S, D, extra))
+        out.append((i + (100 if other else 0), dtype, B, Hkv * G, Hkv, L, S, D, extra))
     return out
 
 
-@pytest.mark.parametrize("case", _backward_cases(), ids=lambda c: "%d-%s-B%d-H%d/%d-L%d-S%d-D%d-%s" % c)
+@pytest.mark.parametrize("case", _backward_cases() + _backward_cases(other=True), ids=lambda c: "%d-%s-B%d-H%d/%d-L%d-S%d-D%d-%s" % c)
 def test_random_backward_shape(case):
     """The same idea for ttsdpa_backward: both kernel families, ragged tiles on both sides, grouped heads, both causal
     alignments, masks, per-batch key counts — against the oracle's gradients."""
