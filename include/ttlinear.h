@@ -45,9 +45,12 @@ int ttlinear_plan(int dtype, const void* x, const void* w, const void* bias, con
  * [N, K] with transB).  (false, true) is ttlinear_forward; FuncLinear::backward (reference
  * src/Function/FuncNNLayer.h:20-33) uses the other two that matter: (false, false) for the input gradient
  * dy[M, N] . w[N, K], and (true, false) for the weight gradient dy^T . x.  lda / ldb / ldo are row strides in elements.
- * workspace: ttlinear_matmul_workspace_bytes() bytes of device scratch, 256-byte aligned — the MFMA route first makes
- * dense row-major copies of the operands that are stored contraction-major; with less (or NULL), or for shapes the MFMA
- * kernel does not take, the vector-ALU kernel reads the operands in place.  Same return codes as ttlinear_forward. */
+ * fp16 / bf16 operands stored contraction-major are read in place by the matrix-core kernel (K a multiple of 64, N a
+ * multiple of 4, 16-byte aligned operands with leading dimensions that are multiples of 8, a contraction-major operand's
+ * row count a multiple of 8): no scratch is used then and workspace may be NULL.
+ * workspace: ttlinear_matmul_workspace_bytes() bytes of device scratch, 256-byte aligned — for fp32 the MFMA route first
+ * makes dense row-major copies of the operands that are stored contraction-major; with less (or NULL), or for shapes the
+ * MFMA kernels do not take, the vector-ALU kernel reads the operands in place.  Same return codes as ttlinear_forward. */
 size_t ttlinear_matmul_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b);
 int ttlinear_matmul(int dtype, const void* a, const void* b, const void* bias, void* out, int64_t M, int64_t N, int64_t K,
                     int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldo, void* workspace,

@@ -198,9 +198,9 @@ typedef struct ttsdpa_backward_params {
 /* Fill *p for dense tensors (ttsdpa_params_init for fwd, dense gradient strides); pointers NULL. */
 void ttsdpa_backward_params_init(ttsdpa_backward_params* p, int dtype, int B, int Hq, int Hkv, int L, int S, int D);
 /* Validate and report the kernels ttsdpa_backward would use: TTSDPA_ROUTE_PREFILL = the MFMA backward kernels
- * (fp16 / bf16 / fp32 — the latter on the fp32 matrix cores —, head_dim 64 or 128, 16-byte aligned rows; an attnMask
- * must have contiguous, 4-aligned keys), TTSDPA_ROUTE_GENERAL = the vector-ALU kernels, TTSDPA_ROUTE_NONE = nothing to
- * compute.  Needs no GPU. */
+ * (fp16 / bf16 with head_dim a multiple of 8 up to 128, fp32 — on the fp32 matrix cores — with head_dim a multiple of 4
+ * up to 128; 16-byte aligned rows; an attnMask must have contiguous, 4-aligned keys), TTSDPA_ROUTE_GENERAL = the
+ * vector-ALU kernels, TTSDPA_ROUTE_NONE = nothing to compute.  Needs no GPU. */
 int ttsdpa_backward_plan(const ttsdpa_backward_params* p, int* route);
 size_t ttsdpa_backward_workspace_bytes(const ttsdpa_backward_params* p);
 int ttsdpa_backward(const ttsdpa_backward_params* p, void* workspace, size_t workspace_bytes, void* stream);
