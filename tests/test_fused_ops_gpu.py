@@ -74,7 +74,9 @@ def test_silu_mul(rows, d, dtype):
 @pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("shape,dim", [((4,), 0), ((3, 7), -1), ((3, 7), 0), ((64, 1000), 1), ((5, 32000), -1),
                                        ((2, 151936), -1), ((4, 9, 6), 1), ((2, 3, 300, 64), 2), ((8, 4096), 1),
-                                       ((2, 70000), 1), ((6, 128, 33), 1)])
+                                       ((2, 70000), 1), ((6, 128, 33), 1),
+                                       # few very long rows (1024 lanes per row): kept whole, kept in part, unaligned
+                                       ((64, 128256), -1), ((3, 40000), 1), ((1, 262144), 0 + 1), ((2, 100003), -1)])
 def test_softmax_and_log_softmax(shape, dim, dtype):
     say("softmax", shape, dim, dtype)
     xh, xd = inputs(400 + sum(shape), 0, shape, dtype, 3.0)

@@ -71,8 +71,8 @@ struct MaxOp {
 };
 
 // Reduction over the LPR lanes of a row; every lane of the row gets the result.  LPR <= 64: butterfly inside the
-// wavefront.  LPR == 256: the workgroup is one row; wavefront totals cross through LDS (`slot` tells successive
-// reductions of one kernel apart, so one barrier per reduction suffices).
+// wavefront.  LPR == 256 or 1024: the workgroup is one row; wavefront totals cross through LDS (`slot` tells successive
+// reductions of one kernel apart, so one barrier per reduction suffices; lds holds 2 slots x LPR/64 floats).
 template <int LPR, typename Op>
 __device__ __forceinline__ float row_reduce(float v, float* lds, int slot) {
   constexpr int W = LPR < 64 ? LPR : 64;
@@ -83,6 +83,14 @@ __device__ __forceinline__ float row_reduce(float v, float* lds, int slot) {
     if ((threadIdx.x & 63) == 0) lds[4 * slot + wave] = v;
     __syncthreads();
     v = Op::apply(Op::apply(lds[4 * slot], lds[4 * slot + 1]), Op::apply(lds[4 * slot + 2], lds[4 * slot + 3]));
+  } else if constexpr (LPR > 256) {
+    constexpr int NW = LPR / 64;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) lds[NW * slot + wave] = v;
+    __syncthreads();
+    v = lds[NW * slot];
+#pragma unroll
+    for (int w = 1; w < NW; w++) v = Op::apply(v, lds[NW * slot + w]);  // the same order in every lane
   }
   return v;
 }
@@ -188,11 +196,17 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const T* x, T* res, const
 // registers (and from a second read for the part of a very long row that was not kept).
 // KEEP: vectors of its row a lane holds in registers between the statistics and the write (16 for rows of one workgroup
 // that would otherwise be read twice: up to 32768 16-bit elements are then read once).
+// LPR == 1024 (a few very long rows: the softmax over a vocabulary for a batch of sequences): a workgroup of 16
+// wavefronts per row.  With 256 lanes such a launch has one small workgroup per row on a quarter of the CUs and four
+// loads per lane in flight: latency-bound (64 rows of 128256 bf16 elements: 30 us, 1.1 TB/s; 19 us with 1024 lanes, of
+// which a third is the row's exponentials on one CU.  Keeping 16 vectors per lane instead of 8 measured the same: a
+// wavefront of such a workgroup has 128 registers, too few to hold a longer row's exponentials as fp32).
 template <typename T, int VEC, int LPR, bool LOG, int KEEP>
-__global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* out, long long rows, int dim) {  // out may be x
+__global__ __launch_bounds__(LPR > 256 ? LPR : 256) void softmax_rows_kernel(const T* x, T* out, long long rows, int dim) {  // out may be x
   typedef typename Pack<T, VEC>::type V;
-  __shared__ float lds[8];
-  constexpr int RPB = 256 / LPR;
+  constexpr int BLK = LPR > 256 ? LPR : 256;
+  __shared__ float lds[LPR > 256 ? 2 * (LPR / 64) : 8];
+  constexpr int RPB = BLK / LPR;
   const int lr = threadIdx.x % LPR;
   const long long row = (long long)blockIdx.x * RPB + threadIdx.x / LPR;
   const bool live = row < rows;
@@ -426,6 +440,8 @@ int launch_softmax_rows(const void* x, void* out, long long rows, int dim, hipSt
     default:
       if (dim / VEC > CACHE * 256 && dim / VEC <= 2 * CACHE * 256)  // a row of 8 to 16 vectors per lane: keep all of it
         hipLaunchKernelGGL((softmax_rows_kernel<T, VEC, 256, LOG, 2 * CACHE>), dim3(grid), dim3(256), 0, s, (const T*)x, (T*)out, rows, dim);
+      else if (dim / VEC > 2 * CACHE * 256 && rows <= 2048)  // few rows, longer than 256 lanes keep: 1024 lanes per row
+        hipLaunchKernelGGL((softmax_rows_kernel<T, VEC, 1024, LOG, CACHE>), dim3((unsigned)rows), dim3(1024), 0, s, (const T*)x, (T*)out, rows, dim);
       else
         TT_SM(256);
       break;
