@@ -49,6 +49,9 @@ CASES = [
     (7, 200, 128, "f16", False, "mfma"),         # ... a partial block of 32 columns
     (33, 96, 192, "bf16", True, "mfma"),         # ... two row blocks, the second nearly empty
     (64, 1536, 2048, "f16", True, "mfma"),
+    (5, 16384, 256, "bf16", True, "mfma"),       # ... many columns: two column blocks per workgroup
+    (40, 16420, 192, "f16", False, "mfma"),      # ... with both row blocks and a partial last pair of column blocks
+    (64, 20000, 128, "bf16", True, "mfma"),
     (2, 3, 5, "f32", True, "general"),
     (70, 90, 100, "f32", True, "general"),
     (129, 65, 200, "bf16", True, "general"),     # K not a multiple of 64

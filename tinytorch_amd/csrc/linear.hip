@@ -613,26 +613,30 @@ __global__ __launch_bounds__(256, 1) void linear256_kernel(LinArgs a) {
 // read back as MFMA operands, 16-byte chunk c of row r at slot c ^ ((r/2) % 8) (conflict-free b128 reads).  No
 // barriers inside the stream: a ring belongs to one wavefront.  out^T[n][m] accumulates with w as the A operand, so a
 // lane ends up with four consecutive n of one row m: 8-byte stores.
-template <int MB>
+template <int MB, int NB>
 struct Skinny {
-  static constexpr int NST = 3;                        // k-blocks of a wavefront in LDS
-  static constexpr int WT = 32 * 128;                  // bytes of a weight tile: 32 rows x 64 k
+  static constexpr int WT = NB * 32 * 128;             // bytes of a weight tile: NB x 32 rows x 64 k
   static constexpr int STG = WT + MB * 32 * 128;       // ... plus the x tile
-  static constexpr int LPB = 4 + 4 * MB;               // load instructions per k-block
+  static constexpr int NST = 4 * 3 * STG <= 160 * 1024 ? 3 : 2;  // k-blocks of a wavefront in LDS (what fits the CU's 160 KiB)
+  static constexpr int LPB = 4 * NB + 4 * MB;          // load instructions per k-block
   static constexpr int LDS = 4 * NST * STG;
-  static_assert(LDS >= 3 * MB * 16 * 64 * 4, "the partial sums of three wavefronts reuse the rings");
+  static_assert(LDS >= 3 * MB * NB * 16 * 64 * 4, "the partial sums of three wavefronts reuse the rings");
 };
 
-template <typename TR, int MB>  // MB = 32-row blocks of x: 1 (M <= 32) or 2 (M <= 64)
+// MB = 32-row blocks of x: 1 (M <= 32) or 2 (M <= 64).  NB = 32-column blocks of the output a workgroup owns: every x
+// tile a wavefront fetches (from L2) serves NB weight tiles (from memory), so the bytes a CU takes in per weight byte
+// fall from 1 + MB to 1 + MB / NB.  At M = 64 the kernel with NB = 1 is bound by what the L2s deliver (three bytes per
+// weight byte).
+template <typename TR, int MB, int NB>
 __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
   typedef typename TR::elem T;
   typedef typename TR::vec8 vec8;
-  typedef Skinny<MB> SK;
+  typedef Skinny<MB, NB> SK;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lq = lane & 31, lh = lane >> 5;
-  const long long n0 = (long long)blockIdx.x * 32;
+  const long long n0 = (long long)blockIdx.x * (32 * NB);
   char* ring = smem + wave * SK::NST * SK::STG;
   const unsigned ring_addr = (unsigned)(unsigned long)(lds_void_t*)ring;
 
@@ -640,13 +644,16 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
   };
   // this lane's part of a load instruction: row 8i + lane/8 of a tile, slot lane%8
-  unsigned woff[4], xoff[MB][4];
+  unsigned woff[NB][4], xoff[MB][4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int row = 8 * i + (lane >> 3);
     const unsigned chunk = (unsigned)((lane & 7) ^ ((row >> 1) & 7));
-    // columns past the end re-read the last weight row (not stored)
-    woff[i] = (unsigned)(((n0 + row < a.N ? row : (int)(a.N - 1 - n0)) * a.ldw + 8 * chunk) * 2);
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+      const long long n = n0 + 32 * nb + row;  // columns past the end re-read the last weight row (not stored)
+      woff[nb][i] = (unsigned)(((n < a.N ? n - n0 : a.N - 1 - n0) * a.ldw + 8 * chunk) * 2);
+    }
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
       const int m = 32 * mb + row;
@@ -660,7 +667,9 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
     const char* wk = wbase + kb * 128;
     const char* xk = xbase + kb * 128;
 #pragma unroll
-    for (int i = 0; i < 4; i++) dma16(wk, woff[i], at + 8 * i * 128);
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) dma16(wk, woff[nb][i], at + (32 * nb + 8 * i) * 128);
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
@@ -671,21 +680,24 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
 #pragma unroll
   for (int j = 0; j < 4; j++) rd[j] = (unsigned)(lq * 128 + 16 * ((4 * lh + j) ^ ((lq >> 1) & 7)));
 
-  f32x16 acc[MB];
+  f32x16 acc[NB][MB];
 #pragma unroll
-  for (int mb = 0; mb < MB; mb++)
+  for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[mb][r] = 0.f;
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[nb][mb][r] = 0.f;
   const long long nkb = a.K / 64;
-  const long long nb = nkb > wave ? (nkb - wave + 3) / 4 : 0;  // k-blocks of this wavefront: wave, wave + 4, ...
-  if (nb > 0) issue(wave, 0);
-  if (nb > 1) issue(wave + 4, 1);
+  const long long nb_ = nkb > wave ? (nkb - wave + 3) / 4 : 0;  // k-blocks of this wavefront: wave, wave + 4, ...
+  constexpr int AHEAD = SK::NST - 1;                             // k-blocks in flight beyond the one in use
+  for (int t = 0; t < AHEAD; t++)
+    if (nb_ > t) issue(wave + 4 * t, t);
   int cur = 0;
-  for (long long t = 0; t < nb; t++) {
-    const int nxt2 = cur == 0 ? 2 : cur - 1;  // (t + 2) % 3
-    if (t + 2 < nb) issue(wave + 4 * (t + 2), nxt2);
+  for (long long t = 0; t < nb_; t++) {
+    const int nxt = cur == 0 ? SK::NST - 1 : cur - 1;  // (t + AHEAD) % NST
+    if (t + AHEAD < nb_) issue(wave + 4 * (t + AHEAD), nxt);
     // block t has landed when only the loads of the blocks issued after it are outstanding
-    const long long later = nb - 1 - t < 2 ? nb - 1 - t : 2;
+    const long long later = nb_ - 1 - t < AHEAD ? nb_ - 1 - t : AHEAD;
     if (later == 2) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SK::LPB) : "memory");
     } else if (later == 1) {
@@ -697,60 +709,75 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a) {
     const char* xt = wt + SK::WT;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      const vec8 wv = *(const vec8*)(wt + rd[j]);
+      vec8 xv[MB];
 #pragma unroll
-      for (int mb = 0; mb < MB; mb++) acc[mb] = TR::mfma32(wv, *(const vec8*)(xt + mb * 32 * 128 + rd[j]), acc[mb]);
+      for (int mb = 0; mb < MB; mb++) xv[mb] = *(const vec8*)(xt + mb * 32 * 128 + rd[j]);
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        const vec8 wv = *(const vec8*)(wt + nb * 32 * 128 + rd[j]);
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) acc[nb][mb] = TR::mfma32(wv, xv[mb], acc[nb][mb]);
+      }
     }
-    cur = cur == 2 ? 0 : cur + 1;
+    cur = cur == SK::NST - 1 ? 0 : cur + 1;
   }
   __syncthreads();  // every ring is drained: the partial sums of wavefronts 1-3 take their place
   float* part = (float*)smem;
   if (wave > 0) {
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+    for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) part[(((wave - 1) * MB + mb) * 16 + r) * 64 + lane] = acc[mb][r];
+      for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) part[((((wave - 1) * NB + nb) * MB + mb) * 16 + r) * 64 + lane] = acc[nb][mb][r];
   }
   __syncthreads();
   if (wave != 0) return;
 #pragma unroll
-  for (int mb = 0; mb < MB; mb++) {
-    const long long m = 32 * mb + lq;
+  for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-    for (int rg = 0; rg < 4; rg++) {
-      const long long n = n0 + 8 * rg + 4 * lh;
-      f32x4 v;
+    for (int mb = 0; mb < MB; mb++) {
+      const long long m = 32 * mb + lq;
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int r = 4 * rg + i;
-        float sum = acc[mb][r];
+      for (int rg = 0; rg < 4; rg++) {
+        const long long n = n0 + 32 * nb + 8 * rg + 4 * lh;
+        f32x4 v;
 #pragma unroll
-        for (int w = 0; w < 3; w++) sum += part[((w * MB + mb) * 16 + r) * 64 + lane];
-        if (a.bias && n + i < a.N) sum += load_as_float((const T*)a.bias + n + i);
-        v[i] = sum;
-      }
-      if (m < a.M && n < a.N) {  // N is a multiple of 4 on this route: a group of four is inside or outside
-        *(typename TR::vec4*)((T*)a.out + m * a.ldo + n) = __builtin_convertvector(v, typename TR::vec4);
+        for (int i = 0; i < 4; i++) {
+          const int r = 4 * rg + i;
+          float sum = acc[nb][mb][r];
+#pragma unroll
+          for (int w = 0; w < 3; w++) sum += part[(((w * NB + nb) * MB + mb) * 16 + r) * 64 + lane];
+          if (a.bias && n + i < a.N) sum += load_as_float((const T*)a.bias + n + i);
+          v[i] = sum;
+        }
+        if (m < a.M && n < a.N) {  // N is a multiple of 4 on this route: a group of four is inside or outside
+          *(typename TR::vec4*)((T*)a.out + m * a.ldo + n) = __builtin_convertvector(v, typename TR::vec4);
+        }
       }
     }
-  }
 }
 
-template <typename TR, int MB>
+template <typename TR, int MB, int NB>
 int launch_skinny_mb(const LinArgs& a, hipStream_t stream) {
   static hipError_t state[kMaxDevices];
   static bool done[kMaxDevices];
-  const hipError_t granted = grant_dynamic_lds((const void*)linear_skinny_kernel<TR, MB>, Skinny<MB>::LDS, state, done);
+  constexpr int lds = Skinny<MB, NB>::LDS;
+  const hipError_t granted = grant_dynamic_lds((const void*)linear_skinny_kernel<TR, MB, NB>, lds, state, done);
   if (granted != hipSuccess) return (int)granted;
-  const long long nwg = (a.N + 31) / 32;
+  const long long nwg = (a.N + 32 * NB - 1) / (32 * NB);
   if (nwg > 0x7fffffffLL) return TTSDPA_ERR_SHAPE;
-  hipLaunchKernelGGL((linear_skinny_kernel<TR, MB>), dim3((unsigned)nwg), dim3(256), Skinny<MB>::LDS, stream, a);
+  hipLaunchKernelGGL((linear_skinny_kernel<TR, MB, NB>), dim3((unsigned)nwg), dim3(256), lds, stream, a);
   return (int)hipGetLastError();
 }
 
+// Two column blocks per workgroup once they still make a workgroup per CU (N >= 16384).  Weights beyond the last-level
+// cache, bf16, K = 4096: N = 28672 (an MLP's up projection) 3.9 -> 4.4 TB/s at M <= 8, 3.4 -> 4.3 at M = 32, 2.8 -> 3.5 at
+// M = 64; N = 6144 and 4096 (96 and 64 workgroups then) 3.0 -> 2.7 and 2.7 -> 2.4: those keep one block.
 template <typename TR>
 int launch_skinny(const LinArgs& a, hipStream_t stream) {
-  return a.M <= 32 ? launch_skinny_mb<TR, 1>(a, stream) : launch_skinny_mb<TR, 2>(a, stream);
+  if (a.N >= 16384) return a.M <= 32 ? launch_skinny_mb<TR, 1, 2>(a, stream) : launch_skinny_mb<TR, 2, 2>(a, stream);
+  return a.M <= 32 ? launch_skinny_mb<TR, 1, 1>(a, stream) : launch_skinny_mb<TR, 2, 1>(a, stream);
 }
 
 // Any element type and shape: 64 x 64 output tile per workgroup, 4 x 4 outputs per lane, K in steps of 16 through LDS.
