@@ -120,7 +120,12 @@ static void test_half_dtypes_and_gqa() {
   const Case cases[] = {{1, 8, 2, 160, 160, 128, true, DType::BFloat16},
                         {2, 4, 4, 96, 96, 128, true, DType::Float16},
                         {2, 8, 2, 1, 700, 128, false, DType::BFloat16},
-                        {1, 4, 2, 40, 56, 64, false, DType::Float32}};
+                        {1, 4, 2, 40, 56, 64, false, DType::Float32},
+                        // head sizes between the matrix-core kernels' own (the reference takes any): prefill, decode, fp32
+                        {1, 4, 2, 200, 200, 80, true, DType::BFloat16},
+                        {2, 8, 2, 1, 700, 96, false, DType::Float16},
+                        {1, 4, 2, 150, 90, 100, false, DType::Float32},
+                        {1, 2, 1, 33, 47, 20, true, DType::BFloat16}};
   for (const Case& c : cases) {
     std::vector<float> q = pseudoRandom(static_cast<size_t>(c.B) * c.Hq * c.L * c.D, 1);
     std::vector<float> k = pseudoRandom(static_cast<size_t>(c.B) * c.Hkv * c.S * c.D, 2);
