@@ -717,6 +717,15 @@ def main():
         summary["backward_f32"] = line["backward"]["fp32"]["roofline"]["frac"]
     if summary:  # fraction of its own roofline for every other line of this run (config1: launch-sized, its kernel ms)
         line["roofline"]["summary"] = summary
+    # said once, in the headline's roofline object: how every line is timed; the secondary line's figures sit in roofline.decode
+    for other in [line.get("secondary"), line.get("fp32")] + list(line.get("other_configs", [])):
+        if other:
+            for key in ("timing", "kernel_ms_mean", "kernel_ms_min"):
+                other["roofline"].pop(key, None)
+    if "decode" in line["roofline"] and "secondary" in line:
+        line["secondary"] = {"workload": line["secondary"]["workload"], "route": line["secondary"]["route"],
+                             "ms_per_step": line["secondary"]["ms_per_step"], "value": line["secondary"]["value"],
+                             "unit": line["secondary"]["unit"], "roofline": "see roofline.decode of the headline"}
     # the figures the metric is quoted on once more as the line's last key: a record that keeps only the end of a
     # long line still holds them
     r = line["roofline"]
