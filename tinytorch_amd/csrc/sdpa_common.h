@@ -201,13 +201,16 @@ struct BwdArgs {
 // measured 1 % slower, 13-20 % with an attnMask).  A split must still get a few tiles.  `groups`: wavefront groups
 // that already share a key block inside a workgroup (2 in the 16-bit head_dim-128 kernel, where splitting 512
 // workgroups of a causal call further measured 4 % slower, 256 of them 7-21 % faster).
-// `per_cu`: workgroups of the kernel that fit a CU (2 at head_dim 64 without an attnMask, else 1); it counts for calls
-// without a causal mask only (head_dim 64, 256 equal workgroups: two splits +28 %; causal with 512: four splits instead
-// of two -2 to -5 %).
+// `per_cu`: workgroups of the kernel that fit a CU (2 at head_dim 64 without an attnMask, else 1): head_dim 64, 256 equal
+// workgroups without a causal mask: two splits +28 %; causal with 512: four splits instead of two -2 to -5 %.
 inline int backward_dkv_splits(int B, int Hkv, int Hq, int L, int S, bool causal, int groups, int per_cu) {
   const long long wgs = (long long)B * Hkv * ((S + 127) / 128) * groups;
   const long long tiles = (long long)(Hq / Hkv) * ((L + 31) / 32) / groups;  // the longest query stream, in 32-row tiles
-  const long long enough = causal ? 1024 : 256 * per_cu;
+  // causal: two rounds of the workgroups a CU holds at a time (one for the 8-wavefront head_dim-128 kernel, whose two
+  // groups make `wgs` count double, and for the fp32 head_dim-128 kernel; two at head_dim 64).  fp32 head_dim 128, 512
+  // workgroups (B2 32q/8kv 4096 x 4096): splitting them in two measured the same time, 60 % more bytes read and a
+  // third kernel for the partial sums; 256 of them (2048 x 2048) two splits 76.5, four 74.1 TFLOP/s.
+  const long long enough = causal ? 512LL * per_cu * groups : 256 * per_cu;
   int n = 1;
   while (n < 4 && wgs * n < enough && tiles >= 16 * n) n *= 2;
   return n;
